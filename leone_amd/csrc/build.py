@@ -1,0 +1,142 @@
+"""Builds the gfx950 kernel library from the sources in this folder.
+
+``hipcc`` cross-compiles without a GPU.  Objects and the shared library go to
+``_build/`` beside the sources; if that folder cannot be written (a read-only
+checkout) a per-user folder under the system's temporary directory is used.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libleone_hip.so"
+ARCH = "gfx950"
+# Packed single-precision instructions are kept off for every device function.
+DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Wno-unused-result"] + DEVICE_FLAGS
+
+
+def sources() -> list[str]:
+    return sorted(f for f in os.listdir(HERE) if f.endswith(".hip"))
+
+
+def _headers() -> list[str]:
+    return sorted(f for f in os.listdir(HERE) if f.endswith(".h"))
+
+
+def source_digest() -> str:
+    digest = hashlib.sha256()
+    for name in sources() + _headers():
+        digest.update(name.encode())
+        with open(os.path.join(HERE, name), "rb") as handle:
+            digest.update(handle.read())
+    digest.update(" ".join(FLAGS).encode())
+    return digest.hexdigest()[:16]
+
+
+def _writable(path: str) -> bool:
+    try:
+        os.makedirs(path, exist_ok=True)
+        probe = os.path.join(path, f".probe{os.getpid()}")
+        with open(probe, "w"):
+            pass
+        os.remove(probe)
+        return True
+    except OSError:
+        return False
+
+
+def build_dir() -> str:
+    in_tree = os.path.join(HERE, "_build")
+    if _writable(in_tree):
+        return in_tree
+    fallback = os.path.join(tempfile.gettempdir(), f"leone_amd_build_{os.getuid()}")
+    os.makedirs(fallback, exist_ok=True)
+    return fallback
+
+
+def library_path() -> str | None:
+    """The built library that matches the present sources, if there is one."""
+    digest = source_digest()
+    for folder in (os.path.join(HERE, "_build"),
+                   os.path.join(tempfile.gettempdir(), f"leone_amd_build_{os.getuid()}")):
+        lib = os.path.join(folder, LIB_NAME)
+        stamp = os.path.join(folder, "digest.txt")
+        if os.path.exists(lib) and os.path.exists(stamp):
+            with open(stamp) as handle:
+                if handle.read().strip() == digest:
+                    return lib
+    return None
+
+
+def hipcc() -> str:
+    found = shutil.which("hipcc")
+    if found:
+        return found
+    candidate = "/opt/rocm/bin/hipcc"
+    if os.path.exists(candidate):
+        return candidate
+    raise RuntimeError("hipcc not found: the kernel library cannot be built")
+
+
+def build(verbose: bool = True, force: bool = True) -> str:
+    """Compiles every source and links the library; returns its path."""
+    if not force:
+        ready = library_path()
+        if ready:
+            return ready
+    out_dir = build_dir()
+    compiler = hipcc()
+    names = sources()
+    started = time.time()
+    done = threading.Event()
+
+    def heartbeat():
+        while not done.wait(10.0):
+            if verbose:
+                print(f"[leone_amd] compiling kernels for {ARCH} ... {time.time() - started:.0f}s",
+                      file=sys.stderr, flush=True)
+
+    def compile_one(name: str) -> str:
+        obj = os.path.join(out_dir, name[:-4] + ".o")
+        cmd = [compiler] + FLAGS + ["-I", HERE, "-c", os.path.join(HERE, name), "-o", obj]
+        result = subprocess.run(cmd, capture_output=True, text=True)
+        if result.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {name}:\n{result.stderr}")
+        return obj
+
+    if verbose:
+        print(f"[leone_amd] building {LIB_NAME} from {len(names)} sources into {out_dir}",
+              file=sys.stderr, flush=True)
+    ticker = threading.Thread(target=heartbeat, daemon=True)
+    ticker.start()
+    try:
+        workers = max(1, min(len(names), int(os.environ.get("MAX_JOBS", "8")), 16))
+        with ThreadPoolExecutor(max_workers=workers) as pool:
+            objects = list(pool.map(compile_one, names))
+        lib = os.path.join(out_dir, LIB_NAME)
+        tmp = lib + f".tmp{os.getpid()}"
+        link = [compiler, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp] + objects
+        result = subprocess.run(link, capture_output=True, text=True)
+        if result.returncode != 0:
+            raise RuntimeError(f"hipcc failed to link {LIB_NAME}:\n{result.stderr}")
+        os.replace(tmp, lib)
+        with open(os.path.join(out_dir, "digest.txt"), "w") as handle:
+            handle.write(source_digest() + "\n")
+    finally:
+        done.set()
+    if verbose:
+        print(f"[leone_amd] built {lib} in {time.time() - started:.0f}s", file=sys.stderr, flush=True)
+    return lib
+
+
+if __name__ == "__main__":
+    print(build())

@@ -1,0 +1,120 @@
+// Shared helpers for the gfx950 kernels: storage types, conversions, wave
+// reductions and the error channel of the C entry points.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+namespace leone {
+
+// Element types as passed over the C boundary.
+enum DType : int { kF32 = 0, kBF16 = 1 };
+
+constexpr int kWave = 64;
+
+// bfloat16 is carried as its 16 bits; all arithmetic is done in float.
+struct bf16_t {
+    uint16_t bits;
+};
+
+__host__ __device__ inline float to_float(float v) { return v; }
+__host__ __device__ inline float to_float(bf16_t v) {
+    union {
+        uint32_t u;
+        float f;
+    } c;
+    c.u = static_cast<uint32_t>(v.bits) << 16;
+    return c.f;
+}
+
+// Round to nearest even; NaN stays NaN.
+__host__ __device__ inline uint16_t bf16_bits_from_float(float f) {
+    union {
+        uint32_t u;
+        float f;
+    } c;
+    c.f = f;
+    uint32_t u = c.u;
+    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+
+template <typename T>
+__host__ __device__ inline T from_float(float f);
+template <>
+__host__ __device__ inline float from_float<float>(float f) {
+    return f;
+}
+template <>
+__host__ __device__ inline bf16_t from_float<bf16_t>(float f) {
+    bf16_t r;
+    r.bits = bf16_bits_from_float(f);
+    return r;
+}
+
+// A gain or table vector that may be stored in either type.
+struct AnyVec {
+    const void* ptr;
+    int dtype;
+};
+__device__ inline float load_any(const AnyVec& v, long i) {
+    return v.dtype == kF32 ? static_cast<const float*>(v.ptr)[i]
+                           : to_float(static_cast<const bf16_t*>(v.ptr)[i]);
+}
+
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// Sum over a block of kThreads (a multiple of 64, at most 1024); every thread
+// gets the result.  `scratch` holds at least kThreads/64 floats.  The order of
+// the additions is fixed, so a launch repeats bit for bit.
+template <int kThreads>
+__device__ inline float block_sum(float v, float* scratch) {
+    v = wave_sum(v);
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < kThreads / kWave; ++w) total += scratch[w];
+    return total;
+}
+
+// ---- error channel -------------------------------------------------------
+// Every entry point returns 0 on success.  On failure it returns nonzero and
+// leaves a message that leone_last_error() hands out.
+void set_error(const char* fmt, ...);
+
+#define LEONE_REQUIRE(cond, ...)          \
+    do {                                  \
+        if (!(cond)) {                    \
+            leone::set_error(__VA_ARGS__); \
+            return 1;                     \
+        }                                 \
+    } while (0)
+
+#define LEONE_LAUNCH_CHECK(name)                                                      \
+    do {                                                                              \
+        hipError_t e_ = hipGetLastError();                                            \
+        if (e_ != hipSuccess) {                                                       \
+            leone::set_error("%s: launch failed: %s", name, hipGetErrorString(e_));   \
+            return 2;                                                                 \
+        }                                                                             \
+    } while (0)
+
+inline int ceil_div(long a, long b) { return static_cast<int>((a + b - 1) / b); }
+
+}  // namespace leone

@@ -1,0 +1,51 @@
+// C entry points of the gfx950 kernel library.  Every function returns 0 on
+// success; otherwise leone_last_error() describes what was refused.  Pointers
+// are device pointers unless said otherwise; `dtype` arguments are 0 for
+// float and 1 for bfloat16.  All work is queued on `stream`.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+extern "C" {
+
+const char* leone_last_error();
+int leone_library_version();
+
+// out[r, :] = table[tokens[r], :] widened to float.
+int leone_embed(const void* table, int dtype, const int* tokens, float* out, int rows, int hidden, int vocab,
+                hipStream_t stream);
+
+// x += delta (delta may be null); y = rmsnorm(x) * gain.  With `rows` given,
+// y[r] is computed from row rows[r] and x is not written.
+int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, const void* gain, int gain_dtype, float eps,
+                      void* y, int y_dtype, const int* rows, int n_rows, int hidden, hipStream_t stream);
+
+// out[r, c] = silu(gate_up[r, c]) * gate_up[r, ffn + c].
+int leone_swiglu(const void* gate_up, void* out, int dtype, int rows, int ffn, hipStream_t stream);
+
+// cos/sin[pos, i] of pos * theta^(-2i/rotary_dim), for pos < positions.
+int leone_rope_table(float* cos_out, float* sin_out, double theta, int rotary_dim, int positions,
+                     hipStream_t stream);
+
+// Per-head RMSNorm (gains may be null), half-split rotation (tables may be
+// null), q to q_out, k and v into the paged cache.
+int leone_qk_norm_rope_write(const void* qkv, void* q_out, void* k_pool, void* v_pool, int dtype,
+                             const void* q_gain, const void* k_gain, int gain_dtype, float eps,
+                             const float* cos_table, const float* sin_table, int table_positions,
+                             const int* positions, const int* row_entry, const int* block_table, int max_blocks,
+                             int rows, int q_heads, int kv_heads, int head_dim, int page_tokens, int write_cache,
+                             hipStream_t stream);
+
+// Attention of each query row over its request's cached keys [first, pos].
+int leone_attention_rows(const void* q, void* out, const void* k_pool, const void* v_pool, int dtype,
+                         const int* positions, const int* row_entry, const int* block_table, int max_blocks,
+                         int rows, int q_heads, int kv_heads, int head_dim, int page_tokens, float scale,
+                         int window, hipStream_t stream);
+
+// C[M,N] = A[M,K] . B[N,K]^T in float.
+int leone_gemm_f32(const float* a, const float* b, float* c, int m, int n, int k, hipStream_t stream);
+
+int leone_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream);
+int leone_sample_temperature(const float* logits, const double* temperature, const double* uniform, int* out,
+                             int rows, int vocab, hipStream_t stream);
+}

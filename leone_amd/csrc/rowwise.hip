@@ -1,0 +1,309 @@
+// Row-wise kernels: embedding gather, residual-add + RMSNorm, SwiGLU, the
+// rotary table, and the fused per-head norm + rotation + cache write.
+//
+// Formulas follow the reference's scalar backend: RMSNorm
+// y = (x * w) * rsqrt(mean(x^2) + eps) (crates/leone/src/cpu.rs:1642-1663),
+// half-split rotary pairs (i, i + D/2) with inverse frequency theta^(-2i/D)
+// (crates/leone/src/cpu.rs:1721-1779), SwiGLU g / (1 + exp(-g)) * u
+// (crates/leone/src/cpu.rs:892-907).  Sums of squares, gains and rotations are
+// computed in float whatever the storage type; rotary angles in double.
+#include "common.h"
+#include "leone_hip.h"
+
+namespace leone {
+
+// ---- embedding -------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
+                             float* __restrict__ out, int hidden, int vocab) {
+    const int row = blockIdx.x;
+    const int token = tokens[row];
+    float* dst = out + static_cast<long>(row) * hidden;
+    if (token < 0 || token >= vocab) {
+        // The host rejects such ids before the launch; never read outside the table.
+        for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = __builtin_nanf("");
+        return;
+    }
+    const T* src = table + static_cast<long>(token) * hidden;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = to_float(src[c]);
+}
+
+// ---- residual add + RMSNorm -------------------------------------------------
+// One block per output row.  With `rows` == nullptr row r of `x` is updated in
+// place (x += delta) and normalised into y[r].  With `rows` given, output row r
+// reads x[rows[r]] (+ delta[rows[r]]) and x is left untouched.
+template <typename TD, typename TY, int kThreads>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                   AnyVec gain, float eps, TY* __restrict__ y,
+                                   const int* __restrict__ rows, int hidden) {
+    __shared__ float scratch[kThreads / kWave];
+    const int out_row = blockIdx.x;
+    const long in_row = rows ? rows[out_row] : out_row;
+    float* xr = x + in_row * hidden;
+    const TD* dr = delta ? delta + in_row * hidden : nullptr;
+    TY* yr = y + static_cast<long>(out_row) * hidden;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < hidden; c += kThreads) {
+        float v = xr[c];
+        if (dr) {
+            v += to_float(dr[c]);
+            if (!rows) xr[c] = v;
+        }
+        ss = fmaf(v, v, ss);
+    }
+    const float total = block_sum<kThreads>(ss, scratch);
+    const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+    for (int c = threadIdx.x; c < hidden; c += kThreads) {
+        float v = xr[c];
+        if (dr && rows) v += to_float(dr[c]);
+        yr[c] = from_float<TY>((v * load_any(gain, c)) * inv);
+    }
+}
+
+// ---- SwiGLU -------------------------------------------------------------------
+// in: [rows, 2F] with the gate in the first F columns, up in the last F.
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long rows, int ffn) {
+    const long total = rows * ffn;
+    for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < total;
+         i += static_cast<long>(gridDim.x) * blockDim.x) {
+        const long r = i / ffn;
+        const int c = static_cast<int>(i - r * ffn);
+        const float g = to_float(gate_up[r * 2 * ffn + c]);
+        const float u = to_float(gate_up[r * 2 * ffn + ffn + c]);
+        out[i] = from_float<T>((g / (1.0f + expf(-g))) * u);
+    }
+}
+
+// ---- rotary table ----------------------------------------------------------------
+// cos/sin of pos * theta^(-2i/D), evaluated in double and stored as float
+// (the reference's device table, crates/leone-cuda/cuda/ie_cuda.cu:2383-2401).
+__global__ void rope_table_kernel(float* __restrict__ cos_out, float* __restrict__ sin_out,
+                                  double theta, int pairs, int rotary_dim, int positions) {
+    const long total = static_cast<long>(positions) * pairs;
+    for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < total;
+         i += static_cast<long>(gridDim.x) * blockDim.x) {
+        const int pos = static_cast<int>(i / pairs);
+        const int p = static_cast<int>(i % pairs);
+        const double inv = pow(theta, -2.0 * static_cast<double>(p) / static_cast<double>(rotary_dim));
+        const double angle = static_cast<double>(pos) * inv;
+        cos_out[i] = static_cast<float>(cos(angle));
+        sin_out[i] = static_cast<float>(sin(angle));
+    }
+}
+
+// ---- per-head norm + rotation + cache write ------------------------------------------
+// One wave per (row, head) of the fused projection output
+// qkv[row] = [q heads | k heads | v heads], each head of D elements.
+//   q heads: optional RMSNorm over D, optional rotation, written to q_out.
+//   k heads: the same, written into the request's page at `position`.
+//   v heads: copied into the page unchanged.
+// A lane owns pairs p = lane, lane + 64, ... (p < D/2): elements p and p + D/2.
+// When `write_cache` is 0 the k and v heads are skipped (a layer that reads
+// another layer's cache).
+constexpr int kMaxPairsPerLane = 4;  // head_dim up to 512
+
+template <typename T>
+__global__ void qk_norm_rope_write_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_pool, T* __restrict__ v_pool,
+    AnyVec q_gain, AnyVec k_gain, float eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, int table_positions, const int* __restrict__ positions,
+    const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
+    int q_heads, int kv_heads, int head_dim, int page_tokens, int write_cache) {
+    const int row = blockIdx.x;
+    const int head = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    const int heads_total = q_heads + (write_cache ? 2 * kv_heads : 0);
+    if (head >= heads_total) return;
+    const int half = head_dim / 2;
+    const int qkv_width = (q_heads + 2 * kv_heads) * head_dim;
+    const T* src = qkv + static_cast<long>(row) * qkv_width + static_cast<long>(head) * head_dim;
+    const int pos = positions[row];
+
+    const bool is_q = head < q_heads;
+    const bool is_k = !is_q && head < q_heads + kv_heads;
+    T* dst;
+    if (is_q) {
+        dst = q_out + (static_cast<long>(row) * q_heads + head) * head_dim;
+    } else {
+        const int kvh = is_k ? head - q_heads : head - q_heads - kv_heads;
+        const int page = block_table[static_cast<long>(row_entry[row]) * max_blocks + pos / page_tokens];
+        if (page < 0) return;  // host reserves pages before the launch
+        const long slot = ((static_cast<long>(page) * kv_heads + kvh) * page_tokens + pos % page_tokens) * head_dim;
+        dst = (is_k ? k_pool : v_pool) + slot;
+    }
+
+    float a[kMaxPairsPerLane], b[kMaxPairsPerLane];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxPairsPerLane; ++i) {
+        const int p = lane + i * kWave;
+        if (p < half) {
+            a[i] = to_float(src[p]);
+            b[i] = to_float(src[p + half]);
+            ss = fmaf(a[i], a[i], ss);
+            ss = fmaf(b[i], b[i], ss);
+        }
+    }
+    if (!is_q && !is_k) {  // value head: plain copy
+#pragma unroll
+        for (int i = 0; i < kMaxPairsPerLane; ++i) {
+            const int p = lane + i * kWave;
+            if (p < half) {
+                dst[p] = from_float<T>(a[i]);
+                dst[p + half] = from_float<T>(b[i]);
+            }
+        }
+        return;
+    }
+    const AnyVec gain = is_q ? q_gain : k_gain;
+    float inv = 1.f;
+    if (gain.ptr) {
+        ss = wave_sum(ss);
+        inv = 1.0f / sqrtf(ss / static_cast<float>(head_dim) + eps);
+    }
+    const bool rotate = cos_table != nullptr;
+    const int tpos = pos < table_positions ? pos : table_positions - 1;  // host checks the bound
+#pragma unroll
+    for (int i = 0; i < kMaxPairsPerLane; ++i) {
+        const int p = lane + i * kWave;
+        if (p < half) {
+            float u = a[i], v = b[i];
+            if (gain.ptr) {
+                u = (u * load_any(gain, p)) * inv;
+                v = (v * load_any(gain, p + half)) * inv;
+            }
+            if (rotate) {
+                const float c = cos_table[static_cast<long>(tpos) * half + p];
+                const float s = sin_table[static_cast<long>(tpos) * half + p];
+                const float ru = u * c - v * s;
+                const float rv = u * s + v * c;
+                u = ru;
+                v = rv;
+            }
+            dst[p] = from_float<T>(u);
+            dst[p + half] = from_float<T>(v);
+        }
+    }
+}
+
+static int check_dtype(int dtype, const char* what) {
+    if (dtype != kF32 && dtype != kBF16) {
+        set_error("%s: unknown element type %d", what, dtype);
+        return 1;
+    }
+    return 0;
+}
+
+}  // namespace leone
+
+using namespace leone;
+
+extern "C" int leone_embed(const void* table, int dtype, const int* tokens, float* out, int rows,
+                           int hidden, int vocab, hipStream_t stream) {
+    if (check_dtype(dtype, "embed")) return 1;
+    LEONE_REQUIRE(table && tokens && out, "embed: null pointer");
+    LEONE_REQUIRE(rows > 0 && hidden > 0 && vocab > 0, "embed: rows %d hidden %d vocab %d must be positive", rows, hidden, vocab);
+    const int threads = hidden >= 1024 ? 256 : 64;
+    if (dtype == kF32)
+        embed_kernel<float><<<rows, threads, 0, stream>>>(static_cast<const float*>(table), tokens, out, hidden, vocab);
+    else
+        embed_kernel<bf16_t><<<rows, threads, 0, stream>>>(static_cast<const bf16_t*>(table), tokens, out, hidden, vocab);
+    LEONE_LAUNCH_CHECK("embed");
+    return 0;
+}
+
+template <typename TD, typename TY>
+static void launch_add_rmsnorm(float* x, const void* delta, AnyVec gain, float eps, void* y,
+                               const int* rows, int n_rows, int hidden, hipStream_t stream) {
+    if (hidden > 512)
+        add_rmsnorm_kernel<TD, TY, 256><<<n_rows, 256, 0, stream>>>(x, static_cast<const TD*>(delta), gain, eps, static_cast<TY*>(y), rows, hidden);
+    else
+        add_rmsnorm_kernel<TD, TY, 64><<<n_rows, 64, 0, stream>>>(x, static_cast<const TD*>(delta), gain, eps, static_cast<TY*>(y), rows, hidden);
+}
+
+extern "C" int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, const void* gain,
+                                 int gain_dtype, float eps, void* y, int y_dtype, const int* rows,
+                                 int n_rows, int hidden, hipStream_t stream) {
+    if (check_dtype(delta_dtype, "add_rmsnorm delta") || check_dtype(gain_dtype, "add_rmsnorm gain") ||
+        check_dtype(y_dtype, "add_rmsnorm output"))
+        return 1;
+    LEONE_REQUIRE(x && gain && y, "add_rmsnorm: null pointer");
+    LEONE_REQUIRE(n_rows > 0 && hidden > 0, "add_rmsnorm: rows %d hidden %d must be positive", n_rows, hidden);
+    LEONE_REQUIRE(eps > 0.f && eps == eps, "add_rmsnorm: eps must be positive");
+    AnyVec g{gain, gain_dtype};
+    if (delta_dtype == kF32 && y_dtype == kF32)
+        launch_add_rmsnorm<float, float>(x, delta, g, eps, y, rows, n_rows, hidden, stream);
+    else if (delta_dtype == kBF16 && y_dtype == kBF16)
+        launch_add_rmsnorm<bf16_t, bf16_t>(x, delta, g, eps, y, rows, n_rows, hidden, stream);
+    else if (delta_dtype == kF32 && y_dtype == kBF16)
+        launch_add_rmsnorm<float, bf16_t>(x, delta, g, eps, y, rows, n_rows, hidden, stream);
+    else
+        launch_add_rmsnorm<bf16_t, float>(x, delta, g, eps, y, rows, n_rows, hidden, stream);
+    LEONE_LAUNCH_CHECK("add_rmsnorm");
+    return 0;
+}
+
+extern "C" int leone_swiglu(const void* gate_up, void* out, int dtype, int rows, int ffn, hipStream_t stream) {
+    if (check_dtype(dtype, "swiglu")) return 1;
+    LEONE_REQUIRE(gate_up && out, "swiglu: null pointer");
+    LEONE_REQUIRE(rows > 0 && ffn > 0, "swiglu: rows %d width %d must be positive", rows, ffn);
+    const long total = static_cast<long>(rows) * ffn;
+    long blocks = (total + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    if (dtype == kF32)
+        swiglu_kernel<float><<<static_cast<int>(blocks), 256, 0, stream>>>(static_cast<const float*>(gate_up), static_cast<float*>(out), rows, ffn);
+    else
+        swiglu_kernel<bf16_t><<<static_cast<int>(blocks), 256, 0, stream>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out), rows, ffn);
+    LEONE_LAUNCH_CHECK("swiglu");
+    return 0;
+}
+
+extern "C" int leone_rope_table(float* cos_out, float* sin_out, double theta, int rotary_dim,
+                                int positions, hipStream_t stream) {
+    LEONE_REQUIRE(cos_out && sin_out, "rope_table: null pointer");
+    LEONE_REQUIRE(rotary_dim > 0 && rotary_dim % 2 == 0, "rope_table: rotary dim %d must be even and positive", rotary_dim);
+    LEONE_REQUIRE(positions > 0, "rope_table: positions %d must be positive", positions);
+    LEONE_REQUIRE(theta > 0.0 && theta == theta, "rope_table: theta must be positive");
+    const int pairs = rotary_dim / 2;
+    const long total = static_cast<long>(positions) * pairs;
+    long blocks = (total + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    rope_table_kernel<<<static_cast<int>(blocks), 256, 0, stream>>>(cos_out, sin_out, theta, pairs, rotary_dim, positions);
+    LEONE_LAUNCH_CHECK("rope_table");
+    return 0;
+}
+
+extern "C" int leone_qk_norm_rope_write(const void* qkv, void* q_out, void* k_pool, void* v_pool, int dtype,
+                                        const void* q_gain, const void* k_gain, int gain_dtype, float eps,
+                                        const float* cos_table, const float* sin_table, int table_positions,
+                                        const int* positions, const int* row_entry, const int* block_table,
+                                        int max_blocks, int rows, int q_heads, int kv_heads, int head_dim,
+                                        int page_tokens, int write_cache, hipStream_t stream) {
+    if (check_dtype(dtype, "qk_norm_rope_write") || check_dtype(gain_dtype, "qk_norm_rope_write gain")) return 1;
+    LEONE_REQUIRE(qkv && q_out && positions, "qk_norm_rope_write: null pointer");
+    LEONE_REQUIRE(!write_cache || (k_pool && v_pool && row_entry && block_table && max_blocks > 0 && page_tokens > 0),
+                  "qk_norm_rope_write: cache write needs pools, row map and block table");
+    LEONE_REQUIRE((q_gain == nullptr) == (k_gain == nullptr), "qk_norm_rope_write: q and k gains come together");
+    LEONE_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "qk_norm_rope_write: cos and sin tables come together");
+    LEONE_REQUIRE(!cos_table || table_positions > 0, "qk_norm_rope_write: empty rotary table");
+    LEONE_REQUIRE(rows > 0 && q_heads > 0 && kv_heads > 0, "qk_norm_rope_write: rows %d heads %d/%d must be positive", rows, q_heads, kv_heads);
+    LEONE_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= 2 * kWave * kMaxPairsPerLane,
+                  "qk_norm_rope_write: head_dim %d must be even and at most %d", head_dim, 2 * kWave * kMaxPairsPerLane);
+    const int heads_total = q_heads + (write_cache ? 2 * kv_heads : 0);
+    const int waves_per_block = 4;
+    dim3 grid(rows, ceil_div(heads_total, waves_per_block));
+    AnyVec qg{q_gain, gain_dtype}, kg{k_gain, gain_dtype};
+    if (dtype == kF32)
+        qk_norm_rope_write_kernel<float><<<grid, waves_per_block * kWave, 0, stream>>>(
+            static_cast<const float*>(qkv), static_cast<float*>(q_out), static_cast<float*>(k_pool),
+            static_cast<float*>(v_pool), qg, kg, eps, cos_table, sin_table, table_positions, positions, row_entry,
+            block_table, max_blocks, q_heads, kv_heads, head_dim, page_tokens, write_cache);
+    else
+        qk_norm_rope_write_kernel<bf16_t><<<grid, waves_per_block * kWave, 0, stream>>>(
+            static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(q_out), static_cast<bf16_t*>(k_pool),
+            static_cast<bf16_t*>(v_pool), qg, kg, eps, cos_table, sin_table, table_positions, positions, row_entry,
+            block_table, max_blocks, q_heads, kv_heads, head_dim, page_tokens, write_cache);
+    LEONE_LAUNCH_CHECK("qk_norm_rope_write");
+    return 0;
+}

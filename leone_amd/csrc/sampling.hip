@@ -1,0 +1,160 @@
+// Token selection on the device.
+//
+// argmax: the highest finite logit, the lowest index on a tie; NaN and
+// infinities never win; a row without a finite value yields -1
+// (crates/leone/src/sampler.rs:787-799, crates/leone/src/cpu.rs:1341-1362).
+// temperature: weights exp(l/t - max/t) over the finite logits in double,
+// the token is the first, in id order, whose running share exceeds the given
+// uniform value; the last eligible token if rounding leaves none
+// (crates/leone/src/sampler.rs:502-534, 843-858).
+#include "common.h"
+#include "leone_hip.h"
+
+#include <math.h>
+
+namespace leone {
+
+constexpr int kSampleThreads = 1024;
+
+struct Best {
+    float value;
+    int index;
+};
+
+__device__ inline Best better(Best a, Best b) {
+    if (b.index < 0) return a;
+    if (a.index < 0) return b;
+    if (b.value > a.value || (b.value == a.value && b.index < a.index)) return b;
+    return a;
+}
+
+__device__ inline Best block_best(Best mine, Best* scratch) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        Best other;
+        other.value = __shfl_xor(mine.value, off, kWave);
+        other.index = __shfl_xor(mine.index, off, kWave);
+        mine = better(mine, other);
+    }
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = mine;
+    __syncthreads();
+    Best total = scratch[0];
+    for (int w = 1; w < kSampleThreads / kWave; ++w) total = better(total, scratch[w]);
+    return total;
+}
+
+__global__ void __launch_bounds__(kSampleThreads)
+argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
+    __shared__ Best scratch[kSampleThreads / kWave];
+    const float* row = logits + static_cast<long>(blockIdx.x) * vocab;
+    Best mine{0.f, -1};
+    for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
+        const float v = row[i];
+        if (!isfinite(v)) continue;
+        if (mine.index < 0 || v > mine.value) mine = Best{v, i};
+    }
+    const Best total = block_best(mine, scratch);
+    if (threadIdx.x == 0) out[blockIdx.x] = total.index;
+}
+
+// Thread t owns the ids [t * chunk, (t + 1) * chunk): running sums follow id order.
+__global__ void __launch_bounds__(kSampleThreads)
+sample_temperature_kernel(const float* __restrict__ logits, const double* __restrict__ temperature,
+                          const double* __restrict__ uniform, int* __restrict__ out, int vocab) {
+    __shared__ Best scratch[kSampleThreads / kWave];
+    __shared__ double sums[kSampleThreads];
+    __shared__ int last_finite[kSampleThreads];
+    __shared__ int chosen_thread;
+    __shared__ double chosen_before, target;
+
+    const float* row = logits + static_cast<long>(blockIdx.x) * vocab;
+    const double t = temperature[blockIdx.x];
+    const int chunk = (vocab + kSampleThreads - 1) / kSampleThreads;
+    const int begin = threadIdx.x * chunk;
+    const int end = begin + chunk < vocab ? begin + chunk : vocab;
+
+    Best mine{0.f, -1};
+    int last = -1;
+    for (int i = begin; i < end; ++i) {
+        const float v = row[i];
+        if (!isfinite(v)) continue;
+        last = i;
+        if (mine.index < 0 || v > mine.value) mine = Best{v, i};
+    }
+    const Best top = block_best(mine, scratch);
+    if (top.index < 0) {
+        if (threadIdx.x == 0) out[blockIdx.x] = -1;
+        return;
+    }
+    const double highest = static_cast<double>(top.value) / t;
+    double sum = 0.0;
+    for (int i = begin; i < end; ++i) {
+        const float v = row[i];
+        if (isfinite(v)) sum += exp(static_cast<double>(v) / t - highest);
+    }
+    sums[threadIdx.x] = sum;
+    last_finite[threadIdx.x] = last;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double total = 0.0;
+        for (int i = 0; i < kSampleThreads; ++i) total += sums[i];
+        target = uniform[blockIdx.x] * total;
+        double running = 0.0;
+        int pick = -1;
+        for (int i = 0; i < kSampleThreads; ++i) {
+            if (sums[i] > 0.0 && target < running + sums[i]) {
+                pick = i;
+                break;
+            }
+            running += sums[i];
+        }
+        chosen_thread = pick;
+        chosen_before = running;
+        if (pick < 0) {  // rounding left the running sum short: the last eligible token
+            int fallback = -1;
+            for (int i = 0; i < kSampleThreads; ++i)
+                if (last_finite[i] > fallback) fallback = last_finite[i];
+            out[blockIdx.x] = fallback;
+        }
+    }
+    __syncthreads();
+    if (static_cast<int>(threadIdx.x) == chosen_thread) {
+        double running = chosen_before;
+        int token = last;
+        for (int i = begin; i < end; ++i) {
+            const float v = row[i];
+            if (!isfinite(v)) continue;
+            const double w = exp(static_cast<double>(v) / t - highest);
+            if (w <= 0.0) continue;
+            running += w;
+            if (target < running) {
+                token = i;
+                break;
+            }
+        }
+        out[blockIdx.x] = token;
+    }
+}
+
+}  // namespace leone
+
+using namespace leone;
+
+extern "C" int leone_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+    LEONE_REQUIRE(logits && out, "argmax: null pointer");
+    LEONE_REQUIRE(rows > 0 && vocab > 0, "argmax: rows %d vocab %d must be positive", rows, vocab);
+    argmax_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, out, vocab);
+    LEONE_LAUNCH_CHECK("argmax");
+    return 0;
+}
+
+extern "C" int leone_sample_temperature(const float* logits, const double* temperature, const double* uniform,
+                                        int* out, int rows, int vocab, hipStream_t stream) {
+    LEONE_REQUIRE(logits && temperature && uniform && out, "sample_temperature: null pointer");
+    LEONE_REQUIRE(rows > 0 && vocab > 0, "sample_temperature: rows %d vocab %d must be positive", rows, vocab);
+    sample_temperature_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, temperature, uniform, out, vocab);
+    LEONE_LAUNCH_CHECK("sample_temperature");
+    return 0;
+}

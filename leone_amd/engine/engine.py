@@ -1,0 +1,185 @@
+"""The step function: a batch of (request, its next tokens) through the model, from the cache.
+
+The reference has three entry points for this work: one token of one request
+(crates/leone/src/runtime.rs:7293), a prompt portion of one request
+(crates/leone/src/runtime.rs:6638) and one token each of several requests
+(crates/leone/src/runtime.rs:7461).  Here one ``step`` takes any mixture: each
+entry brings the next tokens of one request, prompt portions beside single
+decoded tokens, cut anywhere.  Only the given tokens are run; everything
+earlier comes from the cache.  A step is a transaction on the cache: pages are
+reserved first, written by the kernels, and committed only if the step succeeds
+(crates/leone/src/kv.rs:326-370, 856-927).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, OutOfPages
+from ..cache.pools import DevicePools
+from ..parts.context import EntryInfo, StepContext
+from ..parts.model import DecoderModel
+
+
+@dataclass
+class StepEntry:
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()       # indices into ``tokens`` whose logits are asked for
+
+
+@dataclass
+class StepOutput:
+    logits: Optional[torch.Tensor]                 # float32 [wanted, vocab] on the device, or None
+    rows: List[tuple] = field(default_factory=list)  # (request, index into its tokens) per logits row
+
+
+class StepError(ValueError):
+    """A step was refused before anything ran; the cache is unchanged."""
+
+
+class Engine:
+    def __init__(self, model: DecoderModel, *, num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
+                 page_tokens: int = 64, max_requests: int = 64, max_context: Optional[int] = None,
+                 poison_freed: bool = False):
+        if model.embedding is None:
+            raise ValueError("the model has no weights bound")
+        if not torch.cuda.is_available() or model.device.type != "cuda":
+            raise RuntimeError("the engine runs on a GPU only; there is no CPU path")
+        self.model = model
+        self.device = model.device
+        self.dtype = model.dtype
+        self.page_tokens = page_tokens
+        self.max_context = min(max_context or model.spec.max_positions, model.spec.max_positions)
+        if num_pages is None:
+            if max_tokens is None:
+                raise ValueError("give num_pages or max_tokens")
+            num_pages = (max_tokens + page_tokens - 1) // page_tokens
+        self.pools = DevicePools(model.cache_needs(), self.dtype, self.device, num_pages, page_tokens, max_requests)
+        self.cache = CacheManager(self.pools.group_specs, max_requests, self.max_context)
+        self.poison_freed = poison_freed
+        self.vocab_size = model.spec.vocab_size
+
+    # ---- requests -----------------------------------------------------------------
+    def admit(self, request: Hashable) -> int:
+        slot = self.cache.admit(request)
+        self.pools.zero_state(slot)
+        return slot
+
+    def release(self, request: Hashable) -> None:
+        if self.poison_freed:
+            tables = [list(self.cache.table(request, g)) for g in range(len(self.cache.groups))]
+        self.cache.release(request)
+        if self.poison_freed:
+            for g, table in enumerate(tables):
+                self.pools.poison_pages(g, [p for p in table if p >= 0])
+
+    def length(self, request: Hashable) -> int:
+        return self.cache.length(request)
+
+    # ---- the step --------------------------------------------------------------------
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen = set()
+        for e in entries:
+            if e.request in seen:
+                raise StepError(f"request {e.request!r} appears twice in one step")
+            seen.add(e.request)
+            if len(e.tokens) == 0:
+                raise StepError(f"request {e.request!r} brings no tokens")
+            for t in e.tokens:
+                if not 0 <= int(t) < self.vocab_size:
+                    raise StepError(f"request {e.request!r}: token {t} is outside the vocabulary of {self.vocab_size}")
+            for w in e.want:
+                if not 0 <= int(w) < len(e.tokens):
+                    raise StepError(f"request {e.request!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
+
+    def step(self, entries: Sequence[StepEntry]) -> StepOutput:
+        """Admits unknown requests, reserves pages, runs the tokens and commits.  All or nothing."""
+        self._validate(entries)
+        admitted, reserved = [], []
+        try:
+            for e in entries:
+                if not self.cache.has(e.request):
+                    self.admit(e.request)
+                    admitted.append(e.request)
+                self.cache.reserve(e.request, len(e.tokens))
+                reserved.append(e.request)
+        except Exception:
+            for request in reserved:
+                self.cache.rollback(request)
+            for request in admitted:
+                self.cache.release(request)
+            raise
+        return self.run_reserved(entries)
+
+    def run_reserved(self, entries: Sequence[StepEntry]) -> StepOutput:
+        """Runs a step whose pages the caller has reserved; commits on success, rolls back on failure."""
+        try:
+            self._validate(entries)
+            tokens, context, rows = self._build_context(entries)
+            caches = self.pools.views(context.block_tables)
+            logits = self.model.forward(tokens, context, caches)
+        except Exception:
+            for e in entries:
+                if self.cache.has(e.request):
+                    self.cache.rollback(e.request)
+            raise
+        freed_before = None
+        if self.poison_freed:
+            freed_before = [[list(self.cache.table(e.request, g)) for g in range(len(self.cache.groups))]
+                            for e in entries]
+        for e in entries:
+            self.cache.commit(e.request, len(e.tokens))
+        if self.poison_freed:
+            for e, before in zip(entries, freed_before):
+                for g, old in enumerate(before):
+                    new = self.cache.table(e.request, g)
+                    gone = [p for b, p in enumerate(old) if p >= 0 and (b >= len(new) or new[b] != p)]
+                    self.pools.poison_pages(g, gone)
+        return StepOutput(logits, rows)
+
+    def _build_context(self, entries: Sequence[StepEntry]):
+        n_rows = sum(len(e.tokens) for e in entries)
+        n_groups = len(self.cache.groups)
+        tokens = np.empty(n_rows, dtype=np.int32)
+        positions = np.empty(n_rows, dtype=np.int32)
+        row_entry = np.empty(n_rows, dtype=np.int32)
+        slots = np.empty(len(entries), dtype=np.int32)
+        tables = [np.full((len(entries), self.cache.max_blocks(g)), -1, dtype=np.int32) for g in range(n_groups)]
+        want_rows: List[int] = []
+        rows_map: List[tuple] = []
+        infos: List[EntryInfo] = []
+        row = 0
+        for ei, e in enumerate(entries):
+            start = self.cache.length(e.request)
+            n = len(e.tokens)
+            tokens[row:row + n] = np.asarray(e.tokens, dtype=np.int64)
+            positions[row:row + n] = np.arange(start, start + n)
+            row_entry[row:row + n] = ei
+            slots[ei] = self.cache.slot(e.request)
+            for g in range(n_groups):
+                table = self.cache.table(e.request, g)
+                tables[g][ei, :len(table)] = table
+            for w in e.want:
+                want_rows.append(row + int(w))
+                rows_map.append((e.request, int(w)))
+            infos.append(EntryInfo(e.request, int(slots[ei]), row, n, start))
+            row += n
+        # One upload for all step metadata.
+        parts = [tokens, positions, row_entry, slots, np.asarray(want_rows, dtype=np.int32)] + \
+                [t.reshape(-1) for t in tables]
+        packed = torch.from_numpy(np.concatenate(parts)).to(self.device)
+        offsets = np.cumsum([0] + [p.size for p in parts])
+        pieces = [packed[offsets[i]:offsets[i + 1]] for i in range(len(parts))]
+        block_tables = {g: pieces[5 + g].view(len(entries), -1) for g in range(n_groups)}
+        context = StepContext(
+            rows=n_rows, dtype=self.dtype, device=self.device, positions=pieces[1], row_entry=pieces[2],
+            entries=infos, entry_slots=pieces[3], want_rows=pieces[4] if want_rows else None,
+            block_tables=block_tables, max_position=int(positions.max()),
+            decode_only=all(len(e.tokens) == 1 for e in entries))
+        return pieces[0], context, rows_map

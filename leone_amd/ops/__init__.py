@@ -1,0 +1,200 @@
+"""Tensor-level wrappers over the HIP entry points.
+
+Each wrapper checks device, type, shape and contiguity on the host before the
+launch, because a kernel that reads outside its operands can take the whole
+GPU down.  Tensors must live on the GPU: there is no CPU path.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .library import KernelError, call, library
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    try:
+        return _CODES[t.dtype]
+    except KeyError:
+        raise KernelError(f"{what}: element type {t.dtype} is not float32 or bfloat16") from None
+
+
+def _dev(t: Optional[torch.Tensor], what: str, dtype=None, shape=None) -> int:
+    """Checks one operand and returns its device address (0 for None)."""
+    if t is None:
+        return 0
+    if not t.is_cuda:
+        raise KernelError(f"{what}: tensor is on {t.device}; the kernels run on the GPU only")
+    if not t.is_contiguous():
+        raise KernelError(f"{what}: tensor must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{what}: expected {dtype}, found {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{what}: expected shape {tuple(shape)}, found {tuple(t.shape)}")
+    return t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[r] = table[tokens[r]] as float32.  Token ids must have been checked against the table."""
+    vocab, hidden = table.shape
+    rows = tokens.numel()
+    if out is None:
+        out = torch.empty((rows, hidden), dtype=torch.float32, device=table.device)
+    call("leone_embed", _dev(table, "embed table"), _code(table, "embed table"),
+         _dev(tokens, "embed tokens", torch.int32, (rows,)), _dev(out, "embed out", torch.float32, (rows, hidden)),
+         rows, hidden, vocab, _stream())
+    return out
+
+
+def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x += delta, then y = rmsnorm(x) * gain; with ``rows``, y[i] comes from row rows[i] and x is not written."""
+    n, hidden = x.shape
+    n_out = n if rows is None else rows.numel()
+    if out is None:
+        out = torch.empty((n_out, hidden), dtype=out_dtype, device=x.device)
+    delta_code = _code(delta, "add_rmsnorm delta") if delta is not None else _CODES[out_dtype]
+    call("leone_add_rmsnorm", _dev(x, "add_rmsnorm x", torch.float32),
+         _dev(delta, "add_rmsnorm delta", None, (n, hidden)), delta_code,
+         _dev(gain, "add_rmsnorm gain", None, (hidden,)), _code(gain, "add_rmsnorm gain"), float(eps),
+         _dev(out, "add_rmsnorm out", out_dtype, (n_out, hidden)), _CODES[out_dtype],
+         _dev(rows, "add_rmsnorm rows", torch.int32), n_out, hidden, _stream())
+    return out
+
+
+def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    rows, twice = gate_up.shape
+    if twice % 2:
+        raise KernelError("swiglu: input width must be even (gate columns, then up columns)")
+    ffn = twice // 2
+    if out is None:
+        out = torch.empty((rows, ffn), dtype=gate_up.dtype, device=gate_up.device)
+    call("leone_swiglu", _dev(gate_up, "swiglu in"), _dev(out, "swiglu out", gate_up.dtype, (rows, ffn)),
+         _code(gate_up, "swiglu in"), rows, ffn, _stream())
+    return out
+
+
+def rope_table(theta: float, rotary_dim: int, positions: int, device) -> tuple[torch.Tensor, torch.Tensor]:
+    cos = torch.empty((positions, rotary_dim // 2), dtype=torch.float32, device=device)
+    sin = torch.empty_like(cos)
+    call("leone_rope_table", _dev(cos, "rope cos"), _dev(sin, "rope sin"), float(theta), rotary_dim, positions,
+         _stream())
+    return cos, sin
+
+
+def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int,
+                       q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
+                       cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
+                       row_entry: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
+                       k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor], write_cache: bool = True,
+                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Splits the fused projection, normalises and rotates q and k heads, writes k and v into the cache."""
+    rows, width = qkv.shape
+    if width != (q_heads + 2 * kv_heads) * head_dim:
+        raise KernelError(f"qk_norm_rope_write: width {width} is not ({q_heads}+2*{kv_heads})*{head_dim}")
+    if out is None:
+        out = torch.empty((rows, q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    max_blocks = page_tokens = 0
+    if write_cache:
+        if k_pool is None or v_pool is None or block_table is None or row_entry is None:
+            raise KernelError("qk_norm_rope_write: a cache write needs pools, a block table and a row map")
+        pages, pool_heads, page_tokens, pool_dim = k_pool.shape
+        if (pool_heads, pool_dim) != (kv_heads, head_dim) or v_pool.shape != k_pool.shape:
+            raise KernelError(f"qk_norm_rope_write: pool shape {tuple(k_pool.shape)} does not fit "
+                              f"{kv_heads} heads of {head_dim}")
+        max_blocks = block_table.shape[1]
+    table_positions = 0
+    if cos is not None:
+        table_positions = cos.shape[0]
+        if cos.shape[1] != head_dim // 2 or sin is None or sin.shape != cos.shape:
+            raise KernelError("qk_norm_rope_write: rotary table does not fit the head size")
+    gain_code = _code(q_gain, "q gain") if q_gain is not None else F32
+    if q_gain is not None and (k_gain is None or k_gain.dtype != q_gain.dtype):
+        raise KernelError("qk_norm_rope_write: q and k gains must come together in one type")
+    call("leone_qk_norm_rope_write", _dev(qkv, "qkv"), _dev(out, "q out", qkv.dtype),
+         _dev(k_pool if write_cache else None, "k pool", qkv.dtype),
+         _dev(v_pool if write_cache else None, "v pool", qkv.dtype), _code(qkv, "qkv"),
+         _dev(q_gain, "q gain", None, (head_dim,)), _dev(k_gain, "k gain", None, (head_dim,)), gain_code,
+         float(eps), _dev(cos, "rope cos", torch.float32), _dev(sin, "rope sin", torch.float32), table_positions,
+         _dev(positions, "positions", torch.int32, (rows,)),
+         _dev(row_entry if write_cache else None, "row map", torch.int32, (rows,)),
+         _dev(block_table if write_cache else None, "block table", torch.int32), max_blocks, rows, q_heads,
+         kv_heads, head_dim, page_tokens, 1 if write_cache else 0, _stream())
+    return out
+
+
+def attention_rows(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
+                   row_entry: torch.Tensor, block_table: torch.Tensor, q_heads: int, scale: float,
+                   window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Each query row attends its request's cached keys up to its own position."""
+    rows = q.shape[0]
+    pages, kv_heads, page_tokens, head_dim = k_pool.shape
+    if q.shape[1] != q_heads * head_dim:
+        raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
+    if v_pool.shape != k_pool.shape:
+        raise KernelError("attention: key and value pools differ in shape")
+    if out is None:
+        out = torch.empty_like(q)
+    call("leone_attention_rows", _dev(q, "attention q"), _dev(out, "attention out", q.dtype, q.shape),
+         _dev(k_pool, "k pool", q.dtype), _dev(v_pool, "v pool", q.dtype), _code(q, "attention q"),
+         _dev(positions, "positions", torch.int32, (rows,)), _dev(row_entry, "row map", torch.int32, (rows,)),
+         _dev(block_table, "block table", torch.int32), block_table.shape[1], rows, q_heads, kv_heads, head_dim,
+         page_tokens, float(scale), int(window), _stream())
+    return out
+
+
+def gemm_f32(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a[M,K] . b[N,K]^T in true single precision."""
+    m, k = a.shape
+    n, k2 = b.shape
+    if k != k2:
+        raise KernelError(f"gemm_f32: inner sizes {k} and {k2} differ")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    call("leone_gemm_f32", _dev(a, "gemm a", torch.float32), _dev(b, "gemm b", torch.float32),
+         _dev(out, "gemm out", torch.float32, (m, n)), m, n, k, _stream())
+    return out
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """x[R,K] . weight[N,K]^T.  float32 runs the single-precision kernel; bfloat16 inputs accumulate in float."""
+    if x.dtype != weight.dtype:
+        raise KernelError(f"linear: activations are {x.dtype} but the weight is {weight.dtype}")
+    out_dtype = out_dtype or x.dtype
+    if x.dtype == torch.float32:
+        if out_dtype != torch.float32:
+            raise KernelError("linear: the float32 path produces float32")
+        return gemm_f32(x, weight)
+    if not x.is_cuda:
+        raise KernelError("linear: tensor is not on the GPU")
+    y = torch.nn.functional.linear(x, weight)  # library matrix product, float accumulation
+    return y if out_dtype == y.dtype else y.to(out_dtype)
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    rows, vocab = logits.shape
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    call("leone_argmax", _dev(logits, "argmax logits", torch.float32), _dev(out, "argmax out"), rows, vocab,
+         _stream())
+    return out
+
+
+def sample_temperature(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
+    rows, vocab = logits.shape
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    call("leone_sample_temperature", _dev(logits, "sample logits", torch.float32),
+         _dev(temperature, "sample temperature", torch.float64, (rows,)),
+         _dev(uniform, "sample uniform", torch.float64, (rows,)), _dev(out, "sample out"), rows, vocab, _stream())
+    return out
+
+
+__all__ = [name for name in dir() if not name.startswith("_")]

@@ -1,0 +1,62 @@
+"""Loads the gfx950 kernel library and declares its entry points for ctypes.
+
+There is no substitute path: if the library cannot be built or loaded, the
+first kernel call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+from ctypes import c_char_p, c_double, c_float, c_int, c_void_p
+
+from ..csrc import build as _build
+
+
+class KernelError(RuntimeError):
+    """A kernel entry point refused its arguments or failed to launch."""
+
+
+_lock = threading.Lock()
+_lib: ctypes.CDLL | None = None
+
+P = c_void_p
+_PROTOTYPES = {
+    "leone_embed": [P, c_int, P, P, c_int, c_int, c_int, P],
+    "leone_add_rmsnorm": [P, P, c_int, P, c_int, c_float, P, c_int, P, c_int, c_int, P],
+    "leone_swiglu": [P, P, c_int, c_int, c_int, P],
+    "leone_rope_table": [P, P, c_double, c_int, c_int, P],
+    "leone_qk_norm_rope_write": [P, P, P, P, c_int, P, P, c_int, c_float, P, P, c_int, P, P, P, c_int,
+                                 c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "leone_attention_rows": [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                             c_int, P],
+    "leone_gemm_f32": [P, P, P, c_int, c_int, c_int, P],
+    "leone_argmax": [P, P, c_int, c_int, P],
+    "leone_sample_temperature": [P, P, P, P, c_int, c_int, P],
+}
+
+
+def library() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is None:
+            path = _build.library_path()
+            if path is None:
+                path = _build.build(verbose=True)
+            lib = ctypes.CDLL(path)
+            lib.leone_last_error.restype = c_char_p
+            lib.leone_last_error.argtypes = []
+            for name, argtypes in _PROTOTYPES.items():
+                fn = getattr(lib, name)
+                fn.argtypes = argtypes
+                fn.restype = c_int
+            _lib = lib
+    return _lib
+
+
+def call(name: str, *args) -> None:
+    lib = library()
+    status = getattr(lib, name)(*args)
+    if status != 0:
+        raise KernelError(lib.leone_last_error().decode("utf-8", "replace"))

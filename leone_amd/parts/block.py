@@ -1,0 +1,47 @@
+"""How norm, mixer and feed-forward are arranged in one layer."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..weights.loader import TensorSpec
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Part, PartSpec
+from .context import CacheView, StepContext
+
+
+@BLOCKS.register("prenorm")
+class PreNormBlock(Part):
+    """x1 = x + mixer(norm1(x)); x2 = x1 + feed_forward(norm2(x1)).
+
+    Reference layer order: crates/leone/src/runtime.rs:9019-9050.
+    Parameters: ``norm1``, ``mixer``, ``norm2``, ``feed_forward`` (part specs).
+    The residual stream is float32; each delta is added by the following norm's
+    kernel, so the block returns its last delta instead of adding it.
+    """
+
+    def __init__(self, spec: PartSpec, **context):
+        self.norm1 = NORMS.build(spec["norm1"], **context)
+        self.mixer = MIXERS.build(spec["mixer"], **context)
+        self.norm2 = NORMS.build(spec["norm2"], **context)
+        self.feed_forward = FEED_FORWARDS.build(spec["feed_forward"], **context)
+
+    def parts(self):
+        return (self.norm1, self.mixer, self.norm2, self.feed_forward)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for part in self.parts() for s in part.tensor_specs()]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for part in self.parts():
+            part.bind(tensors)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], step: StepContext,
+                cache: Optional[CacheView]) -> torch.Tensor:
+        y = self.norm1.add_norm(x, pending, step.dtype)
+        delta = self.mixer.forward(y, step, cache)
+        y = self.norm2.add_norm(x, delta, step.dtype)
+        return self.feed_forward.forward(y, step)

@@ -1,0 +1,87 @@
+"""Token mixers."""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import ops
+from ..weights.loader import MATRIX, VECTOR, TensorSpec
+from .base import MIXERS, KvNeed, Part, PartSpec
+from .context import KvCacheView, StepContext
+
+
+@MIXERS.register("gqa_attention")
+class GqaAttention(Part):
+    """Grouped-query causal attention over a paged key/value cache.
+
+    q = Wq y, k = Wk y, v = Wv y (no bias); optional per-head RMSNorm of q and
+    k over head_dim, then the position encoding on q and k; k and v go into the
+    cache; each row attends the keys of its own request up to its position
+    (within ``window`` if set) with scale 1/sqrt(head_dim); out = Wo o.
+    Reference: crates/leone/src/runtime.rs:9104-9157 (decode order),
+    crates/leone/src/backend.rs:2182-2208 (per-head norm),
+    crates/leone/src/cpu.rs:2299-2357 (attention).
+
+    Parameters: ``hidden``, ``q_heads``, ``kv_heads``, ``head_dim``, ``qk_norm_eps``
+    (None: no q/k norm), ``window`` (None: all keys), ``position`` (name of a
+    position part) and tensor names ``q``, ``k``, ``v``, ``o``, ``q_norm``, ``k_norm``.
+    """
+
+    def __init__(self, spec: PartSpec, positions: Optional[dict] = None, **_):
+        p = spec.params
+        self.hidden = int(p["hidden"])
+        self.q_heads = int(p["q_heads"])
+        self.kv_heads = int(p["kv_heads"])
+        self.head_dim = int(p["head_dim"])
+        if self.q_heads % self.kv_heads:
+            raise ValueError(f"{self.q_heads} query heads cannot be grouped over {self.kv_heads} kv heads")
+        self.qk_norm_eps = p.get("qk_norm_eps")
+        self.window = p.get("window")
+        self.scale = float(p.get("scale", 1.0 / math.sqrt(self.head_dim)))
+        self.names = {k: p[k] for k in ("q", "k", "v", "o")}
+        if self.qk_norm_eps is not None:
+            self.names.update(q_norm=p["q_norm"], k_norm=p["k_norm"])
+        self.position = (positions or {}).get(p.get("position")) if p.get("position") else None
+        if p.get("position") and self.position is None:
+            raise ValueError(f"attention names position part {p.get('position')!r}, which the model does not define")
+        self.w_qkv = self.w_o = self.q_gain = self.k_gain = None
+
+    def cache_need(self) -> KvNeed:
+        return KvNeed(self.kv_heads, self.head_dim, self.window)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        qw, kvw = self.q_heads * self.head_dim, self.kv_heads * self.head_dim
+        specs = [TensorSpec(self.names["q"], (qw, self.hidden), MATRIX),
+                 TensorSpec(self.names["k"], (kvw, self.hidden), MATRIX),
+                 TensorSpec(self.names["v"], (kvw, self.hidden), MATRIX),
+                 TensorSpec(self.names["o"], (self.hidden, qw), MATRIX)]
+        if self.qk_norm_eps is not None:
+            specs += [TensorSpec(self.names["q_norm"], (self.head_dim,), VECTOR),
+                      TensorSpec(self.names["k_norm"], (self.head_dim,), VECTOR)]
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        # One product for q, k and v: a pure re-layout of the three matrices.
+        self.w_qkv = torch.cat([tensors.pop(self.names["q"]), tensors.pop(self.names["k"]),
+                                tensors.pop(self.names["v"])], dim=0).contiguous()
+        self.w_o = tensors.pop(self.names["o"]).contiguous()
+        if self.qk_norm_eps is not None:
+            self.q_gain = tensors.pop(self.names["q_norm"]).contiguous()
+            self.k_gain = tensors.pop(self.names["k_norm"]).contiguous()
+            if self.q_gain.dtype != self.k_gain.dtype:
+                self.q_gain, self.k_gain = self.q_gain.float(), self.k_gain.float()
+
+    def forward(self, y: torch.Tensor, step: StepContext, cache: KvCacheView) -> torch.Tensor:
+        qkv = ops.linear(y, self.w_qkv)
+        cos, sin = self.position.tables() if self.position is not None else (None, None)
+        if cos is not None and step.max_position >= cos.shape[0]:
+            raise ValueError(f"position {step.max_position} is beyond the rotary table of {cos.shape[0]} positions")
+        q = ops.qk_norm_rope_write(qkv, self.q_heads, self.kv_heads, self.head_dim, self.q_gain, self.k_gain,
+                                   self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin,
+                                   step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
+                                   write_cache=cache.writes)
+        attended = ops.attention_rows(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
+                                      cache.block_table, self.q_heads, self.scale, int(self.window or 0))
+        return ops.linear(attended, self.w_o)

@@ -1,0 +1,123 @@
+"""A decoder model as data (``ModelSpec``) and the object built from it."""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from .. import ops
+from ..weights.loader import MATRIX, TensorSpec
+from .base import BLOCKS, NORMS, POSITIONS, KvNeed, PartSpec, StateNeed
+from .context import CacheView, StepContext
+
+
+@dataclass(frozen=True)
+class LayerRun:
+    """One entry of the execution order.
+
+    ``layer`` indexes ``ModelSpec.layers`` (a layer may be named more than
+    once).  ``cache`` is the cache slot the run works on; two runs that name the
+    same slot share it, and only runs with ``writes`` put new keys, values or
+    state there.
+    """
+    layer: int
+    cache: Optional[int]
+    writes: bool = True
+
+
+@dataclass
+class ModelSpec:
+    hidden_size: int
+    vocab_size: int
+    max_positions: int
+    embedding: str                                  # tensor name of the token table [vocab, hidden]
+    layers: List[PartSpec]                          # block specs
+    schedule: List[LayerRun]
+    final_norm: PartSpec
+    head: Optional[str]                             # tensor name [vocab, hidden]; None = tied to the embedding
+    positions: Dict[str, PartSpec] = field(default_factory=dict)
+    ignore_tensors: Sequence[str] = ()              # names a file may hold that the model does not use
+
+
+def default_schedule(n_layers: int) -> List[LayerRun]:
+    return [LayerRun(i, i, True) for i in range(n_layers)]
+
+
+class DecoderModel:
+    """Embedding, the scheduled layer runs, final norm and the output head."""
+
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"engine type must be float32 or bfloat16, found {dtype}")
+        self.spec = spec
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.positions = {name: POSITIONS.build(s) for name, s in spec.positions.items()}
+        self.layers = [BLOCKS.build(s, positions=self.positions) for s in spec.layers]
+        self.final_norm = NORMS.build(spec.final_norm)
+        self.schedule = list(spec.schedule)
+        for run in self.schedule:
+            if not 0 <= run.layer < len(self.layers):
+                raise ValueError(f"schedule names layer {run.layer}, the model has {len(self.layers)}")
+        self.embedding: Optional[torch.Tensor] = None
+        self.head: Optional[torch.Tensor] = None
+
+    # ---- weights -------------------------------------------------------------
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = [TensorSpec(self.spec.embedding, (self.spec.vocab_size, self.spec.hidden_size), MATRIX)]
+        for layer in self.layers:
+            specs += layer.tensor_specs()
+        specs += self.final_norm.tensor_specs()
+        if self.spec.head is not None:
+            specs.append(TensorSpec(self.spec.head, (self.spec.vocab_size, self.spec.hidden_size), MATRIX))
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        tensors = dict(tensors)
+        self.embedding = tensors.pop(self.spec.embedding).contiguous()
+        self.head = tensors.pop(self.spec.head).contiguous() if self.spec.head is not None else self.embedding
+        for layer in self.layers:
+            layer.bind(tensors)
+        self.final_norm.bind(tensors)
+        for position in self.positions.values():
+            position.prepare(self.spec.max_positions, self.device)
+
+    # ---- cache ---------------------------------------------------------------
+    def cache_needs(self) -> Dict[int, object]:
+        """Cache slot -> what the layer runs on it need (one need per slot)."""
+        needs: Dict[int, object] = {}
+        writers: Dict[int, int] = {}
+        for run in self.schedule:
+            need = self.layers[run.layer].cache_need()
+            if need is None:
+                if run.cache is not None:
+                    raise ValueError(f"layer {run.layer} keeps no cache but its run names slot {run.cache}")
+                continue
+            if run.cache is None:
+                raise ValueError(f"layer {run.layer} needs a cache but its run names none")
+            if run.cache in needs and needs[run.cache] != need:
+                raise ValueError(f"cache slot {run.cache} is shared by layers with different needs")
+            needs[run.cache] = need
+            writers[run.cache] = writers.get(run.cache, 0) + (1 if run.writes else 0)
+        for slot, count in writers.items():
+            if count != 1:
+                raise ValueError(f"cache slot {slot} must have exactly one writing run, found {count}")
+        return needs
+
+    # ---- forward ---------------------------------------------------------------
+    def forward(self, tokens: torch.Tensor, step: StepContext, caches: Dict[int, CacheView]) -> Optional[torch.Tensor]:
+        """Runs the step's rows through every scheduled layer; returns float32 logits of the wanted rows."""
+        x = ops.embed(self.embedding, tokens)
+        pending = None
+        for run in self.schedule:
+            cache = caches.get(run.cache) if run.cache is not None else None
+            if cache is not None and cache.writes != run.writes:
+                cache = type(cache)(**{**cache.__dict__, "writes": run.writes})
+            pending = self.layers[run.layer].forward(x, pending, step, cache)
+        if step.want_rows is None or step.want_rows.numel() == 0:
+            if pending is not None:
+                pass  # nothing reads the last delta when no logits are wanted
+            return None
+        y = self.final_norm.add_norm(x, pending, self.dtype, rows=step.want_rows)
+        return ops.linear(y, self.head, out_dtype=torch.float32)

@@ -1,0 +1,34 @@
+"""Normalisation parts."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from .. import ops
+from ..weights.loader import TensorSpec, VECTOR
+from .base import NORMS, Part, PartSpec
+
+
+@NORMS.register("rmsnorm")
+class RmsNorm(Part):
+    """y = (x * gain) / sqrt(mean(x^2) + eps); the gain multiplies directly (not 1 + gain).
+
+    Reference: crates/leone/src/cpu.rs:1642-1663.  Parameters: ``size``, ``eps``, ``weight`` (tensor name).
+    """
+
+    def __init__(self, spec: PartSpec, **_):
+        self.size = int(spec["size"])
+        self.eps = float(spec["eps"])
+        self.weight_name = spec["weight"]
+        self.gain: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.weight_name, (self.size,), VECTOR)]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.gain = tensors[self.weight_name].contiguous()
+
+    def add_norm(self, x: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype,
+                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.add_rmsnorm(x, delta, self.gain, self.eps, out_dtype, rows)

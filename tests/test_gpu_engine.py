@@ -1,0 +1,106 @@
+"""The engine against the plain implementation, under every way of cutting the work."""
+import numpy as np
+import pytest
+import torch
+
+from tests import schedules
+from tests.plain import qwen3_plain
+from tests.util import TINY, make_model_dir, random_tokens, read_config, read_weights, tolerance
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [1, 7, 33, 64, 100, 18, 47], "B": [5, 40, 130, 66, 90], "C": [70, 150, 35, 81, 3]}
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def cases(tmp_path_factory):
+    """(config name, dtype name) -> model folder, requests and the plain logits of each request."""
+    cache = {}
+
+    def get(name, dtype_name):
+        key = (name, dtype_name)
+        if key not in cache:
+            folder = str(tmp_path_factory.mktemp(f"model_{name}_{dtype_name}"))
+            make_model_dir(folder, TINY[name], seed=11 + len(cache), dtype=DTYPES[dtype_name], sharpen=2.0)
+            config, weights = read_config(folder), read_weights(folder)
+            requests = {f"r{i}": random_tokens(100 * i + 7, n, config["vocab_size"])
+                        for i, n in enumerate(LENGTHS[name])}
+            expected = {rid: qwen3_plain.forward(weights, config, toks).numpy() for rid, toks in requests.items()}
+            cache[key] = (folder, requests, expected)
+        return cache[key]
+
+    return get
+
+
+def run_steps(engine, steps):
+    from leone_amd.engine.engine import StepEntry
+
+    outputs = {}
+    for s in steps:
+        out = engine.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        if out.logits is not None:
+            outputs[s["step"]] = out.logits.float().cpu().numpy()
+        for rid in s["end"]:
+            engine.release(rid)
+        engine.cache.check()
+    return outputs
+
+
+def compare(steps, outputs, expected, tol, what):
+    got = schedules.collect(steps, outputs)
+    assert set(got) == set(expected)
+    for rid, rows in got.items():
+        have = np.stack(rows)
+        want = expected[rid]
+        assert have.shape == want.shape, (what, rid, have.shape, want.shape)
+        assert np.isfinite(have).all(), f"{what}: request {rid} has non-finite logits"
+        err = np.abs(have - want).max(axis=1)
+        worst = int(err.argmax())
+        assert err[worst] <= tol, (f"{what}: request {rid} first wrong position "
+                                   f"{int(np.argmax(err > tol))} of {len(err)}, worst {worst}: {err[worst]:.3e} > {tol}")
+
+
+SCHEDULES = {
+    "whole": schedules.whole,
+    "tail_decoded": schedules.tail_decoded,
+    "portions": schedules.portions,
+    "mixed": schedules.mixed,
+}
+
+
+@pytest.mark.parametrize("page_tokens", [16, 64])
+@pytest.mark.parametrize("schedule", list(SCHEDULES))
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+@pytest.mark.parametrize("name", list(TINY))
+def test_engine_matches_plain(cases, name, dtype_name, schedule, page_tokens):
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+
+    folder, requests, expected = cases(name, dtype_name)
+    steps = SCHEDULES[schedule](requests)
+    # As few pages as the schedule can live with, so that pages given back are used again.
+    pool_tokens = schedules.max_live_tokens(steps, round_to=page_tokens)
+    model = load_model(folder, dtype_name)
+    engine = Engine(model, num_pages=pool_tokens // page_tokens, page_tokens=page_tokens, max_requests=4,
+                    poison_freed=True)
+    outputs = run_steps(engine, steps)
+    compare(steps, outputs, expected, tolerance(dtype_name), f"{name}/{dtype_name}/{schedule}/page{page_tokens}")
+    assert not engine.cache.live_requests()
+    assert all(engine.cache.free_pages(g) == engine.cache.groups[g].num_pages for g in range(len(engine.cache.groups)))
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_rerun_is_bitwise_identical(cases, dtype_name):
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+
+    folder, requests, _ = cases("B", dtype_name)
+    steps = schedules.mixed(requests)
+    model = load_model(folder, dtype_name)
+    results = []
+    for _ in range(2):
+        engine = Engine(model, max_tokens=schedules.max_live_tokens(steps, 16), page_tokens=16, max_requests=4)
+        results.append(run_steps(engine, steps))
+    for step in results[0]:
+        assert np.array_equal(results[0][step], results[1][step]), f"step {step} differs between two runs"

@@ -1,0 +1,251 @@
+"""Each HIP kernel alone against a plain float64 computation, at sizes other than the engine's."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from tests.plain import qwen3_plain as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def close(have, want, atol, rtol, what=""):
+    have, want = have.double().cpu(), want.double().cpu()
+    err = (have - want).abs()
+    bound = atol + rtol * want.abs()
+    bad = err > bound
+    assert not bad.any(), f"{what}: {int(bad.sum())} of {bad.numel()} off, worst {float((err - bound).max()):.3e} over"
+
+
+def tol(dtype):
+    # float32: a few ulps of sums over up to thousands of terms; bfloat16: one rounding of the output (2^-8).
+    return (2e-5, 2e-5) if dtype == torch.float32 else (1e-2, 1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(dtype):
+    from leone_amd import ops
+    torch.manual_seed(0)
+    table = torch.randn(777, 80, device=DEV).to(dtype)
+    tokens = torch.tensor([0, 776, 5, 5, 123], dtype=torch.int32, device=DEV)
+    out = ops.embed(table, tokens)
+    assert out.dtype == torch.float32
+    assert torch.equal(out, table.float()[tokens.long()])
+
+
+@pytest.mark.parametrize("hidden", [80, 1000, 4096, 5120])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_rmsnorm(dtype, hidden):
+    from leone_amd import ops
+    torch.manual_seed(1)
+    x = torch.randn(7, hidden, device=DEV) * 3
+    delta = torch.randn(7, hidden, device=DEV).to(dtype)
+    gain = (1 + 0.1 * torch.randn(hidden, device=DEV))
+    eps = 1e-5
+    x0 = x.clone()
+    y = ops.add_rmsnorm(x, delta, gain, eps, dtype)
+    want_x = x0.double() + delta.double()
+    assert torch.equal(x, (x0 + delta.float()))          # the stream is updated in float
+    close(y, plain.rms_norm(want_x.cpu(), gain.cpu(), eps), *tol(dtype), "add_rmsnorm")
+    # without a delta the stream is untouched
+    x1 = x.clone()
+    y2 = ops.add_rmsnorm(x, None, gain.to(dtype), eps, dtype)
+    assert torch.equal(x, x1)
+    close(y2, plain.rms_norm(x1.cpu(), gain.to(dtype).cpu(), eps), *tol(dtype), "rmsnorm")
+    # gathered rows: x stays, only the chosen rows come out
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    y3 = ops.add_rmsnorm(x, delta, gain, eps, torch.float32, rows=rows)
+    assert torch.equal(x, x1)
+    close(y3, plain.rms_norm((x1.double() + delta.double())[rows.long()].cpu(), gain.cpu(), eps), 2e-5, 2e-5, "gather")
+
+
+def test_rmsnorm_reference_vector():
+    """rows [1,2],[3,4], gain [1,0.5], eps 1e-6: the largest of the four outputs is index 2
+    (crates/leone/src/cpu.rs:2781-2807)."""
+    from leone_amd import ops
+    x = torch.tensor([[1.0, 2.0], [3.0, 4.0]], device=DEV)
+    y = ops.add_rmsnorm(x, None, torch.tensor([1.0, 0.5], device=DEV), 1e-6, torch.float32)
+    assert int(y.flatten().argmax()) == 2
+    assert int(ops.argmax(y.reshape(1, 4))[0]) == 2
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu(dtype):
+    """gate in [-8, 8], up in [-2, 2], 12,289 elements (crates/leone-cuda/tests/gpu.rs:1851-1867)."""
+    from leone_amd import ops
+    torch.manual_seed(2)
+    n = 12289
+    gate = (torch.rand(3, n, device=DEV) * 16 - 8)
+    up = (torch.rand(3, n, device=DEV) * 4 - 2)
+    gu = torch.cat([gate, up], dim=1).to(dtype)
+    out = ops.swiglu(gu)
+    want = plain.swiglu(gu[:, :n].cpu(), gu[:, n:].cpu())
+    atol, rtol = (2e-6, 3e-6) if dtype == torch.float32 else (1e-2, 1e-2)
+    close(out, want, atol, rtol, "swiglu")
+
+
+def test_rope_table():
+    """positions {0, 17, 2048, 8000}, theta 1e6, D 128 within 5e-7 of double (crates/leone-cuda/tests/gpu.rs:1468-1488)."""
+    from leone_amd import ops
+    cos, sin = ops.rope_table(1e6, 128, 8192, DEV)
+    for pos in (0, 17, 2048, 8000):
+        for i in (0, 1, 31, 63):
+            angle = pos * (1e6 ** (-2.0 * i / 128))
+            assert abs(float(cos[pos, i]) - math.cos(angle)) < 5e-7
+            assert abs(float(sin[pos, i]) - math.sin(angle)) < 5e-7
+
+
+def paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed, extra_pages=3):
+    """Random keys/values for several requests scattered over shuffled pages."""
+    g = torch.Generator().manual_seed(seed)
+    blocks = [(n + page_tokens - 1) // page_tokens for n in lengths]
+    n_pages = sum(blocks) + extra_pages
+    order = torch.randperm(n_pages, generator=g).tolist()
+    max_blocks = max(blocks) + 1
+    table = torch.full((len(lengths), max_blocks), -1, dtype=torch.int32)
+    k_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), float("nan"))
+    v_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), float("nan"))
+    keys, values = [], []
+    at = 0
+    for r, n in enumerate(lengths):
+        k = torch.randn(n, kv_heads, head_dim, generator=g).to(dtype).float()
+        v = torch.randn(n, kv_heads, head_dim, generator=g).to(dtype).float()
+        keys.append(k)
+        values.append(v)
+        for b in range(blocks[r]):
+            page = order[at]
+            at += 1
+            table[r, b] = page
+            lo, hi = b * page_tokens, min(n, (b + 1) * page_tokens)
+            k_pool[page, :, :hi - lo] = k[lo:hi].transpose(0, 1)
+            v_pool[page, :, :hi - lo] = v[lo:hi].transpose(0, 1)
+    return table, k_pool.to(dtype), v_pool.to(dtype), keys, values
+
+
+@pytest.mark.parametrize("window", [0, 5, 37])
+@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 1, 32, 64), (5, 5, 48, 16), (8, 2, 128, 32), (3, 3, 256, 16)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_rows(dtype, shape, window):
+    """Rows of several requests, portions and single tokens, over scattered pages; unmapped
+    slots hold NaN and must never be read (crates/leone/tests/cpu_kv_span_attention_oracle.rs:303-309)."""
+    from leone_amd import ops
+    q_heads, kv_heads, head_dim, page_tokens = shape
+    lengths = [1, 17, 70, 130]
+    table, k_pool, v_pool, keys, values = paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed=3)
+    # request 0: its only token; request 1: last token (decode); request 2: rows 40..69 (a portion);
+    # request 3: every row.
+    rows = [(0, 0)] + [(1, 16)] + [(2, p) for p in range(40, 70)] + [(3, p) for p in range(130)]
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn(len(rows), q_heads, head_dim, generator=g).to(dtype)
+    positions = torch.tensor([p for _, p in rows], dtype=torch.int32)
+    row_entry = torch.tensor([r for r, _ in rows], dtype=torch.int32)
+    scale = 1.0 / math.sqrt(head_dim)
+    out = ops.attention_rows(q.reshape(len(rows), -1).to(DEV), k_pool.to(DEV), v_pool.to(DEV), positions.to(DEV),
+                             row_entry.to(DEV), table.to(DEV), q_heads, scale, window)
+    assert torch.isfinite(out.float()).all()
+    want = torch.empty(len(rows), q_heads, head_dim, dtype=torch.float64)
+    for i, (r, p) in enumerate(rows):
+        want[i] = plain.attend_one(q[i].float(), keys[r][:p + 1], values[r][:p + 1], window or None)
+    atol, rtol = (3e-5, 3e-4) if dtype == torch.float32 else (2e-2, 2e-2)
+    close(out.reshape(len(rows), q_heads, head_dim), want, atol, rtol, "attention")
+
+
+def test_attention_reference_vector():
+    """2 heads, 1 kv head, D=2, K rows [1,0],[0,1], V rows [2,4],[6,8], q [1,0] and [0,1] per token
+    (crates/leone/src/cpu.rs:2850-2898)."""
+    from leone_amd import ops
+    k_pool = torch.zeros(1, 1, 16, 2, device=DEV)
+    v_pool = torch.zeros(1, 1, 16, 2, device=DEV)
+    k_pool[0, 0, 0] = torch.tensor([1.0, 0.0]); k_pool[0, 0, 1] = torch.tensor([0.0, 1.0])
+    v_pool[0, 0, 0] = torch.tensor([2.0, 4.0]); v_pool[0, 0, 1] = torch.tensor([6.0, 8.0])
+    q = torch.tensor([[1.0, 0.0, 0.0, 1.0], [1.0, 0.0, 0.0, 1.0]], device=DEV)
+    out = ops.attention_rows(q, k_pool, v_pool, torch.tensor([0, 1], dtype=torch.int32, device=DEV),
+                             torch.zeros(2, dtype=torch.int32, device=DEV),
+                             torch.zeros(1, 1, dtype=torch.int32, device=DEV), 2, 1.0 / math.sqrt(2.0))
+    h = math.exp(1.0 / math.sqrt(2.0))
+    want = torch.tensor([[2.0, 4.0, 2.0, 4.0],
+                         [(h * 2 + 6) / (h + 1), (h * 4 + 8) / (h + 1), (2 + h * 6) / (h + 1), (4 + h * 8) / (h + 1)]])
+    close(out, want, 1e-6, 1e-6, "reference vector")
+
+
+@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 1, 32, 64), (5, 5, 48, 16), (32, 8, 128, 64)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_qk_norm_rope_write(dtype, shape):
+    from leone_amd import ops
+    q_heads, kv_heads, head_dim, page_tokens = shape
+    torch.manual_seed(5)
+    rows_meta = [(0, 3), (0, 4), (1, 16), (1, 17), (2, 8000)]  # (entry, position): page edges and a far position
+    n = len(rows_meta)
+    width = (q_heads + 2 * kv_heads) * head_dim
+    qkv = torch.randn(n, width).to(dtype)
+    q_gain = (1 + 0.1 * torch.randn(head_dim))
+    k_gain = (1 + 0.1 * torch.randn(head_dim))
+    eps, theta = 1e-5, 1e6
+    max_blocks = 8000 // page_tokens + 1
+    n_pages = 6
+    table = torch.full((3, max_blocks), -1, dtype=torch.int32)
+    table[0, 0] = 4
+    table[1, 16 // page_tokens] = 2
+    table[1, 17 // page_tokens] = 2 if 16 // page_tokens == 17 // page_tokens else 5
+    table[2, 8000 // page_tokens] = 1
+    k_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), 7.0).to(dtype)
+    v_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), 7.0).to(dtype)
+    cos, sin = ops.rope_table(theta, head_dim, 8192, DEV)
+    positions = torch.tensor([p for _, p in rows_meta], dtype=torch.int32)
+    row_entry = torch.tensor([e for e, _ in rows_meta], dtype=torch.int32)
+    kp, vp = k_pool.to(DEV), v_pool.to(DEV)
+    q_out = ops.qk_norm_rope_write(qkv.to(DEV), q_heads, kv_heads, head_dim, q_gain.to(DEV), k_gain.to(DEV), eps,
+                                   cos, sin, positions.to(DEV), row_entry.to(DEV), table.to(DEV), kp, vp)
+    x = qkv.float()
+    q = x[:, :q_heads * head_dim].view(n, q_heads, head_dim)
+    k = x[:, q_heads * head_dim:(q_heads + kv_heads) * head_dim].view(n, kv_heads, head_dim)
+    v = x[:, (q_heads + kv_heads) * head_dim:].view(n, kv_heads, head_dim)
+    want_q = plain.rope_half_split(plain.rms_norm(q, q_gain, eps), positions, theta)
+    want_k = plain.rope_half_split(plain.rms_norm(k, k_gain, eps), positions, theta)
+    atol, rtol = (5e-6, 2e-5) if dtype == torch.float32 else (2e-2, 1e-2)
+    close(q_out.view(n, q_heads, head_dim), want_q, atol, rtol, "q")
+    touched = torch.zeros(n_pages, page_tokens, dtype=torch.bool)
+    for i, (e, p) in enumerate(rows_meta):
+        page, off = int(table[e, p // page_tokens]), p % page_tokens
+        touched[page, off] = True
+        close(kp[page, :, off], want_k[i], atol, rtol, f"k row {i}")
+        assert torch.equal(vp[page, :, off].cpu(), v[i].to(dtype))      # values are copied unchanged
+    # every other slot is untouched
+    assert torch.equal(kp.cpu()[~touched], k_pool[~touched])
+    assert torch.equal(vp.cpu()[~touched], v_pool[~touched])
+    # a layer that reads another layer's cache writes nothing
+    kp2, vp2 = k_pool.to(DEV), v_pool.to(DEV)
+    q2 = ops.qk_norm_rope_write(qkv.to(DEV), q_heads, kv_heads, head_dim, q_gain.to(DEV), k_gain.to(DEV), eps, cos,
+                                sin, positions.to(DEV), row_entry.to(DEV), table.to(DEV), kp2, vp2, write_cache=False)
+    assert torch.equal(q2, q_out) and torch.equal(kp2.cpu(), k_pool) and torch.equal(vp2.cpu(), v_pool)
+    # no norm and no rotation: the heads come through as they are
+    q3 = ops.qk_norm_rope_write(qkv.to(DEV), q_heads, kv_heads, head_dim, None, None, eps, None, None,
+                                positions.to(DEV), row_entry.to(DEV), table.to(DEV), kp2, vp2)
+    assert torch.equal(q3.cpu().view(n, q_heads, head_dim), q.to(dtype))
+
+
+@pytest.mark.parametrize("mnk", [(1, 777, 80), (5, 64, 64), (130, 192, 96), (67, 1000, 333), (300, 130, 1029)])
+def test_gemm_f32(mnk):
+    from leone_amd import ops
+    m, n, k = mnk
+    torch.manual_seed(6)
+    a, b = torch.randn(m, k, device=DEV), torch.randn(n, k, device=DEV)
+    out = ops.gemm_f32(a, b)
+    want = a.double() @ b.double().T
+    close(out, want, 1e-5 * math.sqrt(k), 1e-5, "gemm_f32")
+
+
+def test_argmax_rules():
+    """[1, 4, 4, NaN] -> 1; no finite value -> -1 (crates/leone/src/sampler/tests.rs:521-537)."""
+    from leone_amd import ops
+    nan, inf = float("nan"), float("inf")
+    rows = torch.tensor([[1.0, 4.0, 4.0, nan], [nan, -inf, inf, nan], [inf, -5.0, nan, -7.0], [0.0, 0.0, 0.0, 0.0]],
+                        device=DEV)
+    assert ops.argmax(rows).tolist() == [1, -1, 1, 0]
+    torch.manual_seed(7)
+    big = torch.randn(5, 151936, device=DEV)
+    big[2, 1000] = big[2, 150000] = 9.0
+    assert ops.argmax(big).tolist() == [int(r.argmax()) if i != 2 else 1000 for i, r in enumerate(big)]
