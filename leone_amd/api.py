@@ -1,0 +1,130 @@
+"""The Python entry point: load a model folder, generate from token ids or text.
+
+Mirrors the reference's ``Runtime::load`` + ``generate`` / ``generate_tokens``
+(crates/leone/src/runtime.rs:1305, 3524-3540) and its ``GenerateOptions``
+(crates/leone/src/runtime.rs:251-287): ``max_tokens`` there is ``max_new_tokens``
+here, the sampler options keep their command-line names.
+"""
+from __future__ import annotations
+
+import os
+from typing import Callable, Hashable, List, Optional, Sequence, Union
+
+import torch
+
+from .engine.engine import Engine
+from .engine.generate import GenerationResult, GenerationStats, generate_tokens
+from .engine.scheduler import SchedulerPolicy
+from .runtime import load_model, random_model
+from .sampling.sampler import SamplingParams
+
+
+def sampling_params(temperature: Optional[float] = None, seed: int = 0, top_k: Optional[int] = None,
+                    top_p: Optional[float] = None, min_p: Optional[float] = None,
+                    truncations: Optional[Sequence[tuple]] = None, repeat_penalty: float = 1.0,
+                    presence_penalty: float = 0.0, frequency_penalty: float = 0.0,
+                    penalty_window: int = 64) -> SamplingParams:
+    """``temperature`` None is greedy.  ``truncations`` gives stages in order; the named
+    shortcuts are appended as top-k, top-p, min-p."""
+    stages = list(truncations or [])
+    if top_k is not None:
+        stages.append(("top_k", top_k))
+    if top_p is not None:
+        stages.append(("top_p", top_p))
+    if min_p is not None:
+        stages.append(("min_p", min_p))
+    params = SamplingParams(temperature, stages, seed, repeat_penalty, presence_penalty, frequency_penalty,
+                            penalty_window)
+    if stages and temperature is None:
+        raise ValueError("truncation stages need a temperature; greedy takes the highest logit")
+    params.validate()
+    return params
+
+
+def default_num_pages(model, page_tokens: int, max_requests: int, max_context: int, bytes_per_token: int) -> int:
+    wanted = max_requests * ((max_context + page_tokens - 1) // page_tokens)
+    free, _ = torch.cuda.mem_get_info(model.device)
+    affordable = int(free * 0.8) // max(1, bytes_per_token * page_tokens)
+    return max(1, min(wanted, affordable))
+
+
+class Runtime:
+    """A loaded model with its cache, ready to generate."""
+
+    def __init__(self, model, *, num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
+                 page_tokens: int = 64, max_requests: int = 64, max_context: Optional[int] = None,
+                 policy: Optional[SchedulerPolicy] = None, tokenizer=None):
+        self.model = model
+        self.config = getattr(model, "config", None)
+        context = min(max_context or model.spec.max_positions, model.spec.max_positions)
+        if num_pages is None and max_tokens is None:
+            size = torch.empty((), dtype=model.dtype).element_size()
+            per_token = sum(2 * need.kv_heads * need.head_dim * size for need in model.cache_needs().values()
+                            if hasattr(need, "kv_heads"))
+            num_pages = default_num_pages(model, page_tokens, max_requests, context, per_token)
+        self.engine = Engine(model, num_pages=num_pages, max_tokens=max_tokens, page_tokens=page_tokens,
+                             max_requests=max_requests, max_context=context)
+        self.policy = policy or SchedulerPolicy(max_live_requests=max_requests)
+        self.tokenizer = tokenizer
+        self.last_stats: Optional[GenerationStats] = None
+
+    @classmethod
+    def load(cls, model_dir: str, dtype: Union[str, torch.dtype] = "bfloat16", device: Optional[str] = None,
+             **engine_options) -> "Runtime":
+        model = load_model(model_dir, dtype, device)
+        tokenizer = None
+        tokenizer_file = os.path.join(model_dir, "tokenizer.json")
+        if os.path.exists(tokenizer_file):
+            from tokenizers import Tokenizer
+            tokenizer = Tokenizer.from_file(tokenizer_file)
+        return cls(model, tokenizer=tokenizer, **engine_options)
+
+    @classmethod
+    def random(cls, config, seed: int = 0, dtype: Union[str, torch.dtype] = "bfloat16",
+               device: Optional[str] = None, **engine_options) -> "Runtime":
+        return cls(random_model(config, seed, dtype, device), **engine_options)
+
+    @property
+    def eos_token_id(self) -> Optional[int]:
+        return getattr(self.config, "eos_token_id", None)
+
+    def generate_tokens(self, prompts: Sequence[Sequence[int]], max_new_tokens: int,
+                        sampling: Optional[SamplingParams] = None, eos_token_id: Union[int, None, str] = "config",
+                        on_token: Optional[Callable[[Hashable, int], None]] = None,
+                        logit_observer: Optional[Callable] = None) -> List[GenerationResult]:
+        """Token ids in, token ids out, one result per prompt in order."""
+        eos = self.eos_token_id if eos_token_id == "config" else eos_token_id
+        results, stats = generate_tokens(self.engine, prompts, max_new_tokens, sampling, eos, self.policy, on_token,
+                                         logit_observer)
+        self.last_stats = stats
+        return results
+
+    def encode(self, text: str) -> List[int]:
+        if self.tokenizer is None:
+            raise ValueError("the model folder has no tokenizer.json; give token ids instead of text")
+        return list(self.tokenizer.encode(text).ids)
+
+    def decode(self, tokens: Sequence[int]) -> str:
+        if self.tokenizer is None:
+            raise ValueError("the model folder has no tokenizer.json")
+        return self.tokenizer.decode(list(tokens))
+
+    def generate(self, prompts: Sequence[str], max_new_tokens: int, sampling: Optional[SamplingParams] = None,
+                 **options) -> List[str]:
+        results = self.generate_tokens([self.encode(p) for p in prompts], max_new_tokens, sampling, **options)
+        return [self.decode(r.tokens) for r in results]
+
+
+def generate(model: Union[str, dict, Runtime], prompts: Sequence[Sequence[int]], max_new_tokens: int,
+             temperature: Optional[float] = None, seed: int = 0, top_k: Optional[int] = None,
+             top_p: Optional[float] = None, eos_token_id: Union[int, None, str] = "config",
+             dtype: str = "bfloat16", **engine_options) -> List[GenerationResult]:
+    """One call: ``model`` is a model folder, a config.json mapping (random weights from ``seed``) or a Runtime."""
+    if isinstance(model, Runtime):
+        runtime = model
+    elif isinstance(model, dict):
+        runtime = Runtime.random(model, seed, dtype, **engine_options)
+    else:
+        runtime = Runtime.load(model, dtype, **engine_options)
+    return runtime.generate_tokens(prompts, max_new_tokens, sampling_params(temperature, seed, top_k, top_p),
+                                   eos_token_id)

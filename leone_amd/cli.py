@@ -1,0 +1,290 @@
+"""Command line in the reference's manner: ``leone generate -m <model> -p <prompt> -n <tokens>``.
+
+Subcommands and option names follow crates/leone-cli/src/main.rs:418-460 (generate, eval) and
+crates/leone-cli/src/doctor.rs:303-346 (doctor).  Where the reference selects a backend or a
+quantised cache (``--backend``, ``--kv``) this engine has ``--dtype bfloat16|float32``, which sets
+weights, activations and cache alike.  A model without tokenizer.json takes ``--prompt-tokens``.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import struct
+import sys
+import time
+from typing import List, Optional
+
+_STAGE_FLAGS = {"--top-k": "top_k", "--top-p": "top_p", "--min-p": "min_p", "--top-a": "top_a", "--tfs": "tfs",
+                "--typical": "typical", "--epsilon": "epsilon", "--eta": "eta", "--min-k": "min_k",
+                "--top-n-sigma": "top_n_sigma"}
+
+
+class _Stage(argparse.Action):
+    """Truncation stages apply in the order their flags are given."""
+
+    def __call__(self, parser, namespace, values, option_string=None):
+        stages = list(getattr(namespace, "truncations", None) or [])
+        stages.append((_STAGE_FLAGS[option_string], float(values)))
+        namespace.truncations = stages
+
+
+def _add_sampling(parser: argparse.ArgumentParser) -> None:
+    parser.add_argument("--seed", type=int, default=0, help="Seed the sampler. Default: 0")
+    parser.add_argument("--temp", "--temperature", dest="temp", type=float, default=None,
+                        help="Scale logits by 1/t (without it: greedy)")
+    helps = {"--top-k": "Keep the n highest-probability tokens", "--top-p": "Keep the smallest set covering mass p",
+             "--min-p": "Keep tokens with at least p times the highest probability",
+             "--top-a": "Keep tokens with at least a times the highest probability squared",
+             "--tfs": "Tail-free sampling with share z", "--typical": "Locally typical sampling with mass p",
+             "--epsilon": "Keep tokens with probability at least e", "--eta": "Eta sampling with floor e",
+             "--min-k": "Min-k on raw logits with fallback tau", "--top-n-sigma": "Keep raw logits within n deviations"}
+    for flag, text in helps.items():
+        parser.add_argument(flag, action=_Stage, help=text)
+    parser.add_argument("--repeat-penalty", type=float, default=1.0, help="Apply sign-aware scaling to seen logits")
+    parser.add_argument("--presence-penalty", type=float, default=0.0, help="Subtract once from any seen token")
+    parser.add_argument("--frequency-penalty", type=float, default=0.0, help="Subtract once per earlier occurrence")
+    parser.add_argument("--penalty-window", type=int, default=64, help="History the penalties count over; 0 disables")
+
+
+def _sampling_from(args):
+    from .sampling.sampler import SamplingParams
+    params = SamplingParams(args.temp, list(getattr(args, "truncations", None) or []), args.seed,
+                            args.repeat_penalty, args.presence_penalty, args.frequency_penalty, args.penalty_window)
+    if params.truncations and params.temperature is None:
+        raise SystemExit("error: truncation flags need --temp; without it generation is greedy")
+    params.validate()
+    return params
+
+
+def build_parser() -> argparse.ArgumentParser:
+    parser = argparse.ArgumentParser(prog="leone", description="Qwen3 dense inference on MI355X")
+    sub = parser.add_subparsers(dest="command")
+
+    g = sub.add_parser("generate", help="Generate text", usage="leone generate -m <model> -p <prompt> -n <tokens> [options]")
+    g.add_argument("-m", "--model", required=True, help="Model folder (config.json, model.safetensors)")
+    g.add_argument("-p", "--prompt", help="Prompt text (needs tokenizer.json in the model folder)")
+    g.add_argument("--prompt-tokens", help="Prompt as comma-separated token ids")
+    g.add_argument("-n", "--tokens", type=int, required=True, help="Number of tokens to generate")
+    g.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"], help="Weights, activations and cache")
+    g.add_argument("--eager-decode", action="store_true", help="Disable decode graph replay")
+    g.add_argument("--prefill-chunk", type=int, default=2048, help="Longest prompt portion per step")
+    g.add_argument("--max-context", type=int, default=None, help="Context the cache is sized for")
+    g.add_argument("--debug-tokens", help="Write generated token IDs as JSON")
+    g.add_argument("--debug-logits", help="Write the top five logits for each token")
+    g.add_argument("--ignore-eos", action="store_true", help="Do not stop at the end token")
+    _add_sampling(g)
+
+    d = sub.add_parser("doctor", help="Check the platform, the kernel library and a model folder")
+    d.add_argument("-m", "--model", help="Model folder to check (metadata only)")
+    d.add_argument("--probe", action="store_true", help="Also load the weights onto the GPU")
+    d.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+
+    e = sub.add_parser("eval", help="Evaluate model logits for given token ids")
+    e.add_argument("-m", "--model", required=True)
+    e.add_argument("--tokens", required=True, help="Token ids as little-endian u32")
+    e.add_argument("--logits", required=True, help="Output: row-major little-endian f32 logits")
+    e.add_argument("--metadata", help="Write execution metadata as JSON")
+    e.add_argument("--window", type=int, default=512, help="Overlapping evaluation window. Default: 512")
+    e.add_argument("--position-limit", type=int, default=None, help="Score only the first n positions")
+    e.add_argument("--prefill-chunk", type=int, default=None, help="Feed windows in chunks of n tokens")
+    e.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+
+    r = sub.add_parser("random-model", help="Write a model folder with seeded random weights")
+    r.add_argument("--config", required=True, help="config.json to build from")
+    r.add_argument("--seed", type=int, default=0)
+    r.add_argument("--out", required=True)
+    r.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+
+    b = sub.add_parser("bench", help="Measure decode and prefill throughput")
+    b.add_argument("rest", nargs=argparse.REMAINDER)
+    return parser
+
+
+def cmd_generate(args) -> int:
+    from .api import Runtime
+    from .engine.scheduler import SchedulerPolicy
+
+    sampling = _sampling_from(args)
+    if args.tokens <= 0:
+        raise SystemExit("error: -n must be positive")
+    if (args.prompt is None) == (args.prompt_tokens is None):
+        raise SystemExit("error: give exactly one of -p/--prompt and --prompt-tokens")
+    runtime = Runtime.load(args.model, args.dtype, max_requests=1, max_context=args.max_context,
+                           policy=SchedulerPolicy(max_live_requests=1, prefill_chunk_tokens=args.prefill_chunk,
+                                                  max_step_tokens=max(args.prefill_chunk, 1)))
+    if args.prompt is not None:
+        prompt = runtime.encode(args.prompt)
+    else:
+        prompt = [int(t) for t in args.prompt_tokens.replace(",", " ").split()]
+    top_five: List[str] = []
+    observe = None
+    if args.debug_logits:
+        def observe(request, position, row):
+            values, ids = row.topk(min(5, row.numel()))
+            top_five.append(" ".join(f"{int(i)}:{float(v):.6f}:0x{struct.unpack('<I', struct.pack('<f', float(v)))[0]:08x}"
+                                     for v, i in zip(values.tolist(), ids.tolist())))
+
+    def on_token(request, token):
+        if runtime.tokenizer is not None:
+            sys.stdout.write(runtime.decode([token]))
+        else:
+            sys.stdout.write(f"{token} ")
+        sys.stdout.flush()
+
+    eos = None if args.ignore_eos else "config"
+    results = runtime.generate_tokens([prompt], args.tokens, sampling, eos_token_id=eos, on_token=on_token,
+                                      logit_observer=observe)
+    stats = runtime.last_stats
+    sys.stdout.write("\n")
+    if args.debug_tokens:
+        with open(args.debug_tokens, "w") as handle:
+            json.dump(results[0].tokens, handle)
+    if args.debug_logits:
+        with open(args.debug_logits, "w") as handle:
+            handle.write("\n".join(top_five) + "\n")
+    print(file=sys.stderr)
+    print(f"decode: {stats.decode_rate:.2f} tok/s", file=sys.stderr)
+    print(f"prefill: {stats.prefill_rate:.2f} tok/s", file=sys.stderr)
+    print(f"tokens emitted: {stats.emitted_tokens}", file=sys.stderr)
+    print(f"finish: {results[0].finish_reason}", file=sys.stderr)
+    return 0
+
+
+def cmd_doctor(args) -> int:
+    import torch
+
+    print(f"python {sys.version.split()[0]}, torch {torch.__version__}, hip {torch.version.hip}")
+    ok = True
+    if torch.cuda.is_available():
+        props = torch.cuda.get_device_properties(0)
+        print(f"gpu: {props.name}, {props.total_memory / 2**30:.1f} GiB, {props.multi_processor_count} CUs")
+    else:
+        print("gpu: none visible (this engine has no CPU path)")
+        ok = False
+    try:
+        from .csrc import build
+        path = build.library_path() or build.build(verbose=True)
+        print(f"kernel library: {path}")
+    except Exception as error:  # noqa: BLE001 - doctor reports, it does not raise
+        print(f"kernel library: FAILED: {error}")
+        ok = False
+    if args.model:
+        from .architectures import config_from_dir, model_spec_for
+        from .parts.model import DecoderModel
+        from .weights import loader
+        from .weights.safetensors_io import ModelFiles
+        config = config_from_dir(args.model)
+        print(f"architecture: {config.architecture}")
+        print(f"context limit: {config.max_position_embeddings}")
+        model = DecoderModel(model_spec_for(config), torch.float32, "cpu")
+        files = ModelFiles(args.model)
+        total = 0
+        by_type = {}
+        for entry in files.entries.values():
+            total += entry.nbytes
+            by_type[entry.dtype_name] = by_type.get(entry.dtype_name, 0) + entry.nbytes
+        print(f"tensors: {len(files.entries)}, {total / 2**20:.1f} MiB " +
+              ", ".join(f"{k} {v / 2**20:.1f} MiB" for k, v in sorted(by_type.items())))
+        found = {n: (e.shape, e.dtype) for n, e in files.entries.items()}
+        loader.check(model.tensor_specs(), found, args.model, model.spec.ignore_tensors)
+        print("tensor names and shapes: ok")
+        size = 2 if args.dtype == "bfloat16" else 4
+        per_token = sum(2 * need.kv_heads * need.head_dim * size for need in model.cache_needs().values()
+                        if hasattr(need, "kv_heads"))
+        print(f"cache bytes per token ({args.dtype}): {per_token}")
+        if torch.cuda.is_available():
+            free, _ = torch.cuda.mem_get_info(0)
+            room = free - total * (2 if args.dtype == "float32" else 1)
+            print(f"tokens of context that fit beside the weights: {max(0, int(room * 0.9) // max(1, per_token))}")
+        if args.probe:
+            from .runtime import load_model
+            started = time.time()
+            load_model(args.model, args.dtype)
+            print(f"probe: weights loaded in {time.time() - started:.1f}s")
+    return 0 if ok else 1
+
+
+def cmd_eval(args) -> int:
+    """Windows of W tokens, stride W-1, a fresh cache per window; the row after token i scores token i+1
+    (crates/leone/src/runtime.rs:1673-1996, crates/leone-cli/src/eval.rs:526-558)."""
+    import hashlib
+    import numpy as np
+    from .engine.engine import Engine, StepEntry
+    from .runtime import load_model
+
+    tokens = np.fromfile(args.tokens, dtype="<u4").astype(np.int64)
+    if args.position_limit is not None:
+        tokens = tokens[:args.position_limit]
+    if tokens.size < 2:
+        raise SystemExit("error: need at least two tokens")
+    if args.window < 2:
+        raise SystemExit("error: --window must be at least 2")
+    model = load_model(args.model, args.dtype)
+    window = min(args.window, model.spec.max_positions)
+    engine = Engine(model, max_tokens=window + 64, page_tokens=64, max_requests=1, max_context=window)
+    rows = 0
+    digest = hashlib.sha256()
+    with open(args.logits, "wb") as out:
+        start = 0
+        while start < tokens.size - 1:
+            piece = tokens[start:start + window].tolist()
+            feed = piece[:-1]   # the last token of a window is only a target
+            chunk = args.prefill_chunk or 1
+            at = 0
+            while at < len(feed):
+                part = feed[at:at + chunk]
+                logits = engine.step([StepEntry("w", part, list(range(len(part))))]).logits
+                data = logits.cpu().numpy().astype("<f4").tobytes()
+                out.write(data)
+                digest.update(data)
+                rows += len(part)
+                at += len(part)
+            engine.release("w")
+            start += window - 1
+    if args.metadata:
+        with open(args.metadata, "w") as handle:
+            json.dump({"schema": "leone-amd.eval.v1", "model": os.path.abspath(args.model), "dtype": args.dtype,
+                       "window": window, "prefill_chunk": args.prefill_chunk, "tokens": int(tokens.size),
+                       "rows": rows, "vocab": model.spec.vocab_size,
+                       "row_label": "row i of a window holds the logits after feeding its token i",
+                       "logits_sha256": digest.hexdigest()}, handle, indent=2)
+    print(f"wrote {rows} rows of {model.spec.vocab_size} logits", file=sys.stderr)
+    return 0
+
+
+def cmd_random_model(args) -> int:
+    import torch
+    from .architectures import config_from_dict
+    from .weights.random_init import write_model_dir
+    with open(args.config) as handle:
+        config = config_from_dict(json.load(handle))
+    write_model_dir(args.out, config, args.seed, torch.bfloat16 if args.dtype == "bfloat16" else torch.float32)
+    print(args.out)
+    return 0
+
+
+def main(argv: Optional[List[str]] = None) -> int:
+    parser = build_parser()
+    args = parser.parse_args(argv)
+    if args.command is None:
+        from . import __version__
+        print(f"leone-amd {__version__}")
+        return 0
+    if args.command == "generate":
+        return cmd_generate(args)
+    if args.command == "doctor":
+        return cmd_doctor(args)
+    if args.command == "eval":
+        return cmd_eval(args)
+    if args.command == "random-model":
+        return cmd_random_model(args)
+    if args.command == "bench":
+        from .benchmark import main as bench_main
+        return bench_main(args.rest)
+    parser.error(f"unknown command {args.command}")
+    return 2
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -121,6 +121,9 @@ class Engine:
         """Runs a step whose pages the caller has reserved; commits on success, rolls back on failure."""
         try:
             self._validate(entries)
+            for e in entries:
+                if self.cache.length(e.request) == 0:
+                    self.pools.zero_state(self.cache.slot(e.request))   # a request's state starts from zero
             tokens, context, rows = self._build_context(entries)
             caches = self.pools.views(context.block_tables)
             logits = self.model.forward(tokens, context, caches)

@@ -1,0 +1,186 @@
+"""Generation: the scheduler's plans run through the engine's step, tokens chosen by the sampler.
+
+The reference's entry points are ``Runtime::load`` and ``generate`` / ``generate_tokens`` with
+``GenerateOptions`` (crates/leone/src/runtime.rs:1305, 3524-3540, 251-287) returning the generated
+tokens, why generation stopped and timing (crates/leone/src/runtime.rs:442-452, 402-427).
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Callable, Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..sampling import rng
+from ..sampling.sampler import SamplerError, SamplingParams, sample as host_sample
+from .engine import Engine, StepEntry
+from .scheduler import Finished, PlannedEntry, Reject, Request, Scheduler, SchedulerPolicy
+
+
+@dataclass
+class GenerationStats:
+    prompt_tokens: int = 0
+    emitted_tokens: int = 0
+    steps: int = 0
+    prefill_seconds: float = 0.0     # steps that held a prompt portion
+    decode_seconds: float = 0.0      # steps of decoded tokens only
+    prefill_tokens: int = 0
+    decode_tokens: int = 0
+    preemptions: int = 0
+
+    @property
+    def prefill_rate(self) -> float:
+        return self.prefill_tokens / self.prefill_seconds if self.prefill_seconds > 0 else 0.0
+
+    @property
+    def decode_rate(self) -> float:
+        return self.decode_tokens / self.decode_seconds if self.decode_seconds > 0 else 0.0
+
+
+@dataclass
+class GenerationResult:
+    id: Hashable
+    prompt_tokens: List[int]
+    tokens: List[int]
+    finish_reason: str
+
+
+class RequestRejected(ValueError):
+    def __init__(self, request_id, reason: Reject):
+        super().__init__(f"request {request_id!r} rejected: {reason.value}")
+        self.reason = reason
+
+
+def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params: Dict[Hashable, SamplingParams],
+                  histories: Dict[Hashable, Sequence[int]]) -> Dict[Hashable, int]:
+    """One token per sampled entry; ``logits`` has one row per such entry, in order.
+
+    Greedy and plain-temperature rows are chosen by the device kernels; rows with truncation stages
+    or penalties are copied to the host and go through the double-precision sampler."""
+    rows = [e for e in entries if e.sample]
+    if not rows:
+        return {}
+    policies = [params[e.request] or SamplingParams() for e in rows]
+    for p in policies:
+        p.validate()
+    out: Dict[Hashable, int] = {}
+    on_device = [i for i, p in enumerate(policies) if p.device_eligible]
+    greedy = [i for i in on_device if policies[i].greedy]
+    scaled = [i for i in on_device if not policies[i].greedy]
+    if greedy:
+        picked = ops.argmax(logits).cpu().tolist()
+        for i in greedy:
+            out[rows[i].request] = picked[i]
+    if scaled:
+        temps = torch.tensor([policies[i].temperature if i in scaled else 1.0 for i in range(len(rows))],
+                             dtype=torch.float64, device=logits.device)
+        draws = torch.tensor([rng.uniform(policies[i].seed, rows[i].sample_position) for i in range(len(rows))],
+                             dtype=torch.float64, device=logits.device)
+        picked = ops.sample_temperature(logits, temps, draws).cpu().tolist()
+        for i in scaled:
+            out[rows[i].request] = picked[i]
+    host_rows = [i for i in range(len(rows)) if i not in on_device]
+    if host_rows:
+        index = torch.tensor(host_rows, dtype=torch.long, device=logits.device)
+        copied = logits.index_select(0, index).cpu().numpy()
+        for k, i in enumerate(host_rows):
+            e = rows[i]
+            out[e.request] = host_sample(copied[k], policies[i], e.sample_position, histories[e.request])
+    for e in rows:
+        if out[e.request] < 0:
+            raise SamplerError(f"request {e.request!r}: no finite logit at position {e.sample_position}")
+    return out
+
+
+class Generator:
+    """Runs requests to completion: scheduler above, engine below."""
+
+    def __init__(self, engine: Engine, policy: Optional[SchedulerPolicy] = None):
+        self.engine = engine
+        self.scheduler = Scheduler(policy or SchedulerPolicy(max_live_requests=engine.cache.max_requests),
+                                   engine.cache)
+        self.params: Dict[Hashable, SamplingParams] = {}
+        self.stats = GenerationStats()
+        # Called with (request, position, float32 logits row on the device) for every sampled row.
+        self.logit_observer: Optional[Callable[[Hashable, int, torch.Tensor], None]] = None
+
+    def submit(self, request_id: Hashable, prompt: Sequence[int], max_new_tokens: int,
+               sampling: Optional[SamplingParams] = None, eos_token_id: Optional[int] = None) -> None:
+        sampling = sampling or SamplingParams()
+        sampling.validate()
+        for t in prompt:
+            if not 0 <= int(t) < self.engine.vocab_size:
+                raise ValueError(f"request {request_id!r}: token {t} is outside the vocabulary")
+        reason = self.scheduler.submit(Request(request_id, [int(t) for t in prompt], max_new_tokens, sampling,
+                                               eos_token_id))
+        if reason is not None:
+            raise RequestRejected(request_id, reason)
+        self.params[request_id] = sampling
+        self.stats.prompt_tokens += len(prompt)
+
+    def step(self, on_token: Optional[Callable[[Hashable, int], None]] = None) -> List[Finished]:
+        """Plans and runs one step.  Returns the requests that finished in it."""
+        scheduler = self.scheduler
+        plan = scheduler.plan()
+        if not plan:
+            return []
+        started = time.perf_counter()
+        try:
+            entries = [StepEntry(e.request, e.tokens, [len(e.tokens) - 1] if e.sample else []) for e in plan]
+            output = self.engine.run_reserved(entries)
+            histories = {e.request: scheduler.live[e.request].tokens for e in plan if e.sample}
+            sampled = choose_tokens(output.logits, plan, self.params, histories) if output.logits is not None else {}
+            if self.logit_observer is not None and output.logits is not None:
+                for row, e in enumerate([e for e in plan if e.sample]):
+                    self.logit_observer(e.request, e.sample_position, output.logits[row])
+        except Exception:
+            scheduler.abort()
+            raise
+        elapsed = time.perf_counter() - started
+        rows = sum(len(e.tokens) for e in plan)
+        if all(len(e.tokens) == 1 and e.start > 0 for e in plan):
+            self.stats.decode_seconds += elapsed
+            self.stats.decode_tokens += rows
+        else:
+            self.stats.prefill_seconds += elapsed
+            self.stats.prefill_tokens += rows
+        self.stats.steps += 1
+        self.stats.emitted_tokens += len(sampled)
+        if on_token is not None:
+            for e in plan:
+                if e.sample:
+                    on_token(e.request, sampled[e.request])
+        done = scheduler.complete(sampled)
+        self.stats.preemptions = scheduler.stats.preemptions
+        return done
+
+    def run(self, on_token: Optional[Callable[[Hashable, int], None]] = None,
+            cancelled: Optional[Callable[[], bool]] = None) -> List[Finished]:
+        finished: List[Finished] = []
+        while self.scheduler.has_work():
+            if cancelled is not None and cancelled():
+                for rid in list(self.scheduler.live) + [q.request.id for q in self.scheduler.queue]:
+                    self.scheduler.cancel(rid)
+            before = len(self.scheduler.finished)
+            self.step(on_token)
+            finished.extend(self.scheduler.finished[before:])
+        return finished
+
+
+def generate_tokens(engine: Engine, prompts: Sequence[Sequence[int]], max_new_tokens: int,
+                    sampling: Optional[SamplingParams] = None, eos_token_id: Optional[int] = None,
+                    policy: Optional[SchedulerPolicy] = None,
+                    on_token: Optional[Callable[[Hashable, int], None]] = None,
+                    logit_observer: Optional[Callable[[Hashable, int, torch.Tensor], None]] = None):
+    """Generates for every prompt (token ids); returns results in prompt order and the run's statistics."""
+    generator = Generator(engine, policy)
+    generator.logit_observer = logit_observer
+    for i, prompt in enumerate(prompts):
+        generator.submit(i, prompt, max_new_tokens, sampling, eos_token_id)
+    finished = {f.id: f for f in generator.run(on_token)}
+    results = [GenerationResult(i, list(finished[i].prompt), list(finished[i].tokens), finished[i].reason)
+               for i in range(len(prompts))]
+    return results, generator.stats

@@ -1,0 +1,241 @@
+"""Sampling policies, in double precision over a float32 logits row.
+
+Greedy is a policy of its own, not temperature zero: the highest finite logit,
+the lowest index on a tie, no random draw (crates/leone/src/sampler.rs:45-48, 787-799).
+Temperature: candidates are the finite logits sorted descending (ties by lower
+index), weights exp(l/t - l_max/t), normalised (crates/leone/src/sampler.rs:502-534).
+Truncation stages run in the order given, each on the previous stage's
+renormalised distribution, each keeping at least one token; min-k and
+top-n-sigma look at raw logits and run before the others
+(crates/leone/src/sampler.rs:184-234, 536-557, 559-606).  The token is the first, in id
+order, whose cumulative probability exceeds the uniform draw; the last eligible
+token if rounding leaves none (crates/leone/src/sampler.rs:843-858).  Penalties
+rewrite the logits from the token history before all this
+(crates/leone/src/penalty.rs:160-196).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import rng
+
+_FRACTION_STAGES = ("top_p", "min_p", "top_a", "tfs", "typical", "epsilon", "eta")
+_RAW_STAGES = ("min_k", "top_n_sigma")
+STAGES = ("top_k",) + _FRACTION_STAGES + _RAW_STAGES
+
+
+class SamplerError(ValueError):
+    pass
+
+
+@dataclass
+class SamplingParams:
+    """temperature None = greedy.  ``truncations`` is an ordered list of (stage, value)."""
+    temperature: Optional[float] = None
+    truncations: List[Tuple[str, float]] = field(default_factory=list)
+    seed: int = 0
+    repeat_penalty: float = 1.0
+    presence_penalty: float = 0.0
+    frequency_penalty: float = 0.0
+    penalty_window: int = 64          # 0 disables the counting penalties
+
+    def validate(self) -> None:
+        t = self.temperature
+        if t is not None and (not math.isfinite(t) or t <= 0.0):
+            raise SamplerError("temperature must be finite and positive (leave it out for greedy)")
+        for stage, value in self.truncations:
+            if stage not in STAGES:
+                raise SamplerError(f"unknown truncation stage {stage!r}")
+            if stage == "top_k":
+                if int(value) != value or value <= 0:
+                    raise SamplerError("top-k must be a positive integer")
+            elif stage in _RAW_STAGES:
+                if not math.isfinite(value) or value < 0.0:
+                    raise SamplerError(f"{stage} must be finite and not negative")
+            elif not math.isfinite(value) or value <= 0.0 or value > 1.0:
+                raise SamplerError(f"{stage} must lie in (0, 1]")
+        if not math.isfinite(self.repeat_penalty) or self.repeat_penalty <= 0.0:
+            raise SamplerError("repeat penalty must be finite and positive")
+        if not math.isfinite(self.presence_penalty) or not math.isfinite(self.frequency_penalty):
+            raise SamplerError("presence and frequency penalties must be finite")
+        if self.penalty_window < 0:
+            raise SamplerError("penalty window must not be negative")
+
+    @property
+    def greedy(self) -> bool:
+        return self.temperature is None
+
+    @property
+    def penalties_active(self) -> bool:
+        return self.penalty_window > 0 and (self.repeat_penalty != 1.0 or self.presence_penalty != 0.0
+                                            or self.frequency_penalty != 0.0)
+
+    @property
+    def device_eligible(self) -> bool:
+        """Greedy or plain temperature without penalties can be sampled by the device kernels."""
+        return not self.truncations and not self.penalties_active
+
+
+def apply_penalties(logits: np.ndarray, history: Sequence[int], params: SamplingParams) -> np.ndarray:
+    """Positive logits of seen tokens are divided by the repeat penalty, negative ones multiplied;
+    then presence is subtracted once and frequency once per occurrence, over the last
+    ``penalty_window`` tokens of the history (prompt included)."""
+    if not params.penalties_active:
+        return logits
+    out = np.array(logits, dtype=np.float32, copy=True)
+    recent = list(history)[-params.penalty_window:]
+    counts = {}
+    for token in recent:
+        counts[token] = counts.get(token, 0) + 1
+    for token, count in sorted(counts.items()):
+        if not 0 <= token < out.shape[0]:
+            continue
+        value = float(out[token])
+        value = value / params.repeat_penalty if value > 0.0 else value * params.repeat_penalty
+        value -= params.presence_penalty
+        value -= params.frequency_penalty * count
+        out[token] = np.float32(value)
+    return out
+
+
+def argmax(logits: np.ndarray) -> int:
+    """Highest finite value, lowest index on a tie; -1 if nothing is finite."""
+    finite = np.isfinite(logits)
+    if not finite.any():
+        return -1
+    masked = np.where(finite, logits, -np.inf)
+    return int(np.argmax(masked))
+
+
+def _entropy(p: np.ndarray) -> float:
+    q = p[p > 0.0]
+    return float(-(q * np.log(q)).sum())
+
+
+def _renormalise(p: np.ndarray) -> np.ndarray:
+    total = p.sum()
+    if not math.isfinite(total) or total <= 0.0:
+        raise SamplerError("no finite logit")
+    return p / total
+
+
+def _threshold_keep(p: np.ndarray, floor: float) -> int:
+    below = np.nonzero(~(p >= floor))[0]
+    return int(below[0]) if below.size else p.size
+
+
+def _keep(stage: str, value: float, p: np.ndarray) -> Optional[int]:
+    if stage == "top_k":
+        return min(int(value), p.size)
+    if stage == "top_p":
+        reached = np.nonzero(np.cumsum(p) >= value)[0]
+        return int(reached[0]) + 1 if reached.size else p.size
+    if stage == "min_p":
+        return _threshold_keep(p, value * p[0])
+    if stage == "top_a":
+        return _threshold_keep(p, value * p[0] * p[0])
+    if stage == "epsilon":
+        return _threshold_keep(p, value)
+    if stage == "eta":
+        return _threshold_keep(p, min(value, math.sqrt(value) * math.exp(-_entropy(p))))
+    if stage == "tfs":
+        if p.size < 3:
+            return p.size
+        second = np.abs(p[:-2] - 2.0 * p[1:-1] + p[2:])
+        total = second.sum()
+        if not math.isfinite(total) or total <= 0.0:
+            return p.size
+        covered = np.cumsum(second / total)
+        over = np.nonzero(~(covered <= value))[0]
+        return 1 + (int(over[0]) if over.size else second.size)
+    return None
+
+
+def _raw_keep(stage: str, value: float, sorted_logits: np.ndarray) -> int:
+    n = sorted_logits.size
+    if n < 2:
+        return n
+    if stage == "top_n_sigma":
+        deviation = float(np.sqrt(((sorted_logits - sorted_logits.mean()) ** 2).mean()))
+        if not math.isfinite(deviation):
+            return n
+        cut = sorted_logits[0] - value * deviation
+        return max(1, _threshold_keep(sorted_logits, cut))
+    # min-k: the sharpest rank-weighted drop, with a fallback rank for nearly flat rows
+    span = float(sorted_logits[0] - sorted_logits[-1]) + 1e-8
+    if not math.isfinite(span) or span <= 0.0:
+        return n
+    gaps = (sorted_logits[:-1] - sorted_logits[1:]) / span / np.arange(1, n)
+    cliff = int(np.argmax(gaps)) + 1
+    fallback = math.floor(value / span)
+    fallback = min(int(fallback), n) if math.isfinite(fallback) and fallback >= 0 else n
+    return min(max(cliff, fallback, 1), n)
+
+
+def distribution(logits: np.ndarray, params: SamplingParams) -> np.ndarray:
+    """The probabilities (float64, zeros outside the kept set) the policy gives one logits row."""
+    params.validate()
+    logits = np.asarray(logits, dtype=np.float32)
+    if logits.size == 0:
+        raise SamplerError("empty logits row")
+    out = np.zeros(logits.shape[0], dtype=np.float64)
+    if params.greedy:
+        best = argmax(logits)
+        if best < 0:
+            raise SamplerError("no finite logit")
+        out[best] = 1.0
+        return out
+    ids = np.nonzero(np.isfinite(logits))[0]
+    if ids.size == 0:
+        raise SamplerError("no finite logit")
+    values = logits[ids].astype(np.float64)
+    order = ids[np.lexsort((ids, -values))]          # descending logit, ties by lower id
+    sorted_logits = logits[order].astype(np.float64)
+    t = float(params.temperature)
+    kept = _renormalise(np.exp(sorted_logits / t - sorted_logits[0] / t))
+    raw = [(s, v) for s, v in params.truncations if s in _RAW_STAGES]
+    for stage, value in raw:
+        n = max(1, _raw_keep(stage, value, sorted_logits[:order.size]))
+        order, kept = order[:n], kept[:n]
+    if raw:
+        kept = _renormalise(kept)
+    for stage, value in params.truncations:
+        if stage in _RAW_STAGES:
+            continue
+        if stage == "typical":
+            score = np.abs(-np.log(kept) - _entropy(kept))
+            by_score = np.lexsort((np.arange(kept.size), score))
+            reached = np.nonzero(np.cumsum(kept[by_score]) >= value)[0]
+            chosen = np.sort(by_score[:int(reached[0]) + 1 if reached.size else kept.size])
+            order, kept = order[chosen], _renormalise(kept[chosen])
+            continue
+        n = max(1, _keep(stage, value, kept))
+        order, kept = order[:n], _renormalise(kept[:n])
+    out[order] = kept
+    return out
+
+
+def select(probabilities: np.ndarray, u: float) -> int:
+    """First token, in id order, whose cumulative probability exceeds ``u``."""
+    eligible = np.nonzero(probabilities > 0.0)[0]
+    if eligible.size == 0:
+        raise SamplerError("no finite logit")
+    cumulative = np.cumsum(probabilities[eligible])
+    hit = np.nonzero(u < cumulative)[0]
+    return int(eligible[hit[0]] if hit.size else eligible[-1])
+
+
+def sample(logits: np.ndarray, params: SamplingParams, position: int, history: Sequence[int] = ()) -> int:
+    """One token for one row.  ``position`` is the absolute index of the token whose logits these are."""
+    logits = apply_penalties(np.asarray(logits, dtype=np.float32), history, params)
+    if params.greedy:
+        params.validate()
+        best = argmax(logits)
+        if best < 0:
+            raise SamplerError("no finite logit")
+        return best
+    return select(distribution(logits, params), rng.uniform(params.seed, position))

@@ -1,0 +1,142 @@
+"""The cache manager: no page lost, held twice or freed twice, under random orders of requests."""
+import random
+
+import pytest
+
+from leone_amd.cache.manager import CacheError, CacheManager, GroupSpec, OutOfPages, OutOfSlots
+
+
+def test_reserve_commit_release_and_reuse():
+    m = CacheManager([GroupSpec(4, 16)], max_requests=2, max_context=64)
+    m.admit("a")
+    m.reserve("a", 17)
+    assert len(m.table("a", 0)) == 2
+    first_pages = list(m.table("a", 0))
+    m.commit("a")
+    assert m.length("a") == 17 and m.free_pages(0) == 2
+    m.reserve("a", 15)            # fills the second page exactly: no new page
+    assert m.free_pages(0) == 2
+    m.commit("a")
+    m.reserve("a", 1)             # crosses into a third page
+    assert m.free_pages(0) == 1
+    m.commit("a")
+    m.release("a")
+    assert m.free_pages(0) == 4 and m.free_slots() == 2
+    m.admit("b")
+    m.reserve("b", 1)
+    assert m.table("b", 0)[0] in first_pages + [3 - sum(first_pages) % 4, 0, 1, 2, 3]
+    m.check()
+
+
+def test_a_freed_page_is_the_next_one_used():
+    m = CacheManager([GroupSpec(3, 8)], 3, 64)
+    m.admit("a"); m.reserve("a", 8); m.commit("a")
+    page = m.table("a", 0)[0]
+    m.release("a")
+    m.admit("b"); m.reserve("b", 3)
+    assert m.table("b", 0) == [page]
+
+
+def test_failed_reservation_changes_nothing_at_every_cut():
+    # the reference rolls a failed allocation back at every cut point (crates/leone/src/kv.rs:1451-1473)
+    for second_group_pages in range(0, 4):
+        m = CacheManager([GroupSpec(8, 4), GroupSpec(max(1, second_group_pages), 4)], 2, 64)
+        m.admit("a")
+        before = (m.free_pages(0), m.free_pages(1), list(m.table("a", 0)), list(m.table("a", 1)))
+        if second_group_pages < 4:
+            with pytest.raises(OutOfPages) as error:
+                m.reserve("a", 16)
+            assert error.value.group == 1
+            assert before == (m.free_pages(0), m.free_pages(1), list(m.table("a", 0)), list(m.table("a", 1)))
+            m.check()
+
+
+def test_rollback_is_exact():
+    m = CacheManager([GroupSpec(6, 4)], 2, 64)
+    m.admit("a"); m.reserve("a", 6); m.commit("a")
+    snapshot = (list(m.table("a", 0)), m.free_pages(0), m.length("a"))
+    m.reserve("a", 9)
+    assert m.free_pages(0) < snapshot[1]
+    m.rollback("a")
+    assert snapshot == (list(m.table("a", 0)), m.free_pages(0), m.length("a"))
+    m.reserve("a", 2); m.commit("a")
+    assert m.length("a") == 8
+    m.check()
+
+
+def test_contract_violations():
+    m = CacheManager([GroupSpec(4, 4)], 1, 10)
+    with pytest.raises(CacheError):
+        m.reserve("ghost", 1)
+    m.admit("a")
+    with pytest.raises(CacheError):
+        m.admit("a")
+    with pytest.raises(OutOfSlots):
+        m.admit("b")
+    with pytest.raises(CacheError):
+        m.commit("a")                       # nothing reserved
+    m.reserve("a", 3)
+    with pytest.raises(CacheError):
+        m.reserve("a", 1)                   # one transaction at a time
+    with pytest.raises(CacheError):
+        m.commit("a", 2)                    # not what was reserved
+    m.commit("a", 3)
+    with pytest.raises(CacheError):
+        m.reserve("a", 8)                   # beyond the context of 10
+    m.release("a")
+    with pytest.raises(CacheError):
+        m.release("a")                      # freed twice
+    m.check()
+
+
+def test_window_group_gives_pages_back_as_the_window_passes():
+    m = CacheManager([GroupSpec(32, 4), GroupSpec(5, 4, window=6)], 1, 128)
+    m.admit("a")
+    m.reserve("a", 10); m.commit("a")
+    # next query at 10 reads keys >= 5: block 0 (positions 0..3) is out of reach, block 1 (4..7) is not
+    assert m.table("a", 1)[0] == -1 and m.table("a", 1)[1] >= 0
+    assert m.table("a", 0)[0] >= 0            # the full group keeps everything
+    for _ in range(100):
+        m.reserve("a", 1); m.commit("a"); m.check()
+        assert 5 - m.free_pages(1) <= 3        # never more than ceil((6-1)/4)+1 pages
+    m.release("a")
+    assert m.free_pages(1) == 5 and m.free_pages(0) == 32
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_keep_every_page_accounted_for(seed):
+    rng = random.Random(seed)
+    groups = [GroupSpec(24, 8), GroupSpec(12, 8, window=rng.choice([5, 16, 23]))]
+    m = CacheManager(groups, max_requests=4, max_context=96)
+    live, names = {}, iter(range(10**6))
+    for _ in range(1500):
+        action = rng.random()
+        if action < 0.15 and len(live) < 4:
+            rid = next(names)
+            m.admit(rid)
+            live[rid] = 0
+        elif action < 0.75 and live:
+            rid = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 2, 5, 8, 9, 20])
+            if live[rid] + n > 96:
+                continue
+            try:
+                m.reserve(rid, n)
+            except OutOfPages:
+                m.check()
+                continue
+            if rng.random() < 0.15:
+                m.rollback(rid)
+            else:
+                m.commit(rid)
+                live[rid] += n
+            assert m.length(rid) == live[rid]
+        elif live:
+            rid = rng.choice(list(live))
+            m.release(rid)
+            del live[rid]
+        m.check()
+    for rid in list(live):
+        m.release(rid)
+    m.check()
+    assert m.free_pages(0) == 24 and m.free_pages(1) == 12 and m.free_slots() == 4

@@ -22,7 +22,12 @@ def cases(tmp_path_factory):
         key = (name, dtype_name)
         if key not in cache:
             folder = str(tmp_path_factory.mktemp(f"model_{name}_{dtype_name}"))
-            make_model_dir(folder, TINY[name], seed=11 + len(cache), dtype=DTYPES[dtype_name], sharpen=2.0)
+            # float32: q/k gains doubled, so scores spread (std ~4) and a misplaced key moves the logits
+            # far beyond 1e-4.  bfloat16: gains as drawn; sharper scores would only amplify the 2^-9
+            # rounding of q and k, which is no fault (misplaced keys in bfloat16 are pinned by the
+            # kernel tests, where one key dominates).
+            sharpen = 2.0 if dtype_name == "float32" else 1.0
+            make_model_dir(folder, TINY[name], seed=11 + len(cache), dtype=DTYPES[dtype_name], sharpen=sharpen)
             config, weights = read_config(folder), read_weights(folder)
             requests = {f"r{i}": random_tokens(100 * i + 7, n, config["vocab_size"])
                         for i, n in enumerate(LENGTHS[name])}

@@ -1,0 +1,145 @@
+"""Generation through the entry points: greedy against the plain implementation, temperature against
+the slow sampler oracle, device sampling kernels against the double-precision sampler, the CLI."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests.plain import qwen3_plain, sampler_plain
+from tests.util import TINY, make_model_dir, random_tokens, read_config, read_weights
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {name: make_model_dir(str(tmp_path_factory.mktemp(f"gen{name}")), TINY[name], 21, torch.float32, 2.0)
+            for name in ("A", "B")}
+
+
+def plain_greedy(weights, config, prompt, n):
+    tokens = list(prompt)
+    for _ in range(n):
+        tokens.append(int(qwen3_plain.forward(weights, config, tokens)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+def test_greedy_generation_matches_plain(folders):
+    """Config A's workload: prompts of 1, 7, 33 and 64 tokens, 16 greedy tokens each, all live together."""
+    from leone_amd.api import Runtime
+    folder = folders["A"]
+    weights, config = read_weights(folder), read_config(folder)
+    prompts = [random_tokens(40 + i, n, config["vocab_size"]) for i, n in enumerate([1, 7, 33, 64])]
+    runtime = Runtime.load(folder, "float32", max_tokens=4 * 96, page_tokens=16, max_requests=4)
+    results = runtime.generate_tokens(prompts, 16, eos_token_id=None)
+    for prompt, result in zip(prompts, results):
+        assert result.tokens == plain_greedy(weights, config, prompt, 16)
+        assert result.finish_reason == "length"
+    assert runtime.last_stats.emitted_tokens == 64
+    assert not runtime.engine.cache.live_requests()
+
+
+def test_long_decoding_and_preemption_keep_the_tokens(folders):
+    """Few pages: requests are preempted and recomputed, and still produce what they produce alone."""
+    from leone_amd.api import Runtime
+    from leone_amd.engine.scheduler import SchedulerPolicy
+    folder = folders["A"]
+    weights, config = read_weights(folder), read_config(folder)
+    prompts = [random_tokens(60 + i, n, config["vocab_size"]) for i, n in enumerate([20, 35, 9])]
+    alone = Runtime.load(folder, "float32", max_tokens=256, page_tokens=16, max_requests=1)
+    expect = [alone.generate_tokens([p], 120, eos_token_id=None)[0].tokens for p in prompts]
+    assert expect[2][:24] == plain_greedy(weights, config, prompts[2], 24)
+    tight = Runtime.load(folder, "float32", num_pages=14, page_tokens=16, max_requests=3,
+                         policy=SchedulerPolicy(max_live_requests=3, prefill_chunk_tokens=16, max_step_tokens=24))
+    results = tight.generate_tokens(prompts, 120, eos_token_id=None)
+    assert [r.tokens for r in results] == expect
+    assert tight.last_stats.preemptions >= 1
+    tight.engine.cache.check()
+
+
+def test_temperature_sampling_matches_oracle_and_ignores_batching(folders):
+    """Config B's workload: prompts 5/40/130, portions of 32, 24 tokens at temperature 0.8, seeded."""
+    from leone_amd.api import Runtime, sampling_params
+    from leone_amd.engine.scheduler import SchedulerPolicy
+    folder = folders["B"]
+    weights, config = read_weights(folder), read_config(folder)
+    prompts = [random_tokens(80 + i, n, config["vocab_size"]) for i, n in enumerate([5, 40, 130])]
+    params = sampling_params(temperature=0.8, seed=1234)
+    together = Runtime.load(folder, "float32", max_tokens=3 * 192, page_tokens=16, max_requests=3,
+                            policy=SchedulerPolicy(max_live_requests=3, prefill_chunk_tokens=32))
+    results = together.generate_tokens(prompts, 24, params, eos_token_id=None)
+    alone = Runtime.load(folder, "float32", max_tokens=192, page_tokens=64, max_requests=1)
+    for prompt, result in zip(prompts, results):
+        assert alone.generate_tokens([prompt], 24, params, eos_token_id=None)[0].tokens == result.tokens
+    # the first request against the oracle: plain logits, slow double-precision distribution, same draws
+    tokens = list(prompts[0])
+    for _ in range(24):
+        logits = qwen3_plain.forward(weights, config, tokens)[-1].float().tolist()
+        probs = sampler_plain.distribution(logits, 0.8)
+        tokens.append(sampler_plain.select(probs, sampler_plain.uniform(1234, len(tokens) - 1)))
+    assert results[0].tokens == tokens[len(prompts[0]):]
+    # truncation stages take the host path; top-k 1 is the argmax whatever the draw
+    greedy = together.generate_tokens(prompts[:1], 8, eos_token_id=None)[0].tokens
+    top1 = together.generate_tokens(prompts[:1], 8, sampling_params(temperature=1.3, seed=5, top_k=1),
+                                    eos_token_id=None)[0].tokens
+    assert top1 == greedy
+
+
+def test_eos_stops_generation(folders):
+    from leone_amd.api import Runtime
+    folder = folders["A"]
+    runtime = Runtime.load(folder, "float32", max_tokens=128, page_tokens=16, max_requests=1)
+    prompt = random_tokens(99, 12, 512)
+    free = runtime.generate_tokens([prompt], 10, eos_token_id=None)[0].tokens
+    stopped = runtime.generate_tokens([prompt], 10, eos_token_id=free[3])[0]
+    assert stopped.tokens == free[:free.index(free[3]) + 1] and stopped.finish_reason == "eos"
+
+
+def test_device_sampling_kernels_against_the_double_precision_sampler():
+    from leone_amd import ops
+    from leone_amd.sampling.sampler import SamplingParams, distribution, select
+    gen = np.random.default_rng(7)
+    for vocab in (1, 2, 777, 1024, 1025, 151936):
+        rows = 6
+        logits = (gen.standard_normal((rows, vocab)) * 3).astype(np.float32)
+        if vocab > 2:
+            logits[1, vocab // 2] = np.nan
+            logits[2, 0] = -np.inf
+            logits[3, :] = logits[3, 0]                      # all equal: uniform distribution
+        temps = np.array([0.8, 1.0, 0.3, 1.0, 5.0, 0.05])
+        draws = gen.random(rows)
+        draws[4] = 0.0
+        got = ops.sample_temperature(torch.from_numpy(logits).cuda(), torch.from_numpy(temps).cuda(),
+                                     torch.from_numpy(draws).cuda()).cpu().tolist()
+        for r in range(rows):
+            probs = distribution(logits[r], SamplingParams(temperature=float(temps[r])))
+            want = select(probs, float(draws[r]))
+            if got[r] != want:   # only a draw within rounding of a boundary may differ, and then by one neighbour
+                cumulative = np.cumsum(probs)
+                assert abs(cumulative[min(got[r], want)] - draws[r]) < 1e-9, (vocab, r, got[r], want)
+    nothing = torch.full((1, 50), float("nan"), device="cuda")
+    assert ops.sample_temperature(nothing, torch.ones(1, dtype=torch.float64, device="cuda"),
+                                  torch.zeros(1, dtype=torch.float64, device="cuda")).tolist() == [-1]
+
+
+def test_command_line_generate(folders, tmp_path):
+    folder = folders["A"]
+    weights, config = read_weights(folder), read_config(folder)
+    prompt = random_tokens(123, 11, config["vocab_size"])
+    tokens_file, logits_file = tmp_path / "tokens.json", tmp_path / "logits.txt"
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "leone"), "generate", "-m", folder,
+                          "--prompt-tokens", ",".join(map(str, prompt)), "-n", "8", "--dtype", "float32",
+                          "--debug-tokens", str(tokens_file), "--debug-logits", str(logits_file)],
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    expect = plain_greedy(weights, config, prompt, 8)
+    assert json.load(open(tokens_file)) == expect
+    assert [int(t) for t in run.stdout.split()] == expect
+    assert "decode:" in run.stderr and "prefill:" in run.stderr and "tokens emitted: 8" in run.stderr
+    lines = open(logits_file).read().strip().splitlines()
+    assert len(lines) == 8 and int(lines[0].split()[0].split(":")[0]) == expect[0]

@@ -214,8 +214,9 @@ def test_qk_norm_rope_write(dtype, shape):
         close(kp[page, :, off], want_k[i], atol, rtol, f"k row {i}")
         assert torch.equal(vp[page, :, off].cpu(), v[i].to(dtype))      # values are copied unchanged
     # every other slot is untouched
-    assert torch.equal(kp.cpu()[~touched], k_pool[~touched])
-    assert torch.equal(vp.cpu()[~touched], v_pool[~touched])
+    untouched = ~touched[:, None, :].expand(-1, kv_heads, -1)
+    assert torch.equal(kp.cpu()[untouched], k_pool[untouched])
+    assert torch.equal(vp.cpu()[untouched], v_pool[untouched])
     # a layer that reads another layer's cache writes nothing
     kp2, vp2 = k_pool.to(DEV), v_pool.to(DEV)
     q2 = ops.qk_norm_rope_write(qkv.to(DEV), q_heads, kv_heads, head_dim, q_gain.to(DEV), k_gain.to(DEV), eps, cos,

@@ -1,0 +1,306 @@
+"""Each part alone against the plain functions, and the generality of the assembly: a toy mixer with
+state of its own, a windowed layer without rotation, a layer that runs twice and a run that reads
+another run's cache, all defined here and registered without touching the framework's files."""
+import json
+import math
+import os
+from dataclasses import dataclass
+
+import numpy as np
+import pytest
+import torch
+
+from tests import schedules
+from tests.plain import qwen3_plain as plain
+from tests.util import random_tokens
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def step_context(rows_meta, dtype, tables=None):
+    """A StepContext for rows [(entry, position)], in the order given."""
+    from leone_amd.parts.context import EntryInfo, StepContext
+    positions = torch.tensor([p for _, p in rows_meta], dtype=torch.int32, device=DEV)
+    row_entry = torch.tensor([e for e, _ in rows_meta], dtype=torch.int32, device=DEV)
+    n_entries = max(e for e, _ in rows_meta) + 1
+    infos, row = [], 0
+    for e in range(n_entries):
+        mine = [p for ee, p in rows_meta if ee == e]
+        infos.append(EntryInfo(e, e, row, len(mine), mine[0]))
+        row += len(mine)
+    return StepContext(rows=len(rows_meta), dtype=dtype, device=torch.device(DEV), positions=positions,
+                       row_entry=row_entry, entries=infos,
+                       entry_slots=torch.arange(n_entries, dtype=torch.int32, device=DEV), want_rows=None,
+                       block_tables=tables or {}, max_position=max(p for _, p in rows_meta))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from leone_amd.parts import NORMS, PartSpec
+    norm = NORMS.build(PartSpec("rmsnorm", {"size": 80, "eps": 3e-6, "weight": "g"}))
+    assert [(s.name, s.shape) for s in norm.tensor_specs()] == [("g", (80,))]
+    gain = 1 + 0.1 * torch.randn(80)
+    norm.bind({"g": gain.to(DEV)})
+    x = torch.randn(5, 80, device=DEV)
+    delta = torch.randn(5, 80, device=DEV).to(dtype)
+    want = plain.rms_norm(x.cpu().double() + delta.cpu().double(), gain, 3e-6)
+    y = norm.add_norm(x, delta, dtype)
+    tol = 2e-5 if dtype == torch.float32 else 1e-2
+    assert (y.cpu().double() - want).abs().max() < tol * (1 + want.abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    from leone_amd.parts import FEED_FORWARDS, PartSpec
+    ffn = FEED_FORWARDS.build(PartSpec("swiglu", {"hidden": 80, "intermediate": 176, "gate": "g", "up": "u", "down": "d"}))
+    assert [(s.name, s.shape) for s in ffn.tensor_specs()] == [("g", (176, 80)), ("u", (176, 80)), ("d", (80, 176))]
+    w = {"g": torch.randn(176, 80) * 0.1, "u": torch.randn(176, 80) * 0.1, "d": torch.randn(80, 176) * 0.1}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    ffn.bind({k: v.to(DEV) for k, v in w.items()})
+    y = torch.randn(9, 80).to(dtype)
+    out = ffn.forward(y.to(DEV), step_context([(0, i) for i in range(9)], dtype))
+    want = plain.feed_forward(y.float(), {f"p.{k}_proj.weight": v.float() for k, v in
+                                          (("gate", w["g"]), ("up", w["u"]), ("down", w["d"]))}, "p")
+    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    assert (out.cpu().double() - want).abs().max() < tol * (1 + want.abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_part_with_portions_and_two_requests(dtype):
+    """Two requests; the second is fed in two calls (a portion, then one token).  Scores are sharpened
+    by a large q/k gain so that one key dominates each row: a misplaced key changes the result by
+    far more than bfloat16 rounding."""
+    from leone_amd.parts import MIXERS, POSITIONS, PartSpec
+    from leone_amd.parts.context import KvCacheView
+    hidden, q_heads, kv_heads, dim, page = 96, 6, 2, 32, 16
+    rope = POSITIONS.build(PartSpec("rope_half_split", {"rotary_dim": dim, "theta": 1e4}))
+    rope.prepare(256, DEV)
+    names = {k: k for k in ("q", "k", "v", "o", "q_norm", "k_norm")}
+    mixer = MIXERS.build(PartSpec("gqa_attention", dict(hidden=hidden, q_heads=q_heads, kv_heads=kv_heads, head_dim=dim,
+                                                        qk_norm_eps=1e-5, window=None, position="rope", **names)),
+                         positions={"rope": rope})
+    torch.manual_seed(3)
+    w = {"q": torch.randn(q_heads * dim, hidden) * 0.1, "k": torch.randn(kv_heads * dim, hidden) * 0.1,
+         "v": torch.randn(kv_heads * dim, hidden) * 0.1, "o": torch.randn(hidden, q_heads * dim) * 0.1,
+         "q_norm": torch.full((dim,), 3.0), "k_norm": torch.full((dim,), 3.0)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    mixer.bind({k: v.to(DEV) for k, v in w.items()})
+    assert mixer.cache_need().kv_heads == kv_heads
+    lengths = [40, 21]
+    ys = [torch.randn(n, hidden).to(dtype) for n in lengths]
+    pw = {f"a.{k}_proj.weight": w[k].float() for k in ("q", "k", "v", "o")}
+    pw.update({"a.q_norm.weight": w["q_norm"].float(), "a.k_norm.weight": w["k_norm"].float()})
+    cfg = dict(num_attention_heads=q_heads, num_key_value_heads=kv_heads, head_dim=dim, rms_norm_eps=1e-5, rope_theta=1e4)
+    want = [plain.attention_block(y.float(), pw, "a", cfg, list(range(len(y)))) for y in ys]
+    k_pool = torch.full((8, kv_heads, page, dim), float("nan"), dtype=dtype, device=DEV)
+    v_pool = torch.full_like(k_pool, float("nan"))
+    table = torch.tensor([[5, 0, 3, -1], [7, 2, -1, -1]], dtype=torch.int32, device=DEV)
+    cache = KvCacheView(writes=True, k_pool=k_pool, v_pool=v_pool, block_table=table, page_tokens=page)
+    # call 1: all of request 0 and the first 20 tokens of request 1
+    meta = [(0, p) for p in range(40)] + [(1, p) for p in range(20)]
+    out1 = mixer.forward(torch.cat([ys[0], ys[1][:20]]).to(DEV), step_context(meta, dtype, {0: table}), cache)
+    # call 2: the last token of request 1 alone, as entry 0 of its step
+    cache2 = KvCacheView(writes=True, k_pool=k_pool, v_pool=v_pool, block_table=table[1:2].contiguous(), page_tokens=page)
+    out2 = mixer.forward(ys[1][20:21].to(DEV), step_context([(0, 20)], dtype, {0: table[1:2]}), cache2)
+    have = [out1[:40], torch.cat([out1[40:], out2])]
+    tol = 2e-5 if dtype == torch.float32 else 4e-2
+    for r in range(2):
+        err = (have[r].cpu().double() - want[r]).abs().max(dim=1).values
+        assert float(err.max()) < tol * (1 + float(want[r].abs().max())), (r, int(err.argmax()), float(err.max()))
+
+
+# ---- a toy architecture assembled from the framework's parts and one part defined here --------------
+
+DECAY = 0.75
+
+
+def register_toy():
+    from leone_amd.architectures import register_architecture
+    from leone_amd.config.base import FieldReader
+    from leone_amd.parts import MIXERS, Part, PartSpec, StateNeed
+    from leone_amd.parts.model import LayerRun, ModelSpec
+    from leone_amd.weights.loader import MATRIX, TensorSpec
+    from leone_amd import ops
+
+    class DecayMixer(Part):
+        """s_t = decay * s_{t-1} + y_t per request; out_t = W s_t.  Its state lives in the per-request slot."""
+
+        def __init__(self, spec, **_):
+            self.hidden, self.decay, self.name = spec["hidden"], spec["decay"], spec["weight"]
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name, (self.hidden, self.hidden), MATRIX)]
+
+        def bind(self, tensors):
+            self.weight = tensors.pop(self.name).contiguous()
+
+        def cache_need(self):
+            return StateNeed((self.hidden,), torch.float32)
+
+        def forward(self, y, step, cache):
+            states = torch.empty((step.rows, self.hidden), dtype=torch.float32, device=y.device)
+            for entry in step.entries:
+                s = cache.state[entry.slot].clone()
+                for r in range(entry.first_row, entry.first_row + entry.count):
+                    s = self.decay * s + y[r].float()
+                    states[r] = s
+                if cache.writes:
+                    cache.state[entry.slot] = s
+            return ops.linear(states.to(y.dtype), self.weight)
+
+    if "toy_decay" not in MIXERS.kinds():
+        MIXERS.register("toy_decay", DecayMixer)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str
+        hidden: int
+        heads: int
+        kv_heads: int
+        head_dim: int
+        ffn: int
+        vocab: int
+        window: int
+        eps: float
+        max_positions: int
+
+        @classmethod
+        def from_dict(cls, raw):
+            r = FieldReader(raw)
+            return cls("ToyForCausalLM", r.positive_int("hidden"), r.positive_int("heads"), r.positive_int("kv_heads"),
+                       r.positive_int("head_dim"), r.positive_int("ffn"), r.positive_int("vocab"),
+                       r.positive_int("window"), r.positive_float("eps"), r.positive_int("max_positions"))
+
+    def spec(c):
+        def norm(name):
+            return PartSpec("rmsnorm", {"size": c.hidden, "eps": c.eps, "weight": name})
+
+        def ffn(p):
+            return PartSpec("swiglu", {"hidden": c.hidden, "intermediate": c.ffn, "gate": f"{p}.gate", "up": f"{p}.up",
+                                       "down": f"{p}.down"})
+
+        def attention(p, window, rope, qk_norm):
+            params = dict(hidden=c.hidden, q_heads=c.heads, kv_heads=c.kv_heads, head_dim=c.head_dim,
+                          qk_norm_eps=c.eps if qk_norm else None, window=window, position="rope" if rope else None,
+                          q=f"{p}.q", k=f"{p}.k", v=f"{p}.v", o=f"{p}.o")
+            if qk_norm:
+                params.update(q_norm=f"{p}.qn", k_norm=f"{p}.kn")
+            return PartSpec("gqa_attention", params)
+
+        layers = [
+            PartSpec("prenorm", {"norm1": norm("l0.n1"), "mixer": attention("l0", None, True, True),
+                                 "norm2": norm("l0.n2"), "feed_forward": ffn("l0")}),
+            PartSpec("prenorm", {"norm1": norm("l1.n1"),
+                                 "mixer": PartSpec("toy_decay", {"hidden": c.hidden, "decay": DECAY, "weight": "l1.w"}),
+                                 "norm2": norm("l1.n2"), "feed_forward": ffn("l1")}),
+            PartSpec("prenorm", {"norm1": norm("l2.n1"), "mixer": attention("l2", c.window, False, False),
+                                 "norm2": norm("l2.n2"), "feed_forward": ffn("l2")}),
+        ]
+        # layer 1 runs twice, each run with state of its own; the last run is layer 0 again, reading the
+        # keys and values its first run wrote, writing none
+        order = [LayerRun(0, 0), LayerRun(1, 1), LayerRun(2, 2), LayerRun(1, 3), LayerRun(0, 0, writes=False)]
+        return ModelSpec(hidden_size=c.hidden, vocab_size=c.vocab, max_positions=c.max_positions, embedding="emb",
+                         layers=layers, schedule=order, final_norm=norm("final"), head="head",
+                         positions={"rope": PartSpec("rope_half_split", {"rotary_dim": c.head_dim, "theta": 5000.0})})
+
+    register_architecture("ToyForCausalLM", ToyConfig.from_dict, spec)
+
+
+TOY = dict(architectures=["ToyForCausalLM"], hidden=48, heads=3, kv_heads=1, head_dim=16, ffn=80, vocab=301, window=11,
+           eps=1e-5, max_positions=256)
+
+
+def toy_plain(w, tokens):
+    """The toy model with the plain functions, whole sequence."""
+    c = TOY
+    n = len(tokens)
+    positions = list(range(n))
+
+    def ffn(x, p):
+        y = plain.rms_norm(x, w[f"{p}.n2"], c["eps"])
+        return x + plain.linear(plain.swiglu(plain.linear(y, w[f"{p}.gate"]), plain.linear(y, w[f"{p}.up"])), w[f"{p}.down"])
+
+    def heads(y, name, count):
+        return plain.linear(y, w[name]).view(n, count, c["head_dim"])
+
+    x = plain.embedding(w["emb"], tokens)
+    # run 1: layer 0, full attention with q/k norm and rotation; its keys and values are kept
+    y = plain.rms_norm(x, w["l0.n1"], c["eps"])
+    k0 = plain.rope_half_split(plain.rms_norm(heads(y, "l0.k", 1), w["l0.kn"], c["eps"]), positions, 5000.0)
+    v0 = heads(y, "l0.v", 1)
+    q = plain.rope_half_split(plain.rms_norm(heads(y, "l0.q", 3), w["l0.qn"], c["eps"]), positions, 5000.0)
+    x = ffn(x + plain.linear(plain.causal_attention(q, k0, v0).reshape(n, -1), w["l0.o"]), "l0")
+
+    def decay_layer(x):
+        y = plain.rms_norm(x, w["l1.n1"], c["eps"])
+        s, rows = torch.zeros(c["hidden"], dtype=torch.float64), []
+        for t in range(n):
+            s = DECAY * s + y[t]
+            rows.append(s)
+        return ffn(x + plain.linear(torch.stack(rows), w["l1.w"]), "l1")
+
+    x = decay_layer(x)
+    # run 3: layer 2, window of 11 keys, no q/k norm, no rotation
+    y = plain.rms_norm(x, w["l2.n1"], c["eps"])
+    att = plain.causal_attention(heads(y, "l2.q", 3), heads(y, "l2.k", 1), heads(y, "l2.v", 1), window=c["window"])
+    x = ffn(x + plain.linear(att.reshape(n, -1), w["l2.o"]), "l2")
+    x = decay_layer(x)                      # run 4: layer 1 again, state of its own, starting from zero
+    # run 5: layer 0 again: new queries over the keys and values of run 1
+    y = plain.rms_norm(x, w["l0.n1"], c["eps"])
+    q = plain.rope_half_split(plain.rms_norm(heads(y, "l0.q", 3), w["l0.qn"], c["eps"]), positions, 5000.0)
+    x = ffn(x + plain.linear(plain.causal_attention(q, k0, v0).reshape(n, -1), w["l0.o"]), "l0")
+    return plain.linear(plain.rms_norm(x, w["final"], c["eps"]), w["head"])
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_toy_architecture_with_state_window_repeat_and_shared_cache(tmp_path, dtype_name):
+    from leone_amd.architectures import config_from_dict, model_spec_for, unregister_architecture
+    from leone_amd.engine.engine import Engine, StepEntry
+    from leone_amd.parts import MIXERS
+    from leone_amd.parts.model import DecoderModel
+    from leone_amd.runtime import load_model
+    from leone_amd.weights.random_init import host_tensors
+    from leone_amd.weights.safetensors_io import write_file
+
+    register_toy()
+    try:
+        dtype = torch.float32 if dtype_name == "float32" else torch.bfloat16
+        folder = str(tmp_path / "toy")
+        os.makedirs(folder)
+        json.dump(TOY, open(os.path.join(folder, "config.json"), "w"))
+        config = config_from_dict(TOY)
+        specs = DecoderModel(model_spec_for(config), torch.float32, "cpu").tensor_specs()
+        assert len({s.name for s in specs}) == len(specs)
+        tensors = host_tensors(specs, 77, dtype)
+        for name in tensors:
+            if name.endswith(".w"):
+                tensors[name] = (tensors[name].float() * 0.3).to(dtype)     # keep the decaying sum's output small
+        write_file(os.path.join(folder, "model.safetensors"), tensors)
+        model = load_model(folder, dtype_name)
+        needs = model.cache_needs()
+        assert sorted(needs) == [0, 1, 2, 3]
+        engine = Engine(model, num_pages=12, page_tokens=8, max_requests=3, poison_freed=True)
+        assert len(engine.cache.groups) == 2 and sorted(g.window or 0 for g in engine.cache.groups) == [0, 11]
+        requests = {f"t{i}": random_tokens(900 + i, n, TOY["vocab"]) for i, n in enumerate([45, 30, 9, 38])}
+        weights = {k: v.float() for k, v in tensors.items()}
+        expected = {rid: toy_plain(weights, toks).numpy() for rid, toks in requests.items()}
+        tol = 1e-4 if dtype_name == "float32" else 4e-2
+        for mode in ("whole", "portions", "mixed"):
+            steps = getattr(schedules, mode)(requests, **({"max_live": 3} if mode == "mixed" else {}))
+            outputs = {}
+            for s in steps:
+                out = engine.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+                outputs[s["step"]] = out.logits.cpu().numpy()
+                for rid in s["end"]:
+                    engine.release(rid)
+                engine.cache.check()
+            got = schedules.collect(steps, outputs)
+            for rid, rows in got.items():
+                err = np.abs(np.stack(rows) - expected[rid]).max(axis=1)
+                assert np.isfinite(err).all() and err.max() <= tol, (mode, rid, int(err.argmax()), float(err.max()))
+            # the windowed group never holds more than ceil((window - 1 + longest portion) / page) + 1 pages a request
+            assert engine.cache.free_pages(0) == 12 and engine.cache.free_pages(1) == 12
+    finally:
+        unregister_architecture("ToyForCausalLM")
+        MIXERS.unregister("toy_decay")

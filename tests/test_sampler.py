@@ -1,0 +1,96 @@
+"""The double-precision sampler against a slow oracle and the reference's own test vectors."""
+import math
+
+import numpy as np
+import pytest
+
+from leone_amd.sampling import rng
+from leone_amd.sampling.sampler import (SamplerError, SamplingParams, apply_penalties, argmax, distribution, sample,
+                                        select)
+from tests.plain import sampler_plain as oracle
+
+
+def test_greedy_ties_and_nan():
+    # crates/leone/src/sampler/tests.rs:521-537
+    assert argmax(np.array([1, 4, 4, np.nan], dtype=np.float32)) == 1
+    assert argmax(np.array([np.nan, np.inf, -np.inf], dtype=np.float32)) == -1
+    with pytest.raises(SamplerError):
+        sample(np.array([np.nan, np.nan], dtype=np.float32), SamplingParams(), 0)
+
+
+def test_invalid_parameters():
+    # crates/leone/src/sampler/tests.rs:659-668
+    for bad in (0.0, float("nan"), -1.0, float("inf")):
+        with pytest.raises(SamplerError):
+            SamplingParams(temperature=bad).validate()
+    with pytest.raises(SamplerError):
+        SamplingParams(temperature=1.0, truncations=[("top_p", 0.0)]).validate()
+    with pytest.raises(SamplerError):
+        SamplingParams(temperature=1.0, truncations=[("top_k", 0)]).validate()
+
+
+def test_rng_is_pure_and_in_range():
+    # crates/leone/src/sampler/tests.rs:746-760
+    seen = set()
+    for seed in (0, 1, 2**63 + 5):
+        for position in range(50):
+            u = rng.uniform(seed, position)
+            assert 0.0 <= u < 1.0
+            assert u == rng.uniform(seed, position) == oracle.uniform(seed, position)
+            seen.add(u)
+    assert len(seen) == 150
+    assert rng.uniform(3, 7, rng.PURPOSE_SELECT) != rng.uniform(3, 7, rng.PURPOSE_ACCEPT)
+
+
+def test_top_k_keeps_exactly_k_and_min_p_cases():
+    # crates/leone/src/sampler/tests.rs:539-548
+    logits = np.array([0.1, 2.0, 1.5, -1.0, 0.7], dtype=np.float32)
+    d = distribution(logits, SamplingParams(temperature=1.0, truncations=[("top_k", 3)]))
+    assert (d > 0).sum() == 3 and abs(d.sum() - 1) < 1e-12
+    peaked = np.array([10.0, 0.0, 0.0, 0.0], dtype=np.float32)
+    flat = np.array([1.0, 1.0, 1.0, 1.0], dtype=np.float32)
+    assert (distribution(peaked, SamplingParams(temperature=1.0, truncations=[("min_p", 0.5)])) > 0).sum() == 1
+    assert (distribution(flat, SamplingParams(temperature=1.0, truncations=[("min_p", 0.5)])) > 0).sum() == 4
+
+
+def test_low_temperature_concentrates_on_argmax():
+    logits = np.random.default_rng(0).standard_normal(100).astype(np.float32)
+    d = distribution(logits, SamplingParams(temperature=1e-3))
+    assert d[argmax(logits)] > 0.999
+
+
+def test_differential_against_slow_oracle():
+    """Random rows, temperatures and stage pipelines: probabilities within 1e-12, same token
+    (the reference's differential test, crates/leone/src/sampler/tests.rs:453-500)."""
+    gen = np.random.default_rng(1234)
+    for case in range(400):
+        n = int(gen.integers(1, 60))
+        logits = (gen.standard_normal(n) * gen.choice([0.1, 1.0, 5.0, 30.0])).astype(np.float32)
+        if gen.random() < 0.3:
+            logits[gen.integers(0, n)] = gen.choice([np.nan, np.inf, -np.inf])
+        if gen.random() < 0.2 and n > 2:
+            logits[1] = logits[0]
+        if not np.isfinite(logits).any():
+            continue
+        t = float(gen.choice([0.05, 0.5, 0.8, 1.0, 1.7, 10.0]))
+        stages = []
+        for name in gen.permutation(["top_k", "top_p", "min_p"])[:int(gen.integers(0, 4))]:
+            stages.append((str(name), float(gen.integers(1, 8)) if name == "top_k" else float(gen.uniform(0.05, 1.0))))
+        params = SamplingParams(temperature=t, truncations=stages, seed=int(gen.integers(0, 2**62)))
+        have = distribution(logits, params)
+        want = oracle.distribution(logits.tolist(), t, stages)
+        assert np.abs(have - np.array(want)).max() <= 1e-12, (case, stages)
+        position = int(gen.integers(0, 10000))
+        u = oracle.uniform(params.seed, position)
+        assert sample(logits, params, position) == oracle.select(want, u) == select(have, u)
+
+
+def test_penalties():
+    # positive logits divided, negative multiplied, presence once, frequency per occurrence
+    # (crates/leone/src/penalty.rs:160-196)
+    logits = np.array([2.0, -2.0, 1.0, 0.5], dtype=np.float32)
+    params = SamplingParams(repeat_penalty=2.0, presence_penalty=0.25, frequency_penalty=0.5, penalty_window=3)
+    out = apply_penalties(logits, [3, 0, 1, 1], params)   # window keeps [0, 1, 1]
+    assert out.tolist() == [2.0 / 2 - 0.25 - 0.5, -2.0 * 2 - 0.25 - 1.0, 1.0, 0.5]
+    assert apply_penalties(logits, [0, 1], SamplingParams()) is logits
+    assert not SamplingParams(repeat_penalty=2.0, penalty_window=0).penalties_active

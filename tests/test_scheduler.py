@@ -1,0 +1,219 @@
+"""The scheduler's decisions, with a stand-in executor whose tokens are a pure function of the
+request's history, so an interleaved run can be compared with each request run alone
+(the reference's isolated-oracle pattern, crates/leone/src/scheduler.rs:1626-1655)."""
+import random
+
+import pytest
+
+from leone_amd.cache.manager import CacheManager, GroupSpec
+from leone_amd.engine.scheduler import Reject, Request, Scheduler, SchedulerError, SchedulerPolicy
+
+
+def next_token(history):
+    """Deterministic stand-in for model + sampler: depends on every earlier token and the position."""
+    value = 17
+    for i, t in enumerate(history):
+        value = (value * 31 + t * (i + 1)) % 1009
+    return value % 97
+
+
+def run(scheduler, fail_at_step=None):
+    """Drives plans to completion; commits the cache as the engine would."""
+    steps = 0
+    while scheduler.has_work():
+        plan = scheduler.plan()
+        steps += 1
+        if fail_at_step == steps:
+            scheduler.abort()
+            continue
+        sampled = {}
+        for entry in plan:
+            assert scheduler.cache.length(entry.request) == entry.start
+            scheduler.cache.commit(entry.request, len(entry.tokens))
+            if entry.sample:
+                state = scheduler.live[entry.request]
+                assert state.tokens[:entry.start + len(entry.tokens)] == state.tokens
+                sampled[entry.request] = next_token(state.tokens)
+        scheduler.complete(sampled)
+        scheduler.cache.check()
+        assert steps < 100000
+    return steps
+
+
+def isolated(prompt, n, eos=None):
+    tokens = list(prompt)
+    for _ in range(n):
+        tokens.append(next_token(tokens))
+        if eos is not None and tokens[-1] == eos:
+            break
+    return tokens[len(prompt):]
+
+
+def make(pages=64, page_tokens=16, max_requests=8, context=4096, **policy):
+    cache = CacheManager([GroupSpec(pages, page_tokens)], max_requests, context)
+    return Scheduler(SchedulerPolicy(**policy), cache)
+
+
+def test_prompt_is_cut_into_portions_under_the_budget():
+    # prompt 13, chunk 8: portions of 8 and 5, then one token a step (crates/leone/src/scheduler.rs:1723-1764)
+    s = make(prefill_chunk_tokens=8, max_step_tokens=64)
+    assert s.submit(Request("a", list(range(13)), 3)) is None
+    first = s.plan()
+    assert [(e.start, len(e.tokens), e.sample) for e in first] == [(0, 8, False)]
+    s.cache.commit("a"); s.complete({})
+    second = s.plan()
+    assert [(e.start, len(e.tokens), e.sample) for e in second] == [(8, 5, True)]
+    assert second[0].sample_position == 12
+    s.cache.commit("a"); s.complete({"a": 50})
+    third = s.plan()
+    assert [(e.start, e.tokens, e.sample) for e in third] == [(13, [50], True)]
+    s.cache.commit("a"); s.complete({"a": 51})
+    fourth = s.plan()
+    s.cache.commit("a")
+    done = s.complete({"a": 52})
+    assert done[0].tokens == [50, 51, 52] and done[0].reason == "length"
+    assert not s.has_work() and s.cache.free_pages(0) == 64 and s.cache.free_slots() == 8
+
+
+def test_token_budget_covers_decode_rows_first_then_portions():
+    s = make(prefill_chunk_tokens=100, max_step_tokens=10)
+    for i in range(3):
+        s.submit(Request(i, [1, 2], 5))
+    plan = s.plan()
+    assert sorted(len(e.tokens) for e in plan) == [2, 2, 2]
+    for e in plan:
+        s.cache.commit(e.request)
+    s.complete({e.request: 7 for e in plan})
+    s.submit(Request("long", list(range(50)), 2))
+    plan = s.plan()
+    kinds = [(e.request, len(e.tokens)) for e in plan]
+    assert kinds[:3] == [(0, 1), (1, 1), (2, 1)] and kinds[3] == ("long", 7)    # 10 - 3 decode rows
+    assert sum(n for _, n in kinds) == 10
+
+
+def test_typed_rejections_hold_nothing():
+    s = make(pages=4, page_tokens=16, context=100, max_prompt_tokens=40, max_output_tokens=30,
+             max_queued_requests=2)
+    assert s.submit(Request("p0", [], 5)) is Reject.PROMPT_LIMIT
+    assert s.submit(Request("p1", [1] * 41, 5)) is Reject.PROMPT_LIMIT
+    assert s.submit(Request("o0", [1], 0)) is Reject.OUTPUT_LIMIT
+    assert s.submit(Request("o1", [1], 31)) is Reject.OUTPUT_LIMIT
+    assert s.submit(Request("k", [1] * 40, 30)) is Reject.KV_CAPACITY     # 69 tokens > 4 pages of 16
+    assert s.submit(Request("ok1", [1] * 40, 25)) is None                 # 64 tokens fit exactly
+    assert s.submit(Request("ok1", [1], 1)) is Reject.DUPLICATE
+    assert s.submit(Request("ok2", [1], 1)) is None
+    assert s.submit(Request("q", [1], 1)) is Reject.QUEUE_LIMIT
+    assert s.stats.rejected == 7 and s.cache.free_pages(0) == 4 and s.cache.free_slots() == 8
+    small = make(context=10)
+    assert small.submit(Request("c", [1] * 8, 4)) is Reject.CONTEXT_LIMIT  # 8 + 4 - 1 > 10
+    assert small.submit(Request("c", [1] * 8, 3)) is None
+
+
+def test_live_limit_and_admission_order():
+    # a cap of 4 live requests out of 6 (crates/leone/src/scheduler.rs:1853-1859)
+    s = make(max_live_requests=4)
+    for i in range(6):
+        s.submit(Request(i, [i + 1], 2))
+    plan = s.plan()
+    assert [e.request for e in plan] == [0, 1, 2, 3]
+    assert s.stats.max_live == 4
+
+
+def test_interleaved_equals_isolated_with_eos_and_cancel():
+    rng = random.Random(5)
+    s = make(pages=40, page_tokens=8, max_live_requests=5, prefill_chunk_tokens=7, max_step_tokens=16)
+    wanted = {}
+    for i in range(12):
+        prompt = [rng.randrange(97) for _ in range(rng.choice([1, 2, 9, 30, 61]))]
+        n = rng.choice([1, 4, 17])
+        eos = 13 if i % 3 == 0 else None
+        assert s.submit(Request(i, prompt, n, eos_token_id=eos)) is None
+        wanted[i] = isolated(prompt, n, eos)
+    s.cancel(11)                                   # still queued: gone at once
+    run(s)
+    by_id = {f.id: f for f in s.finished}
+    assert by_id[11].reason == "cancelled" and by_id[11].tokens == []
+    for i in range(11):
+        assert by_id[i].tokens == wanted[i], i
+        assert by_id[i].reason == ("eos" if by_id[i].tokens[-1:] == [13] and i % 3 == 0 else "length")
+    assert s.cache.free_pages(0) == 40 and s.cache.free_slots() == 8 and not s.live and not s.queue
+    assert s.stats.max_step_rows <= 16
+
+
+def test_cancel_of_a_live_request_takes_effect_at_the_next_step():
+    s = make()
+    s.submit(Request("a", [1, 2, 3], 10))
+    plan = s.plan(); s.cache.commit("a"); s.complete({"a": 5})
+    assert s.cancel("a") and "a" in s.live
+    assert s.plan() == []
+    assert s.finished[-1].reason == "cancelled" and s.finished[-1].tokens == [5]
+    assert s.cache.free_pages(0) == 64 and not s.cancel("nobody")
+
+
+def test_when_pages_run_out_the_newest_request_is_preempted_and_recomputed():
+    """Two requests that together outgrow the pool: the younger is released, requeued with its
+    generated tokens as prompt, and still ends with the tokens it would produce alone."""
+    s = make(pages=6, page_tokens=4, max_step_tokens=64, prefill_chunk_tokens=64)
+    a, b = [3, 1, 4, 1, 5, 9, 2], [2, 7, 1, 8, 2, 8]
+    s.submit(Request("a", a, 14))
+    s.submit(Request("b", b, 12))
+    run(s)
+    by_id = {f.id: f for f in s.finished}
+    assert by_id["a"].tokens == isolated(a, 14) and by_id["b"].tokens == isolated(b, 12)
+    assert s.stats.preemptions >= 1 and by_id["b"].preemptions >= 1 and by_id["a"].preemptions == 0
+    assert [e for e in s.events if e[0] == "preempt"][0][1] == "b"
+    assert s.cache.free_pages(0) == 6
+
+
+def test_prompt_portion_shrinks_to_the_free_pages_and_older_requests_go_first():
+    s = make(pages=5, page_tokens=4, max_step_tokens=64, prefill_chunk_tokens=64)
+    s.submit(Request("a", list(range(12)), 2))      # 3 pages
+    plan = s.plan(); s.cache.commit("a"); s.complete({"a": 1})
+    s.submit(Request("b", list(range(20)), 1))      # needs 5 pages in all; 2 are free now
+    plan = s.plan()
+    assert [(e.request, len(e.tokens)) for e in plan] == [("a", 1)]      # b waits: its tokens do not fit yet
+    s.cache.commit("a"); s.complete({"a": 2})        # a finishes and frees its pages
+    plan = s.plan()
+    assert [(e.request, len(e.tokens), e.sample) for e in plan] == [("b", 20, True)]
+
+
+def test_failed_step_aborts_its_requests_and_frees_everything():
+    # crates/leone/src/service.rs:270-297
+    s = make()
+    s.submit(Request("a", [1, 2, 3], 4))
+    s.submit(Request("b", [4, 5], 4))
+    run(s, fail_at_step=2)
+    assert {f.id: f.reason for f in s.finished} == {"a": "aborted", "b": "aborted"}
+    assert s.cache.free_pages(0) == 64 and s.cache.free_slots() == 8
+    with pytest.raises(SchedulerError):
+        s.complete({})
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_load_under_page_pressure(seed):
+    rng = random.Random(100 + seed)
+    s = make(pages=rng.choice([10, 14, 24]), page_tokens=rng.choice([4, 8]), max_live_requests=4,
+             prefill_chunk_tokens=rng.choice([3, 16, 64]), max_step_tokens=rng.choice([8, 24, 200]))
+    capacity = s.cache.groups[0].num_pages * s.cache.groups[0].page_tokens
+    wanted = {}
+    for i in range(25):
+        prompt = [rng.randrange(97) for _ in range(rng.randrange(1, 40))]
+        n = rng.randrange(1, 30)
+        result = s.submit(Request(i, prompt, n))
+        if len(prompt) + n - 1 > capacity:
+            assert result is Reject.KV_CAPACITY
+        else:
+            assert result is None
+            wanted[i] = isolated(prompt, n)
+    run(s)
+    assert {f.id: f.tokens for f in s.finished} == wanted
+    assert s.cache.free_pages(0) == s.cache.groups[0].num_pages
+    # events alone show that no request got a position twice after its last preemption
+    fed = {}
+    for event in s.events:
+        if event[0] == "preempt":
+            fed[event[1]] = 0
+        elif event[0] == "step":
+            for rid, start, count, _ in event[1]:
+                assert fed.get(rid, 0) == start
+                fed[rid] = start + count
