@@ -1,0 +1,185 @@
+"""Decode and prefill throughput of the Qwen3-8B shape with random weights, as one JSON line.
+
+Method after the reference's own bench (crates/leone/src/runtime.rs:1998-2002, 11342-11348;
+crates/leone-cli/src/main.rs:4655-4802): fixed token ids, prefill timed to the synchronised end of
+the step, decode timed over contiguous steps including the per-step copy of the chosen tokens to the
+host, rate = tokens / duration, roofline = bytes a step must read / its time.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+from typing import List, Optional
+
+QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=36, hidden_size=4096,
+                num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288,
+                vocab_size=151936, max_position_embeddings=40960, rope_theta=1000000.0, rms_norm_eps=1e-6,
+                tie_word_embeddings=False)
+CONTEXT = 8192
+PREFILL_TOKENS = 2048
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def matmul_params(c) -> int:
+    """Weights every token multiplies with, head excluded."""
+    per_layer = (c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim
+                 + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size)
+    return c.num_hidden_layers * per_layer
+
+
+def prefill_flops(c, tokens: int, start: int = 0) -> float:
+    gemm = 2.0 * tokens * matmul_params(c) + 2.0 * c.hidden_size * c.vocab_size          # head for one row
+    keys = tokens * start + tokens * (tokens + 1) / 2.0                                   # causal pairs
+    attention = c.num_hidden_layers * 4.0 * c.num_attention_heads * c.head_dim * keys
+    return gemm + attention
+
+
+def decode_bytes(c, batch: int, context: float, size: int) -> float:
+    """Bytes one decode step has to read: every weight it uses once, and the cache of the live requests."""
+    norms = c.num_hidden_layers * (2 * c.hidden_size + 2 * c.head_dim) + c.hidden_size
+    weights = (matmul_params(c) + c.vocab_size * c.hidden_size + norms + batch * c.hidden_size) * size
+    cache = batch * context * 2 * c.num_hidden_layers * c.num_key_value_heads * c.head_dim * size
+    return weights + cache
+
+
+def fill_cache(engine, batch: int, tokens: int, seed: int = 0):
+    """Live requests with `tokens` positions each, their pages holding random keys and values (the
+    timed steps read them; what they hold does not change the work)."""
+    import torch
+    gen = torch.Generator(device=engine.device)
+    gen.manual_seed(seed)
+    for k_pool, v_pool in engine.pools.kv.values():
+        for pool in (k_pool, v_pool):
+            flat = pool.view(-1)
+            for at in range(0, flat.numel(), 1 << 28):
+                part = flat[at:at + (1 << 28)]
+                part.copy_(torch.randn(part.numel(), generator=gen, device=engine.device, dtype=torch.float32) * 0.5)
+    for b in range(batch):
+        engine.admit(("bench", b))
+        engine.cache.reserve(("bench", b), tokens)
+        engine.cache.commit(("bench", b))
+
+
+def time_decode(engine, batch: int, start_context: int, steps: int, warmup: int, seed: int = 1):
+    import torch
+    from .engine.engine import StepEntry
+    from . import ops
+    fill_cache(engine, batch, start_context)
+    gen = torch.Generator().manual_seed(seed)
+    tokens = torch.randint(0, engine.vocab_size, (batch,), generator=gen).tolist()
+
+    def one_step(tokens):
+        out = engine.step([StepEntry(("bench", b), [tokens[b]], [0]) for b in range(batch)])
+        return ops.argmax(out.logits).cpu().tolist()       # the per-step copy of the chosen tokens
+
+    for _ in range(warmup):
+        tokens = one_step(tokens)
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    for _ in range(steps):
+        tokens = one_step(tokens)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    for b in range(batch):
+        engine.release(("bench", b))
+    mean_context = start_context + warmup + (steps + 1) / 2.0
+    return elapsed, mean_context
+
+
+def time_prefill(engine, tokens: int, repeats: int = 3, seed: int = 2):
+    import torch
+    from .engine.engine import StepEntry
+    gen = torch.Generator().manual_seed(seed)
+    prompt = torch.randint(0, engine.vocab_size, (tokens,), generator=gen).tolist()
+    best = None
+    for i in range(repeats + 1):
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        out = engine.step([StepEntry("prefill", prompt, [tokens - 1])])
+        out.logits.sum().item()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        engine.release("prefill")
+        if i > 0:                                            # the first run warms up
+            best = elapsed if best is None else min(best, elapsed)
+    return best
+
+
+def main(argv: Optional[List[str]] = None) -> int:
+    parser = argparse.ArgumentParser(prog="bench.py")
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--context", type=int, default=CONTEXT)
+    parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    parser.add_argument("--no-prefill", action="store_true")
+    args = parser.parse_args(argv)
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from .architectures import config_from_dict
+    from .engine.engine import Engine
+    from .runtime import random_model
+
+    raw = dict(QWEN3_8B)
+    full_layers = raw["num_hidden_layers"]
+    if args.layers is not None:
+        raw["num_hidden_layers"] = args.layers
+    config = config_from_dict(raw)
+    size = 2 if args.dtype == "bfloat16" else 4
+    dtype_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    model = random_model(config, seed=0, dtype=args.dtype)
+    page_tokens = 64
+    points_batches = [] if args.no_points else [1, 64]
+    largest = max([args.batch] + points_batches)
+    pages = largest * (args.context // page_tokens + 1) + PREFILL_TOKENS // page_tokens
+    engine = Engine(model, num_pages=pages, page_tokens=page_tokens, max_requests=largest + 1,
+                    max_context=args.context)
+
+    start = args.context - args.steps - args.warmup - 1
+    elapsed, mean_context = time_decode(engine, args.batch, start, args.steps, args.warmup)
+    ms_per_step = elapsed / args.steps * 1e3
+    value = args.batch * args.steps / elapsed
+    step_bytes = decode_bytes(config, args.batch, mean_context, size)
+    achieved = step_bytes / (elapsed / args.steps) / 1e9
+    record = {
+        "metric": "decode tok/s (Qwen3-8B shape)", "value": round(value, 2), "unit": "tok/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": dtype_name, "data": "synthetic",
+        "config": {"model": "Qwen3-8B shape, random weights", "layers": config.num_hidden_layers,
+                   "layers_of_configuration": full_layers, "hidden": config.hidden_size,
+                   "q_heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
+                   "head_dim": config.head_dim, "intermediate": config.intermediate_size, "vocab": config.vocab_size,
+                   "global_batch": args.batch, "seq_len": args.context, "decode_start_context": start,
+                   "prefill_tokens": PREFILL_TOKENS, "page_tokens": page_tokens, "rope_theta": config.rope_theta,
+                   "tied_head": config.tie_word_embeddings, "parallelism": "single GPU"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+    }
+    if not args.no_prefill:
+        seconds = time_prefill(engine, PREFILL_TOKENS)
+        flops = prefill_flops(config, PREFILL_TOKENS)
+        record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
+                             "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[dtype_name], 4)}
+    points = {}
+    for batch in points_batches:
+        steps = max(8, args.steps // 2)
+        warm = max(2, args.warmup // 2)
+        e, _ = time_decode(engine, batch, args.context - steps - warm - 1, steps, warm)
+        points[f"decode_b{batch}"] = round(batch * steps / e, 2)
+    if points:
+        record["points"] = points
+    print(json.dumps(record), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

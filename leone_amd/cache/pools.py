@@ -15,7 +15,8 @@ class DevicePools:
 
     Cache slots with the same key/value need (heads, head size, window) form one
     group and share page ids and block tables; each slot has its own key and
-    value tensor ``[pages, kv_heads, page_tokens, head_dim]``.  A slot with a state
+    value tensor (keys ``[pages, kv_heads, page_tokens, head_dim]``, values transposed
+    ``[pages, kv_heads, head_dim, page_tokens]``).  A slot with a state
     need gets ``[max_requests, *shape]``.
     """
 
@@ -43,9 +44,11 @@ class DevicePools:
             self.group_specs.append(GroupSpec(pages, page_tokens, need.window))
         for slot, gi in self.group_of_slot.items():
             need, pages = self.group_needs[gi], self.group_specs[gi].num_pages
-            shape = (pages, need.kv_heads, page_tokens, need.head_dim)
-            self.kv[slot] = (torch.zeros(shape, dtype=dtype, device=self.device),
-                             torch.zeros(shape, dtype=dtype, device=self.device))
+            # keys [page][head][token][element]; values transposed [page][head][element][token]
+            self.kv[slot] = (torch.zeros((pages, need.kv_heads, page_tokens, need.head_dim), dtype=dtype,
+                                         device=self.device),
+                             torch.zeros((pages, need.kv_heads, need.head_dim, page_tokens), dtype=dtype,
+                                         device=self.device))
 
     def bytes_per_token(self) -> int:
         size = torch.empty((), dtype=self.dtype).element_size()

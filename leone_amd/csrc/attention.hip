@@ -9,7 +9,8 @@
 // table instead of its segment list.  Scores, maxima, sums and the accumulator
 // are float whatever the cache's storage type.
 //
-// Cache layout of one layer: [page][kv head][token in page][head_dim].
+// Cache layout of one layer: keys [page][kv head][token in page][head_dim],
+// values transposed [page][kv head][head_dim][token in page].
 #include "common.h"
 #include "leone_hip.h"
 
@@ -60,9 +61,9 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
             l = __builtin_nanf("");
             continue;
         }
-        const long base = ((static_cast<long>(page) * kv_heads + kvh) * page_tokens + j % page_tokens) * head_dim;
-        const T* kr = k_pool + base;
-        const T* vr = v_pool + base;
+        const long head_base = (static_cast<long>(page) * kv_heads + kvh) * page_tokens * head_dim;
+        const T* kr = k_pool + head_base + static_cast<long>(j % page_tokens) * head_dim;
+        const T* vr = v_pool + head_base + j % page_tokens;   // element d at vr[d * page_tokens]
         float partial = 0.f;
         float vv[kRowDimsPerLane];
 #pragma unroll
@@ -70,7 +71,7 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
             const int d = lane + i * kWave;
             if (d < head_dim) {
                 partial = fmaf(qv[i], to_float(kr[d]), partial);
-                vv[i] = to_float(vr[d]);
+                vv[i] = to_float(vr[static_cast<long>(d) * page_tokens]);
             } else {
                 vv[i] = 0.f;
             }

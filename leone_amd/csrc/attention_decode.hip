@@ -1,0 +1,311 @@
+// Split-KV attention over the paged cache on the matrix cores, bfloat16.
+//
+// One workgroup takes (query row, kv head, up to 16 of its query heads, one
+// split of the keys); its four waves walk 32-key tiles of the split.  For a
+// tile a wave computes S^T = K . Q^T (keys x heads) with
+// v_mfma_f32_16x16x32_bf16, runs the running-maximum softmax of the reference
+// (crates/leone/src/cpu.rs:2299-2357) in float on the accumulator registers,
+// and adds O^T += V^T . P^T with the same instruction.  Keys are stored
+// [token][element] and values transposed [element][token], so that both
+// operands are 16-byte loads straight from the cache, a key or value being
+// read once for all query heads of its group.  The waves' partial results are
+// merged in shared memory, the splits' by a second kernel, both in a fixed
+// order (the reference's partial + reduce pair:
+// crates/leone-cuda/cuda/ie_cuda.cu:4465, 4769).
+//
+// Operand layouts of the 16x16x32 instruction (lane l, c = l % 16, g = l / 16):
+//   A: row c,    k-slots 8g .. 8g+7        B: column c, k-slots 8g .. 8g+7
+//   C/D: column c, rows 4g .. 4g+3
+// Which key or element a k-slot stands for is free as long as A and B agree.
+// For S^T the two 16-key halves of a tile are laid out so that lane (g, c)
+// ends up with the scores of keys 8g .. 8g+7 of the tile: exactly the k-slots
+// it has to supply as P^T for the second product.
+#include "common.h"
+#include "leone_hip.h"
+
+#include <math.h>
+
+namespace leone {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+constexpr int kDecodeWaves = 4;
+constexpr int kDecodeThreads = kDecodeWaves * kWave;
+constexpr int kTileKeys = 32;
+
+__device__ inline bf16x8 load8(const bf16_t* p) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+__device__ inline bf16x8 zero8() {
+    uint4 z = {0u, 0u, 0u, 0u};
+    return __builtin_bit_cast(bf16x8, z);
+}
+
+// kD16 = head_dim / 16.
+template <int kD16>
+__global__ void __launch_bounds__(kDecodeThreads)
+attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
+                        const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
+                        const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
+                        float* __restrict__ part_acc, float* __restrict__ part_ml, int q_heads, int kv_heads,
+                        int page_shift, float scale, int window, int splits) {
+    constexpr int kD = kD16 * 16;
+    constexpr int kSteps = (kD16 + 1) / 2;           // 32-element steps of the q.k product
+    extern __shared__ float smem[];                   // [waves][columns][kD] accumulators, then m and l
+
+    const int group = q_heads / kv_heads;
+    const int col_tiles = (group + 15) / 16;
+    const int row = blockIdx.x;
+    const int kvh = blockIdx.y / col_tiles;
+    const int col0 = (blockIdx.y % col_tiles) * 16;
+    const int cols = group - col0 < 16 ? group - col0 : 16;   // query heads handled here
+    const int split = blockIdx.z;
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int page_tokens = 1 << page_shift;
+    const int page_mask = page_tokens - 1;
+
+    const int n = positions[row] + 1;                                    // keys 0 .. n-1 exist
+    const int lo = (window > 0 && n - window > 0) ? n - window : 0;      // first key in reach
+    const int* table = block_table + static_cast<long>(row_entry[row]) * max_blocks;
+    const int t_begin = lo / kTileKeys, t_end = (n + kTileKeys - 1) / kTileKeys;
+    const int per_split = (t_end - t_begin + splits - 1) / splits;
+    const int my_begin = t_begin + split * per_split;
+    const int my_end = my_begin + per_split < t_end ? my_begin + per_split : t_end;
+
+    // Q^T operand: column c is query head kvh*group + col0 + c.
+    bf16x8 qreg[kSteps];
+    {
+        const bool head_ok = c < cols;
+        const bf16_t* qrow = q + (static_cast<long>(row) * q_heads + kvh * group + col0 + (head_ok ? c : 0)) * kD;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            const int d0 = 32 * s + 8 * g;
+            qreg[s] = (head_ok && d0 < kD) ? load8(qrow + d0) : zero8();
+        }
+    }
+
+    float m_run = -INFINITY, l_run = 0.f;
+    bool unmapped = false;
+    floatx4 acc[kD16];
+#pragma unroll
+    for (int dt = 0; dt < kD16; ++dt) acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    for (int t = my_begin + wave; t < my_end; t += kDecodeWaves) {
+        const int key0 = t * kTileKeys;
+        // ---- S^T = K . Q^T for the two 16-key halves --------------------------------------------
+        floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+        {
+            // A-operand row c of half a is key 8*(c/4) + c%4, of half b four keys further
+            const int ka = key0 + 8 * (c >> 2) + (c & 3);
+            const int kb = ka + 4;
+            bool va = ka >= lo && ka < n, vb = kb >= lo && kb < n;
+            const bf16_t* pa = k_pool;
+            const bf16_t* pb = k_pool;
+            if (va) {
+                const int page = table[ka >> page_shift];
+                if (page < 0) unmapped = true;   // never read outside the pool; the result is poisoned below
+                pa = k_pool + ((static_cast<long>(page) * kv_heads + kvh) * page_tokens + (ka & page_mask)) * kD;
+            }
+            if (vb) {
+                const int page = table[kb >> page_shift];
+                if (page < 0) unmapped = true;
+                pb = k_pool + ((static_cast<long>(page) * kv_heads + kvh) * page_tokens + (kb & page_mask)) * kD;
+            }
+            if (unmapped) va = vb = false;
+#pragma unroll
+            for (int s = 0; s < kSteps; ++s) {
+                const int d0 = 32 * s + 8 * g;
+                const bool in_head = d0 < kD;
+                const bf16x8 xa = (va && in_head) ? load8(pa + d0) : zero8();
+                const bf16x8 xb = (vb && in_head) ? load8(pb + d0) : zero8();
+                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, qreg[s], sa, 0, 0, 0);
+                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb, qreg[s], sb, 0, 0, 0);
+            }
+        }
+        // lane (g, c) now holds, for query column c, the scores of keys key0 + 8g + j, j = 0..7
+        float sc[8];
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int key = key0 + 8 * g + j;
+            const float raw = j < 4 ? sa[j] : sb[j - 4];
+            sc[j] = (key >= lo && key < n) ? raw * scale : -INFINITY;
+            tile_max = fmaxf(tile_max, sc[j]);
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+        const float m_new = fmaxf(m_run, tile_max);      // finite: every tile of the range holds a key in reach
+        const float alpha = __expf(m_run - m_new);
+        float psum = 0.f;
+        bf16x8 pt;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float p = __expf(sc[j] - m_new);
+            psum += p;
+            pt[j] = static_cast<__bf16>(p);
+        }
+        psum += __shfl_xor(psum, 16, kWave);
+        psum += __shfl_xor(psum, 32, kWave);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        // ---- O^T += V^T . P^T ------------------------------------------------------------------
+        const int run0 = key0 + 8 * g;                   // this lane's eight keys: run0 .. run0+7
+        bool any = run0 < n && run0 + 8 > lo;
+        const bool whole = run0 >= lo && run0 + 8 <= n;
+        const bf16_t* pv = v_pool;
+        if (any) {
+            const int page = table[run0 >> page_shift];
+            if (page < 0) {
+                unmapped = true;
+                any = false;
+            }
+            pv = v_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (run0 & page_mask);
+        }
+#pragma unroll
+        for (int dt = 0; dt < kD16; ++dt) {
+            bf16x8 xv = any ? load8(pv + static_cast<long>(16 * dt + c) * page_tokens) : zero8();
+            if (any && !whole) {
+                // slots outside [lo, n) may hold anything, even NaN: clear them, a zero weight is not enough
+                uint4 raw = __builtin_bit_cast(uint4, xv);
+                unsigned* w = reinterpret_cast<unsigned*>(&raw);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int e0 = run0 + 2 * i, e1 = e0 + 1;
+                    unsigned mask = 0u;
+                    if (e0 >= lo && e0 < n) mask |= 0x0000ffffu;
+                    if (e1 >= lo && e1 < n) mask |= 0xffff0000u;
+                    w[i] &= mask;
+                }
+                xv = __builtin_bit_cast(bf16x8, raw);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[dt][r] *= alpha;
+            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv, pt, acc[dt], 0, 0, 0);
+        }
+    }
+
+    // ---- merge the four waves --------------------------------------------------------------------
+    float* sm_acc = smem;                                         // [waves][16][kD]
+    float* sm_m = smem + kDecodeWaves * 16 * kD;                  // [waves][16]
+    float* sm_l = sm_m + kDecodeWaves * 16;
+    if (__any(unmapped)) l_run = __builtin_nanf("");   // a key in reach had no page: say so in the result
+    if (g == 0) {
+        sm_m[wave * 16 + c] = m_run;
+        sm_l[wave * 16 + c] = l_run;
+    }
+#pragma unroll
+    for (int dt = 0; dt < kD16; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sm_acc[(wave * 16 + c) * kD + 16 * dt + 4 * g + r] = acc[dt][r];
+    __syncthreads();
+    for (int i = threadIdx.x; i < cols * kD; i += kDecodeThreads) {
+        const int col = i / kD, d = i % kD;
+        float top = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kDecodeWaves; ++w) top = fmaxf(top, sm_m[w * 16 + col]);
+        float num = 0.f, den = 0.f;
+        if (top != -INFINITY) {
+#pragma unroll
+            for (int w = 0; w < kDecodeWaves; ++w) {
+                const float mw = sm_m[w * 16 + col];
+                const float wgt = mw == -INFINITY ? 0.f : __expf(mw - top);
+                num += sm_acc[(w * 16 + col) * kD + d] * wgt;
+                den += sm_l[w * 16 + col] * wgt;
+            }
+        }
+        const long slot = (static_cast<long>(row) * q_heads + kvh * group + col0 + col) * splits + split;
+        part_acc[slot * kD + d] = num;
+        if (d == 0) {
+            part_ml[slot * 2] = top;
+            part_ml[slot * 2 + 1] = den;
+        }
+    }
+}
+
+// Merges the splits of one (row, query head): out = sum_s acc_s e^(m_s - M) / sum_s l_s e^(m_s - M).
+__global__ void attention_reduce_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                                        bf16_t* __restrict__ out, int head_dim, int splits) {
+    const long rh = blockIdx.x;                      // row * q_heads + head
+    const float* ml = part_ml + rh * splits * 2;
+    float top = -INFINITY;
+    for (int s = 0; s < splits; ++s) top = fmaxf(top, ml[2 * s]);
+    float den = 0.f;
+    for (int s = 0; s < splits; ++s) den += ml[2 * s] == -INFINITY ? 0.f : ml[2 * s + 1] * __expf(ml[2 * s] - top);
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+        float num = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            if (ml[2 * s] == -INFINITY) continue;
+            num += part_acc[(rh * splits + s) * head_dim + d] * __expf(ml[2 * s] - top);
+        }
+        out[rh * head_dim + d] = from_float<bf16_t>(num / den);
+    }
+}
+
+static size_t decode_smem_bytes(int head_dim) {
+    return (static_cast<size_t>(kDecodeWaves) * 16 * head_dim + 2 * kDecodeWaves * 16) * sizeof(float);
+}
+
+template <int kD16>
+static void launch_decode(const void* q, const void* k_pool, const void* v_pool, const int* positions,
+                          const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
+                          float* part_ml, int rows, int q_heads, int kv_heads, int page_shift, float scale,
+                          int window, int splits, hipStream_t stream) {
+    const int group = q_heads / kv_heads;
+    dim3 grid(rows, kv_heads * ((group + 15) / 16), splits);
+    const size_t smem = decode_smem_bytes(kD16 * 16);
+    attention_decode_kernel<kD16><<<grid, kDecodeThreads, smem, stream>>>(
+        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
+        positions, row_entry, block_table, max_blocks, part_acc, part_ml, q_heads, kv_heads, page_shift, scale, window,
+        splits);
+}
+
+}  // namespace leone
+
+using namespace leone;
+
+// Workspace: part_acc holds rows*q_heads*splits*head_dim floats, part_ml rows*q_heads*splits*2.
+extern "C" int leone_attention_decode(const void* q, void* out, const void* k_pool, const void* v_pool,
+                                      const int* positions, const int* row_entry, const int* block_table,
+                                      int max_blocks, float* part_acc, float* part_ml, int rows, int q_heads,
+                                      int kv_heads, int head_dim, int page_tokens, float scale, int window,
+                                      int splits, hipStream_t stream) {
+    LEONE_REQUIRE(q && out && k_pool && v_pool && positions && row_entry && block_table && part_acc && part_ml,
+                  "attention_decode: null pointer");
+    LEONE_REQUIRE(rows > 0 && q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
+                  "attention_decode: rows %d, %d query heads over %d kv heads", rows, q_heads, kv_heads);
+    LEONE_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
+                  "attention_decode: head_dim %d must be a multiple of 16 in 16..256", head_dim);
+    LEONE_REQUIRE(page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0,
+                  "attention_decode: page_tokens %d must be a power of two, at least 16", page_tokens);
+    LEONE_REQUIRE(decode_smem_bytes(head_dim) <= 64 * 1024,
+                  "attention_decode: head_dim %d needs more shared memory than a workgroup may have", head_dim);
+    LEONE_REQUIRE(splits >= 1 && splits <= 65535, "attention_decode: splits %d out of range", splits);
+    LEONE_REQUIRE(window >= 0 && max_blocks > 0, "attention_decode: bad window or block table");
+    const long grid_y = static_cast<long>(kv_heads) * ((q_heads / kv_heads + 15) / 16);
+    LEONE_REQUIRE(grid_y <= 65535, "attention_decode: too many heads for one launch");
+    int page_shift = 0;
+    while ((1 << page_shift) < page_tokens) ++page_shift;
+#define LEONE_DECODE_CASE(N)                                                                                      \
+    case N:                                                                                                       \
+        launch_decode<N>(q, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml,     \
+                         rows, q_heads, kv_heads, page_shift, scale, window, splits, stream);                     \
+        break;
+    switch (head_dim / 16) {
+        LEONE_DECODE_CASE(1) LEONE_DECODE_CASE(2) LEONE_DECODE_CASE(3) LEONE_DECODE_CASE(4)
+        LEONE_DECODE_CASE(5) LEONE_DECODE_CASE(6) LEONE_DECODE_CASE(7) LEONE_DECODE_CASE(8)
+        LEONE_DECODE_CASE(9) LEONE_DECODE_CASE(10) LEONE_DECODE_CASE(11) LEONE_DECODE_CASE(12)
+        LEONE_DECODE_CASE(13) LEONE_DECODE_CASE(14) LEONE_DECODE_CASE(15) LEONE_DECODE_CASE(16)
+        default:
+            set_error("attention_decode: head_dim %d is not supported", head_dim);
+            return 1;
+    }
+#undef LEONE_DECODE_CASE
+    LEONE_LAUNCH_CHECK("attention_decode");
+    attention_reduce_kernel<<<rows * q_heads, head_dim <= 64 ? 64 : 128, 0, stream>>>(
+        part_acc, part_ml, static_cast<bf16_t*>(out), head_dim, splits);
+    LEONE_LAUNCH_CHECK("attention_reduce");
+    return 0;
+}

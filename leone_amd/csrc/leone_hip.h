@@ -42,6 +42,14 @@ int leone_attention_rows(const void* q, void* out, const void* k_pool, const voi
                          int rows, int q_heads, int kv_heads, int head_dim, int page_tokens, float scale,
                          int window, hipStream_t stream);
 
+// The same on the matrix cores for bfloat16, the keys of a row cut into `splits` parts whose
+// partial results (part_acc: rows*q_heads*splits*head_dim floats, part_ml: rows*q_heads*splits*2)
+// are merged by a second kernel.  head_dim a multiple of 16 up to 240, page_tokens a power of two >= 16.
+int leone_attention_decode(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
+                           const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
+                           float* part_ml, int rows, int q_heads, int kv_heads, int head_dim, int page_tokens,
+                           float scale, int window, int splits, hipStream_t stream);
+
 // C[M,N] = A[M,K] . B[N,K]^T in float.
 int leone_gemm_f32(const float* a, const float* b, float* c, int m, int n, int k, hipStream_t stream);
 

@@ -98,6 +98,8 @@ __global__ void rope_table_kernel(float* __restrict__ cos_out, float* __restrict
 //   q heads: optional RMSNorm over D, optional rotation, written to q_out.
 //   k heads: the same, written into the request's page at `position`.
 //   v heads: copied into the page unchanged.
+// Keys lie in a page as [kv head][token][element], values transposed as
+// [kv head][element][token], which is how the attention kernels read them.
 // A lane owns pairs p = lane, lane + 64, ... (p < D/2): elements p and p + D/2.
 // When `write_cache` is 0 the k and v heads are skipped (a layer that reads
 // another layer's cache).
@@ -123,14 +125,20 @@ __global__ void qk_norm_rope_write_kernel(
     const bool is_q = head < q_heads;
     const bool is_k = !is_q && head < q_heads + kv_heads;
     T* dst;
+    long dst_stride = 1;   // distance between consecutive elements of the head at the destination
     if (is_q) {
         dst = q_out + (static_cast<long>(row) * q_heads + head) * head_dim;
     } else {
         const int kvh = is_k ? head - q_heads : head - q_heads - kv_heads;
         const int page = block_table[static_cast<long>(row_entry[row]) * max_blocks + pos / page_tokens];
         if (page < 0) return;  // host reserves pages before the launch
-        const long slot = ((static_cast<long>(page) * kv_heads + kvh) * page_tokens + pos % page_tokens) * head_dim;
-        dst = (is_k ? k_pool : v_pool) + slot;
+        const long head_base = (static_cast<long>(page) * kv_heads + kvh) * page_tokens * head_dim;
+        if (is_k) {
+            dst = k_pool + head_base + static_cast<long>(pos % page_tokens) * head_dim;   // [token][element]
+        } else {
+            dst = v_pool + head_base + pos % page_tokens;                               // [element][token]
+            dst_stride = page_tokens;
+        }
     }
 
     float a[kMaxPairsPerLane], b[kMaxPairsPerLane];
@@ -150,8 +158,8 @@ __global__ void qk_norm_rope_write_kernel(
         for (int i = 0; i < kMaxPairsPerLane; ++i) {
             const int p = lane + i * kWave;
             if (p < half) {
-                dst[p] = from_float<T>(a[i]);
-                dst[p + half] = from_float<T>(b[i]);
+                dst[p * dst_stride] = from_float<T>(a[i]);
+                dst[(p + half) * dst_stride] = from_float<T>(b[i]);
             }
         }
         return;

@@ -108,7 +108,7 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim:
         if k_pool is None or v_pool is None or block_table is None or row_entry is None:
             raise KernelError("qk_norm_rope_write: a cache write needs pools, a block table and a row map")
         pages, pool_heads, page_tokens, pool_dim = k_pool.shape
-        if (pool_heads, pool_dim) != (kv_heads, head_dim) or v_pool.shape != k_pool.shape:
+        if (pool_heads, pool_dim) != (kv_heads, head_dim) or tuple(v_pool.shape) != (pages, kv_heads, head_dim, page_tokens):
             raise KernelError(f"qk_norm_rope_write: pool shape {tuple(k_pool.shape)} does not fit "
                               f"{kv_heads} heads of {head_dim}")
         max_blocks = block_table.shape[1]
@@ -140,8 +140,8 @@ def attention_rows(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, 
     pages, kv_heads, page_tokens, head_dim = k_pool.shape
     if q.shape[1] != q_heads * head_dim:
         raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
-    if v_pool.shape != k_pool.shape:
-        raise KernelError("attention: key and value pools differ in shape")
+    if tuple(v_pool.shape) != (pages, kv_heads, head_dim, page_tokens):
+        raise KernelError("attention: the value pool must be [pages, kv_heads, head_dim, page_tokens]")
     if out is None:
         out = torch.empty_like(q)
     call("leone_attention_rows", _dev(q, "attention q"), _dev(out, "attention out", q.dtype, q.shape),
@@ -149,6 +149,46 @@ def attention_rows(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, 
          _dev(positions, "positions", torch.int32, (rows,)), _dev(row_entry, "row map", torch.int32, (rows,)),
          _dev(block_table, "block table", torch.int32), block_table.shape[1], rows, q_heads, kv_heads, head_dim,
          page_tokens, float(scale), int(window), _stream())
+    return out
+
+
+def decode_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int) -> bool:
+    """Whether the matrix-core kernel takes this case; otherwise ``attention_rows`` does."""
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 240
+            and page_tokens >= 16 and page_tokens & (page_tokens - 1) == 0)
+
+
+def choose_splits(rows: int, kv_heads: int, group: int, max_context: int) -> int:
+    """How many parts the keys of a row are cut into: enough workgroups to fill 256 CUs, at least
+    four 32-key tiles a part so that each of a workgroup's waves has one."""
+    blocks = rows * kv_heads * ((group + 15) // 16)
+    tiles = (max_context + 31) // 32
+    return max(1, min(1024 // max(1, blocks), (tiles + 3) // 4, 256))
+
+
+def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
+                     row_entry: torch.Tensor, block_table: torch.Tensor, q_heads: int, scale: float,
+                     window: int = 0, max_context: int = 1, splits: Optional[int] = None,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Split-KV attention on the matrix cores (bfloat16).  ``max_context`` only steers the number of splits."""
+    rows = q.shape[0]
+    pages, kv_heads, page_tokens, head_dim = k_pool.shape
+    if q.shape[1] != q_heads * head_dim:
+        raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
+    if tuple(v_pool.shape) != (pages, kv_heads, head_dim, page_tokens):
+        raise KernelError("attention: the value pool must be [pages, kv_heads, head_dim, page_tokens]")
+    if splits is None:
+        splits = choose_splits(rows, kv_heads, q_heads // kv_heads, max_context)
+    if out is None:
+        out = torch.empty_like(q)
+    part_acc = torch.empty((rows * q_heads * splits * head_dim,), dtype=torch.float32, device=q.device)
+    part_ml = torch.empty((rows * q_heads * splits * 2,), dtype=torch.float32, device=q.device)
+    call("leone_attention_decode", _dev(q, "attention q", torch.bfloat16),
+         _dev(out, "attention out", torch.bfloat16, q.shape), _dev(k_pool, "k pool", torch.bfloat16),
+         _dev(v_pool, "v pool", torch.bfloat16), _dev(positions, "positions", torch.int32, (rows,)),
+         _dev(row_entry, "row map", torch.int32, (rows,)), _dev(block_table, "block table", torch.int32),
+         block_table.shape[1], _dev(part_acc, "partials"), _dev(part_ml, "partial sums"), rows, q_heads, kv_heads,
+         head_dim, page_tokens, float(scale), int(window), int(splits), _stream())
     return out
 
 

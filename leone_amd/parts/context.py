@@ -47,7 +47,7 @@ class CacheView:
 @dataclass
 class KvCacheView(CacheView):
     k_pool: torch.Tensor = None        # [pages, kv_heads, page_tokens, head_dim]
-    v_pool: torch.Tensor = None
+    v_pool: torch.Tensor = None        # [pages, kv_heads, head_dim, page_tokens] (transposed)
     block_table: torch.Tensor = None   # int32 [entries, max_blocks] of the layer's group
     page_tokens: int = 0
 

@@ -82,6 +82,11 @@ class GqaAttention(Part):
                                    self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin,
                                    step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
                                    write_cache=cache.writes)
-        attended = ops.attention_rows(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
-                                      cache.block_table, self.q_heads, self.scale, int(self.window or 0))
+        if ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens):
+            attended = ops.attention_decode(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
+                                            cache.block_table, self.q_heads, self.scale, int(self.window or 0),
+                                            max_context=step.max_position + 1)
+        else:
+            attended = ops.attention_rows(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
+                                          cache.block_table, self.q_heads, self.scale, int(self.window or 0))
         return ops.linear(attended, self.w_o)

@@ -107,7 +107,7 @@ def paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed, extra_pag
     max_blocks = max(blocks) + 1
     table = torch.full((len(lengths), max_blocks), -1, dtype=torch.int32)
     k_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), float("nan"))
-    v_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), float("nan"))
+    v_pool = torch.full((n_pages, kv_heads, head_dim, page_tokens), float("nan"))     # values lie transposed
     keys, values = [], []
     at = 0
     for r, n in enumerate(lengths):
@@ -121,7 +121,7 @@ def paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed, extra_pag
             table[r, b] = page
             lo, hi = b * page_tokens, min(n, (b + 1) * page_tokens)
             k_pool[page, :, :hi - lo] = k[lo:hi].transpose(0, 1)
-            v_pool[page, :, :hi - lo] = v[lo:hi].transpose(0, 1)
+            v_pool[page, :, :, :hi - lo] = v[lo:hi].permute(1, 2, 0)
     return table, k_pool.to(dtype), v_pool.to(dtype), keys, values
 
 
@@ -158,9 +158,9 @@ def test_attention_reference_vector():
     (crates/leone/src/cpu.rs:2850-2898)."""
     from leone_amd import ops
     k_pool = torch.zeros(1, 1, 16, 2, device=DEV)
-    v_pool = torch.zeros(1, 1, 16, 2, device=DEV)
+    v_pool = torch.zeros(1, 1, 2, 16, device=DEV)
     k_pool[0, 0, 0] = torch.tensor([1.0, 0.0]); k_pool[0, 0, 1] = torch.tensor([0.0, 1.0])
-    v_pool[0, 0, 0] = torch.tensor([2.0, 4.0]); v_pool[0, 0, 1] = torch.tensor([6.0, 8.0])
+    v_pool[0, 0, :, 0] = torch.tensor([2.0, 4.0]); v_pool[0, 0, :, 1] = torch.tensor([6.0, 8.0])
     q = torch.tensor([[1.0, 0.0, 0.0, 1.0], [1.0, 0.0, 0.0, 1.0]], device=DEV)
     out = ops.attention_rows(q, k_pool, v_pool, torch.tensor([0, 1], dtype=torch.int32, device=DEV),
                              torch.zeros(2, dtype=torch.int32, device=DEV),
@@ -192,7 +192,7 @@ def test_qk_norm_rope_write(dtype, shape):
     table[1, 17 // page_tokens] = 2 if 16 // page_tokens == 17 // page_tokens else 5
     table[2, 8000 // page_tokens] = 1
     k_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), 7.0).to(dtype)
-    v_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), 7.0).to(dtype)
+    v_pool = torch.full((n_pages, kv_heads, head_dim, page_tokens), 7.0).to(dtype)
     cos, sin = ops.rope_table(theta, head_dim, 8192, DEV)
     positions = torch.tensor([p for _, p in rows_meta], dtype=torch.int32)
     row_entry = torch.tensor([e for e, _ in rows_meta], dtype=torch.int32)
@@ -212,11 +212,11 @@ def test_qk_norm_rope_write(dtype, shape):
         page, off = int(table[e, p // page_tokens]), p % page_tokens
         touched[page, off] = True
         close(kp[page, :, off], want_k[i], atol, rtol, f"k row {i}")
-        assert torch.equal(vp[page, :, off].cpu(), v[i].to(dtype))      # values are copied unchanged
+        assert torch.equal(vp[page, :, :, off].cpu(), v[i].to(dtype))   # values are copied unchanged, transposed
     # every other slot is untouched
     untouched = ~touched[:, None, :].expand(-1, kv_heads, -1)
     assert torch.equal(kp.cpu()[untouched], k_pool[untouched])
-    assert torch.equal(vp.cpu()[untouched], v_pool[untouched])
+    assert torch.equal(vp.cpu().transpose(2, 3)[untouched], v_pool.transpose(2, 3)[untouched])
     # a layer that reads another layer's cache writes nothing
     kp2, vp2 = k_pool.to(DEV), v_pool.to(DEV)
     q2 = ops.qk_norm_rope_write(qkv.to(DEV), q_heads, kv_heads, head_dim, q_gain.to(DEV), k_gain.to(DEV), eps, cos,
@@ -250,3 +250,63 @@ def test_argmax_rules():
     big = torch.randn(5, 151936, device=DEV)
     big[2, 1000] = big[2, 150000] = 9.0
     assert ops.argmax(big).tolist() == [int(r.argmax()) if i != 2 else 1000 for i, r in enumerate(big)]
+
+
+@pytest.mark.parametrize("splits", [1, 3, None])
+@pytest.mark.parametrize("window", [0, 5, 37])
+@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 1, 32, 64), (5, 5, 48, 16), (32, 8, 128, 64), (40, 8, 128, 16),
+                                   (64, 2, 64, 32), (3, 3, 240, 16)])
+def test_attention_decode(shape, window, splits):
+    """The matrix-core kernel on the same cases as the row kernel, whatever the number of splits."""
+    from leone_amd import ops
+    q_heads, kv_heads, head_dim, page_tokens = shape
+    dtype = torch.bfloat16
+    assert ops.decode_attention_supported(dtype, head_dim, page_tokens)
+    lengths = [1, 17, 70, 130]
+    table, k_pool, v_pool, keys, values = paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed=13)
+    rows = [(0, 0)] + [(1, 16)] + [(2, p) for p in range(40, 70)] + [(3, p) for p in range(0, 130, 3)] + [(3, 129)]
+    g = torch.Generator().manual_seed(14)
+    q = torch.randn(len(rows), q_heads, head_dim, generator=g).to(dtype)
+    positions = torch.tensor([p for _, p in rows], dtype=torch.int32)
+    row_entry = torch.tensor([r for r, _ in rows], dtype=torch.int32)
+    scale = 1.0 / math.sqrt(head_dim)
+    args = (q.reshape(len(rows), -1).to(DEV), k_pool.to(DEV), v_pool.to(DEV), positions.to(DEV), row_entry.to(DEV),
+            table.to(DEV), q_heads, scale, window)
+    out = ops.attention_decode(*args, max_context=130, splits=splits)
+    assert torch.isfinite(out.float()).all()
+    want = torch.stack([plain.attend_one(q[i].float(), keys[r][:p + 1], values[r][:p + 1], window or None)
+                        for i, (r, p) in enumerate(rows)])
+    close(out.reshape(len(rows), q_heads, head_dim), want, 2e-2, 2e-2, "attention_decode")
+    again = ops.attention_decode(*args, max_context=130, splits=splits)
+    assert torch.equal(out, again)                                   # fixed order of additions
+
+
+@pytest.mark.parametrize("kernel", ["rows", "decode"])
+def test_attention_finds_the_one_key_that_matters(kernel):
+    """Each query is a scaled copy of one key far back in its request, so that key takes all the weight
+    and the output must be its value row: a key taken from the wrong page, slot or request shows at once,
+    well above bfloat16 rounding."""
+    from leone_amd import ops
+    q_heads, kv_heads, head_dim, page_tokens = 8, 2, 64, 16
+    dtype = torch.bfloat16
+    lengths = [300, 517]
+    table, k_pool, v_pool, keys, values = paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed=21)
+    picks = [(0, 299, 0), (0, 299, 15), (0, 299, 16), (0, 255, 31), (0, 200, 199), (1, 516, 1), (1, 516, 255),
+             (1, 516, 256), (1, 516, 511), (1, 516, 512), (1, 400, 47), (1, 64, 63), (1, 64, 64)]
+    q = torch.zeros(len(picks), q_heads, head_dim)
+    for i, (r, p, j) in enumerate(picks):
+        for h in range(q_heads):
+            k = keys[r][j, h // (q_heads // kv_heads)]
+            q[i, h] = k * (60.0 * math.sqrt(head_dim) / float(k @ k))     # its own score is 60, others ~N(0, 60/8)
+    q = q.to(dtype)
+    positions = torch.tensor([p for _, p, _ in picks], dtype=torch.int32)
+    row_entry = torch.tensor([r for r, _, _ in picks], dtype=torch.int32)
+    args = (q.reshape(len(picks), -1).to(DEV), k_pool.to(DEV), v_pool.to(DEV), positions.to(DEV), row_entry.to(DEV),
+            table.to(DEV), q_heads, 1.0 / math.sqrt(head_dim))
+    out = (ops.attention_rows(*args) if kernel == "rows" else ops.attention_decode(*args, max_context=517))
+    out = out.float().cpu().view(len(picks), q_heads, head_dim)
+    for i, (r, p, j) in enumerate(picks):
+        want = values[r][j].repeat_interleave(q_heads // kv_heads, dim=0)
+        exact = plain.attend_one(q[i].float(), keys[r][:p + 1], values[r][:p + 1])
+        assert (out[i] - exact).abs().max() < 3e-2, (i, r, p, j)
+        assert (out[i] - want).abs().max() < 0.25, (i, r, p, j)       # nearly all the weight is on key j
