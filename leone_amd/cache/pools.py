@@ -15,8 +15,8 @@ class DevicePools:
 
     Cache slots with the same key/value need (heads, head size, window) form one
     group and share page ids and block tables; each slot has its own key and
-    value tensor (keys ``[pages, kv_heads, page_tokens, head_dim]``, values transposed
-    ``[pages, kv_heads, head_dim, page_tokens]``).  A slot with a state
+    value tensor, packed in runs of 8 (keys ``[pages, kv_heads, head_dim/8, page_tokens, 8]``,
+    values ``[pages, kv_heads, page_tokens/8, head_dim, 8]``).  A slot with a state
     need gets ``[max_requests, *shape]``.
     """
 
@@ -44,10 +44,13 @@ class DevicePools:
             self.group_specs.append(GroupSpec(pages, page_tokens, need.window))
         for slot, gi in self.group_of_slot.items():
             need, pages = self.group_needs[gi], self.group_specs[gi].num_pages
-            # keys [page][head][token][element]; values transposed [page][head][element][token]
-            self.kv[slot] = (torch.zeros((pages, need.kv_heads, page_tokens, need.head_dim), dtype=dtype,
+            # keys [page][head][element / 8][token][8]; values [page][head][token / 8][element][8]
+            if need.head_dim % 8 or page_tokens % 8:
+                raise ValueError(f"the cache packs runs of 8: head_dim {need.head_dim} and page_tokens "
+                                 f"{page_tokens} must be multiples of 8")
+            self.kv[slot] = (torch.zeros((pages, need.kv_heads, need.head_dim // 8, page_tokens, 8), dtype=dtype,
                                          device=self.device),
-                             torch.zeros((pages, need.kv_heads, need.head_dim, page_tokens), dtype=dtype,
+                             torch.zeros((pages, need.kv_heads, page_tokens // 8, need.head_dim, 8), dtype=dtype,
                                          device=self.device))
 
     def bytes_per_token(self) -> int:

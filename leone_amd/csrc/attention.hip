@@ -9,8 +9,8 @@
 // table instead of its segment list.  Scores, maxima, sums and the accumulator
 // are float whatever the cache's storage type.
 //
-// Cache layout of one layer: keys [page][kv head][token in page][head_dim],
-// values transposed [page][kv head][head_dim][token in page].
+// Cache layout of one layer: [page][kv head] blocks of page_tokens * head_dim
+// elements, packed inside as key_offset() and value_offset() say.
 #include "common.h"
 #include "leone_hip.h"
 
@@ -62,16 +62,17 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
             continue;
         }
         const long head_base = (static_cast<long>(page) * kv_heads + kvh) * page_tokens * head_dim;
-        const T* kr = k_pool + head_base + static_cast<long>(j % page_tokens) * head_dim;
-        const T* vr = v_pool + head_base + j % page_tokens;   // element d at vr[d * page_tokens]
+        const T* kr = k_pool + head_base;
+        const T* vr = v_pool + head_base;
+        const int token = j % page_tokens;
         float partial = 0.f;
         float vv[kRowDimsPerLane];
 #pragma unroll
         for (int i = 0; i < kRowDimsPerLane; ++i) {
             const int d = lane + i * kWave;
             if (d < head_dim) {
-                partial = fmaf(qv[i], to_float(kr[d]), partial);
-                vv[i] = to_float(vr[static_cast<long>(d) * page_tokens]);
+                partial = fmaf(qv[i], to_float(kr[key_offset(token, d, page_tokens)]), partial);
+                vv[i] = to_float(vr[value_offset(token, d, head_dim)]);
             } else {
                 vv[i] = 0.f;
             }
@@ -125,6 +126,8 @@ extern "C" int leone_attention_rows(const void* q, void* out, const void* k_pool
     LEONE_REQUIRE(q_heads <= 65535, "attention_rows: at most 65535 query heads");
     LEONE_REQUIRE(head_dim > 0 && head_dim <= kRowMaxHeadDim, "attention_rows: head_dim %d must be in 1..%d", head_dim, kRowMaxHeadDim);
     LEONE_REQUIRE(page_tokens > 0 && max_blocks > 0, "attention_rows: page_tokens %d and max_blocks %d must be positive", page_tokens, max_blocks);
+    LEONE_REQUIRE(head_dim % 8 == 0 && page_tokens % 8 == 0,
+                  "attention_rows: head_dim %d and page_tokens %d must be multiples of 8", head_dim, page_tokens);
     LEONE_REQUIRE(window >= 0, "attention_rows: window %d must not be negative", window);
     dim3 grid(rows, q_heads);
     if (dtype == kF32)

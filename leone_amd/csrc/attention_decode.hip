@@ -5,10 +5,11 @@
 // tile a wave computes S^T = K . Q^T (keys x heads) with
 // v_mfma_f32_16x16x32_bf16, runs the running-maximum softmax of the reference
 // (crates/leone/src/cpu.rs:2299-2357) in float on the accumulator registers,
-// and adds O^T += V^T . P^T with the same instruction.  Keys are stored
-// [token][element] and values transposed [element][token], so that both
-// operands are 16-byte loads straight from the cache, a key or value being
-// read once for all query heads of its group.  The waves' partial results are
+// and adds O^T += V^T . P^T with the same instruction.  The cache packs keys
+// as [element / 8][token][8] and values as [token / 8][element][8], so that
+// both operands are 16-byte loads straight from the cache with the 16 lanes of
+// a quarter wave on neighbouring runs, a key or value being read once for all
+// query heads of its group.  The waves' partial results are
 // merged in shared memory, the splits' by a second kernel, both in a fixed
 // order (the reference's partial + reduce pair:
 // crates/leone-cuda/cuda/ie_cuda.cu:4465, 4769).
@@ -107,20 +108,21 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
             if (va) {
                 const int page = table[ka >> page_shift];
                 if (page < 0) unmapped = true;   // never read outside the pool; the result is poisoned below
-                pa = k_pool + ((static_cast<long>(page) * kv_heads + kvh) * page_tokens + (ka & page_mask)) * kD;
+                pa = k_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (ka & page_mask) * 8;
             }
             if (vb) {
                 const int page = table[kb >> page_shift];
                 if (page < 0) unmapped = true;
-                pb = k_pool + ((static_cast<long>(page) * kv_heads + kvh) * page_tokens + (kb & page_mask)) * kD;
+                pb = k_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (kb & page_mask) * 8;
             }
             if (unmapped) va = vb = false;
 #pragma unroll
             for (int s = 0; s < kSteps; ++s) {
                 const int d0 = 32 * s + 8 * g;
                 const bool in_head = d0 < kD;
-                const bf16x8 xa = (va && in_head) ? load8(pa + d0) : zero8();
-                const bf16x8 xb = (vb && in_head) ? load8(pb + d0) : zero8();
+                const long run = static_cast<long>(4 * s + g) * page_tokens * 8;   // run of elements d0 .. d0+7
+                const bf16x8 xa = (va && in_head) ? load8(pa + run) : zero8();
+                const bf16x8 xb = (vb && in_head) ? load8(pb + run) : zero8();
                 sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, qreg[s], sa, 0, 0, 0);
                 sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb, qreg[s], sb, 0, 0, 0);
             }
@@ -162,11 +164,12 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                 unmapped = true;
                 any = false;
             }
-            pv = v_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (run0 & page_mask);
+            pv = v_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD +
+                 static_cast<long>((run0 & page_mask) >> 3) * kD * 8;
         }
 #pragma unroll
         for (int dt = 0; dt < kD16; ++dt) {
-            bf16x8 xv = any ? load8(pv + static_cast<long>(16 * dt + c) * page_tokens) : zero8();
+            bf16x8 xv = any ? load8(pv + (16 * dt + c) * 8) : zero8();
             if (any && !whole) {
                 // slots outside [lo, n) may hold anything, even NaN: clear them, a zero weight is not enough
                 uint4 raw = __builtin_bit_cast(uint4, xv);

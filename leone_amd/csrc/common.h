@@ -93,6 +93,20 @@ __device__ inline float block_sum(float v, float* scratch) {
     return total;
 }
 
+// ---- cache layout ----------------------------------------------------------
+// One page of one kv head holds page_tokens * head_dim elements.  Both tensors
+// are packed in runs of 8 elements (16 bytes of bfloat16) so that the matrix
+// core kernels read whole runs with neighbouring lanes on neighbouring runs:
+//   keys   [head_dim / 8][token][8 elements]   (run = 8 elements of one token)
+//   values [token / 8][head_dim][8 tokens]     (run = one element of 8 tokens)
+// head_dim and page_tokens are multiples of 8.
+__host__ __device__ inline long key_offset(int token, int element, int page_tokens) {
+    return (static_cast<long>(element >> 3) * page_tokens + token) * 8 + (element & 7);
+}
+__host__ __device__ inline long value_offset(int token, int element, int head_dim) {
+    return (static_cast<long>(token >> 3) * head_dim + element) * 8 + (token & 7);
+}
+
 // ---- error channel -------------------------------------------------------
 // Every entry point returns 0 on success.  On failure it returns nonzero and
 // leaves a message that leone_last_error() hands out.

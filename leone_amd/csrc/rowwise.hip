@@ -98,8 +98,7 @@ __global__ void rope_table_kernel(float* __restrict__ cos_out, float* __restrict
 //   q heads: optional RMSNorm over D, optional rotation, written to q_out.
 //   k heads: the same, written into the request's page at `position`.
 //   v heads: copied into the page unchanged.
-// Keys lie in a page as [kv head][token][element], values transposed as
-// [kv head][element][token], which is how the attention kernels read them.
+// Keys and values go into the page in the packed layouts of key_offset() and value_offset().
 // A lane owns pairs p = lane, lane + 64, ... (p < D/2): elements p and p + D/2.
 // When `write_cache` is 0 the k and v heads are skipped (a layer that reads
 // another layer's cache).
@@ -124,22 +123,23 @@ __global__ void qk_norm_rope_write_kernel(
 
     const bool is_q = head < q_heads;
     const bool is_k = !is_q && head < q_heads + kv_heads;
+    // Where element d of this head goes: q rows are plain; keys and values use the cache's packed layout.
     T* dst;
-    long dst_stride = 1;   // distance between consecutive elements of the head at the destination
+    int kind = 0;  // 0 plain, 1 key page, 2 value page
+    int token = 0;
     if (is_q) {
         dst = q_out + (static_cast<long>(row) * q_heads + head) * head_dim;
     } else {
         const int kvh = is_k ? head - q_heads : head - q_heads - kv_heads;
         const int page = block_table[static_cast<long>(row_entry[row]) * max_blocks + pos / page_tokens];
         if (page < 0) return;  // host reserves pages before the launch
-        const long head_base = (static_cast<long>(page) * kv_heads + kvh) * page_tokens * head_dim;
-        if (is_k) {
-            dst = k_pool + head_base + static_cast<long>(pos % page_tokens) * head_dim;   // [token][element]
-        } else {
-            dst = v_pool + head_base + pos % page_tokens;                               // [element][token]
-            dst_stride = page_tokens;
-        }
+        dst = (is_k ? k_pool : v_pool) + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * head_dim;
+        kind = is_k ? 1 : 2;
+        token = pos % page_tokens;
     }
+    auto place = [&](int d) -> long {
+        return kind == 0 ? d : kind == 1 ? key_offset(token, d, page_tokens) : value_offset(token, d, head_dim);
+    };
 
     float a[kMaxPairsPerLane], b[kMaxPairsPerLane];
     float ss = 0.f;
@@ -158,8 +158,8 @@ __global__ void qk_norm_rope_write_kernel(
         for (int i = 0; i < kMaxPairsPerLane; ++i) {
             const int p = lane + i * kWave;
             if (p < half) {
-                dst[p * dst_stride] = from_float<T>(a[i]);
-                dst[(p + half) * dst_stride] = from_float<T>(b[i]);
+                dst[place(p)] = from_float<T>(a[i]);
+                dst[place(p + half)] = from_float<T>(b[i]);
             }
         }
         return;
@@ -189,8 +189,8 @@ __global__ void qk_norm_rope_write_kernel(
                 u = ru;
                 v = rv;
             }
-            dst[p] = from_float<T>(u);
-            dst[p + half] = from_float<T>(v);
+            dst[place(p)] = from_float<T>(u);
+            dst[place(p + half)] = from_float<T>(v);
         }
     }
 }
@@ -298,6 +298,8 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, void* q_out, void* k_po
     LEONE_REQUIRE(rows > 0 && q_heads > 0 && kv_heads > 0, "qk_norm_rope_write: rows %d heads %d/%d must be positive", rows, q_heads, kv_heads);
     LEONE_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= 2 * kWave * kMaxPairsPerLane,
                   "qk_norm_rope_write: head_dim %d must be even and at most %d", head_dim, 2 * kWave * kMaxPairsPerLane);
+    LEONE_REQUIRE(!write_cache || (head_dim % 8 == 0 && page_tokens % 8 == 0),
+                  "qk_norm_rope_write: the cache needs head_dim %d and page_tokens %d to be multiples of 8", head_dim, page_tokens);
     const int heads_total = q_heads + (write_cache ? 2 * kv_heads : 0);
     const int waves_per_block = 4;
     dim3 grid(rows, ceil_div(heads_total, waves_per_block));

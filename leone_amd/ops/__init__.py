@@ -42,6 +42,30 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+def cache_dims(k_pool: torch.Tensor, v_pool: torch.Tensor):
+    """(pages, kv_heads, page_tokens, head_dim) of a key/value pool pair in the packed cache layout:
+    keys ``[pages, kv_heads, head_dim/8, page_tokens, 8]``, values ``[pages, kv_heads, page_tokens/8, head_dim, 8]``."""
+    if k_pool.dim() != 5 or k_pool.shape[4] != 8:
+        raise KernelError(f"key pool must be [pages, kv_heads, head_dim/8, page_tokens, 8], found {tuple(k_pool.shape)}")
+    pages, kv_heads, d8, page_tokens, _ = k_pool.shape
+    if page_tokens % 8 or tuple(v_pool.shape) != (pages, kv_heads, page_tokens // 8, d8 * 8, 8):
+        raise KernelError(f"value pool must be [pages, kv_heads, page_tokens/8, head_dim, 8] matching the key pool "
+                          f"{tuple(k_pool.shape)}, found {tuple(v_pool.shape)}")
+    return pages, kv_heads, page_tokens, d8 * 8
+
+
+def pack_keys(k: torch.Tensor) -> torch.Tensor:
+    """[..., tokens, head_dim] -> the packed page layout [..., head_dim/8, tokens, 8]."""
+    *lead, tokens, dim = k.shape
+    return k.reshape(*lead, tokens, dim // 8, 8).transpose(-3, -2).contiguous()
+
+
+def pack_values(v: torch.Tensor) -> torch.Tensor:
+    """[..., tokens, head_dim] -> the packed page layout [..., tokens/8, head_dim, 8]."""
+    *lead, tokens, dim = v.shape
+    return v.reshape(*lead, tokens // 8, 8, dim).transpose(-2, -1).contiguous()
+
+
 def embed(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[r] = table[tokens[r]] as float32.  Token ids must have been checked against the table."""
     vocab, hidden = table.shape
@@ -107,8 +131,8 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim:
     if write_cache:
         if k_pool is None or v_pool is None or block_table is None or row_entry is None:
             raise KernelError("qk_norm_rope_write: a cache write needs pools, a block table and a row map")
-        pages, pool_heads, page_tokens, pool_dim = k_pool.shape
-        if (pool_heads, pool_dim) != (kv_heads, head_dim) or tuple(v_pool.shape) != (pages, kv_heads, head_dim, page_tokens):
+        pages, pool_heads, page_tokens, pool_dim = cache_dims(k_pool, v_pool)
+        if (pool_heads, pool_dim) != (kv_heads, head_dim):
             raise KernelError(f"qk_norm_rope_write: pool shape {tuple(k_pool.shape)} does not fit "
                               f"{kv_heads} heads of {head_dim}")
         max_blocks = block_table.shape[1]
@@ -137,11 +161,9 @@ def attention_rows(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, 
                    window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Each query row attends its request's cached keys up to its own position."""
     rows = q.shape[0]
-    pages, kv_heads, page_tokens, head_dim = k_pool.shape
+    pages, kv_heads, page_tokens, head_dim = cache_dims(k_pool, v_pool)
     if q.shape[1] != q_heads * head_dim:
         raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
-    if tuple(v_pool.shape) != (pages, kv_heads, head_dim, page_tokens):
-        raise KernelError("attention: the value pool must be [pages, kv_heads, head_dim, page_tokens]")
     if out is None:
         out = torch.empty_like(q)
     call("leone_attention_rows", _dev(q, "attention q"), _dev(out, "attention out", q.dtype, q.shape),
@@ -172,11 +194,9 @@ def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Split-KV attention on the matrix cores (bfloat16).  ``max_context`` only steers the number of splits."""
     rows = q.shape[0]
-    pages, kv_heads, page_tokens, head_dim = k_pool.shape
+    pages, kv_heads, page_tokens, head_dim = cache_dims(k_pool, v_pool)
     if q.shape[1] != q_heads * head_dim:
         raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
-    if tuple(v_pool.shape) != (pages, kv_heads, head_dim, page_tokens):
-        raise KernelError("attention: the value pool must be [pages, kv_heads, head_dim, page_tokens]")
     if splits is None:
         splits = choose_splits(rows, kv_heads, q_heads // kv_heads, max_context)
     if out is None:

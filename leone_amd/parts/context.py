@@ -46,8 +46,8 @@ class CacheView:
 
 @dataclass
 class KvCacheView(CacheView):
-    k_pool: torch.Tensor = None        # [pages, kv_heads, page_tokens, head_dim]
-    v_pool: torch.Tensor = None        # [pages, kv_heads, head_dim, page_tokens] (transposed)
+    k_pool: torch.Tensor = None        # [pages, kv_heads, head_dim / 8, page_tokens, 8]
+    v_pool: torch.Tensor = None        # [pages, kv_heads, page_tokens / 8, head_dim, 8]
     block_table: torch.Tensor = None   # int32 [entries, max_blocks] of the layer's group
     page_tokens: int = 0
 

@@ -106,8 +106,9 @@ def paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed, extra_pag
     order = torch.randperm(n_pages, generator=g).tolist()
     max_blocks = max(blocks) + 1
     table = torch.full((len(lengths), max_blocks), -1, dtype=torch.int32)
+    # plain [page][head][token][element] first, NaN where nothing lives; packed into the cache layout at the end
     k_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), float("nan"))
-    v_pool = torch.full((n_pages, kv_heads, head_dim, page_tokens), float("nan"))     # values lie transposed
+    v_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), float("nan"))
     keys, values = [], []
     at = 0
     for r, n in enumerate(lengths):
@@ -121,7 +122,9 @@ def paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed, extra_pag
             table[r, b] = page
             lo, hi = b * page_tokens, min(n, (b + 1) * page_tokens)
             k_pool[page, :, :hi - lo] = k[lo:hi].transpose(0, 1)
-            v_pool[page, :, :, :hi - lo] = v[lo:hi].permute(1, 2, 0)
+            v_pool[page, :, :hi - lo] = v[lo:hi].transpose(0, 1)
+    from leone_amd import ops
+    k_pool, v_pool = ops.pack_keys(k_pool), ops.pack_values(v_pool)
     return table, k_pool.to(dtype), v_pool.to(dtype), keys, values
 
 
@@ -157,14 +160,19 @@ def test_attention_reference_vector():
     """2 heads, 1 kv head, D=2, K rows [1,0],[0,1], V rows [2,4],[6,8], q [1,0] and [0,1] per token
     (crates/leone/src/cpu.rs:2850-2898)."""
     from leone_amd import ops
-    k_pool = torch.zeros(1, 1, 16, 2, device=DEV)
-    v_pool = torch.zeros(1, 1, 2, 16, device=DEV)
-    k_pool[0, 0, 0] = torch.tensor([1.0, 0.0]); k_pool[0, 0, 1] = torch.tensor([0.0, 1.0])
-    v_pool[0, 0, :, 0] = torch.tensor([2.0, 4.0]); v_pool[0, 0, :, 1] = torch.tensor([6.0, 8.0])
-    q = torch.tensor([[1.0, 0.0, 0.0, 1.0], [1.0, 0.0, 0.0, 1.0]], device=DEV)
-    out = ops.attention_rows(q, k_pool, v_pool, torch.tensor([0, 1], dtype=torch.int32, device=DEV),
+    # head_dim 2 there; here the heads are padded with zeros to 8, which changes no score as the scale is given
+    k = torch.zeros(1, 1, 16, 8)
+    v = torch.zeros(1, 1, 16, 8)
+    k[0, 0, 0, :2] = torch.tensor([1.0, 0.0]); k[0, 0, 1, :2] = torch.tensor([0.0, 1.0])
+    v[0, 0, 0, :2] = torch.tensor([2.0, 4.0]); v[0, 0, 1, :2] = torch.tensor([6.0, 8.0])
+    q = torch.zeros(2, 2, 8)
+    q[:, 0, 0] = 1.0
+    q[:, 1, 1] = 1.0
+    out = ops.attention_rows(q.reshape(2, 16).to(DEV), ops.pack_keys(k).to(DEV), ops.pack_values(v).to(DEV),
+                             torch.tensor([0, 1], dtype=torch.int32, device=DEV),
                              torch.zeros(2, dtype=torch.int32, device=DEV),
                              torch.zeros(1, 1, dtype=torch.int32, device=DEV), 2, 1.0 / math.sqrt(2.0))
+    out = out.view(2, 2, 8)[:, :, :2].reshape(2, 4)
     h = math.exp(1.0 / math.sqrt(2.0))
     want = torch.tensor([[2.0, 4.0, 2.0, 4.0],
                          [(h * 2 + 6) / (h + 1), (h * 4 + 8) / (h + 1), (2 + h * 6) / (h + 1), (4 + h * 8) / (h + 1)]])
@@ -191,8 +199,13 @@ def test_qk_norm_rope_write(dtype, shape):
     table[1, 16 // page_tokens] = 2
     table[1, 17 // page_tokens] = 2 if 16 // page_tokens == 17 // page_tokens else 5
     table[2, 8000 // page_tokens] = 1
-    k_pool = torch.full((n_pages, kv_heads, page_tokens, head_dim), 7.0).to(dtype)
-    v_pool = torch.full((n_pages, kv_heads, head_dim, page_tokens), 7.0).to(dtype)
+    k_pool = torch.full((n_pages, kv_heads, head_dim // 8, page_tokens, 8), 7.0).to(dtype)
+    v_pool = torch.full((n_pages, kv_heads, page_tokens // 8, head_dim, 8), 7.0).to(dtype)
+
+    def unpack(kp, vp):
+        """Packed pools back to [page][head][token][element]."""
+        return (kp.cpu().transpose(2, 3).reshape(n_pages, kv_heads, page_tokens, head_dim),
+                vp.cpu().transpose(3, 4).reshape(n_pages, kv_heads, page_tokens, head_dim))
     cos, sin = ops.rope_table(theta, head_dim, 8192, DEV)
     positions = torch.tensor([p for _, p in rows_meta], dtype=torch.int32)
     row_entry = torch.tensor([e for e, _ in rows_meta], dtype=torch.int32)
@@ -208,15 +221,15 @@ def test_qk_norm_rope_write(dtype, shape):
     atol, rtol = (5e-6, 2e-5) if dtype == torch.float32 else (2e-2, 1e-2)
     close(q_out.view(n, q_heads, head_dim), want_q, atol, rtol, "q")
     touched = torch.zeros(n_pages, page_tokens, dtype=torch.bool)
+    k_plain, v_plain = unpack(kp, vp)
     for i, (e, p) in enumerate(rows_meta):
         page, off = int(table[e, p // page_tokens]), p % page_tokens
         touched[page, off] = True
-        close(kp[page, :, off], want_k[i], atol, rtol, f"k row {i}")
-        assert torch.equal(vp[page, :, :, off].cpu(), v[i].to(dtype))   # values are copied unchanged, transposed
+        close(k_plain[page, :, off], want_k[i], atol, rtol, f"k row {i}")
+        assert torch.equal(v_plain[page, :, off], v[i].to(dtype))          # values are copied unchanged
     # every other slot is untouched
     untouched = ~touched[:, None, :].expand(-1, kv_heads, -1)
-    assert torch.equal(kp.cpu()[untouched], k_pool[untouched])
-    assert torch.equal(vp.cpu().transpose(2, 3)[untouched], v_pool.transpose(2, 3)[untouched])
+    assert (k_plain[untouched] == 7.0).all() and (v_plain[untouched] == 7.0).all()
     # a layer that reads another layer's cache writes nothing
     kp2, vp2 = k_pool.to(DEV), v_pool.to(DEV)
     q2 = ops.qk_norm_rope_write(qkv.to(DEV), q_heads, kv_heads, head_dim, q_gain.to(DEV), k_gain.to(DEV), eps, cos,

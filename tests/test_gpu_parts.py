@@ -93,8 +93,8 @@ def test_attention_part_with_portions_and_two_requests(dtype):
     pw.update({"a.q_norm.weight": w["q_norm"].float(), "a.k_norm.weight": w["k_norm"].float()})
     cfg = dict(num_attention_heads=q_heads, num_key_value_heads=kv_heads, head_dim=dim, rms_norm_eps=1e-5, rope_theta=1e4)
     want = [plain.attention_block(y.float(), pw, "a", cfg, list(range(len(y)))) for y in ys]
-    k_pool = torch.full((8, kv_heads, page, dim), float("nan"), dtype=dtype, device=DEV)
-    v_pool = torch.full((8, kv_heads, dim, page), float("nan"), dtype=dtype, device=DEV)
+    k_pool = torch.full((8, kv_heads, dim // 8, page, 8), float("nan"), dtype=dtype, device=DEV)
+    v_pool = torch.full((8, kv_heads, page // 8, dim, 8), float("nan"), dtype=dtype, device=DEV)
     table = torch.tensor([[5, 0, 3, -1], [7, 2, -1, -1]], dtype=torch.int32, device=DEV)
     cache = KvCacheView(writes=True, k_pool=k_pool, v_pool=v_pool, block_table=table, page_tokens=page)
     # call 1: all of request 0 and the first 20 tokens of request 1
