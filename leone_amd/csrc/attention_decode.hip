@@ -25,6 +25,7 @@
 #include "leone_hip.h"
 
 #include <math.h>
+#include <type_traits>
 
 namespace leone {
 
@@ -94,47 +95,68 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
 #pragma unroll
     for (int dt = 0; dt < kD16; ++dt) acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    for (int t = my_begin + wave; t < my_end; t += kDecodeWaves) {
+    // One 32-key tile.  `full` tiles lie wholly inside [lo, n) and need no masks; at most the first
+    // and the last tile of a row are not.  All loads of a tile, keys and values, are issued before
+    // the first product, so that they are in flight together.
+    auto do_tile = [&](int t, auto full_tag) {
+        constexpr bool kFull = decltype(full_tag)::value;
         const int key0 = t * kTileKeys;
+        // A-operand row c of half a is key 8*(c/4) + c%4, of half b four keys further
+        const int ka = key0 + 8 * (c >> 2) + (c & 3);
+        const int kb = ka + 4;
+        const int run0 = key0 + 8 * g;                   // this lane's eight keys for the second product
+        bool va = true, vb = true, any = true, whole = true;
+        if constexpr (!kFull) {
+            va = ka >= lo && ka < n;
+            vb = kb >= lo && kb < n;
+            any = run0 < n && run0 + 8 > lo;
+            whole = run0 >= lo && run0 + 8 <= n;
+        }
+        const bf16_t* pk = k_pool;
+        const bf16_t* pv = v_pool;
+        if (va || vb) {                                   // ka and kb share a page: pages hold multiples of 8 keys
+            const int page = table[ka >> page_shift];
+            if (page < 0) {
+                unmapped = true;                          // never read outside the pool; the result is poisoned below
+                va = vb = false;
+            }
+            pk = k_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (ka & page_mask) * 8;
+        }
+        if (any) {
+            const int page = table[run0 >> page_shift];
+            if (page < 0) {
+                unmapped = true;
+                any = false;
+            }
+            pv = v_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD +
+                 static_cast<long>((run0 & page_mask) >> 3) * kD * 8;
+        }
+        bf16x8 xa[kSteps], xb[kSteps], xv[kD16];
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            const bool in_head = 32 * s + 8 * g < kD;
+            const long run = static_cast<long>(4 * s + g) * page_tokens * 8;   // elements 32s+8g .. +7 of the key
+            xa[s] = (va && in_head) ? load8(pk + run) : zero8();
+            xb[s] = (vb && in_head) ? load8(pk + run + 32) : zero8();           // four keys further
+        }
+#pragma unroll
+        for (int dt = 0; dt < kD16; ++dt) xv[dt] = any ? load8(pv + (16 * dt + c) * 8) : zero8();
+
         // ---- S^T = K . Q^T for the two 16-key halves --------------------------------------------
         floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
-        {
-            // A-operand row c of half a is key 8*(c/4) + c%4, of half b four keys further
-            const int ka = key0 + 8 * (c >> 2) + (c & 3);
-            const int kb = ka + 4;
-            bool va = ka >= lo && ka < n, vb = kb >= lo && kb < n;
-            const bf16_t* pa = k_pool;
-            const bf16_t* pb = k_pool;
-            if (va) {
-                const int page = table[ka >> page_shift];
-                if (page < 0) unmapped = true;   // never read outside the pool; the result is poisoned below
-                pa = k_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (ka & page_mask) * 8;
-            }
-            if (vb) {
-                const int page = table[kb >> page_shift];
-                if (page < 0) unmapped = true;
-                pb = k_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (kb & page_mask) * 8;
-            }
-            if (unmapped) va = vb = false;
 #pragma unroll
-            for (int s = 0; s < kSteps; ++s) {
-                const int d0 = 32 * s + 8 * g;
-                const bool in_head = d0 < kD;
-                const long run = static_cast<long>(4 * s + g) * page_tokens * 8;   // run of elements d0 .. d0+7
-                const bf16x8 xa = (va && in_head) ? load8(pa + run) : zero8();
-                const bf16x8 xb = (vb && in_head) ? load8(pb + run) : zero8();
-                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, qreg[s], sa, 0, 0, 0);
-                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb, qreg[s], sb, 0, 0, 0);
-            }
+        for (int s = 0; s < kSteps; ++s) {
+            sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[s], qreg[s], sa, 0, 0, 0);
+            sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb[s], qreg[s], sb, 0, 0, 0);
         }
         // lane (g, c) now holds, for query column c, the scores of keys key0 + 8g + j, j = 0..7
         float sc[8];
         float tile_max = -INFINITY;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const int key = key0 + 8 * g + j;
-            const float raw = j < 4 ? sa[j] : sb[j - 4];
-            sc[j] = (key >= lo && key < n) ? raw * scale : -INFINITY;
+            const int key = run0 + j;
+            const float raw = j < 4 ? sa[j & 3] : sb[j & 3];
+            sc[j] = (kFull || (key >= lo && key < n)) ? raw * scale : -INFINITY;
             tile_max = fmaxf(tile_max, sc[j]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
@@ -154,69 +176,67 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         l_run = l_run * alpha + psum;
         m_run = m_new;
         // ---- O^T += V^T . P^T ------------------------------------------------------------------
-        const int run0 = key0 + 8 * g;                   // this lane's eight keys: run0 .. run0+7
-        bool any = run0 < n && run0 + 8 > lo;
-        const bool whole = run0 >= lo && run0 + 8 <= n;
-        const bf16_t* pv = v_pool;
-        if (any) {
-            const int page = table[run0 >> page_shift];
-            if (page < 0) {
-                unmapped = true;
-                any = false;
-            }
-            pv = v_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD +
-                 static_cast<long>((run0 & page_mask) >> 3) * kD * 8;
-        }
 #pragma unroll
         for (int dt = 0; dt < kD16; ++dt) {
-            bf16x8 xv = any ? load8(pv + (16 * dt + c) * 8) : zero8();
-            if (any && !whole) {
-                // slots outside [lo, n) may hold anything, even NaN: clear them, a zero weight is not enough
-                uint4 raw = __builtin_bit_cast(uint4, xv);
-                unsigned* w = reinterpret_cast<unsigned*>(&raw);
+            if constexpr (!kFull) {
+                if (any && !whole) {
+                    // slots outside [lo, n) may hold anything, even NaN: clear them, a zero weight is not enough
+                    uint4 raw = __builtin_bit_cast(uint4, xv[dt]);
+                    unsigned* w = reinterpret_cast<unsigned*>(&raw);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int e0 = run0 + 2 * i, e1 = e0 + 1;
-                    unsigned mask = 0u;
-                    if (e0 >= lo && e0 < n) mask |= 0x0000ffffu;
-                    if (e1 >= lo && e1 < n) mask |= 0xffff0000u;
-                    w[i] &= mask;
+                    for (int i = 0; i < 4; ++i) {
+                        const int e0 = run0 + 2 * i, e1 = e0 + 1;
+                        unsigned mask = 0u;
+                        if (e0 >= lo && e0 < n) mask |= 0x0000ffffu;
+                        if (e1 >= lo && e1 < n) mask |= 0xffff0000u;
+                        w[i] &= mask;
+                    }
+                    xv[dt] = __builtin_bit_cast(bf16x8, raw);
                 }
-                xv = __builtin_bit_cast(bf16x8, raw);
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[dt][r] *= alpha;
-            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv, pt, acc[dt], 0, 0, 0);
+            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[dt], pt, acc[dt], 0, 0, 0);
         }
+    };
+
+    for (int t = my_begin + wave; t < my_end; t += kDecodeWaves) {
+        const int key0 = t * kTileKeys;
+        if (key0 >= lo && key0 + kTileKeys <= n)
+            do_tile(t, std::true_type{});
+        else
+            do_tile(t, std::false_type{});
     }
 
     // ---- merge the four waves --------------------------------------------------------------------
-    float* sm_acc = smem;                                         // [waves][16][kD]
-    float* sm_m = smem + kDecodeWaves * 16 * kD;                  // [waves][16]
-    float* sm_l = sm_m + kDecodeWaves * 16;
+    float* sm_acc = smem;                                         // [waves][cols][kD]
+    float* sm_m = smem + kDecodeWaves * cols * kD;                // [waves][cols]
+    float* sm_l = sm_m + kDecodeWaves * cols;
     if (__any(unmapped)) l_run = __builtin_nanf("");   // a key in reach had no page: say so in the result
-    if (g == 0) {
-        sm_m[wave * 16 + c] = m_run;
-        sm_l[wave * 16 + c] = l_run;
+    if (g == 0 && c < cols) {
+        sm_m[wave * cols + c] = m_run;
+        sm_l[wave * cols + c] = l_run;
     }
+    if (c < cols) {
 #pragma unroll
-    for (int dt = 0; dt < kD16; ++dt)
+        for (int dt = 0; dt < kD16; ++dt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) sm_acc[(wave * 16 + c) * kD + 16 * dt + 4 * g + r] = acc[dt][r];
+            for (int r = 0; r < 4; ++r) sm_acc[(wave * cols + c) * kD + 16 * dt + 4 * g + r] = acc[dt][r];
+    }
     __syncthreads();
     for (int i = threadIdx.x; i < cols * kD; i += kDecodeThreads) {
         const int col = i / kD, d = i % kD;
         float top = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < kDecodeWaves; ++w) top = fmaxf(top, sm_m[w * 16 + col]);
+        for (int w = 0; w < kDecodeWaves; ++w) top = fmaxf(top, sm_m[w * cols + col]);
         float num = 0.f, den = 0.f;
         if (top != -INFINITY) {
 #pragma unroll
             for (int w = 0; w < kDecodeWaves; ++w) {
-                const float mw = sm_m[w * 16 + col];
+                const float mw = sm_m[w * cols + col];
                 const float wgt = mw == -INFINITY ? 0.f : __expf(mw - top);
-                num += sm_acc[(w * 16 + col) * kD + d] * wgt;
-                den += sm_l[w * 16 + col] * wgt;
+                num += sm_acc[(w * cols + col) * kD + d] * wgt;
+                den += sm_l[w * cols + col] * wgt;
             }
         }
         const long slot = (static_cast<long>(row) * q_heads + kvh * group + col0 + col) * splits + split;
@@ -247,8 +267,9 @@ __global__ void attention_reduce_kernel(const float* __restrict__ part_acc, cons
     }
 }
 
-static size_t decode_smem_bytes(int head_dim) {
-    return (static_cast<size_t>(kDecodeWaves) * 16 * head_dim + 2 * kDecodeWaves * 16) * sizeof(float);
+static size_t decode_smem_bytes(int head_dim, int group) {
+    const int cols = group < 16 ? group : 16;
+    return (static_cast<size_t>(kDecodeWaves) * cols * head_dim + 2 * kDecodeWaves * cols) * sizeof(float);
 }
 
 template <int kD16>
@@ -258,7 +279,7 @@ static void launch_decode(const void* q, const void* k_pool, const void* v_pool,
                           int window, int splits, hipStream_t stream) {
     const int group = q_heads / kv_heads;
     dim3 grid(rows, kv_heads * ((group + 15) / 16), splits);
-    const size_t smem = decode_smem_bytes(kD16 * 16);
+    const size_t smem = decode_smem_bytes(kD16 * 16, group);
     attention_decode_kernel<kD16><<<grid, kDecodeThreads, smem, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
         positions, row_entry, block_table, max_blocks, part_acc, part_ml, q_heads, kv_heads, page_shift, scale, window,
@@ -283,7 +304,7 @@ extern "C" int leone_attention_decode(const void* q, void* out, const void* k_po
                   "attention_decode: head_dim %d must be a multiple of 16 in 16..256", head_dim);
     LEONE_REQUIRE(page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0,
                   "attention_decode: page_tokens %d must be a power of two, at least 16", page_tokens);
-    LEONE_REQUIRE(decode_smem_bytes(head_dim) <= 64 * 1024,
+    LEONE_REQUIRE(decode_smem_bytes(head_dim, q_heads / kv_heads) <= 64 * 1024,
                   "attention_decode: head_dim %d needs more shared memory than a workgroup may have", head_dim);
     LEONE_REQUIRE(splits >= 1 && splits <= 65535, "attention_decode: splits %d out of range", splits);
     LEONE_REQUIRE(window >= 0 && max_blocks > 0, "attention_decode: bad window or block table");

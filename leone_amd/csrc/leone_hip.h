@@ -44,7 +44,7 @@ int leone_attention_rows(const void* q, void* out, const void* k_pool, const voi
 
 // The same on the matrix cores for bfloat16, the keys of a row cut into `splits` parts whose
 // partial results (part_acc: rows*q_heads*splits*head_dim floats, part_ml: rows*q_heads*splits*2)
-// are merged by a second kernel.  head_dim a multiple of 16 up to 240, page_tokens a power of two >= 16.
+// are merged by a second kernel.  head_dim a multiple of 16 up to 256, page_tokens a power of two >= 16.
 int leone_attention_decode(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
                            const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
                            float* part_ml, int rows, int q_heads, int kv_heads, int head_dim, int page_tokens,
@@ -52,6 +52,10 @@ int leone_attention_decode(const void* q, void* out, const void* k_pool, const v
 
 // C[M,N] = A[M,K] . B[N,K]^T in float.
 int leone_gemm_f32(const float* a, const float* b, float* c, int m, int n, int k, hipStream_t stream);
+
+// Y[M,N] = X[M,K] . W[N,K]^T for bfloat16 X and W, M <= 64, K a multiple of 8; Y float or bfloat16.
+int leone_gemm_skinny_bf16(const void* x, const void* w, void* y, int out_dtype, int m, int n, int k,
+                           hipStream_t stream);
 
 int leone_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream);
 int leone_sample_temperature(const float* logits, const double* temperature, const double* uniform, int* out,

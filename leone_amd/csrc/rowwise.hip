@@ -60,6 +60,71 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__
     }
 }
 
+// The same for rows whose length is a multiple of 4 and at most 4 * kThreads * kChunks: every
+// thread keeps its elements in registers, so the row is read once, with 16-byte loads, and the
+// gains are fetched together with it.
+__device__ inline void load4(const float* p, float v[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ inline void load4(const bf16_t* p, float v[4]) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+    v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+__device__ inline void store4(float* p, const float v[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ inline void store4(bf16_t* p, const float v[4]) {
+    uint2 t;
+    t.x = bf16_bits_from_float(v[0]) | (static_cast<uint32_t>(bf16_bits_from_float(v[1])) << 16);
+    t.y = bf16_bits_from_float(v[2]) | (static_cast<uint32_t>(bf16_bits_from_float(v[3])) << 16);
+    *reinterpret_cast<uint2*>(p) = t;
+}
+
+template <typename TD, typename TG, typename TY, int kThreads, int kChunks>
+__global__ void __launch_bounds__(kThreads)
+add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, const TG* __restrict__ gain, float eps,
+                       TY* __restrict__ y, const int* __restrict__ rows, int hidden) {
+    __shared__ float scratch[kThreads / kWave];
+    const int out_row = blockIdx.x;
+    const long in_row = rows ? rows[out_row] : out_row;
+    float* xr = x + in_row * hidden;
+    const TD* dr = delta ? delta + in_row * hidden : nullptr;
+    TY* yr = y + static_cast<long>(out_row) * hidden;
+    float v[kChunks][4], gv[kChunks][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+        const int c = 4 * (threadIdx.x + i * kThreads);
+        if (c < hidden) {
+            load4(xr + c, v[i]);
+            load4(gain + c, gv[i]);
+            if (dr) {
+                float d[4];
+                load4(dr + c, d);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[i][j] += d[j];
+                if (!rows) store4(xr + c, v[i]);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) ss = fmaf(v[i][j], v[i][j], ss);
+        }
+    }
+    const float total = block_sum<kThreads>(ss, scratch);
+    const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+        const int c = 4 * (threadIdx.x + i * kThreads);
+        if (c < hidden) {
+            float o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[j] = (v[i][j] * gv[i][j]) * inv;
+            store4(yr + c, o);
+        }
+    }
+}
+
 // ---- SwiGLU -------------------------------------------------------------------
 // in: [rows, 2F] with the gate in the first F columns, up in the last F.
 template <typename T>
@@ -221,9 +286,32 @@ extern "C" int leone_embed(const void* table, int dtype, const int* tokens, floa
     return 0;
 }
 
+template <typename TD, typename TG, typename TY>
+static void launch_add_rmsnorm_vec(float* x, const void* delta, const void* gain, float eps, void* y,
+                                   const int* rows, int n_rows, int hidden, hipStream_t stream) {
+    const TD* d = static_cast<const TD*>(delta);
+    const TG* g = static_cast<const TG*>(gain);
+    TY* out = static_cast<TY*>(y);
+    if (hidden <= 4 * 64 * 2)
+        add_rmsnorm_vec_kernel<TD, TG, TY, 64, 2><<<n_rows, 64, 0, stream>>>(x, d, g, eps, out, rows, hidden);
+    else if (hidden <= 4 * 256 * 2)
+        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 2><<<n_rows, 256, 0, stream>>>(x, d, g, eps, out, rows, hidden);
+    else if (hidden <= 4 * 256 * 4)
+        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 4><<<n_rows, 256, 0, stream>>>(x, d, g, eps, out, rows, hidden);
+    else
+        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 8><<<n_rows, 256, 0, stream>>>(x, d, g, eps, out, rows, hidden);
+}
+
 template <typename TD, typename TY>
 static void launch_add_rmsnorm(float* x, const void* delta, AnyVec gain, float eps, void* y,
                                const int* rows, int n_rows, int hidden, hipStream_t stream) {
+    if (hidden % 4 == 0 && hidden <= 4 * 256 * 8) {
+        if (gain.dtype == kF32)
+            launch_add_rmsnorm_vec<TD, float, TY>(x, delta, gain.ptr, eps, y, rows, n_rows, hidden, stream);
+        else
+            launch_add_rmsnorm_vec<TD, bf16_t, TY>(x, delta, gain.ptr, eps, y, rows, n_rows, hidden, stream);
+        return;
+    }
     if (hidden > 512)
         add_rmsnorm_kernel<TD, TY, 256><<<n_rows, 256, 0, stream>>>(x, static_cast<const TD*>(delta), gain, eps, static_cast<TY*>(y), rows, hidden);
     else

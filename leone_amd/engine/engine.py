@@ -41,10 +41,59 @@ class StepError(ValueError):
     """A step was refused before anything ran; the cache is unchanged."""
 
 
+class _DecodeGraph:
+    """A recorded decode step for one batch size: static metadata buffers, the graph, its logits.
+
+    The step's metadata (tokens, positions, state slots, block tables) lives in one device buffer
+    that is refilled before each replay; the recorded kernels read everything through it, so one
+    recording serves every step of that batch size (the reference replays one decode graph per
+    context bucket with a device-resident position, crates/leone/src/runtime.rs:4991-5013).
+    """
+
+    def __init__(self, engine: "Engine", rows: int):
+        groups = len(engine.cache.groups)
+        widths = [engine.cache.max_blocks(g) for g in range(groups)]
+        sizes = [rows] * 5 + [rows * w for w in widths]     # tokens, positions, row_entry, slots, want, tables
+        self.offsets = np.cumsum([0] + sizes)
+        total = int(self.offsets[-1])
+        self.host = torch.empty(total, dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(total, dtype=torch.int32, device=engine.device)
+        pieces = [self.dev[self.offsets[i]:self.offsets[i + 1]] for i in range(len(sizes))]
+        self.tokens = pieces[0]
+        self.rows = rows
+        self.widths = widths
+        self.context = StepContext(
+            rows=rows, dtype=engine.dtype, device=engine.device, positions=pieces[1], row_entry=pieces[2],
+            entries=[], entry_slots=pieces[3], want_rows=pieces[4],
+            block_tables={g: pieces[5 + g].view(rows, widths[g]) for g in range(groups)},
+            max_position=engine.max_context - 1, decode_only=True)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+        self.copied = torch.cuda.Event()
+
+    def fill(self, engine: "Engine", entries: Sequence[StepEntry]) -> None:
+        self.copied.synchronize()                     # the last upload has left the pinned buffer
+        rows, o, h = self.rows, self.offsets, self.host_np
+        h[o[2]:o[3]] = np.arange(rows)
+        h[o[4]:o[5]] = np.arange(rows)
+        for i, e in enumerate(entries):
+            h[o[0] + i] = int(e.tokens[0])
+            h[o[1] + i] = engine.cache.length(e.request)
+            h[o[3] + i] = engine.cache.slot(e.request)
+            for g, width in enumerate(self.widths):
+                table = engine.cache.table(e.request, g)
+                base = o[5 + g] + i * width
+                h[base:base + len(table)] = table
+                h[base + len(table):base + width] = -1
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+
+
 class Engine:
     def __init__(self, model: DecoderModel, *, num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  page_tokens: int = 64, max_requests: int = 64, max_context: Optional[int] = None,
-                 poison_freed: bool = False):
+                 poison_freed: bool = False, graphs: bool = True):
         if model.embedding is None:
             raise ValueError("the model has no weights bound")
         if not torch.cuda.is_available() or model.device.type != "cuda":
@@ -62,6 +111,9 @@ class Engine:
         self.cache = CacheManager(self.pools.group_specs, max_requests, self.max_context)
         self.poison_freed = poison_freed
         self.vocab_size = model.spec.vocab_size
+        # Steps of single decoded tokens are recorded once per batch size and replayed.
+        self.graphs = bool(graphs) and model.graph_safe
+        self._decode_graphs: Dict[int, _DecodeGraph] = {}
 
     # ---- requests -----------------------------------------------------------------
     def admit(self, request: Hashable) -> int:
@@ -124,9 +176,12 @@ class Engine:
             for e in entries:
                 if self.cache.length(e.request) == 0:
                     self.pools.zero_state(self.cache.slot(e.request))   # a request's state starts from zero
-            tokens, context, rows = self._build_context(entries)
-            caches = self.pools.views(context.block_tables)
-            logits = self.model.forward(tokens, context, caches)
+            if self.graphs and all(len(e.tokens) == 1 for e in entries):
+                logits, rows = self._run_decode_graph(entries)
+            else:
+                tokens, context, rows = self._build_context(entries)
+                caches = self.pools.views(context.block_tables)
+                logits = self.model.forward(tokens, context, caches)
         except Exception:
             for e in entries:
                 if self.cache.has(e.request):
@@ -145,6 +200,36 @@ class Engine:
                     gone = [p for b, p in enumerate(old) if p >= 0 and (b >= len(new) or new[b] != p)]
                     self.pools.poison_pages(g, gone)
         return StepOutput(logits, rows)
+
+    def _run_decode_graph(self, entries: Sequence[StepEntry]):
+        """One decoded token for each entry, replayed from the recording for this batch size."""
+        state = self._decode_graphs.get(len(entries))
+        if state is None:
+            state = self._decode_graphs[len(entries)] = _DecodeGraph(self, len(entries))
+        state.fill(self, entries)
+        if state.graph is None:
+            # First step of this size: run it for real on the static buffers, then record the same
+            # calls for later steps.  Recording executes nothing, so the cache is written once.
+            caches = self.pools.views(state.context.block_tables)
+            logits = self.model.forward(state.tokens, state.context, caches)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                state.logits = self.model.forward(state.tokens, state.context, caches)
+            state.graph = graph
+        else:
+            state.graph.replay()
+            logits = state.logits
+        wanted, rows_map = [], []
+        for i, e in enumerate(entries):
+            for w in e.want:
+                wanted.append(i)
+                rows_map.append((e.request, int(w)))
+        if not wanted:
+            return None, rows_map
+        if wanted == list(range(len(entries))):
+            return logits.clone(), rows_map                   # the recording's buffer is reused by the next replay
+        index = torch.tensor(wanted, dtype=torch.long, device=self.device)
+        return logits.index_select(0, index), rows_map
 
     def _build_context(self, entries: Sequence[StepEntry]):
         n_rows = sum(len(e.tokens) for e in entries)

@@ -174,18 +174,20 @@ def attention_rows(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, 
     return out
 
 
-def decode_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int) -> bool:
+def decode_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int, group: int = 1) -> bool:
     """Whether the matrix-core kernel takes this case; otherwise ``attention_rows`` does."""
-    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 240
+    cols = min(group, 16)
+    shared = (4 * cols * head_dim + 8 * cols) * 4          # the four waves' partial results
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and shared <= 64 * 1024
             and page_tokens >= 16 and page_tokens & (page_tokens - 1) == 0)
 
 
 def choose_splits(rows: int, kv_heads: int, group: int, max_context: int) -> int:
-    """How many parts the keys of a row are cut into: enough workgroups to fill 256 CUs, at least
-    four 32-key tiles a part so that each of a workgroup's waves has one."""
+    """How many parts the keys of a row are cut into: about two workgroups for each of the 256 CUs,
+    at least four 32-key tiles a part so that each of a workgroup's four waves has one."""
     blocks = rows * kv_heads * ((group + 15) // 16)
     tiles = (max_context + 31) // 32
-    return max(1, min(1024 // max(1, blocks), (tiles + 3) // 4, 256))
+    return max(1, min(512 // max(1, blocks), (tiles + 3) // 4, 256))
 
 
 def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
@@ -225,8 +227,27 @@ def gemm_f32(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = Non
     return out
 
 
+SKINNY_ROWS = 64           # most rows one launch of the weight-streaming kernel takes
+SKINNY_LIBRARY_ROWS = 4    # from here on the library's matrix product is used for bfloat16 results
+
+
+def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x[M,K] . weight[N,K]^T on the matrix cores for M <= 64 (bfloat16 in, float accumulation)."""
+    m, k = x.shape
+    n, k2 = weight.shape
+    if k != k2:
+        raise KernelError(f"gemm_skinny: inner sizes {k} and {k2} differ")
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    call("leone_gemm_skinny_bf16", _dev(x, "gemm x", torch.bfloat16), _dev(weight, "gemm weight", torch.bfloat16),
+         _dev(out, "gemm out", out_dtype, (m, n)), _CODES[out_dtype], m, n, k, _stream())
+    return out
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """x[R,K] . weight[N,K]^T.  float32 runs the single-precision kernel; bfloat16 inputs accumulate in float."""
+    """x[R,K] . weight[N,K]^T.  float32 runs the single-precision kernel.  bfloat16 accumulates in float:
+    up to 64 rows on the weight-streaming kernel, more rows through the library's matrix product."""
     if x.dtype != weight.dtype:
         raise KernelError(f"linear: activations are {x.dtype} but the weight is {weight.dtype}")
     out_dtype = out_dtype or x.dtype
@@ -236,6 +257,17 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtyp
         return gemm_f32(x, weight)
     if not x.is_cuda:
         raise KernelError("linear: tensor is not on the GPU")
+    rows, k = x.shape
+    # The weight-streaming kernel re-reads the activations for every 16 weight rows, which costs more
+    # than the library's product beyond a few rows; float32 results (logits) always come from it.
+    if k % 8 == 0 and (rows <= SKINNY_LIBRARY_ROWS or out_dtype == torch.float32):
+        if rows <= SKINNY_ROWS:
+            return gemm_skinny(x, weight, out_dtype)
+        # float32 results (logits) for many rows: 64 rows at a time, each pass streaming the weight again
+        out = torch.empty((rows, weight.shape[0]), dtype=out_dtype, device=x.device)
+        for at in range(0, rows, SKINNY_ROWS):
+            gemm_skinny(x[at:at + SKINNY_ROWS], weight, out_dtype, out=out[at:at + SKINNY_ROWS])
+        return out
     y = torch.nn.functional.linear(x, weight)  # library matrix product, float accumulation
     return y if out_dtype == y.dtype else y.to(out_dtype)
 

@@ -32,6 +32,7 @@ _PROTOTYPES = {
     "leone_attention_decode": [P, P, P, P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                c_int, P],
     "leone_gemm_f32": [P, P, P, c_int, c_int, c_int, P],
+    "leone_gemm_skinny_bf16": [P, P, P, c_int, c_int, c_int, c_int, P],
     "leone_argmax": [P, P, c_int, c_int, P],
     "leone_sample_temperature": [P, P, P, P, c_int, c_int, P],
 }

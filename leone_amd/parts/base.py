@@ -96,7 +96,14 @@ BLOCKS = Registry("block")
 
 
 class Part:
-    """Common behaviour: a part states its tensors and later receives them."""
+    """Common behaviour: a part states its tensors and later receives them.
+
+    ``graph_safe`` says that the part's forward work depends on the step only through the
+    device arrays of the StepContext and cache views (never through host-side lists, sizes
+    of data or values read back), so that it can be recorded once and replayed.  A model is
+    replayed from a graph only if all its parts say so.
+    """
+    graph_safe = False
 
     def tensor_specs(self) -> List[TensorSpec]:
         return []

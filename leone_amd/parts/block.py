@@ -29,6 +29,10 @@ class PreNormBlock(Part):
     def parts(self):
         return (self.norm1, self.mixer, self.norm2, self.feed_forward)
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", False) for part in self.parts())
+
     def tensor_specs(self) -> List[TensorSpec]:
         return [s for part in self.parts() for s in part.tensor_specs()]
 

@@ -34,7 +34,7 @@ class StepContext:
     entry_slots: torch.Tensor          # int32 [entries]: state slot of each entry
     want_rows: Optional[torch.Tensor]  # int32 [wanted] rows whose logits are asked for
     block_tables: Dict[int, torch.Tensor] = field(default_factory=dict)  # group -> int32 [entries, max_blocks]
-    max_position: int = 0              # largest position in the step (host copy)
+    max_position: int = 0              # largest position in the step (an upper bound when the step is replayed)
     decode_only: bool = False          # every entry brings exactly one row
 
 

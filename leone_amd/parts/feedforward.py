@@ -19,6 +19,8 @@ class SwiGluMlp(Part):
     Parameters: ``hidden``, ``intermediate`` and tensor names ``gate``, ``up``, ``down``.
     """
 
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, **_):
         p = spec.params
         self.hidden = int(p["hidden"])

@@ -29,6 +29,8 @@ class GqaAttention(Part):
     position part) and tensor names ``q``, ``k``, ``v``, ``o``, ``q_norm``, ``k_norm``.
     """
 
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, positions: Optional[dict] = None, **_):
         p = spec.params
         self.hidden = int(p["hidden"])
@@ -82,7 +84,7 @@ class GqaAttention(Part):
                                    self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin,
                                    step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
                                    write_cache=cache.writes)
-        if ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens):
+        if ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens, self.q_heads // self.kv_heads):
             attended = ops.attention_decode(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
                                             cache.block_table, self.q_heads, self.scale, int(self.window or 0),
                                             max_context=step.max_position + 1)

@@ -63,6 +63,12 @@ class DecoderModel:
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a step of this model can be recorded once and replayed (see ``Part.graph_safe``)."""
+        return (all(getattr(layer, "graph_safe", False) for layer in self.layers)
+                and getattr(self.final_norm, "graph_safe", False))
+
     # ---- weights -------------------------------------------------------------
     def tensor_specs(self) -> List[TensorSpec]:
         specs = [TensorSpec(self.spec.embedding, (self.spec.vocab_size, self.spec.hidden_size), MATRIX)]

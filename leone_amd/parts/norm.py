@@ -17,6 +17,8 @@ class RmsNorm(Part):
     Reference: crates/leone/src/cpu.rs:1642-1663.  Parameters: ``size``, ``eps``, ``weight`` (tensor name).
     """
 
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, **_):
         self.size = int(spec["size"])
         self.eps = float(spec["eps"])

@@ -19,6 +19,8 @@ class RotaryHalfSplit(Part):
     evaluated in double on the device and kept as float.
     """
 
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, **_):
         self.rotary_dim = int(spec["rotary_dim"])
         self.theta = float(spec["theta"])
@@ -37,6 +39,8 @@ class RotaryHalfSplit(Part):
 @POSITIONS.register("none")
 class NoPosition(Part):
     """No position encoding: queries and keys are used as projected."""
+
+    graph_safe = True
 
     def __init__(self, spec: PartSpec, **_):
         pass

@@ -268,13 +268,13 @@ def test_argmax_rules():
 @pytest.mark.parametrize("splits", [1, 3, None])
 @pytest.mark.parametrize("window", [0, 5, 37])
 @pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 1, 32, 64), (5, 5, 48, 16), (32, 8, 128, 64), (40, 8, 128, 16),
-                                   (64, 2, 64, 32), (3, 3, 240, 16)])
+                                   (64, 2, 64, 32), (3, 3, 256, 16), (34, 2, 240, 16)])
 def test_attention_decode(shape, window, splits):
     """The matrix-core kernel on the same cases as the row kernel, whatever the number of splits."""
     from leone_amd import ops
     q_heads, kv_heads, head_dim, page_tokens = shape
     dtype = torch.bfloat16
-    assert ops.decode_attention_supported(dtype, head_dim, page_tokens)
+    assert ops.decode_attention_supported(dtype, head_dim, page_tokens, q_heads // kv_heads)
     lengths = [1, 17, 70, 130]
     table, k_pool, v_pool, keys, values = paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed=13)
     rows = [(0, 0)] + [(1, 16)] + [(2, p) for p in range(40, 70)] + [(3, p) for p in range(0, 130, 3)] + [(3, 129)]
@@ -323,3 +323,24 @@ def test_attention_finds_the_one_key_that_matters(kernel):
         exact = plain.attend_one(q[i].float(), keys[r][:p + 1], values[r][:p + 1])
         assert (out[i] - exact).abs().max() < 3e-2, (i, r, p, j)
         assert (out[i] - want).abs().max() < 0.25, (i, r, p, j)       # nearly all the weight is on key j
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mnk", [(1, 777, 80), (5, 64, 64), (8, 6144, 4096), (16, 1000, 96), (17, 130, 1032),
+                                 (33, 48, 176), (64, 4096, 12288), (1, 151936, 256), (3, 20, 8)])
+def test_gemm_skinny(mnk, out_dtype):
+    """Inputs rounded to bfloat16 as the kernel sees them, products summed in double
+    (the reference's way for its matrix-core product, crates/leone-cuda/tests/gpu.rs:287-386)."""
+    from leone_amd import ops
+    m, n, k = mnk
+    torch.manual_seed(8)
+    x, w = torch.randn(m, k, device=DEV).bfloat16(), (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    out = ops.gemm_skinny(x, w, out_dtype)
+    want = x.double() @ w.double().T
+    if out_dtype == torch.float32:
+        close(out, want, 2e-6 * k, 1e-5, "gemm_skinny")
+    else:
+        close(out, want, 2e-6 * k + 1e-3, 8e-3, "gemm_skinny bf16")
+    assert torch.equal(out, ops.gemm_skinny(x, w, out_dtype))
+    # a row alone gives the same bits as the row inside a batch (crates/leone-cuda/tests/gpu.rs:770)
+    assert torch.equal(ops.gemm_skinny(x[m - 1:m].contiguous(), w, out_dtype)[0], out[m - 1])
