@@ -248,21 +248,32 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     }
 }
 
-// Merges the splits of one (row, query head): out = sum_s acc_s e^(m_s - M) / sum_s l_s e^(m_s - M).
-__global__ void attention_reduce_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                                        bf16_t* __restrict__ out, int head_dim, int splits) {
+// Merges the splits of one (row, query head): out = sum_s acc_s e^(m_s - M) / sum_s l_s e^(m_s - M),
+// the sums taken in split order.  The weights e^(m_s - M) are computed once, one thread a split.
+constexpr int kReduceThreads = 128;
+constexpr int kMaxSplits = 256;
+
+__global__ void __launch_bounds__(kReduceThreads)
+attention_reduce_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                        bf16_t* __restrict__ out, int head_dim, int splits) {
+    __shared__ float weight[kMaxSplits];
+    __shared__ float wave_top[kReduceThreads / kWave];
     const long rh = blockIdx.x;                      // row * q_heads + head
     const float* ml = part_ml + rh * splits * 2;
     float top = -INFINITY;
-    for (int s = 0; s < splits; ++s) top = fmaxf(top, ml[2 * s]);
+    for (int s = threadIdx.x; s < splits; s += kReduceThreads) top = fmaxf(top, ml[2 * s]);
+    top = wave_max(top);
+    if (threadIdx.x % kWave == 0) wave_top[threadIdx.x / kWave] = top;
+    __syncthreads();
+    top = fmaxf(wave_top[0], wave_top[1]);
+    for (int s = threadIdx.x; s < splits; s += kReduceThreads)
+        weight[s] = ml[2 * s] == -INFINITY ? 0.f : __expf(ml[2 * s] - top);
+    __syncthreads();
     float den = 0.f;
-    for (int s = 0; s < splits; ++s) den += ml[2 * s] == -INFINITY ? 0.f : ml[2 * s + 1] * __expf(ml[2 * s] - top);
-    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    for (int s = 0; s < splits; ++s) den += ml[2 * s + 1] * weight[s];
+    for (int d = threadIdx.x; d < head_dim; d += kReduceThreads) {
         float num = 0.f;
-        for (int s = 0; s < splits; ++s) {
-            if (ml[2 * s] == -INFINITY) continue;
-            num += part_acc[(rh * splits + s) * head_dim + d] * __expf(ml[2 * s] - top);
-        }
+        for (int s = 0; s < splits; ++s) num += part_acc[(rh * splits + s) * head_dim + d] * weight[s];
         out[rh * head_dim + d] = from_float<bf16_t>(num / den);
     }
 }
@@ -306,7 +317,7 @@ extern "C" int leone_attention_decode(const void* q, void* out, const void* k_po
                   "attention_decode: page_tokens %d must be a power of two, at least 16", page_tokens);
     LEONE_REQUIRE(decode_smem_bytes(head_dim, q_heads / kv_heads) <= 64 * 1024,
                   "attention_decode: head_dim %d needs more shared memory than a workgroup may have", head_dim);
-    LEONE_REQUIRE(splits >= 1 && splits <= 65535, "attention_decode: splits %d out of range", splits);
+    LEONE_REQUIRE(splits >= 1 && splits <= kMaxSplits, "attention_decode: splits %d must be in 1..%d", splits, kMaxSplits);
     LEONE_REQUIRE(window >= 0 && max_blocks > 0, "attention_decode: bad window or block table");
     const long grid_y = static_cast<long>(kv_heads) * ((q_heads / kv_heads + 15) / 16);
     LEONE_REQUIRE(grid_y <= 65535, "attention_decode: too many heads for one launch");
@@ -328,7 +339,7 @@ extern "C" int leone_attention_decode(const void* q, void* out, const void* k_po
     }
 #undef LEONE_DECODE_CASE
     LEONE_LAUNCH_CHECK("attention_decode");
-    attention_reduce_kernel<<<rows * q_heads, head_dim <= 64 ? 64 : 128, 0, stream>>>(
+    attention_reduce_kernel<<<rows * q_heads, kReduceThreads, 0, stream>>>(
         part_acc, part_ml, static_cast<bf16_t*>(out), head_dim, splits);
     LEONE_LAUNCH_CHECK("attention_reduce");
     return 0;

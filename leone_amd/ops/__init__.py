@@ -187,7 +187,7 @@ def choose_splits(rows: int, kv_heads: int, group: int, max_context: int) -> int
     at least four 32-key tiles a part so that each of a workgroup's four waves has one."""
     blocks = rows * kv_heads * ((group + 15) // 16)
     tiles = (max_context + 31) // 32
-    return max(1, min(512 // max(1, blocks), (tiles + 3) // 4, 256))
+    return max(1, min(512 // max(1, blocks), (tiles + 3) // 4, 32))
 
 
 def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
