@@ -50,6 +50,14 @@ int leone_attention_decode(const void* q, void* out, const void* k_pool, const v
                            float* part_ml, int rows, int q_heads, int kv_heads, int head_dim, int page_tokens,
                            float scale, int window, int splits, hipStream_t stream);
 
+// Causal attention of prompt portions on the matrix cores for bfloat16.  `tiles` lists (entry, first
+// row, rows) for runs of at most leone_attention_prefill_tile_rows() consecutive rows of one request;
+// the rows of a tile sit at consecutive positions.  head_dim a multiple of 16 up to 128.
+int leone_attention_prefill_tile_rows();
+int leone_attention_prefill(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
+                            const int* tiles, int n_tiles, const int* block_table, int max_blocks, int q_heads,
+                            int kv_heads, int head_dim, int page_tokens, float scale, int window, hipStream_t stream);
+
 // C[M,N] = A[M,K] . B[N,K]^T in float.
 int leone_gemm_f32(const float* a, const float* b, float* c, int m, int n, int k, hipStream_t stream);
 

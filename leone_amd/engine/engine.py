@@ -232,6 +232,7 @@ class Engine:
         return logits.index_select(0, index), rows_map
 
     def _build_context(self, entries: Sequence[StepEntry]):
+        from ..ops import PREFILL_MIN_ROWS, PREFILL_TILE_ROWS
         n_rows = sum(len(e.tokens) for e in entries)
         n_groups = len(self.cache.groups)
         tokens = np.empty(n_rows, dtype=np.int32)
@@ -239,13 +240,19 @@ class Engine:
         row_entry = np.empty(n_rows, dtype=np.int32)
         slots = np.empty(len(entries), dtype=np.int32)
         tables = [np.full((len(entries), self.cache.max_blocks(g)), -1, dtype=np.int32) for g in range(n_groups)]
-        want_rows: List[int] = []
-        rows_map: List[tuple] = []
+        # Inside the step long prompt portions come first (the prompt attention kernel takes them tile by
+        # tile), short portions and decoded tokens after; logits keep the caller's order of entries.
+        order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) < PREFILL_MIN_ROWS)
+        first_row = [0] * len(entries)
         infos: List[EntryInfo] = []
+        tiles: List[tuple] = []
+        prefill_rows = 0
         row = 0
-        for ei, e in enumerate(entries):
+        for ei, i in enumerate(order):
+            e = entries[i]
             start = self.cache.length(e.request)
             n = len(e.tokens)
+            first_row[i] = row
             tokens[row:row + n] = np.asarray(e.tokens, dtype=np.int64)
             positions[row:row + n] = np.arange(start, start + n)
             row_entry[row:row + n] = ei
@@ -253,21 +260,29 @@ class Engine:
             for g in range(n_groups):
                 table = self.cache.table(e.request, g)
                 tables[g][ei, :len(table)] = table
-            for w in e.want:
-                want_rows.append(row + int(w))
-                rows_map.append((e.request, int(w)))
+            if n >= PREFILL_MIN_ROWS:
+                for at in range(0, n, PREFILL_TILE_ROWS):
+                    tiles.append((ei, row + at, min(PREFILL_TILE_ROWS, n - at)))
+                prefill_rows = row + n
             infos.append(EntryInfo(e.request, int(slots[ei]), row, n, start))
             row += n
+        want_rows: List[int] = []
+        rows_map: List[tuple] = []
+        for i, e in enumerate(entries):
+            for w in e.want:
+                want_rows.append(first_row[i] + int(w))
+                rows_map.append((e.request, int(w)))
         # One upload for all step metadata.
-        parts = [tokens, positions, row_entry, slots, np.asarray(want_rows, dtype=np.int32)] + \
-                [t.reshape(-1) for t in tables]
+        parts = [tokens, positions, row_entry, slots, np.asarray(want_rows, dtype=np.int32),
+                 np.asarray(tiles, dtype=np.int32).reshape(-1)] + [t.reshape(-1) for t in tables]
         packed = torch.from_numpy(np.concatenate(parts)).to(self.device)
         offsets = np.cumsum([0] + [p.size for p in parts])
         pieces = [packed[offsets[i]:offsets[i + 1]] for i in range(len(parts))]
-        block_tables = {g: pieces[5 + g].view(len(entries), -1) for g in range(n_groups)}
+        block_tables = {g: pieces[6 + g].view(len(entries), -1) for g in range(n_groups)}
         context = StepContext(
             rows=n_rows, dtype=self.dtype, device=self.device, positions=pieces[1], row_entry=pieces[2],
             entries=infos, entry_slots=pieces[3], want_rows=pieces[4] if want_rows else None,
             block_tables=block_tables, max_position=int(positions.max()),
-            decode_only=all(len(e.tokens) == 1 for e in entries))
+            decode_only=all(len(e.tokens) == 1 for e in entries),
+            prefill_rows=prefill_rows, q_tiles=pieces[5].view(-1, 3) if tiles else None)
         return pieces[0], context, rows_map

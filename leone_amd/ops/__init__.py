@@ -214,6 +214,35 @@ def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
     return out
 
 
+PREFILL_TILE_ROWS = 128      # rows of one request a workgroup of the prompt kernel takes (checked against the library)
+PREFILL_MIN_ROWS = 16        # shorter portions go through the split-KV kernel row by row
+
+
+def prefill_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int) -> bool:
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 128
+            and page_tokens >= 16 and page_tokens & (page_tokens - 1) == 0)
+
+
+def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                      positions: torch.Tensor, tiles: torch.Tensor, block_table: torch.Tensor, q_heads: int,
+                      scale: float, window: int = 0) -> torch.Tensor:
+    """Attention for the rows that ``tiles`` (int32 [n, 3]: entry, first row, rows) covers; writes into ``out``."""
+    if library().leone_attention_prefill_tile_rows() != PREFILL_TILE_ROWS:
+        raise KernelError("the kernel library was built for another prompt tile size")
+    rows = q.shape[0]
+    pages, kv_heads, page_tokens, head_dim = cache_dims(k_pool, v_pool)
+    if q.shape[1] != q_heads * head_dim:
+        raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
+    if tiles.dim() != 2 or tiles.shape[1] != 3:
+        raise KernelError("attention_prefill: tiles must be int32 [n, 3]")
+    call("leone_attention_prefill", _dev(q, "attention q", torch.bfloat16),
+         _dev(out, "attention out", torch.bfloat16, q.shape), _dev(k_pool, "k pool", torch.bfloat16),
+         _dev(v_pool, "v pool", torch.bfloat16), _dev(positions, "positions", torch.int32, (rows,)),
+         _dev(tiles, "tiles", torch.int32), tiles.shape[0], _dev(block_table, "block table", torch.int32),
+         block_table.shape[1], q_heads, kv_heads, head_dim, page_tokens, float(scale), int(window), _stream())
+    return out
+
+
 def gemm_f32(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a[M,K] . b[N,K]^T in true single precision."""
     m, k = a.shape

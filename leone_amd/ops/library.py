@@ -31,6 +31,7 @@ _PROTOTYPES = {
                              c_int, P],
     "leone_attention_decode": [P, P, P, P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                c_int, P],
+    "leone_attention_prefill": [P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "leone_gemm_f32": [P, P, P, c_int, c_int, c_int, P],
     "leone_gemm_skinny_bf16": [P, P, P, c_int, c_int, c_int, c_int, P],
     "leone_argmax": [P, P, c_int, c_int, P],
@@ -50,6 +51,8 @@ def library() -> ctypes.CDLL:
             lib = ctypes.CDLL(path)
             lib.leone_last_error.restype = c_char_p
             lib.leone_last_error.argtypes = []
+            lib.leone_attention_prefill_tile_rows.restype = c_int
+            lib.leone_attention_prefill_tile_rows.argtypes = []
             for name, argtypes in _PROTOTYPES.items():
                 fn = getattr(lib, name)
                 fn.argtypes = argtypes

@@ -84,11 +84,26 @@ class GqaAttention(Part):
                                    self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin,
                                    step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
                                    write_cache=cache.writes)
-        if ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens, self.q_heads // self.kv_heads):
-            attended = ops.attention_decode(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
-                                            cache.block_table, self.q_heads, self.scale, int(self.window or 0),
-                                            max_context=step.max_position + 1)
-        else:
-            attended = ops.attention_rows(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
-                                          cache.block_table, self.q_heads, self.scale, int(self.window or 0))
+        attended = self._attend(q, step, cache)
         return ops.linear(attended, self.w_o)
+
+    def _attend(self, q: torch.Tensor, step: StepContext, cache: KvCacheView) -> torch.Tensor:
+        """Long prompt portions through the prompt kernel, the other rows through the split-KV kernel; the
+        row kernel takes what the matrix-core kernels refuse (float32, odd sizes)."""
+        window = int(self.window or 0)
+        group = self.q_heads // self.kv_heads
+        if not ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens, group):
+            return ops.attention_rows(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
+                                      cache.block_table, self.q_heads, self.scale, window)
+        first = 0
+        out = torch.empty_like(q)
+        if (step.prefill_rows and step.q_tiles is not None
+                and ops.prefill_attention_supported(q.dtype, self.head_dim, cache.page_tokens)):
+            ops.attention_prefill(q, out, cache.k_pool, cache.v_pool, step.positions, step.q_tiles,
+                                  cache.block_table, self.q_heads, self.scale, window)
+            first = step.prefill_rows
+        if first < step.rows:
+            ops.attention_decode(q[first:], cache.k_pool, cache.v_pool, step.positions[first:],
+                                 step.row_entry[first:], cache.block_table, self.q_heads, self.scale, window,
+                                 max_context=step.max_position + 1, out=out[first:])
+        return out

@@ -344,3 +344,67 @@ def test_gemm_skinny(mnk, out_dtype):
     assert torch.equal(out, ops.gemm_skinny(x, w, out_dtype))
     # a row alone gives the same bits as the row inside a batch (crates/leone-cuda/tests/gpu.rs:770)
     assert torch.equal(ops.gemm_skinny(x[m - 1:m].contiguous(), w, out_dtype)[0], out[m - 1])
+
+
+@pytest.mark.parametrize("window", [0, 5, 37])
+@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 1, 32, 64), (5, 5, 48, 16), (32, 8, 128, 64), (3, 3, 112, 32)])
+def test_attention_prefill(shape, window):
+    """Portions that start at position 0 and in the middle of a request, longer and shorter than a
+    128-row tile, over scattered pages; rows of the step that belong to no tile stay untouched."""
+    from leone_amd import ops
+    q_heads, kv_heads, head_dim, page_tokens = shape
+    dtype = torch.bfloat16
+    assert ops.prefill_attention_supported(dtype, head_dim, page_tokens)
+    lengths = [300, 77, 200]
+    table, k_pool, v_pool, keys, values = paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed=31)
+    portions = [(0, 0, 300), (1, 60, 17), (2, 33, 130)]            # (request, first position, rows)
+    rows, tiles = [], []
+    for entry, (r, start, count) in enumerate(portions):
+        for at in range(0, count, ops.PREFILL_TILE_ROWS):
+            tiles.append((entry, len(rows) + at, min(ops.PREFILL_TILE_ROWS, count - at)))
+        rows += [(r, start + i) for i in range(count)]
+    rows += [(1, 76)]                                               # a row outside every tile
+    g = torch.Generator().manual_seed(32)
+    q = torch.randn(len(rows), q_heads, head_dim, generator=g).to(dtype)
+    positions = torch.tensor([p for _, p in rows], dtype=torch.int32)
+    scale = 1.0 / math.sqrt(head_dim)
+    out = torch.full((len(rows), q_heads * head_dim), 5.0, dtype=dtype, device=DEV)
+    ops.attention_prefill(q.reshape(len(rows), -1).to(DEV), out, k_pool.to(DEV), v_pool.to(DEV), positions.to(DEV),
+                          torch.tensor(tiles, dtype=torch.int32, device=DEV), table.to(DEV), q_heads, scale, window)
+    assert torch.isfinite(out.float()).all()
+    assert (out[-1] == 5.0).all()
+    want = torch.stack([plain.attend_one(q[i].float(), keys[r][:p + 1], values[r][:p + 1], window or None)
+                        for i, (r, p) in enumerate(rows[:-1])])
+    close(out[:-1].reshape(len(rows) - 1, q_heads, head_dim), want, 2e-2, 2e-2, "attention_prefill")
+
+
+def test_attention_prefill_finds_the_one_key_that_matters():
+    from leone_amd import ops
+    q_heads, kv_heads, head_dim, page_tokens = 4, 2, 64, 16
+    dtype = torch.bfloat16
+    lengths = [400]
+    table, k_pool, v_pool, keys, values = paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed=41)
+    start, count = 100, 300
+    rows = [(0, start + i) for i in range(count)]
+    g = torch.Generator().manual_seed(42)
+    targets = [int(torch.randint(0, p + 1, (1,), generator=g)) for _, p in rows]     # any key up to its own position
+    for i in (0, 31, 32, 127, 128, 299):                                              # tile edges look at themselves
+        targets[i] = rows[i][1]
+    for i in (5, 64, 200):                                                            # and at the very first key
+        targets[i] = 0
+    q = torch.zeros(count, q_heads, head_dim)
+    for i, j in enumerate(targets):
+        for h in range(q_heads):
+            k = keys[0][j, h // 2]
+            q[i, h] = k * (60.0 * math.sqrt(head_dim) / float(k @ k))
+    q = q.to(dtype)
+    tiles = [(0, at, min(128, count - at)) for at in range(0, count, 128)]
+    out = torch.zeros((count, q_heads * head_dim), dtype=dtype, device=DEV)
+    ops.attention_prefill(q.reshape(count, -1).to(DEV), out, k_pool.to(DEV), v_pool.to(DEV),
+                          torch.tensor([p for _, p in rows], dtype=torch.int32, device=DEV),
+                          torch.tensor(tiles, dtype=torch.int32, device=DEV), table.to(DEV), q_heads,
+                          1.0 / math.sqrt(head_dim))
+    out = out.float().cpu().view(count, q_heads, head_dim)
+    for i, j in enumerate(targets):
+        want = values[0][j].repeat_interleave(2, dim=0)
+        assert (out[i] - want).abs().max() < 0.25, (i, rows[i][1], j)
