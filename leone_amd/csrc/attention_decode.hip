@@ -77,6 +77,17 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     const int my_begin = t_begin + split * per_split;
     const int my_end = my_begin + per_split < t_end ? my_begin + per_split : t_end;
 
+    // The page ids of this split's keys go to shared memory first: no load of keys or values then
+    // waits on a read of the block table.
+    int* pages = reinterpret_cast<int*>(smem + kDecodeWaves * cols * (kD + 2));
+    const int first_page = (my_begin * kTileKeys) >> page_shift;
+    {
+        const int last_key = (my_end * kTileKeys < n ? my_end * kTileKeys : n) - 1;
+        const int n_pages = my_begin < my_end ? (last_key >> page_shift) - first_page + 1 : 0;
+        for (int i = threadIdx.x; i < n_pages; i += kDecodeThreads) pages[i] = table[first_page + i];
+    }
+    __syncthreads();
+
     // Q^T operand: column c is query head kvh*group + col0 + c.
     bf16x8 qreg[kSteps];
     {
@@ -115,7 +126,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         const bf16_t* pk = k_pool;
         const bf16_t* pv = v_pool;
         if (va || vb) {                                   // ka and kb share a page: pages hold multiples of 8 keys
-            const int page = table[ka >> page_shift];
+            const int page = pages[(ka >> page_shift) - first_page];
             if (page < 0) {
                 unmapped = true;                          // never read outside the pool; the result is poisoned below
                 va = vb = false;
@@ -123,7 +134,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
             pk = k_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (ka & page_mask) * 8;
         }
         if (any) {
-            const int page = table[run0 >> page_shift];
+            const int page = pages[(run0 >> page_shift) - first_page];
             if (page < 0) {
                 unmapped = true;
                 any = false;
@@ -278,9 +289,11 @@ attention_reduce_kernel(const float* __restrict__ part_acc, const float* __restr
     }
 }
 
-static size_t decode_smem_bytes(int head_dim, int group) {
+// The four waves' partial results, and the page ids of a split (at most the whole block table).
+static size_t decode_smem_bytes(int head_dim, int group, int max_blocks) {
     const int cols = group < 16 ? group : 16;
-    return (static_cast<size_t>(kDecodeWaves) * cols * head_dim + 2 * kDecodeWaves * cols) * sizeof(float);
+    return (static_cast<size_t>(kDecodeWaves) * cols * head_dim + 2 * kDecodeWaves * cols) * sizeof(float) +
+           static_cast<size_t>(max_blocks) * sizeof(int);
 }
 
 template <int kD16>
@@ -290,7 +303,7 @@ static void launch_decode(const void* q, const void* k_pool, const void* v_pool,
                           int window, int splits, hipStream_t stream) {
     const int group = q_heads / kv_heads;
     dim3 grid(rows, kv_heads * ((group + 15) / 16), splits);
-    const size_t smem = decode_smem_bytes(kD16 * 16, group);
+    const size_t smem = decode_smem_bytes(kD16 * 16, group, max_blocks);
     attention_decode_kernel<kD16><<<grid, kDecodeThreads, smem, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
         positions, row_entry, block_table, max_blocks, part_acc, part_ml, q_heads, kv_heads, page_shift, scale, window,
@@ -315,7 +328,7 @@ extern "C" int leone_attention_decode(const void* q, void* out, const void* k_po
                   "attention_decode: head_dim %d must be a multiple of 16 in 16..256", head_dim);
     LEONE_REQUIRE(page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0,
                   "attention_decode: page_tokens %d must be a power of two, at least 16", page_tokens);
-    LEONE_REQUIRE(decode_smem_bytes(head_dim, q_heads / kv_heads) <= 64 * 1024,
+    LEONE_REQUIRE(decode_smem_bytes(head_dim, q_heads / kv_heads, max_blocks) <= 64 * 1024,
                   "attention_decode: head_dim %d needs more shared memory than a workgroup may have", head_dim);
     LEONE_REQUIRE(splits >= 1 && splits <= kMaxSplits, "attention_decode: splits %d must be in 1..%d", splits, kMaxSplits);
     LEONE_REQUIRE(window >= 0 && max_blocks > 0, "attention_decode: bad window or block table");

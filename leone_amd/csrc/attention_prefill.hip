@@ -38,7 +38,7 @@ __device__ inline bf16x8 pf_zero8() {
 
 // tiles: [n_tiles][3] = (entry, first row of the tile in the step, rows in the tile).
 template <int kD16>
-__global__ void __launch_bounds__(kPrefillThreads)
+__global__ void __launch_bounds__(kPrefillThreads, 2)
 attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_pool,
                          const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
                          const int* __restrict__ tiles, const int* __restrict__ block_table, int max_blocks,
@@ -53,9 +53,23 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     const int c = lane & 15, g = lane >> 4;
     const int page_tokens = 1 << page_shift, page_mask = page_tokens - 1;
     const int wave_row0 = kRowsPerWave * wave;                 // first row of this wave inside the tile
-    if (wave_row0 >= tile_rows) return;
-    const int wave_rows = tile_rows - wave_row0 < kRowsPerWave ? tile_rows - wave_row0 : kRowsPerWave;
     const int* table = block_table + static_cast<long>(entry) * max_blocks;
+
+    // The page ids of the keys this workgroup reads go to shared memory first, so that no load of keys
+    // or values waits on a read of the block table.
+    extern __shared__ int pages[];
+    int first_page;
+    {
+        const int blk_p0 = positions[tile_row0];
+        const int blk_lo = (window > 0 && blk_p0 - window + 1 > 0) ? blk_p0 - window + 1 : 0;
+        first_page = blk_lo >> page_shift;
+        const int n_pages = ((blk_p0 + tile_rows - 1) >> page_shift) - first_page + 1;
+        for (int i = threadIdx.x; i < n_pages; i += kPrefillThreads) pages[i] = table[first_page + i];
+        __syncthreads();
+    }
+
+    if (wave_row0 >= tile_rows) return;                        // after the workgroup's only barrier
+    const int wave_rows = tile_rows - wave_row0 < kRowsPerWave ? tile_rows - wave_row0 : kRowsPerWave;
 
     // Rows of a portion are consecutive positions: row r of the wave sits at p0 + r.
     const int p0 = positions[tile_row0 + wave_row0];
@@ -109,7 +123,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         const bf16_t* pk = k_pool;
         const bf16_t* pv = v_pool;
         if (va || vb) {
-            const int page = table[ka >> page_shift];
+            const int page = pages[(ka >> page_shift) - first_page];
             if (page < 0) {
                 unmapped = true;
                 va = vb = false;
@@ -117,7 +131,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             pk = k_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (ka & page_mask) * 8;
         }
         if (any) {
-            const int page = table[run0 >> page_shift];
+            const int page = pages[(run0 >> page_shift) - first_page];
             if (page < 0) {
                 unmapped = true;
                 any = false;
@@ -189,12 +203,15 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             psum += __shfl_xor(psum, 32, kWave);
             l_run[j] = l_run[j] * alpha + psum;
             m_run[j] = m_new;
+            if (__any(alpha != 1.0f)) {       // after the first tiles the running maximum seldom moves
 #pragma unroll
-            for (int dt = 0; dt < kD16; ++dt) {
+                for (int dt = 0; dt < kD16; ++dt)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[j][dt][r] *= alpha;
-                acc[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[dt], pt, acc[j][dt], 0, 0, 0);
+                    for (int r = 0; r < 4; ++r) acc[j][dt][r] *= alpha;
             }
+#pragma unroll
+            for (int dt = 0; dt < kD16; ++dt)
+                acc[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[dt], pt, acc[j][dt], 0, 0, 0);
         }
     };
 
@@ -232,7 +249,7 @@ static void launch_prefill(const void* q, void* out, const void* k_pool, const v
                            const int* tiles, int n_tiles, const int* block_table, int max_blocks, int q_heads,
                            int kv_heads, int page_shift, float scale, int window, hipStream_t stream) {
     dim3 grid(n_tiles, q_heads);
-    attention_prefill_kernel<kD16><<<grid, kPrefillThreads, 0, stream>>>(
+    attention_prefill_kernel<kD16><<<grid, kPrefillThreads, static_cast<size_t>(max_blocks) * sizeof(int), stream>>>(
         static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), positions, tiles, block_table, max_blocks, q_heads, kv_heads, page_shift,
         scale, window);
@@ -257,6 +274,8 @@ extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_p
     LEONE_REQUIRE(page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0,
                   "attention_prefill: page_tokens %d must be a power of two, at least 16", page_tokens);
     LEONE_REQUIRE(window >= 0 && max_blocks > 0, "attention_prefill: bad window or block table");
+    LEONE_REQUIRE(static_cast<size_t>(max_blocks) * sizeof(int) <= 64 * 1024,
+                  "attention_prefill: a block table of %d entries does not fit shared memory", max_blocks);
     int page_shift = 0;
     while ((1 << page_shift) < page_tokens) ++page_shift;
 #define LEONE_PREFILL_CASE(N)                                                                                     \

@@ -174,10 +174,11 @@ def attention_rows(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, 
     return out
 
 
-def decode_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int, group: int = 1) -> bool:
+def decode_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int, group: int = 1,
+                               max_blocks: int = 0) -> bool:
     """Whether the matrix-core kernel takes this case; otherwise ``attention_rows`` does."""
     cols = min(group, 16)
-    shared = (4 * cols * head_dim + 8 * cols) * 4          # the four waves' partial results
+    shared = (4 * cols * head_dim + 8 * cols) * 4 + 4 * max_blocks   # the four waves' partial results, page ids
     return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 256 and shared <= 64 * 1024
             and page_tokens >= 16 and page_tokens & (page_tokens - 1) == 0)
 
@@ -218,8 +219,9 @@ PREFILL_TILE_ROWS = 128      # rows of one request a workgroup of the prompt ker
 PREFILL_MIN_ROWS = 16        # shorter portions go through the split-KV kernel row by row
 
 
-def prefill_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int) -> bool:
+def prefill_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int, max_blocks: int = 0) -> bool:
     return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 128
+            and 4 * max_blocks <= 64 * 1024                       # the page ids of a workgroup's keys
             and page_tokens >= 16 and page_tokens & (page_tokens - 1) == 0)
 
 

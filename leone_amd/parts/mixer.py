@@ -92,13 +92,14 @@ class GqaAttention(Part):
         row kernel takes what the matrix-core kernels refuse (float32, odd sizes)."""
         window = int(self.window or 0)
         group = self.q_heads // self.kv_heads
-        if not ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens, group):
+        max_blocks = cache.block_table.shape[1]
+        if not ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens, group, max_blocks):
             return ops.attention_rows(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
                                       cache.block_table, self.q_heads, self.scale, window)
         first = 0
         out = torch.empty_like(q)
         if (step.prefill_rows and step.q_tiles is not None
-                and ops.prefill_attention_supported(q.dtype, self.head_dim, cache.page_tokens)):
+                and ops.prefill_attention_supported(q.dtype, self.head_dim, cache.page_tokens, max_blocks)):
             ops.attention_prefill(q, out, cache.k_pool, cache.v_pool, step.positions, step.q_tiles,
                                   cache.block_table, self.q_heads, self.scale, window)
             first = step.prefill_rows

@@ -18,7 +18,11 @@ TINY_B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden
 TINY_C = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, hidden_size=80,
               num_attention_heads=5, num_key_value_heads=5, head_dim=48, intermediate_size=176, vocab_size=777,
               max_position_embeddings=384, rope_theta=50000.0, rms_norm_eps=3e-6, tie_word_embeddings=False)
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# The head shape of the large models (head_dim 128, four query heads a kv head) at a small width.
+TINY_M = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, hidden_size=512,
+              num_attention_heads=8, num_key_value_heads=2, head_dim=128, intermediate_size=1408, vocab_size=3001,
+              max_position_embeddings=1024, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False)
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "M": TINY_M}
 
 
 def make_model_dir(path: str, raw_config: dict, seed: int, dtype: torch.dtype, sharpen: float = 1.0) -> str:
