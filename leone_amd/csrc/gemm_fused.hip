@@ -1,0 +1,241 @@
+// The weight-streaming matrix product for at most 16 rows with the neighbouring row-wise work
+// folded in, so that a decode step needs one kernel where it had two or three:
+//
+//   input   plain : X is bfloat16 [M,K]
+//           norm  : X is the float32 residual stream; the operand is bf16(x * gain) and the result is
+//                   scaled by 1/sqrt(mean(x^2) + eps) per row afterwards, which is the same RMSNorm
+//                   (crates/leone/src/cpu.rs:1642-1663) because that factor is constant along a row
+//   output  store    : Y[M,N] in bfloat16 or float32
+//           residual : Y is the float32 stream, Y += product (the reference's fused
+//                      matrix-vector + residual, crates/leone/src/runtime.rs:9151-9157, 9311)
+//           gated    : W holds, in every block of 16 rows, 8 gate rows then the 8 up rows that belong to
+//                      them; Y[M,N/2] = silu(gate) * up (crates/leone/src/cpu.rs:892-907)
+//
+// Structure and operand layout are those of gemm_skinny.hip: a workgroup owns 16 rows of W, its waves
+// split K in steps of 64 elements, partial tiles are added in wave order in shared memory.
+#include "common.h"
+#include "leone_hip.h"
+
+#include <math.h>
+
+namespace leone {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+enum FusedIn : int { kInPlain = 0, kInNorm = 1 };
+enum FusedOut : int { kOutStore = 0, kOutResidual = 1, kOutGated = 2 };
+
+struct FusedArgs {
+    const void* x;       // plain: bfloat16 [M,K]; norm: float [*, K]
+    const int* rows;     // norm: row r of the product reads stream row rows[r] (nullptr: r)
+    const void* gain;    // norm: [K]
+    int gain_dtype;
+    float eps;
+    const bf16_t* w;     // [N,K]
+    void* y;
+    int m, n, k;
+};
+
+__device__ inline bf16x8 fz8() {
+    uint4 z = {0u, 0u, 0u, 0u};
+    return __builtin_bit_cast(bf16x8, z);
+}
+__device__ inline bf16x8 fld8(const bf16_t* p) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+__device__ inline void gain8(const void* gain, int dtype, int at, float out[8]) {
+    if (dtype == kF32) {
+        const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(gain) + at);
+        const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(gain) + at + 4);
+        out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+        out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+    } else {
+        const uint4 t = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(gain) + at);
+        const unsigned w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            out[2 * i] = __uint_as_float(w[i] << 16);
+            out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+}
+
+template <int kIn, int kOut, bool kTail, int kWaves, typename TOut>
+__global__ void __launch_bounds__(kWaves * kWave)
+gemm_fused_kernel(FusedArgs a) {
+    __shared__ float partial[kWaves][kWave][4];
+    __shared__ float squares[kWaves][16];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int lane = threadIdx.x % kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int m = a.m, n = a.n, k = a.k;
+    const long n0 = static_cast<long>(blockIdx.x) * 16;
+    // Rows past the end are clamped: they only feed output rows and columns that are never stored.
+    const long wr = n0 + c < n ? n0 + c : n - 1;
+    const bf16_t* wrow = a.w + wr * k + 16 * g;
+    const int xr = c < m ? c : m - 1;
+    const long xrow_index = (kIn == kInNorm && a.rows) ? a.rows[xr] : xr;
+    const bf16_t* xb = static_cast<const bf16_t*>(a.x) + xrow_index * k + 16 * g;   // plain
+    const float* xf = static_cast<const float*>(a.x) + xrow_index * k + 16 * g;     // norm
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    float ss = 0.f;
+
+    // One step: 64 elements of K; this lane's run is elements at + 16g .. + 15, `left` of which exist.
+    auto step = [&](int s, bf16x8 a0, bf16x8 a1, bool tail) {
+        const int at = 64 * s;
+        const int left = tail ? k - (at + 16 * g) : 16;
+        bf16x8 b[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if (left < 8 * (h + 1)) {
+                b[h] = fz8();
+            } else if (kIn == kInPlain) {
+                b[h] = fld8(xb + at + 8 * h);
+            } else {
+                const float4 lo = *reinterpret_cast<const float4*>(xf + at + 8 * h);
+                const float4 hi = *reinterpret_cast<const float4*>(xf + at + 8 * h + 4);
+                const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                float gv[8];
+                gain8(a.gain, a.gain_dtype, at + 16 * g + 8 * h, gv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    ss = fmaf(v[i], v[i], ss);
+                    b[h][i] = static_cast<__bf16>(v[i] * gv[i]);
+                }
+            }
+        }
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b[1], acc, 0, 0, 0);
+    };
+
+    // Each wave takes a contiguous share of K, so that it reads long runs of every weight row.
+    const int whole = k / 64;                        // steps of 64 elements without a tail
+    const int share = (whole + kWaves - 1) / kWaves;
+    const int s_end = (wave + 1) * share < whole ? (wave + 1) * share : whole;
+    constexpr int kUnroll = 4;                       // weight loads of four steps are in flight together
+    int s = wave * share;
+    for (; s + kUnroll <= s_end; s += kUnroll) {
+        bf16x8 wa[kUnroll][2];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            wa[u][0] = fld8(wrow + 64 * (s + u));
+            wa[u][1] = fld8(wrow + 64 * (s + u) + 8);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) step(s + u, wa[u][0], wa[u][1], false);
+    }
+    for (; s < s_end; ++s) step(s, fld8(wrow + 64 * s), fld8(wrow + 64 * s + 8), false);
+    if (kTail && wave == kWaves - 1) {                 // the last wave also takes the step that holds the end of K
+        const int left = k - (64 * whole + 16 * g);
+        step(whole, left >= 8 ? fld8(wrow + 64 * whole) : fz8(), left >= 16 ? fld8(wrow + 64 * whole + 8) : fz8(), true);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) partial[wave][lane][r] = acc[r];
+    if (kIn == kInNorm) {
+        ss += __shfl_xor(ss, 16, kWave);             // the four lanes that share X row c
+        ss += __shfl_xor(ss, 32, kWave);
+        if (g == 0) squares[wave][c] = ss;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    // Wave 0 adds the partial tiles in wave order.  Lane (c, g) holds the product of X row c with
+    // weight rows n0 + 4g .. 4g+3.
+    floatx4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int v = 0; v < kWaves; ++v)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sum[r] += partial[v][lane][r];
+    if (kIn == kInNorm) {
+        float total = 0.f;
+#pragma unroll
+        for (int v = 0; v < kWaves; ++v) total += squares[v][c];
+        const float inv = 1.0f / sqrtf(total / static_cast<float>(k) + a.eps);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) sum[r] *= inv;
+    }
+    const int row = c;
+    if (kOut == kOutGated) {
+        // local rows 0..7 are gate rows, 8..15 the up rows that belong to them: lanes g = 0, 1 hold
+        // gates, lanes g + 2 the matching ups
+        floatx4 up;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) up[r] = __shfl_xor(sum[r], 32, kWave);
+        if (g < 2 && row < m) {
+            bf16_t* out = static_cast<bf16_t*>(a.y) + static_cast<long>(row) * (n / 2) + n0 / 2 + 4 * g;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float gate = sum[r];
+                out[r] = from_float<bf16_t>((gate / (1.0f + expf(-gate))) * up[r]);
+            }
+        }
+        return;
+    }
+    if (row >= m) return;
+    const long col = n0 + 4 * g;
+    if (kOut == kOutResidual) {
+        float* out = static_cast<float*>(a.y) + static_cast<long>(row) * n + col;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (col + r < n) out[r] += sum[r];
+    } else {
+        TOut* out = static_cast<TOut*>(a.y) + static_cast<long>(row) * n + col;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (col + r < n) out[r] = from_float<TOut>(sum[r]);
+    }
+}
+
+template <int kIn, int kOut, typename TOut>
+static void launch_fused(const FusedArgs& a, hipStream_t stream) {
+    const int tiles = ceil_div(a.n, 16);
+    const int steps = ceil_div(a.k, 64);
+    const bool tail = a.k % 64 != 0;
+    const bool many = tiles * 4 >= 4096 || steps < 16;    // as in gemm_skinny: few rows of W split K further
+#define LEONE_FUSED(TAIL, WAVES) \
+    gemm_fused_kernel<kIn, kOut, TAIL, WAVES, TOut><<<tiles, WAVES * kWave, 0, stream>>>(a)
+    if (many) {
+        if (tail) LEONE_FUSED(true, 4); else LEONE_FUSED(false, 4);
+    } else {
+        if (tail) LEONE_FUSED(true, 8); else LEONE_FUSED(false, 8);
+    }
+#undef LEONE_FUSED
+}
+
+}  // namespace leone
+
+using namespace leone;
+
+// in_mode: 0 plain (x bfloat16 [m,k]), 1 norm (x float32 stream, optional rows, gain, eps).
+// out_mode: 0 store (y of out_dtype [m,n]), 1 residual (y float32 [m,n] += product), 2 gated (y bfloat16 [m,n/2]).
+extern "C" int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const void* gain, int gain_dtype,
+                                     float eps, const void* w, void* y, int out_mode, int out_dtype, int m, int n,
+                                     int k, hipStream_t stream) {
+    LEONE_REQUIRE(x && w && y, "gemm_fused: null pointer");
+    LEONE_REQUIRE(m > 0 && m <= 16, "gemm_fused: rows %d must be in 1..16", m);
+    LEONE_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_fused: sizes %d x %d: K must be a positive multiple of 8", n, k);
+    LEONE_REQUIRE(in_mode == kInPlain || in_mode == kInNorm, "gemm_fused: unknown input mode %d", in_mode);
+    LEONE_REQUIRE(in_mode == kInPlain || (gain && eps > 0.f && (gain_dtype == kF32 || gain_dtype == kBF16)),
+                  "gemm_fused: the norm input needs a gain and a positive eps");
+    LEONE_REQUIRE(out_mode >= kOutStore && out_mode <= kOutGated, "gemm_fused: unknown output mode %d", out_mode);
+    LEONE_REQUIRE(out_mode != kOutGated || n % 16 == 0, "gemm_fused: gated output needs N %d to be a multiple of 16", n);
+    LEONE_REQUIRE(out_mode != kOutStore || out_dtype == kF32 || out_dtype == kBF16, "gemm_fused: unknown output type");
+    FusedArgs a{x, rows, gain, gain_dtype, eps, static_cast<const bf16_t*>(w), y, m, n, k};
+#define LEONE_FUSED_OUT(IN)                                                                  \
+    switch (out_mode) {                                                                      \
+        case kOutStore:                                                                      \
+            if (out_dtype == kF32) launch_fused<IN, kOutStore, float>(a, stream);            \
+            else launch_fused<IN, kOutStore, bf16_t>(a, stream);                             \
+            break;                                                                           \
+        case kOutResidual: launch_fused<IN, kOutResidual, float>(a, stream); break;          \
+        default: launch_fused<IN, kOutGated, bf16_t>(a, stream); break;                      \
+    }
+    if (in_mode == kInPlain) {
+        LEONE_FUSED_OUT(kInPlain)
+    } else {
+        LEONE_FUSED_OUT(kInNorm)
+    }
+#undef LEONE_FUSED_OUT
+    LEONE_LAUNCH_CHECK("gemm_fused");
+    return 0;
+}

@@ -20,8 +20,6 @@ namespace leone {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
-constexpr int kSkinnyWaves = 4;
-constexpr int kSkinnyThreads = kSkinnyWaves * kWave;
 
 __device__ inline bf16x8 ld8(const bf16_t* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
@@ -43,9 +41,10 @@ __device__ inline void store4<bf16_t>(bf16_t* p, floatx4 v) {
     for (int r = 0; r < 4; ++r) p[r] = from_float<bf16_t>(v[r]);
 }
 
-// kMT: 16-row tiles of X (M <= 16 * kMT).  kTail: K is not a multiple of 64.
-template <int kMT, bool kTail, typename TOut>
-__global__ void __launch_bounds__(kSkinnyThreads)
+// kMT: 16-row tiles of X (M <= 16 * kMT).  kTail: K is not a multiple of 64.  kSkinnyWaves: waves of a
+// workgroup, which split K between them (more for matrices with few rows, so that the chip is filled).
+template <int kMT, bool kTail, int kSkinnyWaves, typename TOut>
+__global__ void __launch_bounds__(kSkinnyWaves * kWave)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, TOut* __restrict__ y, int m, int n,
                    int k) {
     __shared__ float partial[kSkinnyWaves][kMT][kWave][4];
@@ -79,24 +78,26 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
         }
     };
 
-    const int steps = (k + 63) / 64;
-    const int whole = k / 64;                        // steps without a tail
+    // Each wave takes a contiguous share of K, so that it reads long runs of every weight row.
+    const int whole = k / 64;                        // steps of 64 elements without a tail
+    const int share = (whole + kSkinnyWaves - 1) / kSkinnyWaves;
+    const int s_end = (wave + 1) * share < whole ? (wave + 1) * share : whole;
     constexpr int kUnroll = 4;                       // weight loads of four steps are in flight together
-    int s = wave;
-    for (; s + (kUnroll - 1) * kSkinnyWaves < whole; s += kUnroll * kSkinnyWaves) {
+    int s = wave * share;
+    for (; s + kUnroll <= s_end; s += kUnroll) {
         bf16x8 a[kUnroll][2];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            a[u][0] = ld8(wrow + 64 * (s + u * kSkinnyWaves));
-            a[u][1] = ld8(wrow + 64 * (s + u * kSkinnyWaves) + 8);
+            a[u][0] = ld8(wrow + 64 * (s + u));
+            a[u][1] = ld8(wrow + 64 * (s + u) + 8);
         }
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) step(s + u * kSkinnyWaves, a[u][0], a[u][1], false);
+        for (int u = 0; u < kUnroll; ++u) step(s + u, a[u][0], a[u][1], false);
     }
-    for (; s < whole; s += kSkinnyWaves) step(s, ld8(wrow + 64 * s), ld8(wrow + 64 * s + 8), false);
-    if (kTail && s < steps) {                        // the one step that holds the end of K
-        const int left = k - (64 * s + 16 * g);
-        step(s, left >= 8 ? ld8(wrow + 64 * s) : z8(), left >= 16 ? ld8(wrow + 64 * s + 8) : z8(), true);
+    for (; s < s_end; ++s) step(s, ld8(wrow + 64 * s), ld8(wrow + 64 * s + 8), false);
+    if (kTail && wave == kSkinnyWaves - 1) {                 // the last wave also takes the step that holds the end of K
+        const int left = k - (64 * whole + 16 * g);
+        step(whole, left >= 8 ? ld8(wrow + 64 * whole) : z8(), left >= 16 ? ld8(wrow + 64 * whole + 8) : z8(), true);
     }
 #pragma unroll
     for (int t = 0; t < kMT; ++t)
@@ -126,15 +127,28 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, T
     }
 }
 
-template <int kMT, typename TOut>
-static void launch_skinny(const void* x, const void* w, void* y, int m, int n, int k, hipStream_t stream) {
+template <int kMT, int kWaves, typename TOut>
+static void launch_skinny_waves(const void* x, const void* w, void* y, int m, int n, int k, hipStream_t stream) {
     const int blocks = ceil_div(n, 16);
     if (k % 64 == 0)
-        gemm_skinny_kernel<kMT, false, TOut><<<blocks, kSkinnyThreads, 0, stream>>>(
+        gemm_skinny_kernel<kMT, false, kWaves, TOut><<<blocks, kWaves * kWave, 0, stream>>>(
             static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TOut*>(y), m, n, k);
     else
-        gemm_skinny_kernel<kMT, true, TOut><<<blocks, kSkinnyThreads, 0, stream>>>(
+        gemm_skinny_kernel<kMT, true, kWaves, TOut><<<blocks, kWaves * kWave, 0, stream>>>(
             static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<TOut*>(y), m, n, k);
+}
+
+// Enough waves to fill 256 CUs with several waves a SIMD: matrices with few rows split K further.
+// The choice does not depend on the number of rows of X, so a row's result has the same bits
+// whatever batch it is part of.
+template <int kMT, typename TOut>
+static void launch_skinny(const void* x, const void* w, void* y, int m, int n, int k, hipStream_t stream) {
+    const int tiles = ceil_div(n, 16);
+    const int steps = ceil_div(k, 64);
+    if (tiles * 4 >= 4096 || steps < 16)
+        launch_skinny_waves<kMT, 4, TOut>(x, w, y, m, n, k, stream);
+    else
+        launch_skinny_waves<kMT, 8, TOut>(x, w, y, m, n, k, stream);
 }
 
 template <typename TOut>

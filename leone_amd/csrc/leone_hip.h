@@ -20,7 +20,8 @@ int leone_embed(const void* table, int dtype, const int* tokens, float* out, int
 int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, const void* gain, int gain_dtype, float eps,
                       void* y, int y_dtype, const int* rows, int n_rows, int hidden, hipStream_t stream);
 
-// out[r, c] = silu(gate_up[r, c]) * gate_up[r, ffn + c].
+// out[r, c] = silu(gate) * up, where gate_up[r] holds, in every block of 16 columns, 8 gate values
+// and then the 8 up values that belong to them; ffn is a multiple of 8.
 int leone_swiglu(const void* gate_up, void* out, int dtype, int rows, int ffn, hipStream_t stream);
 
 // cos/sin[pos, i] of pos * theta^(-2i/rotary_dim), for pos < positions.
@@ -64,6 +65,14 @@ int leone_gemm_f32(const float* a, const float* b, float* c, int m, int n, int k
 // Y[M,N] = X[M,K] . W[N,K]^T for bfloat16 X and W, M <= 64, K a multiple of 8; Y float or bfloat16.
 int leone_gemm_skinny_bf16(const void* x, const void* w, void* y, int out_dtype, int m, int n, int k,
                            hipStream_t stream);
+
+// The same product for M <= 16 with row-wise neighbours folded in.  in_mode 0: x is bfloat16 [M,K];
+// 1: x is the float32 stream (row r reads rows[r] if rows is given), the operand is x * gain and the
+// result is scaled by 1/sqrt(mean(x^2) + eps).  out_mode 0: y[M,N] of out_dtype; 1: y float32 [M,N] +=
+// product; 2: W interleaves 8 gate rows with their 8 up rows, y bfloat16 [M,N/2] = silu(gate) * up.
+int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const void* gain, int gain_dtype, float eps,
+                          const void* w, void* y, int out_mode, int out_dtype, int m, int n, int k,
+                          hipStream_t stream);
 
 int leone_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream);
 int leone_sample_temperature(const float* logits, const double* temperature, const double* uniform, int* out,

@@ -126,7 +126,8 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, cons
 }
 
 // ---- SwiGLU -------------------------------------------------------------------
-// in: [rows, 2F] with the gate in the first F columns, up in the last F.
+// in: [rows, 2F]; every block of 16 columns holds 8 gate values, then the 8 up values that belong to
+// them (the order in which the fused gate/up weight keeps its rows).
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long rows, int ffn) {
     const long total = rows * ffn;
@@ -134,8 +135,9 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
          i += static_cast<long>(gridDim.x) * blockDim.x) {
         const long r = i / ffn;
         const int c = static_cast<int>(i - r * ffn);
-        const float g = to_float(gate_up[r * 2 * ffn + c]);
-        const float u = to_float(gate_up[r * 2 * ffn + ffn + c]);
+        const long at = r * 2 * ffn + 16 * (c >> 3) + (c & 7);
+        const float g = to_float(gate_up[at]);
+        const float u = to_float(gate_up[at + 8]);
         out[i] = from_float<T>((g / (1.0f + expf(-g))) * u);
     }
 }
@@ -343,7 +345,7 @@ extern "C" int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, c
 extern "C" int leone_swiglu(const void* gate_up, void* out, int dtype, int rows, int ffn, hipStream_t stream) {
     if (check_dtype(dtype, "swiglu")) return 1;
     LEONE_REQUIRE(gate_up && out, "swiglu: null pointer");
-    LEONE_REQUIRE(rows > 0 && ffn > 0, "swiglu: rows %d width %d must be positive", rows, ffn);
+    LEONE_REQUIRE(rows > 0 && ffn > 0 && ffn % 8 == 0, "swiglu: rows %d, width %d: the width must be a positive multiple of 8", rows, ffn);
     const long total = static_cast<long>(rows) * ffn;
     long blocks = (total + 255) / 256;
     if (blocks > 16384) blocks = 16384;

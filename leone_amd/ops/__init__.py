@@ -260,6 +260,34 @@ def gemm_f32(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = Non
 
 SKINNY_ROWS = 64           # most rows one launch of the weight-streaming kernel takes
 SKINNY_LIBRARY_ROWS = 4    # from here on the library's matrix product is used for bfloat16 results
+FUSED_ROWS = 16            # up to here gate and residual are folded into the weight-streaming kernel
+FUSED_NORM_WEIGHT_ROWS = 1024   # a norm is folded into the product only for weights of at most this many rows
+
+
+class NormedRows:
+    """Rows of the float32 stream that are to be RMS-normalised: a norm not yet carried out, so that
+    the product that consumes it can fold it in.  ``rows`` (int32 indices) picks rows of ``x``."""
+
+    def __init__(self, x: torch.Tensor, gain: torch.Tensor, eps: float, dtype: torch.dtype,
+                 rows: Optional[torch.Tensor] = None):
+        self.x, self.gain, self.eps, self.dtype, self.rows = x, gain, float(eps), dtype, rows
+        self.shape = (x.shape[0] if rows is None else rows.numel(), x.shape[1])
+
+    def materialize(self) -> torch.Tensor:
+        return add_rmsnorm(self.x, None, self.gain, self.eps, self.dtype, self.rows)
+
+
+def materialize(x) -> torch.Tensor:
+    return x.materialize() if isinstance(x, NormedRows) else x
+
+
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """The fused gate/up weight: 8 gate rows, the 8 up rows that belong to them, and so on; the order in
+    which ``swiglu`` and the gated product expect the columns of the product."""
+    ffn, hidden = gate.shape
+    if ffn % 8 or up.shape != gate.shape:
+        raise KernelError(f"gate and up must both be [F, H] with F a multiple of 8, found {tuple(gate.shape)}")
+    return torch.stack([gate.view(ffn // 8, 8, hidden), up.view(ffn // 8, 8, hidden)], dim=1).reshape(2 * ffn, hidden)
 
 
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,
@@ -276,31 +304,75 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,
     return out
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """x[R,K] . weight[N,K]^T.  float32 runs the single-precision kernel.  bfloat16 accumulates in float:
-    up to 64 rows on the weight-streaming kernel, more rows through the library's matrix product."""
-    if x.dtype != weight.dtype:
-        raise KernelError(f"linear: activations are {x.dtype} but the weight is {weight.dtype}")
-    out_dtype = out_dtype or x.dtype
-    if x.dtype == torch.float32:
+def gemm_fused(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+               residual: Optional[torch.Tensor] = None, gated: bool = False) -> Optional[torch.Tensor]:
+    """The product for at most 16 rows with its neighbours folded in: ``x`` may be ``NormedRows``;
+    with ``residual`` the product is added into that float32 tensor and None is returned; with ``gated``
+    the weight is an interleaved gate/up weight and silu(gate) * up comes out."""
+    m, k = x.shape
+    n, k2 = weight.shape
+    if k != k2:
+        raise KernelError(f"gemm_fused: inner sizes {k} and {k2} differ")
+    normed = isinstance(x, NormedRows)
+    if residual is not None and gated:
+        raise KernelError("gemm_fused: a gated product cannot also be added into the stream")
+    if residual is not None:
+        out, mode, out_dtype = residual, 1, torch.float32
+    elif gated:
+        out, mode, out_dtype = torch.empty((m, n // 2), dtype=torch.bfloat16, device=weight.device), 2, torch.bfloat16
+    else:
+        out, mode = torch.empty((m, n), dtype=out_dtype, device=weight.device), 0
+    call("leone_gemm_fused_bf16",
+         _dev(x.x, "stream", torch.float32) if normed else _dev(x, "gemm x", torch.bfloat16, (m, k)),
+         1 if normed else 0, _dev(x.rows, "rows", torch.int32) if normed else 0,
+         _dev(x.gain, "gain", None, (k,)) if normed else 0, _code(x.gain, "gain") if normed else 0,
+         x.eps if normed else 0.0, _dev(weight, "gemm weight", torch.bfloat16),
+         _dev(out, "gemm out", out_dtype, (m, n // 2 if gated else n)), mode, _CODES[out_dtype], m, n, k, _stream())
+    return None if residual is not None else out
+
+
+def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           residual: Optional[torch.Tensor] = None, gated: bool = False) -> Optional[torch.Tensor]:
+    """x[R,K] . weight[N,K]^T, with optional neighbours.
+
+    ``x`` is a tensor or ``NormedRows`` (a norm still to be done).  ``gated``: the weight is an
+    interleaved gate/up weight and the result is silu(gate) * up, ``[R, N/2]``.  ``residual``: the caller
+    wants the product added into this float32 tensor; if the kernel in use can do that, it does and None
+    is returned, otherwise the product is returned for the caller to add later.
+
+    float32 runs the single-precision kernel.  bfloat16 accumulates in float: up to 16 rows on the
+    weight-streaming kernel with everything folded in, more rows through the library's matrix product;
+    float32 results (logits) always come from the weight-streaming kernel.
+    """
+    dtype = x.dtype if isinstance(x, NormedRows) else x.dtype
+    if dtype != weight.dtype:
+        raise KernelError(f"linear: activations are {dtype} but the weight is {weight.dtype}")
+    out_dtype = out_dtype or dtype
+    rows, k = x.shape
+    if dtype == torch.bfloat16 and weight.is_cuda and k % 8 == 0 and rows <= FUSED_ROWS \
+            and (not gated or weight.shape[0] % 16 == 0):
+        # Every workgroup (16 weight rows) would redo a folded norm for its own use: that pays only for
+        # matrices with few rows; for the others the norm kernel runs once and the product reads its result.
+        if isinstance(x, NormedRows) and weight.shape[0] > FUSED_NORM_WEIGHT_ROWS:
+            x = x.materialize()
+        return gemm_fused(x, weight, out_dtype, residual, gated)
+    x = materialize(x)
+    if dtype == torch.float32:
         if out_dtype != torch.float32:
             raise KernelError("linear: the float32 path produces float32")
-        return gemm_f32(x, weight)
-    if not x.is_cuda:
+        y = gemm_f32(x, weight)
+    elif not x.is_cuda:
         raise KernelError("linear: tensor is not on the GPU")
-    rows, k = x.shape
-    # The weight-streaming kernel re-reads the activations for every 16 weight rows, which costs more
-    # than the library's product beyond a few rows; float32 results (logits) always come from it.
-    if k % 8 == 0 and (rows <= SKINNY_LIBRARY_ROWS or out_dtype == torch.float32):
-        if rows <= SKINNY_ROWS:
-            return gemm_skinny(x, weight, out_dtype)
-        # float32 results (logits) for many rows: 64 rows at a time, each pass streaming the weight again
-        out = torch.empty((rows, weight.shape[0]), dtype=out_dtype, device=x.device)
+    elif k % 8 == 0 and out_dtype == torch.float32:
+        # float32 results for many rows: 64 rows at a time, each pass streaming the weight again
+        y = torch.empty((rows, weight.shape[0]), dtype=out_dtype, device=x.device)
         for at in range(0, rows, SKINNY_ROWS):
-            gemm_skinny(x[at:at + SKINNY_ROWS], weight, out_dtype, out=out[at:at + SKINNY_ROWS])
-        return out
-    y = torch.nn.functional.linear(x, weight)  # library matrix product, float accumulation
-    return y if out_dtype == y.dtype else y.to(out_dtype)
+            gemm_skinny(x[at:at + SKINNY_ROWS], weight, out_dtype, out=y[at:at + SKINNY_ROWS])
+    else:
+        y = torch.nn.functional.linear(x, weight)  # library matrix product, float accumulation
+        if out_dtype != y.dtype:
+            y = y.to(out_dtype)
+    return swiglu(y) if gated else y
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:

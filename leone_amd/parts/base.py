@@ -15,6 +15,10 @@ position      ``prepare(max_positions, device)``; what it exposes to a mixer is
 mixer         ``tensor_specs()``, ``bind(tensors)``, ``cache_need()`` -> ``KvNeed`` /
               ``StateNeed`` / ``None``, ``forward(y, step, cache)`` -> delta ``[rows, hidden]``.
 feed_forward  ``tensor_specs()``, ``bind(tensors)``, ``forward(y, step)`` -> delta.
+              A mixer or feed-forward that sets ``fused_io = True`` is instead called with
+              ``forward(y, step[, cache], residual=x)``: ``y`` may then be an ``ops.NormedRows`` (a norm
+              not yet carried out, which ``ops.linear`` folds into the product), and the part may add its
+              result into the float32 stream ``residual`` itself and return None.
 block         ``tensor_specs()``, ``bind(tensors)``, ``cache_need()``,
               ``forward(x, pending, step, cache)`` -> new pending delta.
 

@@ -44,8 +44,22 @@ class PreNormBlock(Part):
         return self.mixer.cache_need()
 
     def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], step: StepContext,
-                cache: Optional[CacheView]) -> torch.Tensor:
-        y = self.norm1.add_norm(x, pending, step.dtype)
-        delta = self.mixer.forward(y, step, cache)
-        y = self.norm2.add_norm(x, delta, step.dtype)
+                cache: Optional[CacheView]) -> Optional[torch.Tensor]:
+        """Returns the delta that is still to be added to ``x``, or None if everything has been added."""
+        y = self._normed(self.norm1, x, pending, step, self.mixer)
+        if getattr(self.mixer, "fused_io", False):
+            delta = self.mixer.forward(y, step, cache, residual=x)
+        else:
+            delta = self.mixer.forward(y, step, cache)
+        y = self._normed(self.norm2, x, delta, step, self.feed_forward)
+        if getattr(self.feed_forward, "fused_io", False):
+            return self.feed_forward.forward(y, step, residual=x)
         return self.feed_forward.forward(y, step)
+
+    @staticmethod
+    def _normed(norm, x, delta, step, consumer):
+        # A consumer with fused_io takes a norm that is only described and may fold it into its first
+        # product; any other gets the normalised rows.
+        if getattr(consumer, "fused_io", False) and hasattr(norm, "lazy"):
+            return norm.lazy(x, delta, step.dtype)
+        return norm.add_norm(x, delta, step.dtype)

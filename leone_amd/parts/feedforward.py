@@ -1,7 +1,7 @@
 """Feed-forward parts."""
 from __future__ import annotations
 
-from typing import Dict, List
+from typing import Dict, List, Optional
 
 import torch
 
@@ -33,12 +33,19 @@ class SwiGluMlp(Part):
                 TensorSpec(self.names["up"], (self.intermediate, self.hidden), MATRIX),
                 TensorSpec(self.names["down"], (self.hidden, self.intermediate), MATRIX)]
 
+    fused_io = True
+
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        # Gate rows first, then up rows: one product, then the activation splits the columns.
-        self.w_gate_up = torch.cat([tensors.pop(self.names["gate"]), tensors.pop(self.names["up"])],
-                                   dim=0).contiguous()
+        # One product for gate and up: 8 gate rows, their 8 up rows, and so on (a pure re-layout), which
+        # lets the activation be applied where the product is finished.
+        if self.intermediate % 8:
+            raise ValueError(f"the fused gate/up product needs an intermediate size that is a multiple of 8, "
+                             f"found {self.intermediate}")
+        self.w_gate_up = ops.interleave_gate_up(tensors.pop(self.names["gate"]),
+                                                tensors.pop(self.names["up"])).contiguous()
         self.w_down = tensors.pop(self.names["down"]).contiguous()
 
-    def forward(self, y: torch.Tensor, step: StepContext) -> torch.Tensor:
-        gate_up = ops.linear(y, self.w_gate_up)
-        return ops.linear(ops.swiglu(gate_up), self.w_down)
+    def forward(self, y, step: StepContext, residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned)."""
+        activated = ops.linear(y, self.w_gate_up, gated=True)
+        return ops.linear(activated, self.w_down, residual=residual)

@@ -75,7 +75,11 @@ class GqaAttention(Part):
             if self.q_gain.dtype != self.k_gain.dtype:
                 self.q_gain, self.k_gain = self.q_gain.float(), self.k_gain.float()
 
-    def forward(self, y: torch.Tensor, step: StepContext, cache: KvCacheView) -> torch.Tensor:
+    fused_io = True
+
+    def forward(self, y, step: StepContext, cache: KvCacheView,
+                residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned)."""
         qkv = ops.linear(y, self.w_qkv)
         cos, sin = self.position.tables() if self.position is not None else (None, None)
         if cos is not None and step.max_position >= cos.shape[0]:
@@ -85,7 +89,7 @@ class GqaAttention(Part):
                                    step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
                                    write_cache=cache.writes)
         attended = self._attend(q, step, cache)
-        return ops.linear(attended, self.w_o)
+        return ops.linear(attended, self.w_o, residual=residual)
 
     def _attend(self, q: torch.Tensor, step: StepContext, cache: KvCacheView) -> torch.Tensor:
         """Long prompt portions through the prompt kernel, the other rows through the split-KV kernel; the

@@ -125,5 +125,8 @@ class DecoderModel:
             if pending is not None:
                 pass  # nothing reads the last delta when no logits are wanted
             return None
-        y = self.final_norm.add_norm(x, pending, self.dtype, rows=step.want_rows)
+        if hasattr(self.final_norm, "lazy"):
+            y = self.final_norm.lazy(x, pending, self.dtype, rows=step.want_rows)
+        else:
+            y = self.final_norm.add_norm(x, pending, self.dtype, rows=step.want_rows)
         return ops.linear(y, self.head, out_dtype=torch.float32)

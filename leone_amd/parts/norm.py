@@ -34,3 +34,11 @@ class RmsNorm(Part):
     def add_norm(self, x: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype,
                  rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         return ops.add_rmsnorm(x, delta, self.gain, self.eps, out_dtype, rows)
+
+    def lazy(self, x: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype,
+             rows: Optional[torch.Tensor] = None):
+        """The same, but if there is nothing to add the norm is only described (``ops.NormedRows``), so
+        that the product that consumes it can carry it out itself."""
+        if delta is not None:
+            return self.add_norm(x, delta, out_dtype, rows)
+        return ops.NormedRows(x, self.gain, self.eps, out_dtype, rows)

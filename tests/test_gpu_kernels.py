@@ -74,17 +74,23 @@ def test_rmsnorm_reference_vector():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_swiglu(dtype):
-    """gate in [-8, 8], up in [-2, 2], 12,289 elements (crates/leone-cuda/tests/gpu.rs:1851-1867)."""
+    """gate in [-8, 8], up in [-2, 2], about 12,289 elements (crates/leone-cuda/tests/gpu.rs:1851-1867).  The input
+    holds 8 gate values, then their 8 up values, and so on, as the fused gate/up weight orders its rows."""
     from leone_amd import ops
     torch.manual_seed(2)
-    n = 12289
-    gate = (torch.rand(3, n, device=DEV) * 16 - 8)
-    up = (torch.rand(3, n, device=DEV) * 4 - 2)
-    gu = torch.cat([gate, up], dim=1).to(dtype)
+    n = 12296
+    gate = (torch.rand(3, n, device=DEV) * 16 - 8).to(dtype)
+    up = (torch.rand(3, n, device=DEV) * 4 - 2).to(dtype)
+    gu = torch.stack([gate.view(3, n // 8, 8), up.view(3, n // 8, 8)], dim=2).reshape(3, 2 * n).contiguous()
     out = ops.swiglu(gu)
-    want = plain.swiglu(gu[:, :n].cpu(), gu[:, n:].cpu())
+    want = plain.swiglu(gate.cpu(), up.cpu())
     atol, rtol = (2e-6, 3e-6) if dtype == torch.float32 else (1e-2, 1e-2)
     close(out, want, atol, rtol, "swiglu")
+    # the same order as rows of a weight: interleave_gate_up(Wg, Wu) @ x gives the layout above
+    wg, wu = torch.randn(16, 5), torch.randn(16, 5)
+    x = torch.randn(5)
+    fused = ops.interleave_gate_up(wg, wu) @ x
+    assert torch.equal(fused.view(2, 2, 8)[:, 0].reshape(-1), wg @ x) and torch.equal(fused.view(2, 2, 8)[:, 1].reshape(-1), wu @ x)
 
 
 def test_rope_table():
@@ -408,3 +414,71 @@ def test_attention_prefill_finds_the_one_key_that_matters():
     for i, j in enumerate(targets):
         want = values[0][j].repeat_interleave(2, dim=0)
         assert (out[i] - want).abs().max() < 0.25, (i, rows[i][1], j)
+
+
+@pytest.mark.parametrize("gain_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mnk", [(1, 6144, 4096), (5, 777, 80), (16, 1000, 176), (8, 96, 1032), (3, 4096, 12288)])
+def test_gemm_fused_norm_and_store(mnk, gain_dtype):
+    """The norm folded into the product equals norm, then product: the row factor 1/rms commutes with the sum."""
+    from leone_amd import ops
+    m, n, k = mnk
+    torch.manual_seed(9)
+    stream = torch.randn(m + 3, k, device=DEV) * 2
+    gain = (1 + 0.1 * torch.randn(k, device=DEV)).to(gain_dtype)
+    w = (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    eps = 1e-5
+    rows = torch.tensor([(3 * i + 1) % (m + 3) for i in range(m)], dtype=torch.int32, device=DEV)
+    for picked in (None, rows):
+        x = stream[:m] if picked is None else stream
+        lazy = ops.NormedRows(x.contiguous(), gain, eps, torch.bfloat16, picked)
+        out = ops.gemm_fused(lazy, w, torch.float32)
+        src = x[:m] if picked is None else x[picked.long()]
+        # the kernel's operand is bf16(x * gain); its rounding is the only difference from double
+        operand = (src * gain.float()).bfloat16().double()
+        inv = 1.0 / torch.sqrt((src.double() ** 2).mean(dim=1, keepdim=True) + eps)
+        want = (operand @ w.double().T) * inv
+        close(out, want, 2e-6 * k, 2e-5, "norm + product")
+        assert torch.equal(out, ops.gemm_fused(lazy, w, torch.float32))
+        # and it agrees with the unfused pair within bfloat16 rounding of the normalised rows
+        unfused = ops.gemm_skinny(lazy.materialize(), w, torch.float32)
+        close(out, unfused.double(), 2e-2 * math.sqrt(k) * 0.05 * 3, 2e-2, "fused against unfused")
+
+
+@pytest.mark.parametrize("mnk", [(1, 4096, 4096), (7, 80, 176), (16, 777, 64)])
+def test_gemm_fused_residual(mnk):
+    from leone_amd import ops
+    m, n, k = mnk
+    torch.manual_seed(10)
+    x = torch.randn(m, k, device=DEV).bfloat16()
+    w = (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    stream = torch.randn(m, n, device=DEV)
+    before = stream.clone()
+    assert ops.gemm_fused(x, w, residual=stream) is None
+    want = before.double() + x.double() @ w.double().T
+    close(stream, want, 2e-6 * k, 1e-5, "product added into the stream")
+    # the same bits as product, then one float addition (crates/leone-cuda/tests/gpu.rs:1921)
+    assert torch.equal(stream, before + ops.gemm_fused(x, w, torch.float32))
+
+
+@pytest.mark.parametrize("mfk", [(1, 12288, 4096), (6, 88, 80), (16, 256, 96)])
+def test_gemm_fused_gated(mfk):
+    from leone_amd import ops
+    m, f, k = mfk
+    torch.manual_seed(11)
+    stream = torch.randn(m, k, device=DEV)
+    gain = 1 + 0.1 * torch.randn(k, device=DEV)
+    wg, wu = (torch.randn(f, k, device=DEV) * 0.1).bfloat16(), (torch.randn(f, k, device=DEV) * 0.1).bfloat16()
+    w = ops.interleave_gate_up(wg, wu).contiguous()
+    lazy = ops.NormedRows(stream, gain, 1e-6, torch.bfloat16)
+    out = ops.gemm_fused(lazy, w, gated=True)
+    assert out.shape == (m, f) and out.dtype == torch.bfloat16
+    operand = (stream * gain).bfloat16().double()
+    inv = 1.0 / torch.sqrt((stream.double() ** 2).mean(dim=1, keepdim=True) + 1e-6)
+    want = plain.swiglu((operand @ wg.double().T) * inv, (operand @ wu.double().T) * inv)
+    close(out, want, 1e-2, 1e-2, "gated product")
+    # through linear(): the same call falls back to product + swiglu kernel beyond 16 rows
+    many = torch.randn(40, k, device=DEV)
+    lazy40 = ops.NormedRows(many, gain, 1e-6, torch.bfloat16)
+    got = ops.linear(lazy40, w, gated=True)
+    y = lazy40.materialize().double().cpu()
+    close(got, plain.swiglu(y @ wg.double().cpu().T, y @ wu.double().cpu().T), 3e-2, 3e-2, "unfused gated")
