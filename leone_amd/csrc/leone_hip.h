@@ -74,7 +74,11 @@ int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const voi
                           const void* w, void* y, int out_mode, int out_dtype, int m, int n, int k,
                           hipStream_t stream);
 
-int leone_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream);
+// Highest finite logit of each row, lowest index on ties, -1 if none.  Workspace: part_value and
+// part_index with rows * ceil(vocab / leone_argmax_chunk()) entries each.
+int leone_argmax_chunk();
+int leone_argmax(const float* logits, int* out, float* part_value, int* part_index, int rows, int vocab,
+                 hipStream_t stream);
 int leone_sample_temperature(const float* logits, const double* temperature, const double* uniform, int* out,
                              int rows, int vocab, hipStream_t stream);
 }

@@ -45,16 +45,38 @@ __device__ inline Best block_best(Best mine, Best* scratch) {
     return total;
 }
 
+// Two stages, as the reference's pair of kernels (crates/leone-cuda/cuda/ie_cuda.cu:4840, 4870): every
+// workgroup finds the best of one chunk of a row, then one workgroup a row picks among the chunks.
+// `better` prefers the lower index on equal values, so the result does not depend on the cut.
+constexpr int kArgmaxChunk = 4096;
+
 __global__ void __launch_bounds__(kSampleThreads)
-argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
+argmax_partial_kernel(const float* __restrict__ logits, float* __restrict__ part_value,
+                      int* __restrict__ part_index, int vocab, int chunks) {
     __shared__ Best scratch[kSampleThreads / kWave];
-    const float* row = logits + static_cast<long>(blockIdx.x) * vocab;
+    const int chunk = blockIdx.x;
+    const float* row = logits + static_cast<long>(blockIdx.y) * vocab;
+    const int end = (chunk + 1) * kArgmaxChunk < vocab ? (chunk + 1) * kArgmaxChunk : vocab;
     Best mine{0.f, -1};
-    for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
+    for (int i = chunk * kArgmaxChunk + threadIdx.x; i < end; i += kSampleThreads) {
         const float v = row[i];
         if (!isfinite(v)) continue;
         if (mine.index < 0 || v > mine.value) mine = Best{v, i};
     }
+    const Best total = block_best(mine, scratch);
+    if (threadIdx.x == 0) {
+        part_value[blockIdx.y * chunks + chunk] = total.value;
+        part_index[blockIdx.y * chunks + chunk] = total.index;
+    }
+}
+
+__global__ void __launch_bounds__(kSampleThreads)
+argmax_final_kernel(const float* __restrict__ part_value, const int* __restrict__ part_index,
+                    int* __restrict__ out, int chunks) {
+    __shared__ Best scratch[kSampleThreads / kWave];
+    Best mine{0.f, -1};
+    for (int i = threadIdx.x; i < chunks; i += kSampleThreads)
+        mine = better(mine, Best{part_value[blockIdx.x * chunks + i], part_index[blockIdx.x * chunks + i]});
     const Best total = block_best(mine, scratch);
     if (threadIdx.x == 0) out[blockIdx.x] = total.index;
 }
@@ -142,10 +164,17 @@ sample_temperature_kernel(const float* __restrict__ logits, const double* __rest
 
 using namespace leone;
 
-extern "C" int leone_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
-    LEONE_REQUIRE(logits && out, "argmax: null pointer");
-    LEONE_REQUIRE(rows > 0 && vocab > 0, "argmax: rows %d vocab %d must be positive", rows, vocab);
-    argmax_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, out, vocab);
+extern "C" int leone_argmax_chunk() { return kArgmaxChunk; }
+
+// part_value and part_index hold rows * ceil(vocab / leone_argmax_chunk()) entries each.
+extern "C" int leone_argmax(const float* logits, int* out, float* part_value, int* part_index, int rows, int vocab,
+                            hipStream_t stream) {
+    LEONE_REQUIRE(logits && out && part_value && part_index, "argmax: null pointer");
+    LEONE_REQUIRE(rows > 0 && rows <= 65535 && vocab > 0, "argmax: rows %d vocab %d out of range", rows, vocab);
+    const int chunks = ceil_div(vocab, kArgmaxChunk);
+    argmax_partial_kernel<<<dim3(chunks, rows), kSampleThreads, 0, stream>>>(logits, part_value, part_index, vocab, chunks);
+    LEONE_LAUNCH_CHECK("argmax");
+    argmax_final_kernel<<<rows, kSampleThreads, 0, stream>>>(part_value, part_index, out, chunks);
     LEONE_LAUNCH_CHECK("argmax");
     return 0;
 }

@@ -259,7 +259,6 @@ def gemm_f32(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = Non
 
 
 SKINNY_ROWS = 64           # most rows one launch of the weight-streaming kernel takes
-SKINNY_LIBRARY_ROWS = 4    # from here on the library's matrix product is used for bfloat16 results
 FUSED_ROWS = 16            # up to here gate and residual are folded into the weight-streaming kernel
 FUSED_NORM_WEIGHT_ROWS = 1024   # a norm is folded into the product only for weights of at most this many rows
 
@@ -363,11 +362,9 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         y = gemm_f32(x, weight)
     elif not x.is_cuda:
         raise KernelError("linear: tensor is not on the GPU")
-    elif k % 8 == 0 and out_dtype == torch.float32:
-        # float32 results for many rows: 64 rows at a time, each pass streaming the weight again
-        y = torch.empty((rows, weight.shape[0]), dtype=out_dtype, device=x.device)
-        for at in range(0, rows, SKINNY_ROWS):
-            gemm_skinny(x[at:at + SKINNY_ROWS], weight, out_dtype, out=y[at:at + SKINNY_ROWS])
+    elif out_dtype == torch.float32:
+        # float32 results (logits) for many rows: the library's product with float output
+        y = torch.mm(x, weight.t(), out_dtype=torch.float32)
     else:
         y = torch.nn.functional.linear(x, weight)  # library matrix product, float accumulation
         if out_dtype != y.dtype:
@@ -377,8 +374,12 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:
     rows, vocab = logits.shape
+    chunks = -(-vocab // library().leone_argmax_chunk())
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-    call("leone_argmax", _dev(logits, "argmax logits", torch.float32), _dev(out, "argmax out"), rows, vocab,
+    part_value = torch.empty((rows * chunks,), dtype=torch.float32, device=logits.device)
+    part_index = torch.empty((rows * chunks,), dtype=torch.int32, device=logits.device)
+    call("leone_argmax", _dev(logits, "argmax logits", torch.float32), _dev(out, "argmax out"),
+         _dev(part_value, "argmax partial values"), _dev(part_index, "argmax partial indices"), rows, vocab,
          _stream())
     return out
 

@@ -35,7 +35,7 @@ _PROTOTYPES = {
     "leone_gemm_f32": [P, P, P, c_int, c_int, c_int, P],
     "leone_gemm_skinny_bf16": [P, P, P, c_int, c_int, c_int, c_int, P],
     "leone_gemm_fused_bf16": [P, c_int, P, P, c_int, c_float, P, P, c_int, c_int, c_int, c_int, c_int, P],
-    "leone_argmax": [P, P, c_int, c_int, P],
+    "leone_argmax": [P, P, P, P, c_int, c_int, P],
     "leone_sample_temperature": [P, P, P, P, c_int, c_int, P],
 }
 
@@ -54,6 +54,8 @@ def library() -> ctypes.CDLL:
             lib.leone_last_error.argtypes = []
             lib.leone_attention_prefill_tile_rows.restype = c_int
             lib.leone_attention_prefill_tile_rows.argtypes = []
+            lib.leone_argmax_chunk.restype = c_int
+            lib.leone_argmax_chunk.argtypes = []
             for name, argtypes in _PROTOTYPES.items():
                 fn = getattr(lib, name)
                 fn.argtypes = argtypes

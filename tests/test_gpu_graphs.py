@@ -65,3 +65,29 @@ def test_a_part_that_is_not_graph_safe_keeps_the_model_eager(tmp_path):
         graph_safe = False
 
     assert not Part.graph_safe and GqaAttention.graph_safe and not HostDependent.graph_safe
+
+
+def test_replay_with_many_rows_uses_the_library_product_inside_the_graph(tmp_path):
+    """More than 16 decode rows take the library's matrix product; a recording that holds it is
+    replayed several times, with eager steps between, and every replay is compared with the eager engine."""
+    from leone_amd.engine.engine import Engine, StepEntry
+    from leone_amd.runtime import load_model
+
+    folder = make_model_dir(str(tmp_path / "m"), TINY["M"], 6, torch.bfloat16)
+    model = load_model(folder, "bfloat16")
+    engines = [Engine(model, num_pages=64, page_tokens=16, max_requests=24, graphs=flag) for flag in (True, False)]
+    vocab = TINY["M"]["vocab_size"]
+    n = 20
+    prompts = [random_tokens(700 + i, 3 + (i * 7) % 19, vocab) for i in range(n)]
+    for e in engines:
+        e.step([StepEntry(i, prompts[i], []) for i in range(n)])
+    for step in range(6):
+        tokens = random_tokens(800 + step, n, vocab)
+        outs = [e.step([StepEntry(i, [tokens[i]], [0]) for i in range(n)]).logits.cpu().numpy() for e in engines]
+        assert np.isfinite(outs[0]).all()
+        assert np.abs(outs[0] - outs[1]).max() < 3e-2, f"replay {step}"
+        if step % 2 == 0:                                      # eager work between the replays
+            for e in engines:
+                e.step([StepEntry("other", random_tokens(900 + step, 21, vocab), [20])])
+                e.release("other")
+    assert engines[0]._decode_graphs[n].graph is not None
