@@ -15,12 +15,25 @@ fixed-size pages:
   undoes an uncommitted reservation; ``release`` returns everything a request
   holds, pages and state slot, at once;
 * a *state slot* is an index into per-request storage of fixed size, handed out
-  on admission and returned on release.
+  on admission and returned on release;
+* ``fork`` lets a new request share the full pages of another request's prefix
+  (the reference's fork shares committed, immutable segments and gives the writer
+  a private tail, crates/leone/src/kv.rs:307-324, 676-691): pages carry reference
+  counts, a page goes back to the free list when its last holder lets go, and a
+  shared page is never written because sharing stops at a page boundary and all
+  appends go to pages of the request's own; ``truncate`` cuts a request back
+  (crates/leone/src/kv.rs:929-950).
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional
+
+
+def _gcd(a: int, b: int) -> int:
+    while b:
+        a, b = b, a % b
+    return a
 
 
 class OutOfPages(RuntimeError):
@@ -71,6 +84,7 @@ class CacheManager:
         # LIFO free lists: a page given back is the next one handed out.
         self._free: List[List[int]] = [list(range(g.num_pages - 1, -1, -1)) for g in self.groups]
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
+        self._refs: List[List[int]] = [[0] * g.num_pages for g in self.groups]   # holders of every page
         self._requests: Dict[Hashable, _Request] = {}
         self.pages_high_water = [0 for _ in self.groups]
 
@@ -122,6 +136,88 @@ class CacheManager:
         self._requests[request] = _Request(slot, len(self.groups))
         return slot
 
+    def _take(self, gi: int) -> int:
+        page = self._free[gi].pop()
+        self._refs[gi][page] = 1
+        return page
+
+    def _drop(self, gi: int, page: int) -> None:
+        """One holder lets go of a page; the last one puts it back on the free list."""
+        if self._refs[gi][page] <= 0:
+            raise CacheError(f"group {gi}: page {page} is given back more often than it was taken")
+        self._refs[gi][page] -= 1
+        if self._refs[gi][page] == 0:
+            self._free[gi].append(page)
+
+    def holders(self, group: int, page: int) -> int:
+        return self._refs[group][page]
+
+    def shared_pages(self, group: int) -> int:
+        return sum(1 for r in self._refs[group] if r > 1)
+
+    def fork(self, parent: Hashable, child: Hashable, tokens: Optional[int] = None) -> int:
+        """Admits ``child`` holding the full pages of the first ``tokens`` tokens of ``parent`` (all it has
+        committed if None).  Returns how many tokens the child holds: ``tokens`` rounded down to a page
+        boundary of every group; what lies beyond, the child computes for itself."""
+        source = self._get(parent)
+        if source.pending_tokens:
+            raise CacheError(f"request {parent!r} has an uncommitted reservation")
+        limit = source.length if tokens is None else min(int(tokens), source.length)
+        if limit < 0:
+            raise CacheError("a fork cannot share a negative number of tokens")
+        unit = 1
+        for g in self.groups:
+            unit = unit * g.page_tokens // _gcd(unit, g.page_tokens)
+        shared = limit // unit * unit
+        plans = []
+        for gi, g in enumerate(self.groups):
+            blocks = shared // g.page_tokens
+            first = 0 if g.window is None else max(0, shared - (g.window - 1)) // g.page_tokens
+            table = source.tables[gi]
+            for b in range(first, blocks):
+                if b >= len(table) or table[b] < 0:
+                    raise CacheError(f"group {gi}: the parent's window has passed block {b}; fork later tokens")
+            plans.append([table[b] if first <= b else -1 for b in range(blocks)])
+        self.admit(child)
+        state = self._requests[child]
+        for gi, pages in enumerate(plans):
+            state.tables[gi] = list(pages)
+            for page in pages:
+                if page >= 0:
+                    self._refs[gi][page] += 1
+        state.length = shared
+        return shared
+
+    def truncate(self, request: Hashable, position: int) -> None:
+        """Cuts a request back to ``position`` tokens.  Pages wholly beyond go back; the page that holds
+        ``position`` stays and must be the request's own unless ``position`` is a page boundary."""
+        state = self._get(request)
+        if state.pending_tokens:
+            raise CacheError(f"request {request!r} has an uncommitted reservation")
+        if not 0 <= position <= state.length:
+            raise CacheError(f"cannot truncate {request!r} of length {state.length} to {position}")
+        for gi, g in enumerate(self.groups):
+            table = state.tables[gi]
+            keep = (position + g.page_tokens - 1) // g.page_tokens
+            if position % g.page_tokens and keep <= len(table) and table[keep - 1] >= 0 \
+                    and self._refs[gi][table[keep - 1]] > 1:
+                raise CacheError(f"group {gi}: the page holding position {position} is shared; "
+                                 f"truncate to a multiple of {g.page_tokens}")
+        for gi, g in enumerate(self.groups):
+            table = state.tables[gi]
+            keep = (position + g.page_tokens - 1) // g.page_tokens
+            if g.window is not None:
+                reach = max(0, position - (g.window - 1)) // g.page_tokens
+                for b in range(reach, min(keep, len(table))):
+                    if table[b] < 0:
+                        raise CacheError(f"group {gi}: keys before position {position} have left the window; "
+                                         f"they cannot be brought back by truncation")
+            for b in range(keep, len(table)):
+                if table[b] >= 0:
+                    self._drop(gi, table[b])
+            del table[keep:]
+        state.length = position
+
     def _blocks_to_map(self, state: _Request, gi: int, start: int, tokens: int) -> List[int]:
         if tokens <= 0:
             return []
@@ -154,7 +250,7 @@ class CacheManager:
             for b in blocks:
                 while len(table) <= b:
                     table.append(-1)
-                table[b] = self._free[gi].pop()
+                table[b] = self._take(gi)
             state.pending_pages[gi] = blocks
             used = self.groups[gi].num_pages - len(self._free[gi])
             self.pages_high_water[gi] = max(self.pages_high_water[gi], used)
@@ -178,7 +274,7 @@ class CacheManager:
             table = state.tables[gi]
             for b in range(min(len(table), max(0, reach) // g.page_tokens)):
                 if table[b] >= 0:
-                    self._free[gi].append(table[b])
+                    self._drop(gi, table[b])
                     table[b] = -1
 
     def rollback(self, request: Hashable) -> None:
@@ -187,7 +283,7 @@ class CacheManager:
         for gi in range(len(self.groups)):
             table = state.tables[gi]
             for b in reversed(state.pending_pages[gi]):
-                self._free[gi].append(table[b])
+                self._drop(gi, table[b])
                 table[b] = -1
             while table and table[-1] < 0 and len(table) * self.groups[gi].page_tokens > self._covered(state, gi):
                 table.pop()
@@ -206,27 +302,38 @@ class CacheManager:
         for gi in range(len(self.groups)):
             for page in state.tables[gi]:
                 if page >= 0:
-                    self._free[gi].append(page)
+                    self._drop(gi, page)
         self._free_slots.append(state.slot)
 
     # ---- invariants ---------------------------------------------------------------
     def check(self) -> None:
         """No page lost, held twice or free twice; slots likewise.  Raises CacheError."""
         for gi, g in enumerate(self.groups):
-            seen: Dict[int, str] = {}
+            free = set()
             for page in self._free[gi]:
-                if page in seen:
+                if page in free:
                     raise CacheError(f"group {gi}: page {page} is on the free list twice")
-                seen[page] = "free"
+                free.add(page)
+            holders = [0] * g.num_pages
             for request, state in self._requests.items():
+                mine = set()
                 for page in state.tables[gi]:
                     if page < 0:
                         continue
-                    if page in seen:
-                        raise CacheError(f"group {gi}: page {page} held by {request!r} is also {seen[page]}")
-                    seen[page] = f"held by {request!r}"
-            if len(seen) != g.num_pages or any(not 0 <= p < g.num_pages for p in seen):
-                raise CacheError(f"group {gi}: {len(seen)} pages accounted for, {g.num_pages} exist")
+                    if not 0 <= page < g.num_pages:
+                        raise CacheError(f"group {gi}: {request!r} holds page {page}, which does not exist")
+                    if page in mine:
+                        raise CacheError(f"group {gi}: {request!r} holds page {page} twice")
+                    if page in free:
+                        raise CacheError(f"group {gi}: page {page} held by {request!r} is also free")
+                    mine.add(page)
+                    holders[page] += 1
+            for page in range(g.num_pages):
+                if holders[page] != self._refs[gi][page]:
+                    raise CacheError(f"group {gi}: page {page} has {holders[page]} holders but a count of "
+                                     f"{self._refs[gi][page]}")
+                if holders[page] == 0 and page not in free:
+                    raise CacheError(f"group {gi}: page {page} is lost (neither held nor free)")
             for request, state in self._requests.items():
                 total = state.length + state.pending_tokens
                 first = 0 if g.window is None else max(0, state.length - (g.window - 1)) // g.page_tokens

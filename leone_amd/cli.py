@@ -111,6 +111,7 @@ def cmd_generate(args) -> int:
     if (args.prompt is None) == (args.prompt_tokens is None):
         raise SystemExit("error: give exactly one of -p/--prompt and --prompt-tokens")
     runtime = Runtime.load(args.model, args.dtype, max_requests=1, max_context=args.max_context,
+                           graphs=not args.eager_decode,
                            policy=SchedulerPolicy(max_live_requests=1, prefill_chunk_tokens=args.prefill_chunk,
                                                   max_step_tokens=max(args.prefill_chunk, 1)))
     if args.prompt is not None:

@@ -127,10 +127,24 @@ class Engine:
         self.cache.release(request)
         if self.poison_freed:
             for g, table in enumerate(tables):
-                self.pools.poison_pages(g, [p for p in table if p >= 0])
+                self.pools.poison_pages(g, [p for p in table if p >= 0 and self.cache.holders(g, p) == 0])
 
     def length(self, request: Hashable) -> int:
         return self.cache.length(request)
+
+    def fork(self, parent: Hashable, child: Hashable, tokens: Optional[int] = None) -> int:
+        """A new request that shares the full cache pages of ``parent``'s first ``tokens`` tokens.  Returns the
+        number of tokens the child holds (a page boundary); the caller feeds it whatever comes after."""
+        if self.pools.state:
+            raise StepError("a model with per-request state cannot share a prefix: its state exists only "
+                            "for the parent's latest position")
+        return self.cache.fork(parent, child, tokens)
+
+    def truncate(self, request: Hashable, position: int) -> None:
+        """Cuts a request back to its first ``position`` tokens."""
+        if self.pools.state:
+            raise StepError("a model with per-request state cannot be cut back")
+        self.cache.truncate(request, position)
 
     # ---- the step --------------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]) -> None:
@@ -197,7 +211,8 @@ class Engine:
             for e, before in zip(entries, freed_before):
                 for g, old in enumerate(before):
                     new = self.cache.table(e.request, g)
-                    gone = [p for b, p in enumerate(old) if p >= 0 and (b >= len(new) or new[b] != p)]
+                    gone = [p for b, p in enumerate(old)
+                            if p >= 0 and (b >= len(new) or new[b] != p) and self.cache.holders(g, p) == 0]
                     self.pools.poison_pages(g, gone)
         return StepOutput(logits, rows)
 

@@ -140,3 +140,97 @@ def test_random_orders_keep_every_page_accounted_for(seed):
         m.release(rid)
     m.check()
     assert m.free_pages(0) == 24 and m.free_pages(1) == 12 and m.free_slots() == 4
+
+
+def test_fork_shares_full_pages_and_appends_go_to_private_ones():
+    # fork shares storage, appends go to a private tail (crates/leone/src/kv.rs:1238-1274)
+    m = CacheManager([GroupSpec(10, 4)], max_requests=3, max_context=64)
+    m.admit("a"); m.reserve("a", 10); m.commit("a")                 # pages for blocks 0, 1, 2 (the last half full)
+    shared = m.fork("a", "b")
+    assert shared == 8 and m.length("b") == 8                        # rounded down to a page boundary
+    assert m.table("b", 0) == m.table("a", 0)[:2] and m.shared_pages(0) == 2
+    assert m.free_pages(0) == 7                                      # sharing took no page
+    m.reserve("b", 3); m.commit("b")                                 # b's own tokens 8..10 go to a page of its own
+    assert m.table("b", 0)[2] != m.table("a", 0)[2] and m.free_pages(0) == 6
+    m.reserve("a", 5); m.commit("a")                                 # a goes on in its own tail
+    assert m.table("a", 0)[:2] == m.table("b", 0)[:2]
+    m.check()
+    m.release("a")                                                   # shared pages stay while b holds them
+    assert m.free_pages(0) == 10 - 3 and m.shared_pages(0) == 0
+    m.check()
+    m.release("b")
+    assert m.free_pages(0) == 10
+    m.check()
+    # a fork of fewer tokens, and a fork of a fork
+    m.admit("p"); m.reserve("p", 16); m.commit("p")
+    assert m.fork("p", "q", tokens=9) == 8 and m.fork("q", "r") == 8
+    assert m.holders(0, m.table("p", 0)[0]) == 3 and m.holders(0, m.table("p", 0)[2]) == 1
+    with pytest.raises(CacheError):
+        m.fork("p", "q")                                             # already admitted
+    with pytest.raises(OutOfSlots):
+        m.fork("p", "s")
+    m.check()
+
+
+def test_truncate_keeps_the_shared_prefix():
+    # crates/leone/src/kv.rs:1276
+    m = CacheManager([GroupSpec(10, 4)], 2, 64)
+    m.admit("a"); m.reserve("a", 14); m.commit("a")
+    m.fork("a", "b")                                                 # shares 12 tokens, 3 pages
+    m.truncate("a", 13)                                              # inside a's private page: fine
+    assert m.length("a") == 13 and len(m.table("a", 0)) == 4
+    with pytest.raises(CacheError):
+        m.truncate("a", 10)                                          # the page holding 10 is shared
+    m.truncate("a", 8)                                               # a page boundary: a lets go of block 2, b keeps it
+    assert m.table("a", 0) == m.table("b", 0)[:2] and m.holders(0, m.table("b", 0)[2]) == 1
+    m.reserve("a", 2); m.commit("a")                                 # and writes on in a fresh page
+    assert m.table("a", 0)[2] != m.table("b", 0)[2]
+    with pytest.raises(CacheError):
+        m.truncate("a", 11)
+    m.check()
+    m.release("a"); m.release("b"); m.check()
+    assert m.free_pages(0) == 10
+
+
+def test_fork_from_a_windowed_group_needs_the_pages_in_reach():
+    m = CacheManager([GroupSpec(20, 4), GroupSpec(6, 4, window=6)], 3, 128)
+    m.admit("a"); m.reserve("a", 20); m.commit("a")                  # window group has dropped blocks 0..2
+    assert m.fork("a", "b") == 20 and m.table("b", 1)[:3] == [-1, -1, -1] and m.table("b", 1)[3] >= 0
+    with pytest.raises(CacheError):
+        m.fork("a", "c", tokens=8)                                   # keys 3..7 have left a's window
+    m.check()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_orders_with_forks(seed):
+    rng = random.Random(50 + seed)
+    m = CacheManager([GroupSpec(30, 4)], max_requests=5, max_context=80)
+    live, names = {}, iter(range(10**6))
+    for _ in range(1200):
+        action = rng.random()
+        if action < 0.12 and len(live) < 5:
+            rid = next(names); m.admit(rid); live[rid] = 0
+        elif action < 0.22 and live and len(live) < 5:
+            parent = rng.choice(list(live)); rid = next(names)
+            live[rid] = m.fork(parent, rid, rng.choice([None, live[parent] // 2]))
+            assert live[rid] % 4 == 0 and live[rid] <= live[parent]
+        elif action < 0.75 and live:
+            rid = rng.choice(list(live)); n = rng.choice([1, 1, 2, 5, 9])
+            if live[rid] + n > 80:
+                continue
+            try:
+                m.reserve(rid, n)
+            except OutOfPages:
+                continue
+            m.commit(rid); live[rid] += n
+        elif action < 0.82 and live:
+            rid = rng.choice(list(live))
+            m.truncate(rid, live[rid] // 4 * 4 - (4 if live[rid] >= 4 and rng.random() < 0.5 else 0))
+            live[rid] = m.length(rid)
+        elif live:
+            rid = rng.choice(list(live)); m.release(rid); del live[rid]
+        m.check()
+    for rid in list(live):
+        m.release(rid)
+    m.check()
+    assert m.free_pages(0) == 30 and m.shared_pages(0) == 0

@@ -110,3 +110,43 @@ def test_rerun_is_bitwise_identical(cases, dtype_name):
         results.append(run_steps(engine, steps))
     for step in results[0]:
         assert np.array_equal(results[0][step], results[1][step]), f"step {step} differs between two runs"
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_forked_requests_share_prefix_pages_and_agree_with_plain(cases, dtype_name):
+    """A second request takes over the full pages of the first one's prefix, computes only what lies
+    beyond, and both go on independently; cutting a request back and feeding other tokens likewise."""
+    from leone_amd.engine.engine import Engine, StepEntry
+    from leone_amd.runtime import load_model
+
+    folder, _, _ = cases("B", dtype_name)
+    config, weights = read_config(folder), read_weights(folder)
+    vocab, tol = config["vocab_size"], tolerance(dtype_name)
+    model = load_model(folder, dtype_name)
+    engine = Engine(model, num_pages=16, page_tokens=16, max_requests=3, poison_freed=True)
+    a = random_tokens(1, 90, vocab)
+    b = a[:64] + random_tokens(2, 45, vocab)                    # the same first four pages, then its own way
+    want_a = qwen3_plain.forward(weights, config, a).numpy()
+    want_b = qwen3_plain.forward(weights, config, b).numpy()
+
+    def feed(rid, tokens, start, want):
+        out = engine.step([StepEntry(rid, tokens, list(range(len(tokens))))]).logits.cpu().numpy()
+        err = np.abs(out - want[start:start + len(tokens)]).max()
+        assert np.isfinite(out).all() and err <= tol, (rid, start, float(err))
+
+    feed("a", a[:70], 0, want_a)
+    free_before = engine.cache.free_pages(0)
+    assert engine.fork("a", "b") == 64 and engine.cache.free_pages(0) == free_before
+    assert engine.cache.shared_pages(0) == 4
+    feed("b", b[64:100], 64, want_b)                             # a portion right after the shared pages
+    feed("a", a[70:71], 70, want_a)                              # the parent decodes on in its own tail
+    feed("b", b[100:], 100, want_b)
+    engine.release("a")                                          # its private pages are poisoned, the shared ones live on
+    engine.cache.check()
+    c = b[:80] + random_tokens(3, 20, vocab)
+    want_c = qwen3_plain.forward(weights, config, c).numpy()
+    engine.truncate("b", 80)
+    feed("b", c[80:], 80, want_c)
+    engine.release("b")
+    engine.cache.check()
+    assert engine.cache.free_pages(0) == 16
