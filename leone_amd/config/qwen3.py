@@ -62,8 +62,20 @@ class Qwen3Config:
             head_dim = hidden // heads
         if head_dim % 2 != 0:
             raise ConfigError("head_dim", f"rotary pairs need an even head_dim, found {head_dim}")
-        if read.optional("rope_scaling") is not None:
+        scaling = read.optional("rope_scaling")
+        if scaling is not None and not (isinstance(scaling, dict) and
+                                        scaling.get("rope_type", scaling.get("type")) == "default"):
             raise ConfigError("rope_scaling", "rotary scaling is not supported")
+        # Newer checkpoints keep the rotary base in a rope_parameters object.
+        rope = read.optional("rope_parameters")
+        theta_from_rope = None
+        if rope is not None:
+            if not isinstance(rope, dict) or rope.get("rope_type", "default") != "default":
+                raise ConfigError("rope_parameters", "only the default rotary encoding is supported")
+            theta_from_rope = rope.get("rope_theta")
+        layer_types = read.optional("layer_types")
+        if layer_types is not None and any(kind != "full_attention" for kind in layer_types):
+            raise ConfigError("layer_types", "this architecture runs full attention in every layer")
         if read.optional("attention_bias") not in (None, False):
             raise ConfigError("attention_bias", "projection biases are not supported")
         if read.optional("use_sliding_window") not in (None, False):
@@ -89,7 +101,7 @@ class Qwen3Config:
             intermediate_size=read.positive_int("intermediate_size"),
             vocab_size=read.positive_int("vocab_size"),
             max_position_embeddings=read.positive_int("max_position_embeddings"),
-            rope_theta=read.positive_float("rope_theta", 10000.0),
+            rope_theta=read.positive_float("rope_theta", 10000.0 if theta_from_rope is None else theta_from_rope),
             rms_norm_eps=read.positive_float("rms_norm_eps", 1e-6),
             tie_word_embeddings=read.boolean("tie_word_embeddings", False),
             eos_token_id=eos,

@@ -49,6 +49,8 @@ def test_defaults_and_head_dim_not_tied_to_hidden():
     ({"hidden_act": "gelu"}, "hidden_act"),
     ({"tie_word_embeddings": "yes"}, "tie_word_embeddings"),
     ({"model_type": "llama"}, "model_type"),
+    ({"layer_types": ["full_attention", "sliding_attention"]}, "layer_types"),
+    ({"rope_parameters": {"rope_type": "yarn", "rope_theta": 1e6, "factor": 4.0}}, "rope_parameters"),
     ({"intermediate_size": None}, "intermediate_size"),
 ])
 def test_errors_name_the_field(change, field):
@@ -95,3 +97,10 @@ def test_model_spec_is_built_from_parts_layer_by_layer():
     assert spec.layers[2]["feed_forward"].kind == "swiglu" and spec.layers[2]["feed_forward"]["intermediate"] == 256
     assert spec.positions["rope"]["theta"] == 1e6 and spec.head == "lm_head.weight"
     assert model_spec_for(config_from_dict(TINY_A)).head is None
+
+
+def test_rotary_base_from_rope_parameters_and_harmless_extras():
+    raw = {k: v for k, v in TINY_A.items() if k != "rope_theta"}
+    raw.update(rope_parameters={"rope_type": "default", "rope_theta": 123456.0}, layer_types=["full_attention"] * 2,
+               rope_scaling={"rope_type": "default"}, sliding_window=4096, use_sliding_window=False)
+    assert config_from_dict(raw).rope_theta == 123456.0

@@ -143,3 +143,34 @@ def test_command_line_generate(folders, tmp_path):
     assert "decode:" in run.stderr and "prefill:" in run.stderr and "tokens emitted: 8" in run.stderr
     lines = open(logits_file).read().strip().splitlines()
     assert len(lines) == 8 and int(lines[0].split()[0].split(":")[0]) == expect[0]
+
+
+def test_command_line_eval_and_doctor(folders, tmp_path):
+    """`leone eval`: windows of W tokens with stride W-1, a fresh cache per window, the row after token i
+    scores token i+1 (crates/leone/src/runtime.rs:1673-1996); here against the plain logits of each window."""
+    folder = folders["B"]
+    weights, config = read_weights(folder), read_config(folder)
+    tokens = random_tokens(5, 70, config["vocab_size"])
+    tokens_file, logits_file, meta_file = tmp_path / "t.bin", tmp_path / "l.bin", tmp_path / "m.json"
+    np.asarray(tokens, dtype="<u4").tofile(tokens_file)
+    for chunk in (None, 7):
+        cmd = [sys.executable, os.path.join(ROOT, "bin", "leone"), "eval", "-m", folder, "--tokens", str(tokens_file),
+               "--logits", str(logits_file), "--window", "32", "--dtype", "float32", "--metadata", str(meta_file)]
+        if chunk:
+            cmd += ["--prefill-chunk", str(chunk)]
+        run = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+        assert run.returncode == 0, run.stderr
+        rows = np.fromfile(logits_file, dtype="<f4").reshape(-1, config["vocab_size"])
+        expect = []
+        start = 0
+        while start < len(tokens) - 1:
+            window = tokens[start:start + 32]
+            expect.append(qwen3_plain.forward(weights, config, window).numpy()[:len(window) - 1])
+            start += 31
+        expect = np.concatenate(expect)
+        assert rows.shape == expect.shape and np.abs(rows - expect).max() < 1e-4
+        assert json.load(open(meta_file))["rows"] == rows.shape[0]
+    doctor = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "leone"), "doctor", "-m", folder, "--probe"],
+                            capture_output=True, text=True, timeout=300)
+    assert doctor.returncode == 0, doctor.stdout + doctor.stderr
+    assert "Qwen3ForCausalLM" in doctor.stdout and "tensor names and shapes: ok" in doctor.stdout
