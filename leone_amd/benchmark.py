@@ -108,6 +108,71 @@ def time_prefill(engine, tokens: int, repeats: int = 3, seed: int = 2):
     return best
 
 
+QWEN3_14B = dict(QWEN3_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)
+QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
+
+# Serving scenarios beside the headline figure: continuous batching with chunked prefill, and page pressure.
+SCENARIOS = {
+    # 32 requests, prompts uniform in 128..4096, prompt portions of 512, 128 greedy tokens each
+    "mixed14b": dict(config=QWEN3_14B, requests=32, prompt=(128, 4096), new_tokens=128, chunk=512, temperature=None,
+                     live=32, pool_fraction=1.0),
+    # 16 requests of 4096 tokens, 256 tokens at temperature 0.7, the page pool at 60 % of what all would need
+    "pressure32b": dict(config=QWEN3_32B, requests=16, prompt=(4096, 4096), new_tokens=256, chunk=1024,
+                        temperature=0.7, live=16, pool_fraction=0.6),
+}
+
+
+def run_scenario(name: str, dtype: str = "bfloat16", layers: Optional[int] = None) -> dict:
+    import torch
+    from .architectures import config_from_dict
+    from .engine.engine import Engine
+    from .engine.generate import Generator
+    from .engine.scheduler import SchedulerPolicy
+    from .runtime import random_model
+    from .sampling.sampler import SamplingParams
+
+    sc = SCENARIOS[name]
+    raw = dict(sc["config"])
+    full_layers = raw["num_hidden_layers"]
+    if layers is not None:
+        raw["num_hidden_layers"] = layers
+    config = config_from_dict(raw)
+    model = random_model(config, seed=0, dtype=dtype)
+    gen = torch.Generator().manual_seed(7)
+    lo, hi = sc["prompt"]
+    lengths = [int(torch.randint(lo, hi + 1, (1,), generator=gen)) for _ in range(sc["requests"])]
+    prompts = [torch.randint(0, config.vocab_size, (n,), generator=gen).tolist() for n in lengths]
+    page_tokens = 64
+    needed = sum((n + sc["new_tokens"] + page_tokens - 1) // page_tokens for n in lengths)
+    pages = max(int(needed * sc["pool_fraction"]), (max(lengths) + sc["new_tokens"]) // page_tokens + 2)
+    engine = Engine(model, num_pages=pages, page_tokens=page_tokens, max_requests=sc["live"],
+                    max_context=max(lengths) + sc["new_tokens"] + 1)
+    policy = SchedulerPolicy(max_live_requests=sc["live"], prefill_chunk_tokens=sc["chunk"],
+                             max_step_tokens=sc["chunk"] + sc["live"])
+    generator = Generator(engine, policy)
+    sampling = SamplingParams(temperature=sc["temperature"], seed=11)
+    for i, prompt in enumerate(prompts):
+        generator.submit(i, prompt, sc["new_tokens"], sampling, None)
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    finished = generator.run()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    engine.cache.check()
+    assert len(finished) == sc["requests"] and all(len(f.tokens) == sc["new_tokens"] for f in finished)
+    assert not engine.cache.live_requests()
+    stats, sched = generator.stats, generator.scheduler.stats
+    return {"metric": f"generated tok/s, scenario {name}", "value": round(stats.emitted_tokens / elapsed, 2),
+            "unit": "tok/s", "n_gpus": 1, "seconds": round(elapsed, 3), "dtype": "bf16" if dtype == "bfloat16" else "fp32",
+            "data": "synthetic",
+            "config": {"model": name, "layers": config.num_hidden_layers, "layers_of_configuration": full_layers,
+                       "requests": sc["requests"], "prompt_tokens": sum(lengths), "new_tokens": sc["new_tokens"],
+                       "prefill_chunk": sc["chunk"], "pages": pages, "pages_needed_for_all": needed,
+                       "page_tokens": page_tokens},
+            "steps": stats.steps, "prefill_tok_s": round(stats.prefill_rate, 1), "decode_tok_s": round(stats.decode_rate, 1),
+            "preemptions": sched.preemptions, "max_step_rows": sched.max_step_rows, "max_live": sched.max_live}
+
+
 def main(argv: Optional[List[str]] = None) -> int:
     parser = argparse.ArgumentParser(prog="bench.py")
     parser.add_argument("--gpus", type=int, default=1)
@@ -119,10 +184,15 @@ def main(argv: Optional[List[str]] = None) -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--scenario", choices=sorted(SCENARIOS), help="run a serving scenario instead of the headline figure")
     args = parser.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+
+    if args.scenario:
+        print(json.dumps(run_scenario(args.scenario, args.dtype, args.layers)), flush=True)
+        return 0
 
     import torch
     from .architectures import config_from_dict
