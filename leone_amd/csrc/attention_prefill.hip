@@ -1,8 +1,8 @@
 // Causal attention of prompt portions over the paged cache on the matrix cores, bfloat16.
 //
-// A portion's rows are cut into tiles of 128 consecutive rows (the host lists them: entry, first
-// row, row count); a workgroup takes one tile and one query head, each of its four waves 32 rows
-// as two 16-column operands.  A wave walks the 32-key tiles its rows can see, from the cache, and
+// A portion's rows are cut into tiles of 32 consecutive rows (the host lists them: entry, first
+// row, row count); a wave takes one tile and one query head, its rows as two 16-column operands;
+// a workgroup is one to four such waves.  A wave walks the 32-key tiles its rows can see, from the cache, and
 // keeps the running maximum, sum and accumulator of the reference's recurrence
 // (crates/leone/src/cpu.rs:2359-2421) per query in registers; nothing of size rows x keys is ever
 // stored (the reference's prefill materialises the scores, crates/leone-cuda/cuda/ie_cuda.cu:5124-5220).
@@ -24,8 +24,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 constexpr int kPrefillWaves = 4;
 constexpr int kPrefillThreads = kPrefillWaves * kWave;
 constexpr int kColsPerWave = 2;                                  // 16-query operands a wave carries
-constexpr int kRowsPerWave = 16 * kColsPerWave;
-constexpr int kRowsPerTile = kRowsPerWave * kPrefillWaves;       // 128
+constexpr int kRowsPerWave = 16 * kColsPerWave;                  // rows of a tile
 constexpr int kKeysPerTile = 32;
 
 __device__ inline bf16x8 pf_load8(const bf16_t* p) {
@@ -36,40 +35,45 @@ __device__ inline bf16x8 pf_zero8() {
     return __builtin_bit_cast(bf16x8, z);
 }
 
-// tiles: [n_tiles][3] = (entry, first row of the tile in the step, rows in the tile).
+// tiles: [n_tiles][3] = (entry, first row of the tile in the step, rows in the tile), at most 32 rows a
+// tile.  Wave w of workgroup b takes tile b * waves + w; waves share nothing but the launch, so tiles of
+// different requests may sit in one workgroup.
 template <int kD16>
 __global__ void __launch_bounds__(kPrefillThreads, 2)
 attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_pool,
                          const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
-                         const int* __restrict__ tiles, const int* __restrict__ block_table, int max_blocks,
-                         int q_heads, int kv_heads, int page_shift, float scale, int window) {
+                         const int* __restrict__ tiles, int n_tiles, const int* __restrict__ block_table,
+                         int max_blocks, int q_heads, int kv_heads, int page_shift, float scale, int window) {
     constexpr int kD = kD16 * 16;
     constexpr int kSteps = (kD16 + 1) / 2;
-    const int entry = tiles[3 * blockIdx.x], tile_row0 = tiles[3 * blockIdx.x + 1], tile_rows = tiles[3 * blockIdx.x + 2];
-    const int head = blockIdx.y;
-    const int kvh = head / (q_heads / kv_heads);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int lane = threadIdx.x % kWave;
+    const int tile = blockIdx.x * (blockDim.x / kWave) + wave;
+    const bool has_tile = tile < n_tiles;
+    const int entry = has_tile ? tiles[3 * tile] : 0;
+    const int tile_row0 = has_tile ? tiles[3 * tile + 1] : 0;
+    const int wave_rows = has_tile ? tiles[3 * tile + 2] : 0;
+    const int head = blockIdx.y;
+    const int kvh = head / (q_heads / kv_heads);
     const int c = lane & 15, g = lane >> 4;
     const int page_tokens = 1 << page_shift, page_mask = page_tokens - 1;
-    const int wave_row0 = kRowsPerWave * wave;                 // first row of this wave inside the tile
+    const int wave_row0 = 0;
     const int* table = block_table + static_cast<long>(entry) * max_blocks;
 
-    // The page ids of the keys this workgroup reads go to shared memory first, so that no load of keys
-    // or values waits on a read of the block table.
-    extern __shared__ int pages[];
-    int first_page;
-    {
-        const int blk_p0 = positions[tile_row0];
-        const int blk_lo = (window > 0 && blk_p0 - window + 1 > 0) ? blk_p0 - window + 1 : 0;
-        first_page = blk_lo >> page_shift;
-        const int n_pages = ((blk_p0 + tile_rows - 1) >> page_shift) - first_page + 1;
-        for (int i = threadIdx.x; i < n_pages; i += kPrefillThreads) pages[i] = table[first_page + i];
-        __syncthreads();
+    // The page ids of the keys a wave reads go to its part of shared memory first, so that no load of
+    // keys or values waits on a read of the block table.
+    extern __shared__ int all_pages[];
+    int* pages = all_pages + wave * max_blocks;
+    int first_page = 0;
+    if (has_tile) {
+        const int tile_p0 = positions[tile_row0];
+        const int tile_lo = (window > 0 && tile_p0 - window + 1 > 0) ? tile_p0 - window + 1 : 0;
+        first_page = tile_lo >> page_shift;
+        const int n_pages = ((tile_p0 + wave_rows - 1) >> page_shift) - first_page + 1;
+        for (int i = lane; i < n_pages; i += kWave) pages[i] = table[first_page + i];
     }
-
-    if (wave_row0 >= tile_rows) return;                        // after the workgroup's only barrier
-    const int wave_rows = tile_rows - wave_row0 < kRowsPerWave ? tile_rows - wave_row0 : kRowsPerWave;
+    __syncthreads();
+    if (!has_tile) return;                                     // after the workgroup's only barrier
 
     // Rows of a portion are consecutive positions: row r of the wave sits at p0 + r.
     const int p0 = positions[tile_row0 + wave_row0];
@@ -248,18 +252,22 @@ template <int kD16>
 static void launch_prefill(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
                            const int* tiles, int n_tiles, const int* block_table, int max_blocks, int q_heads,
                            int kv_heads, int page_shift, float scale, int window, hipStream_t stream) {
-    dim3 grid(n_tiles, q_heads);
-    attention_prefill_kernel<kD16><<<grid, kPrefillThreads, static_cast<size_t>(max_blocks) * sizeof(int), stream>>>(
+    // Four tiles a workgroup when there are plenty (their waves read the same keys, which the caches
+    // then serve once), fewer when the chip would otherwise stay half empty.
+    const long wave_tiles = static_cast<long>(n_tiles) * q_heads;
+    const int waves = wave_tiles >= 2048 ? 4 : wave_tiles >= 1024 ? 2 : 1;
+    dim3 grid(ceil_div(n_tiles, waves), q_heads);
+    attention_prefill_kernel<kD16><<<grid, waves * kWave, static_cast<size_t>(waves) * max_blocks * sizeof(int), stream>>>(
         static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_pool),
-        static_cast<const bf16_t*>(v_pool), positions, tiles, block_table, max_blocks, q_heads, kv_heads, page_shift,
-        scale, window);
+        static_cast<const bf16_t*>(v_pool), positions, tiles, n_tiles, block_table, max_blocks, q_heads, kv_heads,
+        page_shift, scale, window);
 }
 
 }  // namespace leone
 
 using namespace leone;
 
-extern "C" int leone_attention_prefill_tile_rows() { return kRowsPerTile; }
+extern "C" int leone_attention_prefill_tile_rows() { return kRowsPerWave; }
 
 extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_pool, const void* v_pool,
                                        const int* positions, const int* tiles, int n_tiles, const int* block_table,
@@ -274,7 +282,7 @@ extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_p
     LEONE_REQUIRE(page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0,
                   "attention_prefill: page_tokens %d must be a power of two, at least 16", page_tokens);
     LEONE_REQUIRE(window >= 0 && max_blocks > 0, "attention_prefill: bad window or block table");
-    LEONE_REQUIRE(static_cast<size_t>(max_blocks) * sizeof(int) <= 64 * 1024,
+    LEONE_REQUIRE(static_cast<size_t>(kPrefillWaves) * max_blocks * sizeof(int) <= 64 * 1024,
                   "attention_prefill: a block table of %d entries does not fit shared memory", max_blocks);
     int page_shift = 0;
     while ((1 << page_shift) < page_tokens) ++page_shift;

@@ -215,13 +215,13 @@ def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
     return out
 
 
-PREFILL_TILE_ROWS = 128      # rows of one request a workgroup of the prompt kernel takes (checked against the library)
+PREFILL_TILE_ROWS = 32       # rows of one request a wave of the prompt kernel takes (checked against the library)
 PREFILL_MIN_ROWS = 16        # shorter portions go through the split-KV kernel row by row
 
 
 def prefill_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int, max_blocks: int = 0) -> bool:
     return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 128
-            and 4 * max_blocks <= 64 * 1024                       # the page ids of a workgroup's keys
+            and 16 * max_blocks <= 64 * 1024                      # the page ids of four waves' keys
             and page_tokens >= 16 and page_tokens & (page_tokens - 1) == 0)
 
 

@@ -10,7 +10,7 @@ from tests.util import TINY, make_model_dir, random_tokens, read_config, read_we
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [1, 7, 33, 64, 100, 18, 47], "B": [5, 40, 130, 66, 90], "C": [70, 150, 35, 81, 3],
-           "M": [300, 45, 170, 129, 20]}
+           "M": [300, 45, 170, 129, 20], "D": [90, 17, 64, 2]}
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 
