@@ -96,6 +96,12 @@ def build_parser() -> argparse.ArgumentParser:
     r.add_argument("--out", required=True)
     r.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
 
+    q = sub.add_parser("quality", help="Compare two logit files: KL divergence and top-1 agreement")
+    q.add_argument("--oracle", required=True, help="Reference logits (row-major little-endian f32)")
+    q.add_argument("--subject", required=True, help="Logits under test, same shape")
+    q.add_argument("--vocab", type=int, help="Vocabulary size (or give -m)")
+    q.add_argument("-m", "--model", help="Model folder to take the vocabulary size from")
+
     b = sub.add_parser("bench", help="Measure decode and prefill throughput")
     b.add_argument("rest", nargs=argparse.REMAINDER)
     return parser
@@ -254,6 +260,49 @@ def cmd_eval(args) -> int:
     return 0
 
 
+def quality_stats(oracle, subject):
+    """KL(oracle || subject) per row in nats (mean, median, 99th percentile, maximum) and how often the
+    two agree on the highest logit: the reference's quality figures (crates/leone-cli/src/quality.rs:33-95)."""
+    import numpy as np
+    oracle = np.asarray(oracle, dtype=np.float64)
+    subject = np.asarray(subject, dtype=np.float64)
+    if oracle.shape != subject.shape or oracle.ndim != 2:
+        raise ValueError(f"logit arrays differ in shape: {oracle.shape} and {subject.shape}")
+
+    def log_softmax(x):
+        x = x - x.max(axis=1, keepdims=True)
+        return x - np.log(np.exp(x).sum(axis=1, keepdims=True))
+    lo, ls = log_softmax(oracle), log_softmax(subject)
+    kld = (np.exp(lo) * (lo - ls)).sum(axis=1)
+    return {"samples": int(oracle.shape[0]), "kld_mean": float(kld.mean()), "kld_p50": float(np.percentile(kld, 50)),
+            "kld_p99": float(np.percentile(kld, 99)), "kld_max": float(kld.max()),
+            "top1_agreement": float((oracle.argmax(axis=1) == subject.argmax(axis=1)).mean()),
+            "max_abs": float(np.abs(oracle - subject).max())}
+
+
+def cmd_quality(args) -> int:
+    import numpy as np
+    vocab = args.vocab
+    if vocab is None:
+        if not args.model:
+            raise SystemExit("error: give --vocab or -m")
+        from .architectures import config_from_dir
+        vocab = config_from_dir(args.model).vocab_size
+    oracle = np.fromfile(args.oracle, dtype="<f4")
+    subject = np.fromfile(args.subject, dtype="<f4")
+    if oracle.size != subject.size or oracle.size % vocab:
+        raise SystemExit(f"error: {oracle.size} and {subject.size} values do not make equal rows of {vocab}")
+    stats = quality_stats(oracle.reshape(-1, vocab), subject.reshape(-1, vocab))
+    print(f"samples: {stats['samples']}")
+    print(f"KLD mean: {stats['kld_mean']:.9f} nats")
+    print(f"KLD p50:  {stats['kld_p50']:.9f} nats")
+    print(f"KLD p99:  {stats['kld_p99']:.9f} nats")
+    print(f"KLD max:  {stats['kld_max']:.9f} nats")
+    print(f"top1 agreement: {stats['top1_agreement']:.9f}")
+    print(f"max abs difference: {stats['max_abs']:.6f}")
+    return 0
+
+
 def cmd_random_model(args) -> int:
     import torch
     from .architectures import config_from_dict
@@ -278,6 +327,8 @@ def main(argv: Optional[List[str]] = None) -> int:
         return cmd_doctor(args)
     if args.command == "eval":
         return cmd_eval(args)
+    if args.command == "quality":
+        return cmd_quality(args)
     if args.command == "random-model":
         return cmd_random_model(args)
     if args.command == "bench":

@@ -304,3 +304,66 @@ def test_toy_architecture_with_state_window_repeat_and_shared_cache(tmp_path, dt
     finally:
         unregister_architecture("ToyForCausalLM")
         MIXERS.unregister("toy_decay")
+
+
+def test_position_part():
+    from leone_amd.parts import POSITIONS, PartSpec
+    rope = POSITIONS.build(PartSpec("rope_half_split", {"rotary_dim": 48, "theta": 50000.0}))
+    rope.prepare(300, DEV)
+    cos, sin = rope.tables()
+    assert cos.shape == (300, 24) and cos.dtype == torch.float32
+    for pos in (0, 1, 77, 299):
+        for i in (0, 5, 23):
+            angle = pos * 50000.0 ** (-2.0 * i / 48)
+            assert abs(float(cos[pos, i]) - math.cos(angle)) < 5e-7 and abs(float(sin[pos, i]) - math.sin(angle)) < 5e-7
+    none = POSITIONS.build(PartSpec("none", {}))
+    none.prepare(10, DEV)
+    assert none.tables() == (None, None)
+    with pytest.raises(ValueError):
+        POSITIONS.build(PartSpec("rope_half_split", {"rotary_dim": 15, "theta": 1e4}))
+    with pytest.raises(ValueError):
+        POSITIONS.build(PartSpec("alibi", {}))
+
+
+@pytest.mark.parametrize("rows", [9, 40])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_part(dtype, rows):
+    """One pre-norm block alone: x1 = x + attention(norm1 x), x2 = x1 + feed_forward(norm2 x1).  With few
+    rows the bfloat16 products add into the stream themselves; with many the block hands back a delta."""
+    from leone_amd.parts import BLOCKS, POSITIONS, PartSpec
+    from leone_amd.parts.context import KvCacheView
+    hidden, heads, kv, dim, ffn, page = 64, 4, 2, 16, 96, 16
+    rope = POSITIONS.build(PartSpec("rope_half_split", {"rotary_dim": dim, "theta": 1e4}))
+    rope.prepare(64, DEV)
+    spec = PartSpec("prenorm", {
+        "norm1": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-5, "weight": "n1"}),
+        "mixer": PartSpec("gqa_attention", dict(hidden=hidden, q_heads=heads, kv_heads=kv, head_dim=dim, qk_norm_eps=1e-5,
+                                                window=None, position="rope", q="a.q_proj.weight", k="a.k_proj.weight",
+                                                v="a.v_proj.weight", o="a.o_proj.weight", q_norm="a.q_norm.weight",
+                                                k_norm="a.k_norm.weight")),
+        "norm2": PartSpec("rmsnorm", {"size": hidden, "eps": 1e-5, "weight": "n2"}),
+        "feed_forward": PartSpec("swiglu", {"hidden": hidden, "intermediate": ffn, "gate": "f.gate_proj.weight",
+                                            "up": "f.up_proj.weight", "down": "f.down_proj.weight"})})
+    block = BLOCKS.build(spec, positions={"rope": rope})
+    torch.manual_seed(12)
+    w = {s.name: (torch.randn(s.shape) * 0.08 if len(s.shape) == 2 else 1 + 0.1 * torch.randn(s.shape)).to(dtype)
+         for s in block.tensor_specs()}
+    assert len(w) == 11
+    block.bind({k: v.to(DEV) for k, v in w.items()})
+    x0 = torch.randn(rows, hidden)
+    k_pool = torch.zeros((4, kv, dim // 8, page, 8), dtype=dtype, device=DEV)
+    v_pool = torch.zeros((4, kv, page // 8, dim, 8), dtype=dtype, device=DEV)
+    table = torch.tensor([[2, 0, 3, 1]], dtype=torch.int32, device=DEV)
+    cache = KvCacheView(writes=True, k_pool=k_pool, v_pool=v_pool, block_table=table, page_tokens=page)
+    step = step_context([(0, i) for i in range(rows)], dtype, {0: table})
+    x = x0.to(DEV)
+    pending = block.forward(x, None, step, cache)
+    got = x.cpu().double() + (0 if pending is None else pending.cpu().double())
+    if dtype == torch.bfloat16:
+        assert (pending is None) == (rows <= 16)
+    wf = {k: v.float() for k, v in w.items()}
+    cfg = dict(num_attention_heads=heads, num_key_value_heads=kv, head_dim=dim, rms_norm_eps=1e-5, rope_theta=1e4)
+    x1 = x0.double() + plain.attention_block(plain.rms_norm(x0, wf["n1"], 1e-5), wf, "a", cfg, list(range(rows)))
+    want = x1 + plain.feed_forward(plain.rms_norm(x1, wf["n2"], 1e-5), wf, "f")
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    assert (got - want).abs().max() < tol
