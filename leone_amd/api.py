@@ -23,9 +23,12 @@ def sampling_params(temperature: Optional[float] = None, seed: int = 0, top_k: O
                     top_p: Optional[float] = None, min_p: Optional[float] = None,
                     truncations: Optional[Sequence[tuple]] = None, repeat_penalty: float = 1.0,
                     presence_penalty: float = 0.0, frequency_penalty: float = 0.0,
-                    penalty_window: int = 64) -> SamplingParams:
+                    penalty_window: int = 64, dry_multiplier: float = 0.0, dry_base: float = 1.75,
+                    dry_allowed_length: int = 2, dry_window: int = 64, dry_breakers: Sequence[int] = (),
+                    mirostat: Optional[tuple] = None) -> SamplingParams:
     """``temperature`` None is greedy.  ``truncations`` gives stages in order; the named
-    shortcuts are appended as top-k, top-p, min-p."""
+    shortcuts are appended as top-k, top-p, min-p.  ``dry_multiplier`` above zero turns the
+    repeated-suffix penalty on; ``mirostat`` is (target surprise in nats, learning rate)."""
     stages = list(truncations or [])
     if top_k is not None:
         stages.append(("top_k", top_k))
@@ -34,7 +37,8 @@ def sampling_params(temperature: Optional[float] = None, seed: int = 0, top_k: O
     if min_p is not None:
         stages.append(("min_p", min_p))
     params = SamplingParams(temperature, stages, seed, repeat_penalty, presence_penalty, frequency_penalty,
-                            penalty_window)
+                            penalty_window, dry_multiplier, dry_base, dry_allowed_length, dry_window,
+                            tuple(int(t) for t in dry_breakers), mirostat)
     if stages and temperature is None:
         raise ValueError("truncation stages need a temperature; greedy takes the highest logit")
     params.validate()

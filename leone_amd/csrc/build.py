@@ -1,8 +1,11 @@
-"""Builds the gfx950 kernel library from the sources in this folder.
+"""Builds the two native libraries from the sources in this folder.
 
-``hipcc`` cross-compiles without a GPU.  Objects and the shared library go to
-``_build/`` beside the sources; if that folder cannot be written (a read-only
-checkout) a per-user folder under the system's temporary directory is used.
+``libleone_hip.so`` holds the gfx950 kernels (the ``.hip`` files here); ``hipcc``
+cross-compiles them without a GPU.  ``libleone_host.so`` holds the host runtime
+(cache manager, scheduler, step layout; plain C++ under ``host/``) and needs only
+a C++ compiler.  Objects and libraries go to ``_build/`` beside the sources; if
+that folder cannot be written (a read-only checkout) a per-user folder under the
+system's temporary directory is used.
 """
 from __future__ import annotations
 
@@ -42,6 +45,26 @@ def source_digest() -> str:
     return digest.hexdigest()[:16]
 
 
+HOST_DIR = os.path.join(HERE, "host")
+HOST_LIB_NAME = "libleone_host.so"
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
+
+
+def host_sources() -> list[str]:
+    return sorted(f for f in os.listdir(HOST_DIR) if f.endswith(".cpp"))
+
+
+def host_digest() -> str:
+    digest = hashlib.sha256()
+    for name in sorted(os.listdir(HOST_DIR)):
+        if name.endswith((".cpp", ".h")):
+            digest.update(name.encode())
+            with open(os.path.join(HOST_DIR, name), "rb") as handle:
+                digest.update(handle.read())
+    digest.update(" ".join(HOST_FLAGS).encode())
+    return digest.hexdigest()[:16]
+
+
 def _writable(path: str) -> bool:
     try:
         os.makedirs(path, exist_ok=True)
@@ -63,18 +86,60 @@ def build_dir() -> str:
     return fallback
 
 
-def library_path() -> str | None:
-    """The built library that matches the present sources, if there is one."""
-    digest = source_digest()
+def _built(lib_name: str, stamp_name: str, digest: str) -> str | None:
     for folder in (os.path.join(HERE, "_build"),
                    os.path.join(tempfile.gettempdir(), f"leone_amd_build_{os.getuid()}")):
-        lib = os.path.join(folder, LIB_NAME)
-        stamp = os.path.join(folder, "digest.txt")
+        lib = os.path.join(folder, lib_name)
+        stamp = os.path.join(folder, stamp_name)
         if os.path.exists(lib) and os.path.exists(stamp):
             with open(stamp) as handle:
                 if handle.read().strip() == digest:
                     return lib
     return None
+
+
+def library_path() -> str | None:
+    """The built kernel library that matches the present sources, if there is one."""
+    return _built(LIB_NAME, "digest.txt", source_digest())
+
+
+def host_library_path() -> str | None:
+    """The built host library that matches the present sources, if there is one."""
+    return _built(HOST_LIB_NAME, "digest_host.txt", host_digest())
+
+
+def host_compiler() -> str:
+    for name in ("g++", "c++", "clang++"):
+        found = shutil.which(name)
+        if found:
+            return found
+    return hipcc()      # its clang compiles plain C++ as well
+
+
+def build_host(verbose: bool = True, force: bool = True) -> str:
+    """Compiles the host runtime; returns the library's path."""
+    if not force:
+        ready = host_library_path()
+        if ready:
+            return ready
+    out_dir = build_dir()
+    started = time.time()
+    lib = os.path.join(out_dir, HOST_LIB_NAME)
+    tmp = lib + f".tmp{os.getpid()}"
+    cmd = ([host_compiler()] + HOST_FLAGS + ["-shared", "-I", HOST_DIR, "-o", tmp]
+           + [os.path.join(HOST_DIR, name) for name in host_sources()])
+    if verbose:
+        print(f"[leone_amd] building {HOST_LIB_NAME} from {len(host_sources())} sources into {out_dir}",
+              file=sys.stderr, flush=True)
+    result = subprocess.run(cmd, capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"the C++ compiler failed on the host library:\n{result.stderr}")
+    os.replace(tmp, lib)
+    with open(os.path.join(out_dir, "digest_host.txt"), "w") as handle:
+        handle.write(host_digest() + "\n")
+    if verbose:
+        print(f"[leone_amd] built {lib} in {time.time() - started:.0f}s", file=sys.stderr, flush=True)
+    return lib
 
 
 def hipcc() -> str:
@@ -139,4 +204,5 @@ def build(verbose: bool = True, force: bool = True) -> str:
 
 
 if __name__ == "__main__":
+    print(build_host())
     print(build())

@@ -12,12 +12,15 @@ reserved first, written by the kernels, and committed only if the step succeeds
 """
 from __future__ import annotations
 
+import ctypes
+from ctypes import c_int, c_int64, c_long
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence
 
 import numpy as np
 import torch
 
+from .. import hostlib, ops
 from ..cache.manager import CacheManager, OutOfPages
 from ..cache.pools import DevicePools
 from ..parts.context import EntryInfo, StepContext
@@ -41,6 +44,63 @@ class StepError(ValueError):
     """A step was refused before anything ran; the cache is unchanged."""
 
 
+class _PackedStep:
+    """One step's metadata as the native layout routine wrote it into a host buffer."""
+
+    def __init__(self, engine: "Engine", entries: Sequence[StepEntry], all_rows_wanted: bool,
+                 host: Optional[torch.Tensor] = None):
+        cache = engine.cache
+        n = len(entries)
+        lib = hostlib.library()
+        requests = (c_int64 * max(1, n))()
+        counts, want_counts = (c_int * max(1, n))(), (c_int * max(1, n))()
+        flat_tokens: List[int] = []
+        flat_wants: List[int] = []
+        for i, e in enumerate(entries):
+            key = cache.keys.key(e.request)
+            if key is None:
+                raise StepError(f"request {e.request!r} is not admitted")
+            requests[i], counts[i], want_counts[i] = key, len(e.tokens), len(e.want)
+            flat_tokens.extend(e.tokens)
+            flat_wants.extend(e.want)
+        try:
+            tokens = np.asarray(flat_tokens, dtype=np.int64)
+            wants = np.asarray(flat_wants, dtype=np.int64)
+        except (TypeError, ValueError, OverflowError) as error:
+            raise StepError(f"tokens and wanted places must be integers: {error}") from None
+        limit = np.iinfo(np.int32)
+        if tokens.size and (tokens.min() < limit.min or tokens.max() > limit.max):
+            raise StepError(f"a token lies outside the vocabulary of {engine.vocab_size}")
+        if wants.size and (wants.min() < limit.min or wants.max() > limit.max):
+            raise StepError("a wanted place lies outside its entry")
+        tokens, wants = tokens.astype(np.int32), wants.astype(np.int32)
+        shape = (c_int * 4)(engine.vocab_size, ops.PREFILL_TILE_ROWS, ops.PREFILL_MIN_ROWS, int(all_rows_wanted))
+        sections = (c_long * (7 + len(cache.groups)))()
+        summary, placed = (c_int * 6)(), (c_int * (5 * max(1, n)))()
+        as_i32 = lambda a: a.ctypes.data_as(hostlib.PI32)
+        args = (cache.handle, n, requests, counts, want_counts, as_i32(tokens), as_i32(wants), shape)
+        total = lib.leone_step_pack(*args, None, 0, sections, None, None)
+        if total >= 0:
+            if host is None:
+                host = torch.empty(max(1, total), dtype=torch.int32)
+            elif host.numel() < total:
+                raise StepError("the step does not fit the recorded layout")
+            total = lib.leone_step_pack(*args, ctypes.cast(host.data_ptr(), hostlib.PI32), host.numel(), sections,
+                                        summary, placed)
+        if total < 0:
+            raise StepError(hostlib.last_error())
+        self.host = host
+        self.total = int(total)
+        self.offsets = list(sections)
+        self.rows, self.prefill_rows, self.max_position, self.tiles, self.wanted = list(summary)[:5]
+        self.decode_only = bool(summary[5])
+        # Entries in the order they run in: (index in the caller's list, slot, first row, rows, start).
+        self.placed = [tuple(placed[5 * i:5 * i + 5]) for i in range(n)]
+
+    def pieces(self, packed: torch.Tensor) -> List[torch.Tensor]:
+        return [packed[self.offsets[i]:self.offsets[i + 1]] for i in range(len(self.offsets) - 1)]
+
+
 class _DecodeGraph:
     """A recorded decode step for one batch size: static metadata buffers, the graph, its logits.
 
@@ -53,20 +113,18 @@ class _DecodeGraph:
     def __init__(self, engine: "Engine", rows: int):
         groups = len(engine.cache.groups)
         widths = [engine.cache.max_blocks(g) for g in range(groups)]
-        sizes = [rows] * 5 + [rows * w for w in widths]     # tokens, positions, row_entry, slots, want, tables
-        self.offsets = np.cumsum([0] + sizes)
-        total = int(self.offsets[-1])
+        sizes = [rows] * 5 + [0] + [rows * w for w in widths]   # tokens, positions, row_entry, slots, want, tiles, tables
+        self.offsets = [int(v) for v in np.cumsum([0] + sizes)]
+        total = self.offsets[-1]
         self.host = torch.empty(total, dtype=torch.int32).pin_memory()
-        self.host_np = self.host.numpy()
         self.dev = torch.zeros(total, dtype=torch.int32, device=engine.device)
         pieces = [self.dev[self.offsets[i]:self.offsets[i + 1]] for i in range(len(sizes))]
         self.tokens = pieces[0]
         self.rows = rows
-        self.widths = widths
         self.context = StepContext(
             rows=rows, dtype=engine.dtype, device=engine.device, positions=pieces[1], row_entry=pieces[2],
             entries=[], entry_slots=pieces[3], want_rows=pieces[4],
-            block_tables={g: pieces[5 + g].view(rows, widths[g]) for g in range(groups)},
+            block_tables={g: pieces[6 + g].view(rows, widths[g]) for g in range(groups)},
             max_position=engine.max_context - 1, decode_only=True)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
@@ -74,18 +132,9 @@ class _DecodeGraph:
 
     def fill(self, engine: "Engine", entries: Sequence[StepEntry]) -> None:
         self.copied.synchronize()                     # the last upload has left the pinned buffer
-        rows, o, h = self.rows, self.offsets, self.host_np
-        h[o[2]:o[3]] = np.arange(rows)
-        h[o[4]:o[5]] = np.arange(rows)
-        for i, e in enumerate(entries):
-            h[o[0] + i] = int(e.tokens[0])
-            h[o[1] + i] = engine.cache.length(e.request)
-            h[o[3] + i] = engine.cache.slot(e.request)
-            for g, width in enumerate(self.widths):
-                table = engine.cache.table(e.request, g)
-                base = o[5 + g] + i * width
-                h[base:base + len(table)] = table
-                h[base + len(table):base + width] = -1
+        packed = _PackedStep(engine, entries, all_rows_wanted=True, host=self.host)
+        if packed.offsets != self.offsets:
+            raise StepError("the step does not fit the recorded layout")
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
 
@@ -148,6 +197,7 @@ class Engine:
 
     # ---- the step --------------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]) -> None:
+        """Refuses a malformed step before anything is reserved (the layout routine checks again)."""
         if not entries:
             raise StepError("a step needs at least one entry")
         seen = set()
@@ -157,9 +207,9 @@ class Engine:
             seen.add(e.request)
             if len(e.tokens) == 0:
                 raise StepError(f"request {e.request!r} brings no tokens")
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    raise StepError(f"request {e.request!r}: token {t} is outside the vocabulary of {self.vocab_size}")
+            tokens = np.asarray(e.tokens)
+            if tokens.dtype.kind not in "iu" or tokens.min() < 0 or tokens.max() >= self.vocab_size:
+                raise StepError(f"request {e.request!r}: a token is outside the vocabulary of {self.vocab_size}")
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise StepError(f"request {e.request!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
@@ -186,7 +236,6 @@ class Engine:
     def run_reserved(self, entries: Sequence[StepEntry]) -> StepOutput:
         """Runs a step whose pages the caller has reserved; commits on success, rolls back on failure."""
         try:
-            self._validate(entries)
             for e in entries:
                 if self.cache.length(e.request) == 0:
                     self.pools.zero_state(self.cache.slot(e.request))   # a request's state starts from zero
@@ -247,57 +296,18 @@ class Engine:
         return logits.index_select(0, index), rows_map
 
     def _build_context(self, entries: Sequence[StepEntry]):
-        from ..ops import PREFILL_MIN_ROWS, PREFILL_TILE_ROWS
-        n_rows = sum(len(e.tokens) for e in entries)
+        """The step's metadata, laid out by the native routine and uploaded in one copy."""
+        packed = _PackedStep(self, entries, all_rows_wanted=False)
+        device = packed.host[:max(1, packed.total)].to(self.device)
+        pieces = packed.pieces(device)
+        infos = [EntryInfo(entries[given].request, slot, first_row, count, start)
+                 for given, slot, first_row, count, start in packed.placed]
+        rows_map = [(e.request, int(w)) for e in entries for w in e.want]
         n_groups = len(self.cache.groups)
-        tokens = np.empty(n_rows, dtype=np.int32)
-        positions = np.empty(n_rows, dtype=np.int32)
-        row_entry = np.empty(n_rows, dtype=np.int32)
-        slots = np.empty(len(entries), dtype=np.int32)
-        tables = [np.full((len(entries), self.cache.max_blocks(g)), -1, dtype=np.int32) for g in range(n_groups)]
-        # Inside the step long prompt portions come first (the prompt attention kernel takes them tile by
-        # tile), short portions and decoded tokens after; logits keep the caller's order of entries.
-        order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) < PREFILL_MIN_ROWS)
-        first_row = [0] * len(entries)
-        infos: List[EntryInfo] = []
-        tiles: List[tuple] = []
-        prefill_rows = 0
-        row = 0
-        for ei, i in enumerate(order):
-            e = entries[i]
-            start = self.cache.length(e.request)
-            n = len(e.tokens)
-            first_row[i] = row
-            tokens[row:row + n] = np.asarray(e.tokens, dtype=np.int64)
-            positions[row:row + n] = np.arange(start, start + n)
-            row_entry[row:row + n] = ei
-            slots[ei] = self.cache.slot(e.request)
-            for g in range(n_groups):
-                table = self.cache.table(e.request, g)
-                tables[g][ei, :len(table)] = table
-            if n >= PREFILL_MIN_ROWS:
-                for at in range(0, n, PREFILL_TILE_ROWS):
-                    tiles.append((ei, row + at, min(PREFILL_TILE_ROWS, n - at)))
-                prefill_rows = row + n
-            infos.append(EntryInfo(e.request, int(slots[ei]), row, n, start))
-            row += n
-        want_rows: List[int] = []
-        rows_map: List[tuple] = []
-        for i, e in enumerate(entries):
-            for w in e.want:
-                want_rows.append(first_row[i] + int(w))
-                rows_map.append((e.request, int(w)))
-        # One upload for all step metadata.
-        parts = [tokens, positions, row_entry, slots, np.asarray(want_rows, dtype=np.int32),
-                 np.asarray(tiles, dtype=np.int32).reshape(-1)] + [t.reshape(-1) for t in tables]
-        packed = torch.from_numpy(np.concatenate(parts)).to(self.device)
-        offsets = np.cumsum([0] + [p.size for p in parts])
-        pieces = [packed[offsets[i]:offsets[i + 1]] for i in range(len(parts))]
-        block_tables = {g: pieces[6 + g].view(len(entries), -1) for g in range(n_groups)}
         context = StepContext(
-            rows=n_rows, dtype=self.dtype, device=self.device, positions=pieces[1], row_entry=pieces[2],
-            entries=infos, entry_slots=pieces[3], want_rows=pieces[4] if want_rows else None,
-            block_tables=block_tables, max_position=int(positions.max()),
-            decode_only=all(len(e.tokens) == 1 for e in entries),
-            prefill_rows=prefill_rows, q_tiles=pieces[5].view(-1, 3) if tiles else None)
+            rows=packed.rows, dtype=self.dtype, device=self.device, positions=pieces[1], row_entry=pieces[2],
+            entries=infos, entry_slots=pieces[3], want_rows=pieces[4] if packed.wanted else None,
+            block_tables={g: pieces[6 + g].view(len(entries), -1) for g in range(n_groups)},
+            max_position=packed.max_position, decode_only=packed.decode_only,
+            prefill_rows=packed.prefill_rows, q_tiles=pieces[5].view(-1, 3) if packed.tiles else None)
         return pieces[0], context, rows_map

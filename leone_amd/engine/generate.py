@@ -15,7 +15,7 @@ import torch
 
 from .. import ops
 from ..sampling import rng
-from ..sampling.sampler import SamplerError, SamplingParams, sample as host_sample
+from ..sampling.sampler import MirostatState, SamplerError, SamplingParams, sample as host_sample
 from .engine import Engine, StepEntry
 from .scheduler import Finished, PlannedEntry, Reject, Request, Scheduler, SchedulerPolicy
 
@@ -55,7 +55,8 @@ class RequestRejected(ValueError):
 
 
 def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params: Dict[Hashable, SamplingParams],
-                  histories: Dict[Hashable, Sequence[int]]) -> Dict[Hashable, int]:
+                  histories: Dict[Hashable, Sequence[int]],
+                  controllers: Optional[Dict[Hashable, MirostatState]] = None) -> Dict[Hashable, int]:
     """One token per sampled entry; ``logits`` has one row per such entry, in order.
 
     Greedy and plain-temperature rows are chosen by the device kernels; rows with truncation stages
@@ -88,7 +89,8 @@ def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params:
         copied = logits.index_select(0, index).cpu().numpy()
         for k, i in enumerate(host_rows):
             e = rows[i]
-            out[e.request] = host_sample(copied[k], policies[i], e.sample_position, histories[e.request])
+            out[e.request] = host_sample(copied[k], policies[i], e.sample_position, histories[e.request],
+                                         (controllers or {}).get(e.request))
     for e in rows:
         if out[e.request] < 0:
             raise SamplerError(f"request {e.request!r}: no finite logit at position {e.sample_position}")
@@ -103,6 +105,8 @@ class Generator:
         self.scheduler = Scheduler(policy or SchedulerPolicy(max_live_requests=engine.cache.max_requests),
                                    engine.cache)
         self.params: Dict[Hashable, SamplingParams] = {}
+        # Mirostat bounds live with the request, across portions and preemptions.
+        self.controllers: Dict[Hashable, MirostatState] = {}
         self.stats = GenerationStats()
         # Called with (request, position, float32 logits row on the device) for every sampled row.
         self.logit_observer: Optional[Callable[[Hashable, int, torch.Tensor], None]] = None
@@ -119,6 +123,8 @@ class Generator:
         if reason is not None:
             raise RequestRejected(request_id, reason)
         self.params[request_id] = sampling
+        if sampling.mirostat is not None:
+            self.controllers[request_id] = MirostatState(*sampling.mirostat)
         self.stats.prompt_tokens += len(prompt)
 
     def step(self, on_token: Optional[Callable[[Hashable, int], None]] = None) -> List[Finished]:
@@ -132,7 +138,7 @@ class Generator:
             entries = [StepEntry(e.request, e.tokens, [len(e.tokens) - 1] if e.sample else []) for e in plan]
             output = self.engine.run_reserved(entries)
             histories = {e.request: scheduler.live[e.request].tokens for e in plan if e.sample}
-            sampled = choose_tokens(output.logits, plan, self.params, histories) if output.logits is not None else {}
+            sampled = choose_tokens(output.logits, plan, self.params, histories, self.controllers) if output.logits is not None else {}
             if self.logit_observer is not None and output.logits is not None:
                 for row, e in enumerate([e for e in plan if e.sample]):
                     self.logit_observer(e.request, e.sample_position, output.logits[row])
@@ -154,6 +160,8 @@ class Generator:
                 if e.sample:
                     on_token(e.request, sampled[e.request])
         done = scheduler.complete(sampled)
+        for f in done:
+            self.controllers.pop(f.id, None)
         self.stats.preemptions = scheduler.stats.preemptions
         return done
 
@@ -164,6 +172,7 @@ class Generator:
             if cancelled is not None and cancelled():
                 for rid in list(self.scheduler.live) + [q.request.id for q in self.scheduler.queue]:
                     self.scheduler.cancel(rid)
+                    self.controllers.pop(rid, None)
             before = len(self.scheduler.finished)
             self.step(on_token)
             finished.extend(self.scheduler.finished[before:])

@@ -3,7 +3,9 @@
 It decides; it runs nothing.  Each ``plan()`` yields the entries of one step
 with their pages already reserved; the caller runs them (which commits the
 cache) and reports the sampled tokens to ``complete()``.  It needs only the
-host-side cache manager, so its decisions can be tested without a GPU.
+host-side cache manager, so its decisions can be tested without a GPU.  The
+scheduler itself is C++ (``csrc/host/scheduler.cpp``); this class binds it and
+keeps what only this side knows: the requests' names and sampling settings.
 
 What is kept from the reference's scheduler (crates/leone/src/scheduler.rs):
 typed admission rejects with nothing reserved on rejection (:99-110, :587-636);
@@ -27,12 +29,14 @@ is shortened to the free pages or waits; it never preempts.
 """
 from __future__ import annotations
 
-from collections import deque
-from dataclasses import dataclass, field
+import ctypes
+from ctypes import c_int, c_int32, c_int64
+from dataclasses import dataclass, fields
 from enum import Enum
-from typing import Deque, Dict, Hashable, List, Optional, Sequence
+from typing import Dict, Hashable, List, Optional, Sequence
 
-from ..cache.manager import CacheManager, OutOfPages
+from .. import hostlib
+from ..cache.manager import CacheManager
 
 
 class Reject(Enum):
@@ -115,16 +119,30 @@ class SchedulerStats:
     max_live: int = 0
 
 
-class _Live:
-    __slots__ = ("request", "tokens", "prompt_len", "order", "cancelled", "preemptions")
+_REJECTS = [None, Reject.PROMPT_LIMIT, Reject.OUTPUT_LIMIT, Reject.CONTEXT_LIMIT, Reject.KV_CAPACITY,
+            Reject.QUEUE_LIMIT, Reject.DUPLICATE]
+_REASONS = ["eos", "length", "cancelled", "aborted"]
 
-    def __init__(self, request: Request, order: int):
-        self.request = request
-        self.tokens: List[int] = list(request.prompt)   # prompt, then generated tokens
-        self.prompt_len = len(self.tokens)
-        self.order = order
-        self.cancelled = False
-        self.preemptions = 0
+
+class _Known:
+    """A queued or live request as this side sees it; its tokens are read from the native scheduler."""
+    __slots__ = ("request", "_scheduler", "_key")
+
+    def __init__(self, request: Request, scheduler: "Scheduler", key: int):
+        self.request, self._scheduler, self._key = request, scheduler, key
+
+    @property
+    def tokens(self) -> List[int]:
+        """Prompt, then generated tokens."""
+        return self._scheduler._history(self._key)
+
+    @property
+    def prompt_len(self) -> int:
+        return self._scheduler._info(self._key)[0]
+
+    @property
+    def preemptions(self) -> int:
+        return self._scheduler._info(self._key)[1]
 
     @property
     def generated(self) -> List[int]:
@@ -135,265 +153,189 @@ class Scheduler:
     def __init__(self, policy: SchedulerPolicy, cache: CacheManager):
         self.policy = policy.validate()
         self.cache = cache
-        self.queue: Deque[_Live] = deque()
-        self.live: Dict[Hashable, _Live] = {}
         self.finished: List[Finished] = []
-        self.stats = SchedulerStats()
-        self.events: List[tuple] = []
-        self._order = 0
-        self._planned: Optional[List[PlannedEntry]] = None
+        self._lib = hostlib.library()
+        values = (c_int64 * 6)(policy.max_live_requests, policy.max_queued_requests, policy.max_step_tokens,
+                               policy.prefill_chunk_tokens, policy.max_prompt_tokens, policy.max_output_tokens)
+        self.handle = self._lib.leone_scheduler_create(cache.handle, values)
+        if not self.handle:
+            raise SchedulerError(hostlib.last_error())
+        self._known: Dict[Hashable, _Known] = {}        # queued and live requests
+        self._names: Dict[int, Hashable] = {}           # every key ever used, for the event log
+        self._capacity = 0
+        self._grow(64)
+
+    def __del__(self):
+        handle, self.handle = getattr(self, "handle", None), None
+        if handle:
+            self._lib.leone_scheduler_destroy(handle)
+
+    def _grow(self, n: int) -> None:
+        if n > self._capacity:
+            self._capacity = max(n, 2 * self._capacity)
+            self._keys = (c_int64 * self._capacity)()
+            self._starts = (c_int * self._capacity)()
+            self._counts = (c_int * self._capacity)()
+            self._samples = (c_int * self._capacity)()
+            self._sampled = (c_int32 * self._capacity)()
+
+    def _checked(self, code: int) -> int:
+        if code < 0:
+            raise SchedulerError(hostlib.last_error())
+        return code
+
+    def _history(self, key: int) -> List[int]:
+        n = self._checked(self._lib.leone_scheduler_history(self.handle, key, None, 0))
+        out = (c_int32 * max(1, n))()
+        self._checked(self._lib.leone_scheduler_history(self.handle, key, out, n))
+        return out[:n]
+
+    def _info(self, key: int):
+        prompt, preemptions = c_int(), c_int()
+        self._checked(self._lib.leone_scheduler_request_info(self.handle, key, ctypes.byref(prompt),
+                                                             ctypes.byref(preemptions)))
+        return prompt.value, preemptions.value
 
     # ---- admission ---------------------------------------------------------------------
     def submit(self, request: Request) -> Optional[Reject]:
         """Queues a request, or says why not.  A rejected request holds nothing."""
-        self.stats.submitted += 1
-        reason = self._reject_reason(request)
-        if reason is not None:
-            self.stats.rejected += 1
-            self.events.append(("reject", request.id, reason.value))
-            return reason
-        self._order += 1
-        self.queue.append(_Live(request, self._order))
-        self.stats.max_queue_depth = max(self.stats.max_queue_depth, len(self.queue))
-        self.events.append(("submit", request.id))
-        return None
-
-    def _reject_reason(self, request: Request) -> Optional[Reject]:
-        prompt, out = len(request.prompt), request.max_new_tokens
-        if request.id in self.live or any(q.request.id == request.id for q in self.queue):
-            return Reject.DUPLICATE
-        if prompt == 0 or prompt > self.policy.max_prompt_tokens:
-            return Reject.PROMPT_LIMIT
-        if out <= 0 or out > self.policy.max_output_tokens:
-            return Reject.OUTPUT_LIMIT
-        # The last generated token is never fed back, so the cache holds prompt + out - 1 tokens
-        # (crates/leone/src/runtime.rs:3597-3615).
-        held = prompt + out - 1
-        if held > self.cache.max_context:
-            return Reject.CONTEXT_LIMIT
-        for g in self.cache.groups:
-            if g.window is None:
-                need = (held + g.page_tokens - 1) // g.page_tokens
-            else:
-                span = min(held, g.window - 1 + min(self.policy.prefill_chunk_tokens, self.policy.max_step_tokens))
-                need = (span + g.page_tokens - 1) // g.page_tokens + 1
-            if need > g.num_pages:
-                return Reject.KV_CAPACITY
-        if len(self.queue) >= self.policy.max_queued_requests:
-            return Reject.QUEUE_LIMIT
+        known = request.id in self._known
+        key = self.cache.keys.pin(request.id)
+        self._names[key] = request.id
+        prompt = (c_int32 * max(1, len(request.prompt)))(*[int(t) for t in request.prompt])
+        eos = -1 if request.eos_token_id is None else int(request.eos_token_id)
+        code = self._checked(self._lib.leone_scheduler_submit(self.handle, key, prompt, len(request.prompt),
+                                                              int(request.max_new_tokens), eos))
+        if code != 0:
+            if not known:
+                self.cache.keys.unpin(request.id, held=self.cache.has(request.id))
+            return _REJECTS[code]
+        self._known[request.id] = _Known(request, self, key)
         return None
 
     def cancel(self, request_id: Hashable) -> bool:
         """A queued request goes at once; a live one at the next step boundary."""
-        for queued in list(self.queue):
-            if queued.request.id == request_id:
-                self.queue.remove(queued)
-                self._finish(queued, "cancelled", held=False)
-                return True
-        if request_id in self.live:
-            self.live[request_id].cancelled = True
-            return True
-        return False
+        state = self._known.get(request_id)
+        if state is None:
+            return False
+        found = self._checked(self._lib.leone_scheduler_cancel(self.handle, state._key)) == 1
+        self._collect_finished()
+        return found
+
+    # ---- views ---------------------------------------------------------------------------
+    def _listed(self, call) -> List[_Known]:
+        n = self._checked(call(self.handle, None, 0))
+        self._grow(n)
+        self._checked(call(self.handle, self._keys, self._capacity))
+        return [self._known[self._names[self._keys[i]]] for i in range(n)]
+
+    @property
+    def live(self) -> Dict[Hashable, _Known]:
+        """Admitted requests, oldest first."""
+        return {state.request.id: state for state in self._listed(self._lib.leone_scheduler_live)}
+
+    @property
+    def queue(self) -> List[_Known]:
+        """Waiting requests, the next to be admitted first."""
+        return self._listed(self._lib.leone_scheduler_queued)
+
+    def history(self, request_id: Hashable) -> List[int]:
+        """Prompt, then generated tokens, of a queued or live request."""
+        return self._known[request_id].tokens
+
+    @property
+    def stats(self) -> SchedulerStats:
+        values = (c_int64 * 15)()
+        self._lib.leone_scheduler_stats(self.handle, values)
+        return SchedulerStats(*values)
+
+    @property
+    def events(self) -> List[tuple]:
+        """The decision log: ("reject", id, reason), ("submit", id), ("step", [(id, start, tokens, sample)]),
+        ("admit", id), ("preempt", id, tokens known), ("token", id, position, token), ("finish", id, reason)."""
+        n = self._checked(self._lib.leone_scheduler_event_count(self.handle))
+        kinds, a, b, c = (c_int * max(1, n))(), (c_int * max(1, n))(), (c_int * max(1, n))(), (c_int * max(1, n))()
+        keys = (c_int64 * max(1, n))()
+        self._checked(self._lib.leone_scheduler_events(self.handle, 0, n, kinds, keys, a, b, c))
+        out: List[tuple] = []
+        i = 0
+        while i < n:
+            kind = kinds[i]
+            name = self._names.get(keys[i])
+            if kind == 0:
+                out.append(("reject", name, _REJECTS[a[i]].value))
+            elif kind == 1:
+                out.append(("submit", name))
+            elif kind == 2:
+                rows = [(self._names[keys[j]], a[j], b[j], bool(c[j])) for j in range(i + 1, i + 1 + a[i])]
+                out.append(("step", rows))
+                i += a[i]
+            elif kind == 4:
+                out.append(("admit", name))
+            elif kind == 5:
+                out.append(("preempt", name, a[i]))
+            elif kind == 6:
+                out.append(("token", name, a[i], b[i]))
+            elif kind == 7:
+                out.append(("finish", name, _REASONS[a[i]]))
+            i += 1
+        return out
 
     # ---- planning ------------------------------------------------------------------------
     def has_work(self) -> bool:
-        return bool(self.queue or self.live)
+        return self._lib.leone_scheduler_has_work(self.handle) == 1
 
     def plan(self) -> List[PlannedEntry]:
         """Decides the next step and reserves its pages.  Empty only if there is nothing to do."""
-        if self._planned is not None:
-            raise SchedulerError("the previous step was neither completed nor aborted")
-        for state in [s for s in self.live.values() if s.cancelled]:
-            self._finish(state, "cancelled", held=True)
-        entries: List[PlannedEntry] = []
-        for _ in range(len(self.live) + len(self.queue) + 1):
-            entries = self._plan_once()
-            if entries or not self.live:
-                break
-            # Every live request waits for pages that only another live request could free.
-            self._preempt(self._newest(), planned=[])
-        if not entries and (self.live or self.queue):
-            raise SchedulerError("no request can make progress")
-        self._planned = entries
-        if entries:
-            self.stats.steps += 1
-            rows = sum(len(e.tokens) for e in entries)
-            self.stats.max_step_rows = max(self.stats.max_step_rows, rows)
-            self.events.append(("step", [(e.request, e.start, len(e.tokens), e.sample) for e in entries]))
+        n = self._lib.leone_scheduler_plan(self.handle)
+        self._collect_finished()            # requests cancelled since the last step end here
+        self._checked(n)
+        self._grow(n)
+        self._checked(self._lib.leone_scheduler_planned(self.handle, self._keys, self._starts, self._counts,
+                                                        self._samples, self._capacity))
+        entries = []
+        for i in range(n):
+            key, start, count = self._keys[i], self._starts[i], self._counts[i]
+            tokens = (c_int32 * count)()
+            self._checked(self._lib.leone_scheduler_tokens(self.handle, key, start, count, tokens))
+            entries.append(PlannedEntry(self._names[key], list(tokens), start, bool(self._samples[i])))
         return entries
-
-    def _newest(self) -> _Live:
-        return max(self.live.values(), key=lambda s: s.order)
-
-    def _plan_once(self) -> List[PlannedEntry]:
-        entries: List[PlannedEntry] = []
-        budget = self.policy.max_step_tokens
-        by_age = sorted(self.live.values(), key=lambda s: s.order)
-        # 1. one token for every request that is decoding, oldest first
-        for state in by_age:
-            if budget == 0:
-                break
-            if state.request.id not in self.live:
-                continue  # preempted a moment ago
-            cached = self.cache.length(state.request.id)
-            if len(state.tokens) - cached != 1:
-                continue
-            while True:
-                try:
-                    self.cache.reserve(state.request.id, 1)
-                except OutOfPages:
-                    victim = self._newest()
-                    self._preempt(victim, entries)
-                    if victim is state:
-                        break
-                    continue
-                entries.append(PlannedEntry(state.request.id, [state.tokens[cached]], cached, True))
-                budget -= 1
-                self.stats.decode_rows += 1
-                break
-        # 2. prompt portions for the live requests that still have some, oldest first
-        starved = False
-        for state in by_age:
-            if budget == 0 or starved:
-                break
-            if state.request.id not in self.live:
-                continue
-            cached = self.cache.length(state.request.id)
-            remaining = len(state.tokens) - cached
-            if remaining <= 1:
-                continue
-            taken = self._reserve_portion(state, cached, min(remaining, self.policy.prefill_chunk_tokens, budget))
-            if taken == 0:
-                starved = True   # younger requests must not take the pages an older one waits for
-                break
-            entries.append(PlannedEntry(state.request.id, state.tokens[cached:cached + taken], cached,
-                                        taken == remaining))
-            budget -= taken
-            self.stats.prefill_portions += 1
-            self.stats.prefill_tokens += taken
-        # 3. admit from the queue
-        while (self.queue and not starved and budget > 0 and len(self.live) < self.policy.max_live_requests
-               and self.cache.free_slots() > 0):
-            state = self.queue[0]
-            remaining = len(state.tokens)
-            # Admit only when the pages for everything the request already holds are free now,
-            # so that a request just preempted is not taken back in only to be preempted again.
-            if self.live and not self._room_for(remaining):
-                break
-            self.cache.admit(state.request.id)
-            taken = self._reserve_portion(state, 0, min(remaining, self.policy.prefill_chunk_tokens, budget))
-            if taken == 0:
-                self.cache.release(state.request.id)
-                break
-            self.queue.popleft()
-            self.live[state.request.id] = state
-            self.stats.admitted += 1
-            self.stats.max_live = max(self.stats.max_live, len(self.live))
-            self.events.append(("admit", state.request.id))
-            entries.append(PlannedEntry(state.request.id, state.tokens[:taken], 0, taken == remaining))
-            budget -= taken
-            if remaining > 1 or taken > 1:
-                self.stats.prefill_portions += 1
-                self.stats.prefill_tokens += taken
-            else:
-                self.stats.decode_rows += 1
-        return entries
-
-    def _reserve_portion(self, state: _Live, cached: int, wanted: int) -> int:
-        """Reserves the longest portion of at most ``wanted`` tokens that the free pages allow."""
-        rid = state.request.id
-        n = wanted
-        while n > 0:
-            try:
-                self.cache.reserve(rid, n)
-                return n
-            except OutOfPages:
-                lo, hi = 0, n - 1       # largest count whose pages are free
-                while lo < hi:
-                    mid = (lo + hi + 1) // 2
-                    if self._fits(rid, mid):
-                        lo = mid
-                    else:
-                        hi = mid - 1
-                n = lo
-        return 0
-
-    def _room_for(self, tokens: int) -> bool:
-        for gi, g in enumerate(self.cache.groups):
-            span = tokens if g.window is None else min(tokens, g.window - 1 + self.policy.prefill_chunk_tokens)
-            if (span + g.page_tokens - 1) // g.page_tokens > self.cache.free_pages(gi):
-                return False
-        return True
-
-    def _fits(self, rid: Hashable, tokens: int) -> bool:
-        if tokens == 0:
-            return True
-        needed = self.cache.pages_needed(rid, tokens)
-        return all(needed[g] <= self.cache.free_pages(g) for g in range(len(needed)))
-
-    def _preempt(self, victim: _Live, planned: List[PlannedEntry]) -> None:
-        rid = victim.request.id
-        for entry in [e for e in planned if e.request == rid]:
-            planned.remove(entry)
-        self.cache.rollback(rid)
-        self.cache.release(rid)
-        del self.live[rid]
-        victim.preemptions += 1
-        self.queue.appendleft(victim)
-        self.stats.preemptions += 1
-        self.events.append(("preempt", rid, len(victim.tokens)))
 
     # ---- after the step ----------------------------------------------------------------------
     def complete(self, sampled: Dict[Hashable, int]) -> List[Finished]:
         """The planned step ran and its cache writes are committed.  ``sampled`` holds a token for
         every entry planned with ``sample``.  Returns the requests that finished."""
-        if self._planned is None:
-            raise SchedulerError("no step is planned")
-        planned, self._planned = self._planned, None
-        done: List[Finished] = []
-        for entry in planned:
-            state = self.live[entry.request]
-            if self.cache.length(entry.request) != entry.start + len(entry.tokens):
-                raise SchedulerError(f"request {entry.request!r}: the step was not committed to the cache")
-            if not entry.sample:
+        self._grow(len(sampled))
+        n = 0
+        for name, token in sampled.items():
+            state = self._known.get(name)
+            if state is None:
                 continue
-            if entry.request not in sampled:
-                raise SchedulerError(f"request {entry.request!r}: the step returned no token")
-            token = int(sampled[entry.request])
-            state.tokens.append(token)
-            self.stats.emitted_tokens += 1
-            self.events.append(("token", entry.request, entry.sample_position, token))
-            eos = state.request.eos_token_id
-            if eos is not None and token == eos:
-                done.append(self._finish(state, "eos", held=True))
-            elif len(state.generated) >= state.request.max_new_tokens:
-                done.append(self._finish(state, "length", held=True))
-        return done
+            self._keys[n], self._sampled[n] = state._key, int(token)
+            n += 1
+        self._checked(self._lib.leone_scheduler_complete(self.handle, self._keys, self._sampled, n))
+        return self._collect_finished()
 
     def abort(self) -> List[Finished]:
         """The planned step failed: every request in it ends as aborted and gives back what it holds."""
-        if self._planned is None:
-            raise SchedulerError("no step is planned")
-        planned, self._planned = self._planned, None
-        out = []
-        for entry in planned:
-            state = self.live[entry.request]
-            self.cache.rollback(entry.request)
-            out.append(self._finish(state, "aborted", held=True))
-        return out
+        self._checked(self._lib.leone_scheduler_abort(self.handle))
+        return self._collect_finished()
 
-    def _finish(self, state: _Live, reason: str, held: bool) -> Finished:
-        rid = state.request.id
-        if held:
-            self.cache.release(rid)
-            del self.live[rid]
-        result = Finished(rid, list(state.request.prompt), state.generated, reason, state.preemptions)
-        self.finished.append(result)
-        if reason == "cancelled":
-            self.stats.cancelled += 1
-        elif reason == "aborted":
-            self.stats.aborted += 1
-        else:
-            self.stats.finished += 1
-        self.events.append(("finish", rid, reason))
-        return result
+    def _collect_finished(self) -> List[Finished]:
+        total = self._checked(self._lib.leone_scheduler_finished_count(self.handle))
+        new: List[Finished] = []
+        for index in range(len(self.finished), total):
+            key, reason, preemptions, n_prompt, n_out = c_int64(), c_int(), c_int(), c_int(), c_int()
+            self._checked(self._lib.leone_scheduler_finished_info(
+                self.handle, index, ctypes.byref(key), ctypes.byref(reason), ctypes.byref(preemptions),
+                ctypes.byref(n_prompt), ctypes.byref(n_out)))
+            prompt, out = (c_int32 * max(1, n_prompt.value))(), (c_int32 * max(1, n_out.value))()
+            self._checked(self._lib.leone_scheduler_finished_tokens(self.handle, index, prompt, out))
+            name = self._names[key.value]
+            record = Finished(name, prompt[:n_prompt.value], out[:n_out.value], _REASONS[reason.value],
+                              preemptions.value)
+            self.finished.append(record)
+            new.append(record)
+            self._known.pop(name, None)
+            self.cache.keys.unpin(name, held=False)
+        return new

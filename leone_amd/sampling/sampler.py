@@ -10,8 +10,11 @@ top-n-sigma look at raw logits and run before the others
 (crates/leone/src/sampler.rs:184-234, 536-557, 559-606).  The token is the first, in id
 order, whose cumulative probability exceeds the uniform draw; the last eligible
 token if rounding leaves none (crates/leone/src/sampler.rs:843-858).  Penalties
-rewrite the logits from the token history before all this
-(crates/leone/src/penalty.rs:160-196).
+rewrite the logits from the token history before all this: the counting ones
+(crates/leone/src/penalty.rs:160-196), then the repeated-suffix penalty
+(crates/leone/src/penalty.rs:198-249).  A Mirostat v2 controller, when one is
+given, filters the final distribution by surprise before the draw and learns
+from the drawn token (crates/leone/src/sampler.rs:398-446).
 """
 from __future__ import annotations
 
@@ -42,6 +45,12 @@ class SamplingParams:
     presence_penalty: float = 0.0
     frequency_penalty: float = 0.0
     penalty_window: int = 64          # 0 disables the counting penalties
+    dry_multiplier: float = 0.0       # 0 disables the repeated-suffix penalty
+    dry_base: float = 1.75
+    dry_allowed_length: int = 2
+    dry_window: int = 64
+    dry_breakers: Tuple[int, ...] = ()
+    mirostat: Optional[Tuple[float, float]] = None   # (target surprise in nats, learning rate in (0, 1])
 
     def validate(self) -> None:
         t = self.temperature
@@ -64,20 +73,40 @@ class SamplingParams:
             raise SamplerError("presence and frequency penalties must be finite")
         if self.penalty_window < 0:
             raise SamplerError("penalty window must not be negative")
+        if not math.isfinite(self.dry_multiplier) or self.dry_multiplier < 0.0:
+            raise SamplerError("the DRY multiplier must be finite and not negative")
+        if not math.isfinite(self.dry_base) or self.dry_base <= 0.0:
+            raise SamplerError("the DRY base must be finite and positive")
+        if self.dry_allowed_length < 1 or self.dry_window < 0:
+            raise SamplerError("the DRY allowed length must be at least 1 and its window not negative")
+        if self.mirostat is not None:
+            target, rate = self.mirostat
+            if not math.isfinite(target) or target <= 0.0:
+                raise SamplerError("the Mirostat target must be finite and greater than zero")
+            if not math.isfinite(rate) or rate <= 0.0 or rate > 1.0:
+                raise SamplerError("the Mirostat learning rate must be finite and in (0, 1]")
 
     @property
     def greedy(self) -> bool:
         return self.temperature is None
 
     @property
-    def penalties_active(self) -> bool:
+    def counting_active(self) -> bool:
         return self.penalty_window > 0 and (self.repeat_penalty != 1.0 or self.presence_penalty != 0.0
                                             or self.frequency_penalty != 0.0)
 
     @property
+    def dry_active(self) -> bool:
+        return self.dry_multiplier > 0.0 and self.dry_window > 0
+
+    @property
+    def penalties_active(self) -> bool:
+        return self.counting_active or self.dry_active
+
+    @property
     def device_eligible(self) -> bool:
         """Greedy or plain temperature without penalties can be sampled by the device kernels."""
-        return not self.truncations and not self.penalties_active
+        return not self.truncations and not self.penalties_active and self.mirostat is None
 
 
 def apply_penalties(logits: np.ndarray, history: Sequence[int], params: SamplingParams) -> np.ndarray:
@@ -87,19 +116,86 @@ def apply_penalties(logits: np.ndarray, history: Sequence[int], params: Sampling
     if not params.penalties_active:
         return logits
     out = np.array(logits, dtype=np.float32, copy=True)
-    recent = list(history)[-params.penalty_window:]
-    counts = {}
-    for token in recent:
-        counts[token] = counts.get(token, 0) + 1
-    for token, count in sorted(counts.items()):
-        if not 0 <= token < out.shape[0]:
-            continue
-        value = float(out[token])
-        value = value / params.repeat_penalty if value > 0.0 else value * params.repeat_penalty
-        value -= params.presence_penalty
-        value -= params.frequency_penalty * count
-        out[token] = np.float32(value)
+    history = list(history)
+    if params.counting_active:
+        counts = {}
+        for token in history[-params.penalty_window:]:
+            counts[token] = counts.get(token, 0) + 1
+        for token, count in sorted(counts.items()):
+            if not 0 <= token < out.shape[0]:
+                continue
+            value = float(out[token])
+            value = value / params.repeat_penalty if value > 0.0 else value * params.repeat_penalty
+            value -= params.presence_penalty
+            value -= params.frequency_penalty * count
+            out[token] = np.float32(value)
+    if params.dry_active:
+        for token, penalty in sorted(dry_penalties(history[-params.dry_window:], params).items()):
+            if 0 <= token < out.shape[0]:
+                out[token] = np.float32(float(out[token]) - penalty)
     return out
+
+
+def dry_penalties(recent: Sequence[int], params: SamplingParams) -> dict:
+    """Token -> penalty for every token that would extend a repeat of earlier history.
+
+    An earlier occurrence of the last token starts a candidate; the match runs backwards from
+    there while the tokens agree and no breaker is crossed.  A match of at least the allowed
+    length costs multiplier * base**(length - allowed) on the token that followed the earlier
+    occurrence, unless that token is a breaker; the longest repeat decides
+    (crates/leone/src/penalty.rs:213-249)."""
+    penalties: dict = {}
+    if len(recent) < 2:
+        return penalties
+    last = len(recent) - 1
+    breakers = set(params.dry_breakers)
+    for start in range(last):
+        if recent[start] != recent[last]:
+            continue
+        length = 1
+        while (length <= start and recent[start - length] == recent[last - length]
+               and recent[last - length] not in breakers):
+            length += 1
+        if length < params.dry_allowed_length:
+            continue
+        continuation = recent[start + 1]
+        if continuation in breakers:
+            continue
+        penalty = params.dry_multiplier * params.dry_base ** (length - params.dry_allowed_length)
+        penalties[continuation] = max(penalties.get(continuation, 0.0), penalty)
+    return penalties
+
+
+class MirostatState:
+    """Mirostat v2: keeps tokens whose surprise -ln p is at most a moving bound, the most likely
+    token alone if none is; after the draw the bound moves against the error between the drawn
+    token's surprise, measured on the unfiltered distribution, and the target.  The bound starts
+    at twice the target and never falls to zero (crates/leone/src/sampler.rs:130-146, 398-446)."""
+
+    def __init__(self, target_surprise: float, learning_rate: float, maximum_surprise: Optional[float] = None):
+        self.target_surprise = float(target_surprise)
+        self.learning_rate = float(learning_rate)
+        self.maximum_surprise = 2.0 * self.target_surprise if maximum_surprise is None else float(maximum_surprise)
+        if not math.isfinite(self.maximum_surprise) or self.maximum_surprise <= 0.0:
+            raise SamplerError("the Mirostat state must be finite and greater than zero")
+
+    def select(self, probabilities: np.ndarray, u: float) -> int:
+        positive = probabilities > 0.0
+        if not positive.any():
+            raise SamplerError("no finite logit")
+        surprise = np.full(probabilities.shape, np.inf)
+        surprise[positive] = -np.log(probabilities[positive])
+        kept = np.where(surprise <= self.maximum_surprise, probabilities, 0.0)
+        total = kept.sum()
+        if total == 0.0:
+            best = int(np.argmax(probabilities))        # the first of equal maxima, as a strict > scan
+            kept[best] = probabilities[best]
+            total = kept[best]
+        token = select(kept / total, u)
+        observed = -math.log(float(probabilities[token]))
+        self.maximum_surprise -= self.learning_rate * (observed - self.target_surprise)
+        self.maximum_surprise = max(self.maximum_surprise, float(np.finfo(np.float64).eps))
+        return token
 
 
 def argmax(logits: np.ndarray) -> int:
@@ -229,9 +325,12 @@ def select(probabilities: np.ndarray, u: float) -> int:
     return int(eligible[hit[0]] if hit.size else eligible[-1])
 
 
-def sample(logits: np.ndarray, params: SamplingParams, position: int, history: Sequence[int] = ()) -> int:
+def sample(logits: np.ndarray, params: SamplingParams, position: int, history: Sequence[int] = (),
+           mirostat: Optional[MirostatState] = None) -> int:
     """One token for one row.  ``position`` is the absolute index of the token whose logits these are."""
     logits = apply_penalties(np.asarray(logits, dtype=np.float32), history, params)
+    if mirostat is not None:
+        return mirostat.select(distribution(logits, params), rng.uniform(params.seed, position))
     if params.greedy:
         params.validate()
         best = argmax(logits)

@@ -82,3 +82,45 @@ def select(probs, u):
         if u < running:
             return i
     return last
+
+
+def dry(logits, history, multiplier, base, allowed, window, breakers=()):
+    """The repeated-suffix penalty, by comparing suffixes outright: for every earlier position
+    holding the last token, the longest common run ending there and at the end, cut where a
+    breaker would be crossed; a run of at least ``allowed`` costs multiplier * base^(run - allowed)
+    on the token after the earlier position (crates/leone/src/penalty.rs:198-249)."""
+    out = [float(v) for v in logits]
+    recent = list(history)[-window:] if window > 0 else []
+    if multiplier <= 0 or len(recent) < 2:
+        return out
+    end = len(recent) - 1
+    best = {}
+    for at in range(end):
+        run = 0
+        while run <= at and recent[at - run] == recent[end - run] and (run == 0 or recent[end - run] not in breakers):
+            run += 1
+        if run == 0 or run < allowed:
+            continue
+        follower = recent[at + 1]
+        if follower in breakers:
+            continue
+        cost = multiplier
+        for _ in range(run - allowed):
+            cost *= base
+        best[follower] = max(best.get(follower, 0.0), cost)
+    for token, cost in best.items():
+        if token < len(out):
+            out[token] -= cost
+    return out
+
+
+def mirostat(probs, bound, target, rate, u):
+    """One Mirostat v2 draw: (token, new bound) (crates/leone/src/sampler.rs:398-446)."""
+    kept = [p if p > 0.0 and -math.log(p) <= bound else 0.0 for p in probs]
+    if sum(kept) == 0.0:
+        top = max(range(len(probs)), key=lambda i: (probs[i], -i))
+        kept[top] = probs[top]
+    total = math.fsum(kept)
+    token = select([p / total for p in kept], u)
+    bound = bound - rate * (-math.log(probs[token]) - target)
+    return token, max(bound, 2.0 ** -52)

@@ -90,6 +90,30 @@ def test_temperature_sampling_matches_oracle_and_ignores_batching(folders):
     assert top1 == greedy
 
 
+def test_mirostat_and_dry_generation_matches_oracle(folders):
+    """The controller's bound and the repeated-suffix penalty follow a request through portions and a batch."""
+    from leone_amd.api import Runtime, sampling_params
+    from leone_amd.engine.scheduler import SchedulerPolicy
+    folder = folders["A"]
+    weights, config = read_weights(folder), read_config(folder)
+    # a prompt that repeats itself, so that the penalty has something to act on
+    prompts = [random_tokens(60, 9, config["vocab_size"]) * 3, random_tokens(61, 21, config["vocab_size"])]
+    params = sampling_params(temperature=1.1, seed=77, mirostat=(2.5, 0.4), dry_multiplier=0.8, dry_base=1.5,
+                             dry_allowed_length=2, dry_window=32)
+    runtime = Runtime.load(folder, "float32", max_tokens=256, page_tokens=16, max_requests=2,
+                           policy=SchedulerPolicy(max_live_requests=2, prefill_chunk_tokens=8))
+    results = runtime.generate_tokens(prompts, 16, params, eos_token_id=None)
+    for prompt, result in zip(prompts, results):
+        tokens, bound = list(prompt), 5.0
+        for _ in range(16):
+            logits = qwen3_plain.forward(weights, config, tokens)[-1].float().tolist()
+            logits = np.array(sampler_plain.dry(logits, tokens, 0.8, 1.5, 2, 32), dtype=np.float32).tolist()
+            probs = sampler_plain.distribution(logits, 1.1)
+            token, bound = sampler_plain.mirostat(probs, bound, 2.5, 0.4, sampler_plain.uniform(77, len(tokens) - 1))
+            tokens.append(token)
+        assert result.tokens == tokens[len(prompt):]
+
+
 def test_eos_stops_generation(folders):
     from leone_amd.api import Runtime
     folder = folders["A"]

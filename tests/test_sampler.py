@@ -94,3 +94,69 @@ def test_penalties():
     assert out.tolist() == [2.0 / 2 - 0.25 - 0.5, -2.0 * 2 - 0.25 - 1.0, 1.0, 0.5]
     assert apply_penalties(logits, [0, 1], SamplingParams()) is logits
     assert not SamplingParams(repeat_penalty=2.0, penalty_window=0).penalties_active
+
+
+def _dry_params(**kw):
+    base = dict(dry_multiplier=1.0, dry_base=2.0, dry_allowed_length=2, dry_window=64)
+    base.update(kw)
+    return SamplingParams(**base)
+
+
+def test_dry_reference_vectors():
+    # crates/leone/src/penalty.rs:440-505: the expected values of the reference's own tests.
+    zeros = np.zeros(8, dtype=np.float32)
+    out = apply_penalties(zeros, [1, 2, 3, 4, 9, 1, 2, 3], _dry_params())
+    assert out[4] == -2.0 and np.count_nonzero(out) == 1
+    out = apply_penalties(zeros, [7, 1, 2, 3, 4, 9, 7, 1, 2, 3], _dry_params())
+    assert out[4] == -4.0
+    out = apply_penalties(zeros, [1, 2, 3, 4, 9, 1, 2, 3], _dry_params(dry_allowed_length=4))
+    assert not out.any()
+    out = apply_penalties(zeros, [1, 9, 2, 3, 5, 1, 9, 2], _dry_params(dry_breakers=(9,)))
+    assert not out.any()
+    with pytest.raises(SamplerError):
+        _dry_params(dry_base=0.0).validate()
+
+
+def test_dry_against_slow_oracle():
+    gen = np.random.default_rng(11)
+    for _ in range(400):
+        vocab = int(gen.integers(1, 12))
+        history = gen.integers(0, vocab, size=int(gen.integers(1, 40))).tolist()
+        logits = gen.uniform(-8, 8, size=vocab).astype(np.float32)
+        breakers = (int(gen.integers(0, vocab)),) if gen.random() < 0.3 else ()
+        params = _dry_params(dry_multiplier=float(gen.uniform(0.1, 2)), dry_base=float(gen.uniform(1, 3)),
+                             dry_allowed_length=int(gen.integers(1, 5)), dry_window=int(gen.integers(1, 48)),
+                             dry_breakers=breakers)
+        want = oracle.dry(logits, history, params.dry_multiplier, params.dry_base, params.dry_allowed_length,
+                         params.dry_window, breakers)
+        got = apply_penalties(logits, history, params)
+        np.testing.assert_allclose(got, np.array(want, dtype=np.float32), rtol=1e-6, atol=1e-6)
+
+
+def test_mirostat_controller():
+    from leone_amd.sampling.sampler import MirostatState
+    probs = np.array([0.5, 0.25, 0.125, 0.125, 0.0])
+    # A generous bound keeps everything: the draw is the plain one and the bound moves by the error.
+    state = MirostatState(1.0, 0.5, maximum_surprise=10.0)
+    assert state.select(probs, 0.6) == 1
+    assert state.maximum_surprise == pytest.approx(10.0 - 0.5 * (-np.log(0.25) - 1.0))
+    # A bound below every surprise leaves the most likely token alone, whatever the draw.
+    state = MirostatState(1.0, 1.0, maximum_surprise=0.1)
+    assert state.select(probs, 0.99) == 0
+    # The bound cuts the tail: with ln 4 < bound < ln 8 the two rarest tokens are gone and the rest renormalised.
+    state = MirostatState(3.0, 0.1, maximum_surprise=1.5)
+    assert state.select(probs, 0.7) == 1          # cumulative 2/3, 1 over {0.5, 0.25} / 0.75
+    assert MirostatState(2.0, 0.1).maximum_surprise == 4.0
+    with pytest.raises(SamplerError):
+        SamplingParams(temperature=1.0, mirostat=(0.0, 0.1)).validate()
+    with pytest.raises(SamplerError):
+        SamplingParams(temperature=1.0, mirostat=(1.0, 1.5)).validate()
+    # Against the loop oracle over a run of draws.
+    gen = np.random.default_rng(5)
+    state, bound = MirostatState(2.0, 0.3), 4.0
+    for step in range(200):
+        p = gen.dirichlet(np.full(9, 0.3))
+        u = float(gen.random())
+        token, bound = oracle.mirostat(p.tolist(), bound, 2.0, 0.3, u)
+        assert state.select(p, u) == token
+        assert state.maximum_surprise == pytest.approx(bound, rel=1e-12)
