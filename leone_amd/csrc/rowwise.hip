@@ -128,17 +128,28 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, cons
 // ---- SwiGLU -------------------------------------------------------------------
 // in: [rows, 2F]; every block of 16 columns holds 8 gate values, then the 8 up values that belong to
 // them (the order in which the fused gate/up weight keeps its rows).
+// A thread takes one block of 16 columns: two loads of 8 values, one store of 8 results.
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long rows, int ffn) {
-    const long total = rows * ffn;
-    for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < total;
-         i += static_cast<long>(gridDim.x) * blockDim.x) {
-        const long r = i / ffn;
-        const int c = static_cast<int>(i - r * ffn);
-        const long at = r * 2 * ffn + 16 * (c >> 3) + (c & 7);
-        const float g = to_float(gate_up[at]);
-        const float u = to_float(gate_up[at + 8]);
-        out[i] = from_float<T>((g / (1.0f + expf(-g))) * u);
+struct alignas(8 * sizeof(T)) Run8 {
+    T v[8];
+};
+template <typename T>
+__global__ void __launch_bounds__(256)
+swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long rows, int ffn) {
+    const int groups = ffn / 8;
+    const int group = blockIdx.x * blockDim.x + threadIdx.x;
+    if (group >= groups) return;
+    for (long r = blockIdx.y; r < rows; r += gridDim.y) {
+        const T* in = gate_up + r * 2 * ffn + 16 * static_cast<long>(group);
+        const Run8<T> gate = *reinterpret_cast<const Run8<T>*>(in);
+        const Run8<T> up = *reinterpret_cast<const Run8<T>*>(in + 8);
+        Run8<T> y;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float g = to_float(gate.v[i]);
+            y.v[i] = from_float<T>((g / (1.0f + expf(-g))) * to_float(up.v[i]));
+        }
+        *reinterpret_cast<Run8<T>*>(out + r * ffn + 8 * static_cast<long>(group)) = y;
     }
 }
 
@@ -346,13 +357,14 @@ extern "C" int leone_swiglu(const void* gate_up, void* out, int dtype, int rows,
     if (check_dtype(dtype, "swiglu")) return 1;
     LEONE_REQUIRE(gate_up && out, "swiglu: null pointer");
     LEONE_REQUIRE(rows > 0 && ffn > 0 && ffn % 8 == 0, "swiglu: rows %d, width %d: the width must be a positive multiple of 8", rows, ffn);
-    const long total = static_cast<long>(rows) * ffn;
-    long blocks = (total + 255) / 256;
-    if (blocks > 16384) blocks = 16384;
+    const uintptr_t run = 8 * (dtype == kF32 ? sizeof(float) : sizeof(bf16_t));
+    LEONE_REQUIRE(reinterpret_cast<uintptr_t>(gate_up) % run == 0 && reinterpret_cast<uintptr_t>(out) % run == 0,
+                  "swiglu: input and output must be aligned to %d bytes", static_cast<int>(run));
+    const dim3 grid(ceil_div(ffn / 8, 256), rows < 32768 ? rows : 32768);
     if (dtype == kF32)
-        swiglu_kernel<float><<<static_cast<int>(blocks), 256, 0, stream>>>(static_cast<const float*>(gate_up), static_cast<float*>(out), rows, ffn);
+        swiglu_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(gate_up), static_cast<float*>(out), rows, ffn);
     else
-        swiglu_kernel<bf16_t><<<static_cast<int>(blocks), 256, 0, stream>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out), rows, ffn);
+        swiglu_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out), rows, ffn);
     LEONE_LAUNCH_CHECK("swiglu");
     return 0;
 }

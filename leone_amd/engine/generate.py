@@ -55,12 +55,13 @@ class RequestRejected(ValueError):
 
 
 def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params: Dict[Hashable, SamplingParams],
-                  histories: Dict[Hashable, Sequence[int]],
+                  history: Callable[[Hashable], Sequence[int]],
                   controllers: Optional[Dict[Hashable, MirostatState]] = None) -> Dict[Hashable, int]:
     """One token per sampled entry; ``logits`` has one row per such entry, in order.
 
     Greedy and plain-temperature rows are chosen by the device kernels; rows with truncation stages
-    or penalties are copied to the host and go through the double-precision sampler."""
+    or penalties are copied to the host and go through the double-precision sampler, which reads a
+    request's tokens so far through ``history``."""
     rows = [e for e in entries if e.sample]
     if not rows:
         return {}
@@ -89,7 +90,7 @@ def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params:
         copied = logits.index_select(0, index).cpu().numpy()
         for k, i in enumerate(host_rows):
             e = rows[i]
-            out[e.request] = host_sample(copied[k], policies[i], e.sample_position, histories[e.request],
+            out[e.request] = host_sample(copied[k], policies[i], e.sample_position, history(e.request),
                                          (controllers or {}).get(e.request))
     for e in rows:
         if out[e.request] < 0:
@@ -137,8 +138,7 @@ class Generator:
         try:
             entries = [StepEntry(e.request, e.tokens, [len(e.tokens) - 1] if e.sample else []) for e in plan]
             output = self.engine.run_reserved(entries)
-            histories = {e.request: scheduler.live[e.request].tokens for e in plan if e.sample}
-            sampled = choose_tokens(output.logits, plan, self.params, histories, self.controllers) if output.logits is not None else {}
+            sampled = choose_tokens(output.logits, plan, self.params, scheduler.history, self.controllers) if output.logits is not None else {}
             if self.logit_observer is not None and output.logits is not None:
                 for row, e in enumerate([e for e in plan if e.sample]):
                     self.logit_observer(e.request, e.sample_position, output.logits[row])

@@ -37,13 +37,17 @@ class SwiGluMlp(Part):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         # One product for gate and up: 8 gate rows, their 8 up rows, and so on (a pure re-layout), which
-        # lets the activation be applied where the product is finished.
-        if self.intermediate % 8:
-            raise ValueError(f"the fused gate/up product needs an intermediate size that is a multiple of 8, "
-                             f"found {self.intermediate}")
-        self.w_gate_up = ops.interleave_gate_up(tensors.pop(self.names["gate"]),
-                                                tensors.pop(self.names["up"])).contiguous()
-        self.w_down = tensors.pop(self.names["down"]).contiguous()
+        # lets the activation be applied where the product is finished.  An intermediate size that is no
+        # multiple of 8 is filled up with zero rows; they give silu(0) * 0 = 0 and meet zero columns of
+        # the down projection, so the result is unchanged.
+        gate, up, down = (tensors.pop(self.names[k]) for k in ("gate", "up", "down"))
+        pad = -self.intermediate % 8
+        if pad:
+            gate = torch.nn.functional.pad(gate, (0, 0, 0, pad))
+            up = torch.nn.functional.pad(up, (0, 0, 0, pad))
+            down = torch.nn.functional.pad(down, (0, pad))
+        self.w_gate_up = ops.interleave_gate_up(gate, up).contiguous()
+        self.w_down = down.contiguous()
 
     def forward(self, y, step: StepContext, residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned)."""

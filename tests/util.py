@@ -22,9 +22,10 @@ TINY_C = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden
 TINY_M = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, hidden_size=512,
               num_attention_heads=8, num_key_value_heads=2, head_dim=128, intermediate_size=1408, vocab_size=3001,
               max_position_embeddings=1024, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False)
-# A width that is no multiple of 8, so that no product can take the 16-byte-run kernels.
+# A width that is no multiple of 8, so that no product can take the 16-byte-run kernels, and an
+# intermediate size that the fused gate/up layout has to fill up.
 TINY_D = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, hidden_size=100,
-              num_attention_heads=2, num_key_value_heads=1, head_dim=16, intermediate_size=72, vocab_size=333,
+              num_attention_heads=2, num_key_value_heads=1, head_dim=16, intermediate_size=75, vocab_size=333,
               max_position_embeddings=128, rope_theta=20000.0, rms_norm_eps=2e-6, tie_word_embeddings=True)
 TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "M": TINY_M, "D": TINY_D}
 
