@@ -30,6 +30,7 @@ fixed-size pages:
 from __future__ import annotations
 
 import ctypes
+import re
 from ctypes import c_int, c_int64
 from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional
@@ -85,6 +86,13 @@ class RequestKeys:
     def name(self, key: int) -> Hashable:
         return self._name[key]
 
+    def named(self, message: str) -> str:
+        """A message of the native side with its request keys turned back into names."""
+        def swap(match):
+            key = int(match.group(1))
+            return f"request {self._name[key]!r}" if key in self._name else match.group(0)
+        return re.sub(r"request (\d+)", swap, message)
+
     def pin(self, name: Hashable) -> int:
         key = self.key(name, create=True)
         self._pinned.add(name)
@@ -131,7 +139,7 @@ class CacheManager:
 
     # ---- errors ---------------------------------------------------------------
     def _raise(self, code: int):
-        message = hostlib.last_error()
+        message = self.keys.named(hostlib.last_error())
         if code == hostlib.OUT_OF_PAGES:
             group, needed, free = c_int(), c_int(), c_int()
             self._lib.leone_cache_shortage(ctypes.byref(group), ctypes.byref(needed), ctypes.byref(free))

@@ -1,20 +1,29 @@
 // Causal attention of prompt portions over the paged cache on the matrix cores, bfloat16.
 //
-// A portion's rows are cut into tiles of 32 consecutive rows (the host lists them: entry, first
-// row, row count); a wave takes one tile and one query head, its rows as two 16-column operands;
-// a workgroup is one to four such waves.  A wave walks the 32-key tiles its rows can see, from the cache, and
-// keeps the running maximum, sum and accumulator of the reference's recurrence
+// A portion's rows are cut into tiles of 32 consecutive rows; a wave takes one tile and one query
+// head, its rows as two 16-column operands.  A workgroup is four waves whose tiles belong to the
+// same request (the host lists them: entry, first row, row count, four to a workgroup).  The
+// workgroup walks the keys its tiles can see once, 64 at a time: all threads copy the next 64
+// keys and values from the cache to shared memory while the waves work on the present 64, and
+// every wave takes from shared memory the 32-key halves its own rows can see.  A wave keeps the
+// running reference, sum and accumulator of the reference's recurrence
 // (crates/leone/src/cpu.rs:2359-2421) per query in registers; nothing of size rows x keys is ever
 // stored (the reference's prefill materialises the scores, crates/leone-cuda/cuda/ie_cuda.cu:5124-5220).
-// Products and operand layouts are those of the decode kernel: S^T = K . Q^T and O^T += V^T . P^T with
-// v_mfma_f32_16x16x32_bf16, keys and values read as 16-byte runs of the packed cache layout, a tile of
-// keys and values loaded once for both column operands.  Waves do not share data, so no barrier is
-// needed; the four waves of a workgroup read the same keys, which the caches serve.
+// Products and operand layouts are those of the decode kernel: S^T = K . Q^T and O^T += V^T . P^T
+// with v_mfma_f32_16x16x32_bf16 on 16-byte runs of the packed cache layout.  Keys are stored in
+// shared memory in the order the first product's operand wants them, so that neighbouring lanes
+// read neighbouring runs.
+//
+// The recurrence is kept in base-2 units: t = score * scale * log2(e), p = 2^(t - m).  m is a
+// reference, not always the maximum: it is raised (and sums and accumulators rescaled) only when
+// a score exceeds it by more than 8, so that in the common case a pass needs no exchange between
+// lanes; p stays below 2^8 and the quotient of accumulator and sum does not depend on m.  The sum
+// of a query's p is one more row of the second product (a row of ones in V^T), so that numerator
+// and denominator are sums of the same rounded values.
 #include "common.h"
 #include "leone_hip.h"
 
 #include <math.h>
-#include <type_traits>
 
 namespace leone {
 
@@ -25,64 +34,95 @@ constexpr int kPrefillWaves = 4;
 constexpr int kPrefillThreads = kPrefillWaves * kWave;
 constexpr int kColsPerWave = 2;                                  // 16-query operands a wave carries
 constexpr int kRowsPerWave = 16 * kColsPerWave;                  // rows of a tile
-constexpr int kKeysPerTile = 32;
+constexpr int kStageKeys = 64;                                   // keys copied to shared memory at a time
+constexpr int kKeysPerPass = 32;                                 // keys of one pass of a wave
+constexpr float kRaise = 8.0f;                                   // a score this far above the reference raises it
 
-__device__ inline bf16x8 pf_load8(const bf16_t* p) {
-    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
-}
-__device__ inline bf16x8 pf_zero8() {
-    uint4 z = {0u, 0u, 0u, 0u};
-    return __builtin_bit_cast(bf16x8, z);
-}
+__device__ inline bf16x8 pf_bits(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
 
-// tiles: [n_tiles][3] = (entry, first row of the tile in the step, rows in the tile), at most 32 rows a
-// tile.  Wave w of workgroup b takes tile b * waves + w; waves share nothing but the launch, so tiles of
-// different requests may sit in one workgroup.
+// Runs of 16 bytes one stage holds: keys [head_dim / 8][64], values [8][head_dim].
+__host__ __device__ constexpr int stage_runs(int head_dim) { return (head_dim / 8) * kStageKeys + 8 * head_dim; }
+
+// tiles: [n_groups][4][3] = (entry, first row of the tile in the step, rows in the tile); a tile has at
+// most 32 rows, 0 rows marks an unused place; the tiles of a group belong to one entry.
 template <int kD16>
 __global__ void __launch_bounds__(kPrefillThreads, 2)
 attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_pool,
                          const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
-                         const int* __restrict__ tiles, int n_tiles, const int* __restrict__ block_table,
+                         const int* __restrict__ tiles, int n_groups, const int* __restrict__ block_table,
                          int max_blocks, int q_heads, int kv_heads, int page_shift, float scale, int window) {
     constexpr int kD = kD16 * 16;
-    constexpr int kSteps = (kD16 + 1) / 2;
+    constexpr int kRuns = kD / 8;                      // 16-byte runs of one key
+    constexpr int kSteps = (kD16 + 1) / 2;             // 32-element steps of the first product
+    constexpr int kKeyRuns = kRuns * kStageKeys;       // runs of the keys of one stage; the values take as many
+    constexpr int kStageRuns = stage_runs(kD);
+    constexpr int kCopies = (kKeyRuns + kPrefillThreads - 1) / kPrefillThreads;   // runs a thread copies, keys and values each
+
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int lane = threadIdx.x % kWave;
-    const int tile = blockIdx.x * (blockDim.x / kWave) + wave;
-    const bool has_tile = tile < n_tiles;
-    const int entry = has_tile ? tiles[3 * tile] : 0;
-    const int tile_row0 = has_tile ? tiles[3 * tile + 1] : 0;
-    const int wave_rows = has_tile ? tiles[3 * tile + 2] : 0;
-    const int head = blockIdx.y;
-    const int kvh = head / (q_heads / kv_heads);
+    const int tid = threadIdx.x;
     const int c = lane & 15, g = lane >> 4;
-    const int page_tokens = 1 << page_shift, page_mask = page_tokens - 1;
-    const int wave_row0 = 0;
-    const int* table = block_table + static_cast<long>(entry) * max_blocks;
 
-    // The page ids of the keys a wave reads go to its part of shared memory first, so that no load of
-    // keys or values waits on a read of the block table.
-    extern __shared__ int all_pages[];
-    int* pages = all_pages + wave * max_blocks;
-    int first_page = 0;
-    if (has_tile) {
-        const int tile_p0 = positions[tile_row0];
-        const int tile_lo = (window > 0 && tile_p0 - window + 1 > 0) ? tile_p0 - window + 1 : 0;
-        first_page = tile_lo >> page_shift;
-        const int n_pages = ((tile_p0 + wave_rows - 1) >> page_shift) - first_page + 1;
-        for (int i = lane; i < n_pages; i += kWave) pages[i] = table[first_page + i];
+    // Workgroups go round the chip's eight dies in turn, each die has a cache of its own, and a compute
+    // unit holds two workgroups.  Work is numbered with a key/value head's query heads and tile groups
+    // together; a die gets a run of neighbouring numbers (few key/value heads, whose keys its cache then
+    // keeps), and within a die the second half of the workgroups takes the groups in falling order, so
+    // that a compute unit tends to hold a group that sees few keys beside one that sees many.
+    constexpr int kDies = 8;
+    const int launched = gridDim.x;
+    int head, group;
+    if (launched % (2 * kDies) == 0 && n_groups % 2 == 0) {
+        const int per_die = launched / kDies, spot = blockIdx.x / kDies;
+        const int heads_here = per_die / n_groups;                     // per_die = heads_here * n_groups
+        const int late = spot / (per_die / 2), r = spot % (per_die / 2);
+        const int pair = r / heads_here;
+        head = (blockIdx.x % kDies) * heads_here + r % heads_here;
+        group = late ? n_groups - 1 - pair : pair;
+    } else {
+        head = blockIdx.x / n_groups;
+        group = blockIdx.x % n_groups;
     }
-    __syncthreads();
-    if (!has_tile) return;                                     // after the workgroup's only barrier
+    const int kvh = head / (q_heads / kv_heads);
+    const int page_tokens = 1 << page_shift, page_mask = page_tokens - 1;
 
-    // Rows of a portion are consecutive positions: row r of the wave sits at p0 + r.
-    const int p0 = positions[tile_row0 + wave_row0];
+    extern __shared__ uint4 shared[];
+    int* pages = reinterpret_cast<int*>(shared + 2 * kStageRuns);
+    __shared__ int wave_lo[kPrefillWaves], wave_hi[kPrefillWaves];
+    __shared__ int unmapped_seen;
+
+    // This wave's tile.
+    const int* my_tile = tiles + 3 * (static_cast<long>(group) * kPrefillWaves + wave);
+    const int entry = tiles[3 * static_cast<long>(group) * kPrefillWaves];
+    const int tile_row0 = my_tile[1];
+    const int wave_rows = my_tile[2];
+    const int p0 = wave_rows > 0 ? positions[tile_row0] : 0;    // rows of a portion are consecutive positions
     const int p_last = p0 + wave_rows - 1;
-    const int key_hi = p_last + 1;                                              // keys the wave may read: [key_lo, key_hi)
+    const int key_hi = wave_rows > 0 ? p_last + 1 : 0;          // keys the wave may read: [key_lo, key_hi)
     const int key_lo = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
-    // A tile wholly inside [full_lo, full_hi) is visible to every row of the wave: no masks.
+    // A pass wholly inside [full_lo, full_hi) is visible to every row of the wave: no masks.
     const int full_hi = p0 + 1;
     const int full_lo = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+    if (lane == 0) {
+        wave_lo[wave] = wave_rows > 0 ? key_lo : 0x7fffffff;
+        wave_hi[wave] = key_hi;
+    }
+    if (tid == 0) unmapped_seen = 0;
+    __syncthreads();
+    int group_lo = 0x7fffffff, group_hi = 0;
+#pragma unroll
+    for (int w = 0; w < kPrefillWaves; ++w) {
+        group_lo = wave_lo[w] < group_lo ? wave_lo[w] : group_lo;
+        group_hi = wave_hi[w] > group_hi ? wave_hi[w] : group_hi;
+    }
+    if (group_hi <= group_lo) return;                            // a group without rows (every wave agrees)
+
+    // The page ids of the keys the group reads go to shared memory first, so that no load of keys or
+    // values waits on a read of the block table.
+    const int first_page = group_lo >> page_shift;
+    const int n_pages = ((group_hi - 1) >> page_shift) - first_page + 1;
+    const int* table = block_table + static_cast<long>(entry) * max_blocks;
+    for (int i = tid; i < n_pages; i += kPrefillThreads) pages[i] = table[first_page + i];
+    __syncthreads();
 
     // Q^T operands and each column's own position.
     bf16x8 qreg[kColsPerWave][kSteps];
@@ -92,84 +132,133 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         const int r = 16 * j + c;
         const bool ok = r < wave_rows;
         col_pos[j] = ok ? p0 + r : -1;                                          // -1: the column sees no key
-        const bf16_t* qrow = q + (static_cast<long>(tile_row0 + wave_row0 + (ok ? r : 0)) * q_heads + head) * kD;
+        const bf16_t* qrow = q + (static_cast<long>(tile_row0 + (ok ? r : 0)) * q_heads + head) * kD;
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) {
             const int d0 = 32 * s + 8 * g;
-            qreg[j][s] = (ok && d0 < kD) ? pf_load8(qrow + d0) : pf_zero8();
+            qreg[j][s] = (ok && d0 < kD) ? pf_bits(*reinterpret_cast<const uint4*>(qrow + d0)) : pf_bits(uint4{0u, 0u, 0u, 0u});
         }
     }
 
-    float m_run[kColsPerWave], l_run[kColsPerWave];
-    floatx4 acc[kColsPerWave][kD16];
+    // Per column: the reference m (base-2 units), the accumulator, and the sum of p as one more
+    // accumulator tile (every row of it holds the sum).
+    float m_ref[kColsPerWave];
+    floatx4 acc[kColsPerWave][kD16], acc_sum[kColsPerWave];
 #pragma unroll
     for (int j = 0; j < kColsPerWave; ++j) {
-        m_run[j] = -INFINITY;
-        l_run[j] = 0.f;
+        m_ref[j] = -INFINITY;
+        acc_sum[j] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int dt = 0; dt < kD16; ++dt) acc[j][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
-    bool unmapped = false;
+    const float to_log2 = scale * 1.44269504088896340736f;
+    const bf16x8 ones = pf_bits(uint4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
 
-    auto do_tile = [&](int t, auto full_tag) {
-        constexpr bool kFull = decltype(full_tag)::value;
-        const int key0 = t * kKeysPerTile;
-        const int ka = key0 + 8 * (c >> 2) + (c & 3);          // A-operand row c of half a; half b is four keys on
-        const int kb = ka + 4;
-        const int run0 = key0 + 8 * g;                         // the lane's eight keys in the second product
-        bool va = true, vb = true, any = true, whole = true;
-        if constexpr (!kFull) {
-            va = ka >= key_lo && ka < key_hi;
-            vb = kb >= key_lo && kb < key_hi;
-            any = run0 < key_hi && run0 + 8 > key_lo;
-            whole = run0 >= key_lo && run0 + 8 <= key_hi;
-        }
-        const bf16_t* pk = k_pool;
-        const bf16_t* pv = v_pool;
-        if (va || vb) {
-            const int page = pages[(ka >> page_shift) - first_page];
-            if (page < 0) {
-                unmapped = true;
-                va = vb = false;
-            }
-            pk = k_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (ka & page_mask) * 8;
-        }
-        if (any) {
-            const int page = pages[(run0 >> page_shift) - first_page];
-            if (page < 0) {
-                unmapped = true;
-                any = false;
-            }
-            pv = v_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD +
-                 static_cast<long>((run0 & page_mask) >> 3) * kD * 8;
-        }
-        bf16x8 xa[kSteps], xb[kSteps], xv[kD16];
+    // ---- copying a stage: keys [64 t, 64 t + 64) from the cache into registers, then into shared memory.
+    // Copy i of a thread is run `idx / 64` of key `idx % 64` and, of the values, element `idx % kD`
+    // of the eight keys from `8 (idx / kD)`, with idx = i * threads + tid.
+    const long page_elems = static_cast<long>(page_tokens) * kD;
+    const long head_elems = static_cast<long>(kvh) * page_elems;
+    const long pool_stride = static_cast<long>(kv_heads) * page_elems;
+    uint4 held_k[kCopies], held_v[kCopies];
+    // A stage that lies inside one page and inside the group's keys needs one page id and no masks:
+    // its loads are issued back to back.
+    auto fetch_plain = [&](int key_base, int page) {
+        const int in_page = key_base & page_mask;
+        const bf16_t* kp = k_pool + page * pool_stride + head_elems + static_cast<long>(in_page) * 8;
+        const bf16_t* vp = v_pool + page * pool_stride + head_elems + static_cast<long>(in_page >> 3) * kD * 8;
 #pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-            const bool in_head = 32 * s + 8 * g < kD;
-            const long run = static_cast<long>(4 * s + g) * page_tokens * 8;
-            xa[s] = (va && in_head) ? pf_load8(pk + run) : pf_zero8();
-            xb[s] = (vb && in_head) ? pf_load8(pk + run + 32) : pf_zero8();
+        for (int i = 0; i < kCopies; ++i) {
+            const int idx = i * kPrefillThreads + tid;
+            if (kKeyRuns % kPrefillThreads != 0 && idx >= kKeyRuns) continue;
+            held_k[i] = *reinterpret_cast<const uint4*>(kp + (static_cast<long>(idx / kStageKeys) * page_tokens + idx % kStageKeys) * 8);
+            held_v[i] = *reinterpret_cast<const uint4*>(vp + static_cast<long>(idx) * 8);   // (8 tg / 8 * kD + d) * 8 with idx = tg * kD + d
         }
+    };
+    auto fetch_any = [&](int key_base) {
 #pragma unroll
-        for (int dt = 0; dt < kD16; ++dt) {
-            xv[dt] = any ? pf_load8(pv + (16 * dt + c) * 8) : pf_zero8();
-            if constexpr (!kFull) {
-                if (any && !whole) {   // slots the wave may not read can hold anything: clear them
-                    uint4 raw = __builtin_bit_cast(uint4, xv[dt]);
-                    unsigned* w = reinterpret_cast<unsigned*>(&raw);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int e0 = run0 + 2 * i, e1 = e0 + 1;
-                        unsigned mask = 0u;
-                        if (e0 >= key_lo && e0 < key_hi) mask |= 0x0000ffffu;
-                        if (e1 >= key_lo && e1 < key_hi) mask |= 0xffff0000u;
-                        w[i] &= mask;
+        for (int i = 0; i < kCopies; ++i) {
+            const int idx = i * kPrefillThreads + tid;
+            held_k[i] = uint4{0u, 0u, 0u, 0u};
+            held_v[i] = uint4{0u, 0u, 0u, 0u};
+            if (kKeyRuns % kPrefillThreads != 0 && idx >= kKeyRuns) continue;
+            {
+                const int run = idx / kStageKeys, key = key_base + idx % kStageKeys;
+                if (key >= group_lo && key < group_hi) {
+                    const int page = pages[(key >> page_shift) - first_page];
+                    if (page < 0) {
+                        unmapped_seen = 1;
+                    } else {
+                        held_k[i] = *reinterpret_cast<const uint4*>(
+                            k_pool + page * pool_stride + head_elems + (static_cast<long>(run) * page_tokens + (key & page_mask)) * 8);
                     }
-                    xv[dt] = __builtin_bit_cast(bf16x8, raw);
+                }
+            }
+            {
+                const int tg = idx / kD, d = idx % kD, key = key_base + 8 * tg;
+                if (key < group_hi && key + 8 > group_lo) {
+                    const int page = pages[(key >> page_shift) - first_page];
+                    if (page < 0) {
+                        unmapped_seen = 1;
+                    } else {
+                        uint4 raw = *reinterpret_cast<const uint4*>(
+                            v_pool + page * pool_stride + head_elems + (static_cast<long>((key & page_mask) >> 3) * kD + d) * 8);
+                        if (key < group_lo || key + 8 > group_hi) {   // slots outside the range can hold anything: clear them
+                            unsigned* w = reinterpret_cast<unsigned*>(&raw);
+#pragma unroll
+                            for (int h = 0; h < 4; ++h) {
+                                const int e0 = key + 2 * h, e1 = e0 + 1;
+                                unsigned mask = 0u;
+                                if (e0 >= group_lo && e0 < group_hi) mask |= 0x0000ffffu;
+                                if (e1 >= group_lo && e1 < group_hi) mask |= 0xffff0000u;
+                                w[h] &= mask;
+                            }
+                        }
+                        held_v[i] = raw;
+                    }
                 }
             }
         }
+    };
+    auto fetch = [&](int t) {
+        const int key_base = t * kStageKeys;
+        if (page_shift >= 6 && key_base >= group_lo && key_base + kStageKeys <= group_hi) {
+            const int page = __builtin_amdgcn_readfirstlane(pages[(key_base >> page_shift) - first_page]);
+            if (page >= 0) {
+                fetch_plain(key_base, page);
+                return;
+            }
+        }
+        fetch_any(key_base);
+    };
+    auto deposit = [&](uint4* to) {
+#pragma unroll
+        for (int i = 0; i < kCopies; ++i) {
+            const int idx = i * kPrefillThreads + tid;
+            if (kKeyRuns % kPrefillThreads != 0 && idx >= kKeyRuns) continue;
+            // Key kk of a 32-key half sits where the first product's operand row reads it: rows 0..15 are
+            // keys 8 (r / 4) + r % 4, rows 16..31 the keys four further on.
+            const int run = idx / kStageKeys, kl = idx % kStageKeys;
+            const int half = kl >> 5, kk = kl & 31;
+            const int place = ((kk >> 2) & 1) * 16 + 4 * (kk >> 3) + (kk & 3);
+            to[(half * kRuns + run) * 32 + place] = held_k[i];
+            to[kKeyRuns + idx] = held_v[i];
+        }
+    };
+
+    // ---- one pass of a wave: 32 keys against its 32 rows
+    auto pass = [&](const uint4* from, int key0, int half, bool full) {
+        const int run0 = key0 + 8 * g;                         // the lane's eight keys in the second product
+        bf16x8 xa[kSteps], xb[kSteps];
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            const bool in_head = 4 * s + g < kRuns;
+            const uint4* row = from + (half * kRuns + 4 * s + g) * 32;
+            xa[s] = in_head ? pf_bits(row[c]) : pf_bits(uint4{0u, 0u, 0u, 0u});
+            xb[s] = in_head ? pf_bits(row[16 + c]) : pf_bits(uint4{0u, 0u, 0u, 0u});
+        }
+        float sc[kColsPerWave][8];
+        float top[kColsPerWave];
 #pragma unroll
         for (int j = 0; j < kColsPerWave; ++j) {
             floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
@@ -179,62 +268,89 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                 sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb[s], qreg[j][s], sb, 0, 0, 0);
             }
             // lane (g, c): scores of keys run0 .. run0+7 for the query of column c
-            const int p = col_pos[j];
-            const int p_lo = (window > 0) ? p - window + 1 : 0;
-            float sc[8];
-            float tile_max = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int key = run0 + i;
-                const float raw = i < 4 ? sa[i & 3] : sb[i & 3];
-                sc[i] = (kFull || (key <= p && key >= p_lo)) ? raw * scale : -INFINITY;
-                tile_max = fmaxf(tile_max, sc[i]);
-            }
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
-            const float m_new = fmaxf(m_run[j], tile_max);
-            const float m_safe = m_new == -INFINITY ? 0.f : m_new;   // a column that has seen no key yet
-            const float alpha = __expf(m_run[j] - m_safe);
-            float psum = 0.f;
-            bf16x8 pt;
+            for (int i = 0; i < 8; ++i) sc[j][i] = i < 4 ? sa[i & 3] : sb[i & 3];
+        }
+        if (!full) {                                           // the same for the whole wave
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float e = __expf(sc[i] - m_safe);
-                psum += e;
-                pt[i] = static_cast<__bf16>(e);
+            for (int j = 0; j < kColsPerWave; ++j) {
+                const int p = col_pos[j];
+                const int p_lo = (window > 0) ? p - window + 1 : 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int key = run0 + i;
+                    sc[j][i] = (key <= p && key >= p_lo) ? sc[j][i] : -INFINITY;
+                }
             }
-            psum += __shfl_xor(psum, 16, kWave);
-            psum += __shfl_xor(psum, 32, kWave);
-            l_run[j] = l_run[j] * alpha + psum;
-            m_run[j] = m_new;
-            if (__any(alpha != 1.0f)) {       // after the first tiles the running maximum seldom moves
+        }
+        bool raise = false;
+#pragma unroll
+        for (int j = 0; j < kColsPerWave; ++j) {
+            top[j] = fmaxf(fmaxf(fmaxf(sc[j][0], sc[j][1]), fmaxf(sc[j][2], sc[j][3])),
+                           fmaxf(fmaxf(sc[j][4], sc[j][5]), fmaxf(sc[j][6], sc[j][7]))) * to_log2;
+            raise = raise || top[j] > m_ref[j] + kRaise;       // -inf + 8 is -inf: the first scores always raise
+        }
+        if (__any(raise)) {
+            // Some score outgrew its reference: every column takes its true maximum so far as the new one.
+#pragma unroll
+            for (int j = 0; j < kColsPerWave; ++j) {
+                float col_top = fmaxf(top[j], __shfl_xor(top[j], 16, kWave));
+                col_top = fmaxf(col_top, __shfl_xor(col_top, 32, kWave));
+                const float m_new = fmaxf(m_ref[j], col_top);
+                const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_ref[j] - m_new);   // 2^-inf = 0
+                m_ref[j] = m_new;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc_sum[j][r] *= alpha;
 #pragma unroll
                 for (int dt = 0; dt < kD16; ++dt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) acc[j][dt][r] *= alpha;
             }
+        }
+        bf16x8 pt[kColsPerWave];
 #pragma unroll
-            for (int dt = 0; dt < kD16; ++dt)
-                acc[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[dt], pt, acc[j][dt], 0, 0, 0);
+        for (int j = 0; j < kColsPerWave; ++j) {
+            const float shift = m_ref[j] == -INFINITY ? 0.f : -m_ref[j];   // a column that has seen no key yet
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                pt[j][i] = static_cast<__bf16>(__builtin_amdgcn_exp2f(fmaf(sc[j][i], to_log2, shift)));
+            acc_sum[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pt[j], acc_sum[j], 0, 0, 0);
+        }
+#pragma unroll
+        for (int dt = 0; dt < kD16; ++dt) {
+            const bf16x8 xv = pf_bits(from[kKeyRuns + (4 * half + g) * kD + 16 * dt + c]);
+#pragma unroll
+            for (int j = 0; j < kColsPerWave; ++j)
+                acc[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv, pt[j], acc[j][dt], 0, 0, 0);
         }
     };
 
-    const int t_begin = key_lo / kKeysPerTile, t_end = (key_hi + kKeysPerTile - 1) / kKeysPerTile;
+    const int t_begin = group_lo / kStageKeys, t_end = (group_hi + kStageKeys - 1) / kStageKeys;
+    fetch(t_begin);
+    deposit(shared);
+    __syncthreads();
+    int cur = 0;
     for (int t = t_begin; t < t_end; ++t) {
-        const int key0 = t * kKeysPerTile;
-        if (key0 >= full_lo && key0 + kKeysPerTile <= full_hi)
-            do_tile(t, std::true_type{});
-        else
-            do_tile(t, std::false_type{});
+        const bool more = t + 1 < t_end;
+        if (more) fetch(t + 1);                                  // in flight while the waves work
+#pragma unroll
+        for (int half = 0; half < kStageKeys / kKeysPerPass; ++half) {
+            const int key0 = t * kStageKeys + half * kKeysPerPass;
+            if (key0 >= key_hi || key0 + kKeysPerPass <= key_lo) continue;      // nothing of it for this wave
+            pass(shared + cur * kStageRuns, key0, half, key0 >= full_lo && key0 + kKeysPerPass <= full_hi);
+        }
+        if (more) deposit(shared + (cur ^ 1) * kStageRuns);      // the other stage was last read before the barrier below
+        __syncthreads();
+        cur ^= 1;
     }
 
-    const bool poisoned = __any(unmapped);
+    const bool poisoned = unmapped_seen != 0;                    // every write to it came before the last barrier
 #pragma unroll
     for (int j = 0; j < kColsPerWave; ++j) {
         const int r = 16 * j + c;
         if (r >= wave_rows) continue;
-        const float inv = poisoned ? __builtin_nanf("") : 1.0f / l_run[j];
-        bf16_t* orow = out + (static_cast<long>(tile_row0 + wave_row0 + r) * q_heads + head) * kD;
+        const float inv = poisoned ? __builtin_nanf("") : 1.0f / acc_sum[j][0];
+        bf16_t* orow = out + (static_cast<long>(tile_row0 + r) * q_heads + head) * kD;
 #pragma unroll
         for (int dt = 0; dt < kD16; ++dt) {
             // lane (g, c) holds elements 16dt + 4g .. +3 of query column c
@@ -249,18 +365,25 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 }
 
 template <int kD16>
-static void launch_prefill(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
-                           const int* tiles, int n_tiles, const int* block_table, int max_blocks, int q_heads,
-                           int kv_heads, int page_shift, float scale, int window, hipStream_t stream) {
-    // Four tiles a workgroup when there are plenty (their waves read the same keys, which the caches
-    // then serve once), fewer when the chip would otherwise stay half empty.
-    const long wave_tiles = static_cast<long>(n_tiles) * q_heads;
-    const int waves = wave_tiles >= 2048 ? 4 : wave_tiles >= 1024 ? 2 : 1;
-    dim3 grid(ceil_div(n_tiles, waves), q_heads);
-    attention_prefill_kernel<kD16><<<grid, waves * kWave, static_cast<size_t>(waves) * max_blocks * sizeof(int), stream>>>(
+static int launch_prefill(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
+                          const int* tiles, int n_groups, const int* block_table, int max_blocks, int q_heads,
+                          int kv_heads, int page_shift, float scale, int window, hipStream_t stream) {
+    const size_t shared = 2 * static_cast<size_t>(stage_runs(16 * kD16)) * sizeof(uint4) + static_cast<size_t>(max_blocks) * sizeof(int);
+    static size_t allowed = 48 * 1024;                 // what a kernel may use without asking
+    if (shared > allowed) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<kD16>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shared));
+        if (e != hipSuccess) {
+            set_error("attention_prefill: %zu bytes of shared memory were refused: %s", shared, hipGetErrorString(e));
+            return 1;
+        }
+        allowed = shared;
+    }
+    attention_prefill_kernel<kD16><<<n_groups * q_heads, kPrefillThreads, shared, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_pool),
-        static_cast<const bf16_t*>(v_pool), positions, tiles, n_tiles, block_table, max_blocks, q_heads, kv_heads,
+        static_cast<const bf16_t*>(v_pool), positions, tiles, n_groups, block_table, max_blocks, q_heads, kv_heads,
         page_shift, scale, window);
+    return 0;
 }
 
 }  // namespace leone
@@ -268,28 +391,32 @@ static void launch_prefill(const void* q, void* out, const void* k_pool, const v
 using namespace leone;
 
 extern "C" int leone_attention_prefill_tile_rows() { return kRowsPerWave; }
+extern "C" int leone_attention_prefill_group_tiles() { return kPrefillWaves; }
 
+// tiles holds n_groups * leone_attention_prefill_group_tiles() entries of (entry, first row, rows).
 extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_pool, const void* v_pool,
-                                       const int* positions, const int* tiles, int n_tiles, const int* block_table,
+                                       const int* positions, const int* tiles, int n_groups, const int* block_table,
                                        int max_blocks, int q_heads, int kv_heads, int head_dim, int page_tokens,
                                        float scale, int window, hipStream_t stream) {
     LEONE_REQUIRE(q && out && k_pool && v_pool && positions && tiles && block_table, "attention_prefill: null pointer");
-    LEONE_REQUIRE(n_tiles > 0 && q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
-                  "attention_prefill: %d tiles, %d query heads over %d kv heads", n_tiles, q_heads, kv_heads);
-    LEONE_REQUIRE(q_heads <= 65535, "attention_prefill: at most 65535 query heads");
+    LEONE_REQUIRE(n_groups > 0 && q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
+                  "attention_prefill: %d tile groups, %d query heads over %d kv heads", n_groups, q_heads, kv_heads);
+    LEONE_REQUIRE(static_cast<long>(n_groups) * q_heads <= 0x7fffffffL, "attention_prefill: too many tile groups");
     LEONE_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 128,
                   "attention_prefill: head_dim %d must be a multiple of 16 in 16..128", head_dim);
     LEONE_REQUIRE(page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0,
                   "attention_prefill: page_tokens %d must be a power of two, at least 16", page_tokens);
     LEONE_REQUIRE(window >= 0 && max_blocks > 0, "attention_prefill: bad window or block table");
-    LEONE_REQUIRE(static_cast<size_t>(kPrefillWaves) * max_blocks * sizeof(int) <= 64 * 1024,
+    LEONE_REQUIRE(scale > 0.f, "attention_prefill: the score scale must be positive");
+    LEONE_REQUIRE(static_cast<size_t>(max_blocks) * sizeof(int) <= 16 * 1024,
                   "attention_prefill: a block table of %d entries does not fit shared memory", max_blocks);
     int page_shift = 0;
     while ((1 << page_shift) < page_tokens) ++page_shift;
-#define LEONE_PREFILL_CASE(N)                                                                                     \
-    case N:                                                                                                       \
-        launch_prefill<N>(q, out, k_pool, v_pool, positions, tiles, n_tiles, block_table, max_blocks, q_heads,    \
-                          kv_heads, page_shift, scale, window, stream);                                           \
+    int status = 0;
+#define LEONE_PREFILL_CASE(N)                                                                                      \
+    case N:                                                                                                        \
+        status = launch_prefill<N>(q, out, k_pool, v_pool, positions, tiles, n_groups, block_table, max_blocks,    \
+                                   q_heads, kv_heads, page_shift, scale, window, stream);                          \
         break;
     switch (head_dim / 16) {
         LEONE_PREFILL_CASE(1) LEONE_PREFILL_CASE(2) LEONE_PREFILL_CASE(3) LEONE_PREFILL_CASE(4)
@@ -299,6 +426,7 @@ extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_p
             return 1;
     }
 #undef LEONE_PREFILL_CASE
+    if (status) return status;
     LEONE_LAUNCH_CHECK("attention_prefill");
     return 0;
 }

@@ -311,8 +311,9 @@ long leone_step_pack(void* cache, int n_entries, const int64_t* requests, const 
             token_at += std::max(counts[i], 0);
             want_at += std::max(want_counts[i], 0);
         }
-        const StepShape step_shape{shape[0], shape[1], shape[2], shape[3] != 0};
-        if (step_shape.tile_rows <= 0) throw std::invalid_argument("step_pack: tile_rows must be positive");
+        const StepShape step_shape{shape[0], shape[1], shape[2], shape[3] != 0, shape[4]};
+        if (step_shape.tile_rows <= 0 || step_shape.group_tiles <= 0)
+            throw std::invalid_argument("step_pack: tile_rows and group_tiles must be positive");
         const StepSections layout = step_sections(manager, entries, step_shape);
         std::copy(layout.offsets.begin(), layout.offsets.end(), sections);
         if (!out || capacity < layout.total()) return layout.total();

@@ -81,7 +81,7 @@ void leone_scheduler_stats(void* scheduler, int64_t* out15);
 
 // ---- step layout.  Entries are given flat: request, token count and wanted count per entry, then
 // all tokens and all wanted places in entry order.  shape: vocab_size, tile_rows, min_tile_rows,
-// all_rows_wanted.  Returns the words the packed step takes; writes nothing but `sections`
+// all_rows_wanted, group_tiles.  Returns the words the packed step takes; writes nothing but `sections`
 // (7 + groups offsets) if `capacity` is smaller.  summary: rows, prefill_rows, max_position, tiles,
 // wanted, decode_only.  placed: per entry in running order given_index, slot, first_row, count, start.
 long leone_step_pack(void* cache, int n_entries, const int64_t* requests, const int* counts, const int* want_counts,

@@ -10,6 +10,12 @@ namespace {
 
 bool tiled(const StepEntryView& e, const StepShape& shape) { return !shape.all_rows_wanted && e.count >= shape.min_tile_rows; }
 
+// Places the tiles of a portion of `count` rows take: whole groups.
+long tile_places(int count, const StepShape& shape) {
+    const long tiles = (count + shape.tile_rows - 1) / shape.tile_rows;
+    return (tiles + shape.group_tiles - 1) / shape.group_tiles * shape.group_tiles;
+}
+
 void check(const std::vector<StepEntryView>& entries, const StepShape& shape) {
     if (entries.empty()) throw StepRefused("a step needs at least one entry");
     std::unordered_set<RequestKey> seen;
@@ -35,7 +41,7 @@ StepSections step_sections(const CacheManager& cache, const std::vector<StepEntr
     for (const StepEntryView& e : entries) {
         rows += e.count;
         wanted += e.want_count;
-        if (tiled(e, shape)) tiles += (e.count + shape.tile_rows - 1) / shape.tile_rows;
+        if (tiled(e, shape)) tiles += tile_places(e.count, shape);
     }
     if (shape.all_rows_wanted) wanted = rows;
     const long n = static_cast<long>(entries.size());
@@ -86,10 +92,14 @@ StepSummary pack_step(const CacheManager& cache, const std::vector<StepEntryView
             std::fill(dst + held, dst + width, -1);
         }
         if (tiled(e, shape)) {
-            for (int at = 0; at < e.count; at += shape.tile_rows) {
+            const int n_tiles = (e.count + shape.tile_rows - 1) / shape.tile_rows;
+            const long places = tile_places(e.count, shape);
+            for (long index = 0; index < places; ++index) {
+                const bool used = index < n_tiles;
+                const int at = static_cast<int>(index) * shape.tile_rows;
                 tiles[3 * tile] = ei;
-                tiles[3 * tile + 1] = row + at;
-                tiles[3 * tile + 2] = std::min(shape.tile_rows, e.count - at);
+                tiles[3 * tile + 1] = used ? row + at : row;
+                tiles[3 * tile + 2] = used ? std::min(shape.tile_rows, e.count - at) : 0;
                 ++tile;
             }
             summary.prefill_rows = row + e.count;

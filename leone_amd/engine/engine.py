@@ -44,12 +44,12 @@ class StepError(ValueError):
     """A step was refused before anything ran; the cache is unchanged."""
 
 
-class _PackedStep:
-    """One step's metadata as the native layout routine wrote it into a host buffer."""
+class PackedStep:
+    """One step's metadata as the native layout routine wrote it into a host buffer (int32 words):
+    tokens, positions, row -> entry, state slots, wanted rows, query tiles, one block table per cache group."""
 
-    def __init__(self, engine: "Engine", entries: Sequence[StepEntry], all_rows_wanted: bool,
+    def __init__(self, cache: CacheManager, vocab_size: int, entries: Sequence[StepEntry], all_rows_wanted: bool = False,
                  host: Optional[torch.Tensor] = None):
-        cache = engine.cache
         n = len(entries)
         lib = hostlib.library()
         requests = (c_int64 * max(1, n))()
@@ -70,11 +70,12 @@ class _PackedStep:
             raise StepError(f"tokens and wanted places must be integers: {error}") from None
         limit = np.iinfo(np.int32)
         if tokens.size and (tokens.min() < limit.min or tokens.max() > limit.max):
-            raise StepError(f"a token lies outside the vocabulary of {engine.vocab_size}")
+            raise StepError(f"a token lies outside the vocabulary of {vocab_size}")
         if wants.size and (wants.min() < limit.min or wants.max() > limit.max):
             raise StepError("a wanted place lies outside its entry")
         tokens, wants = tokens.astype(np.int32), wants.astype(np.int32)
-        shape = (c_int * 4)(engine.vocab_size, ops.PREFILL_TILE_ROWS, ops.PREFILL_MIN_ROWS, int(all_rows_wanted))
+        shape = (c_int * 5)(vocab_size, ops.PREFILL_TILE_ROWS, ops.PREFILL_MIN_ROWS, int(all_rows_wanted),
+                            ops.PREFILL_GROUP_TILES)
         sections = (c_long * (7 + len(cache.groups)))()
         summary, placed = (c_int * 6)(), (c_int * (5 * max(1, n)))()
         as_i32 = lambda a: a.ctypes.data_as(hostlib.PI32)
@@ -88,7 +89,7 @@ class _PackedStep:
             total = lib.leone_step_pack(*args, ctypes.cast(host.data_ptr(), hostlib.PI32), host.numel(), sections,
                                         summary, placed)
         if total < 0:
-            raise StepError(hostlib.last_error())
+            raise StepError(cache.keys.named(hostlib.last_error()))
         self.host = host
         self.total = int(total)
         self.offsets = list(sections)
@@ -132,7 +133,7 @@ class _DecodeGraph:
 
     def fill(self, engine: "Engine", entries: Sequence[StepEntry]) -> None:
         self.copied.synchronize()                     # the last upload has left the pinned buffer
-        packed = _PackedStep(engine, entries, all_rows_wanted=True, host=self.host)
+        packed = PackedStep(engine.cache, engine.vocab_size, entries, all_rows_wanted=True, host=self.host)
         if packed.offsets != self.offsets:
             raise StepError("the step does not fit the recorded layout")
         self.dev.copy_(self.host, non_blocking=True)
@@ -297,7 +298,7 @@ class Engine:
 
     def _build_context(self, entries: Sequence[StepEntry]):
         """The step's metadata, laid out by the native routine and uploaded in one copy."""
-        packed = _PackedStep(self, entries, all_rows_wanted=False)
+        packed = PackedStep(self.cache, self.vocab_size, entries)
         device = packed.host[:max(1, packed.total)].to(self.device)
         pieces = packed.pieces(device)
         infos = [EntryInfo(entries[given].request, slot, first_row, count, start)

@@ -181,7 +181,7 @@ class Scheduler:
 
     def _checked(self, code: int) -> int:
         if code < 0:
-            raise SchedulerError(hostlib.last_error())
+            raise SchedulerError(self.cache.keys.named(hostlib.last_error()))
         return code
 
     def _history(self, key: int) -> List[int]:

@@ -216,6 +216,7 @@ def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
 
 
 PREFILL_TILE_ROWS = 32       # rows of one request a wave of the prompt kernel takes (checked against the library)
+PREFILL_GROUP_TILES = 4      # tiles of one request a workgroup of the prompt kernel takes (likewise)
 PREFILL_MIN_ROWS = 16        # shorter portions go through the split-KV kernel row by row
 
 
@@ -228,21 +229,38 @@ def prefill_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: 
 def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                       positions: torch.Tensor, tiles: torch.Tensor, block_table: torch.Tensor, q_heads: int,
                       scale: float, window: int = 0) -> torch.Tensor:
-    """Attention for the rows that ``tiles`` (int32 [n, 3]: entry, first row, rows) covers; writes into ``out``."""
-    if library().leone_attention_prefill_tile_rows() != PREFILL_TILE_ROWS:
+    """Attention for the rows that ``tiles`` covers; writes into ``out``.
+
+    ``tiles`` is int32 [n, 3]: (entry, first row, rows) with at most PREFILL_TILE_ROWS consecutive rows of one
+    request each, PREFILL_GROUP_TILES to a group, all tiles of a group of the same entry, unused places with
+    0 rows (``prefill_tiles`` builds such a list)."""
+    if (library().leone_attention_prefill_tile_rows() != PREFILL_TILE_ROWS
+            or library().leone_attention_prefill_group_tiles() != PREFILL_GROUP_TILES):
         raise KernelError("the kernel library was built for another prompt tile size")
     rows = q.shape[0]
     pages, kv_heads, page_tokens, head_dim = cache_dims(k_pool, v_pool)
     if q.shape[1] != q_heads * head_dim:
         raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
-    if tiles.dim() != 2 or tiles.shape[1] != 3:
-        raise KernelError("attention_prefill: tiles must be int32 [n, 3]")
+    if tiles.dim() != 2 or tiles.shape[1] != 3 or tiles.shape[0] % PREFILL_GROUP_TILES:
+        raise KernelError(f"attention_prefill: tiles must be int32 [n, 3] with n a multiple of {PREFILL_GROUP_TILES}")
     call("leone_attention_prefill", _dev(q, "attention q", torch.bfloat16),
          _dev(out, "attention out", torch.bfloat16, q.shape), _dev(k_pool, "k pool", torch.bfloat16),
          _dev(v_pool, "v pool", torch.bfloat16), _dev(positions, "positions", torch.int32, (rows,)),
-         _dev(tiles, "tiles", torch.int32), tiles.shape[0], _dev(block_table, "block table", torch.int32),
+         _dev(tiles, "tiles", torch.int32), tiles.shape[0] // PREFILL_GROUP_TILES,
+         _dev(block_table, "block table", torch.int32),
          block_table.shape[1], q_heads, kv_heads, head_dim, page_tokens, float(scale), int(window), _stream())
     return out
+
+
+def prefill_tiles(portions) -> torch.Tensor:
+    """The tile list of ``attention_prefill`` for portions given as (entry, first row, rows): tiles in order,
+    every portion's last group filled up with unused places (as the native step layout lists a step's own)."""
+    tiles = []
+    for entry, first_row, rows in portions:
+        mine = [(entry, first_row + at, min(PREFILL_TILE_ROWS, rows - at)) for at in range(0, rows, PREFILL_TILE_ROWS)]
+        mine += [(entry, first_row, 0)] * (-len(mine) % PREFILL_GROUP_TILES)
+        tiles += mine
+    return torch.tensor(tiles, dtype=torch.int32).view(-1, 3)
 
 
 def gemm_f32(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -54,6 +54,8 @@ def library() -> ctypes.CDLL:
             lib.leone_last_error.argtypes = []
             lib.leone_attention_prefill_tile_rows.restype = c_int
             lib.leone_attention_prefill_tile_rows.argtypes = []
+            lib.leone_attention_prefill_group_tiles.restype = c_int
+            lib.leone_attention_prefill_group_tiles.argtypes = []
             lib.leone_argmax_chunk.restype = c_int
             lib.leone_argmax_chunk.argtypes = []
             for name, argtypes in _PROTOTYPES.items():

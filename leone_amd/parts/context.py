@@ -37,7 +37,8 @@ class StepContext:
     max_position: int = 0              # largest position in the step (an upper bound when the step is replayed)
     decode_only: bool = False          # every entry brings exactly one row
     # Long prompt portions come first in a step: rows [0, prefill_rows) belong to them, cut into
-    # q_tiles (int32 [n, 3]: entry, first row, rows; at most 32 consecutive rows of one request each).
+    # q_tiles (int32 [n, 3]: entry, first row, rows; tiles of consecutive rows of one request, in the groups
+    # the prompt-attention kernel takes; places of no rows fill a group up).
     prefill_rows: int = 0
     q_tiles: Optional[torch.Tensor] = None
 

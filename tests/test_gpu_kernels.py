@@ -364,19 +364,19 @@ def test_attention_prefill(shape, window):
     lengths = [300, 77, 200]
     table, k_pool, v_pool, keys, values = paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed=31)
     portions = [(0, 0, 300), (1, 60, 17), (2, 33, 130)]            # (request, first position, rows)
-    rows, tiles = [], []
+    rows, listed = [], []
     for entry, (r, start, count) in enumerate(portions):
-        for at in range(0, count, ops.PREFILL_TILE_ROWS):
-            tiles.append((entry, len(rows) + at, min(ops.PREFILL_TILE_ROWS, count - at)))
+        listed.append((entry, len(rows), count))
         rows += [(r, start + i) for i in range(count)]
     rows += [(1, 76)]                                               # a row outside every tile
+    tiles = ops.prefill_tiles(listed)
     g = torch.Generator().manual_seed(32)
     q = torch.randn(len(rows), q_heads, head_dim, generator=g).to(dtype)
     positions = torch.tensor([p for _, p in rows], dtype=torch.int32)
     scale = 1.0 / math.sqrt(head_dim)
     out = torch.full((len(rows), q_heads * head_dim), 5.0, dtype=dtype, device=DEV)
     ops.attention_prefill(q.reshape(len(rows), -1).to(DEV), out, k_pool.to(DEV), v_pool.to(DEV), positions.to(DEV),
-                          torch.tensor(tiles, dtype=torch.int32, device=DEV), table.to(DEV), q_heads, scale, window)
+                          tiles.to(DEV), table.to(DEV), q_heads, scale, window)
     assert torch.isfinite(out.float()).all()
     assert (out[-1] == 5.0).all()
     want = torch.stack([plain.attend_one(q[i].float(), keys[r][:p + 1], values[r][:p + 1], window or None)
@@ -384,7 +384,10 @@ def test_attention_prefill(shape, window):
     close(out[:-1].reshape(len(rows) - 1, q_heads, head_dim), want, 2e-2, 2e-2, "attention_prefill")
 
 
-def test_attention_prefill_finds_the_one_key_that_matters():
+@pytest.mark.parametrize("dealt", [False, True])
+def test_attention_prefill_finds_the_one_key_that_matters(dealt):
+    """``dealt``: the tiles of the portion stand in another order, first and last tiles together in a group;
+    the kernel takes the tiles of a group as they come."""
     from leone_amd import ops
     q_heads, kv_heads, head_dim, page_tokens = 4, 2, 64, 16
     dtype = torch.bfloat16
@@ -404,12 +407,16 @@ def test_attention_prefill_finds_the_one_key_that_matters():
             k = keys[0][j, h // 2]
             q[i, h] = k * (60.0 * math.sqrt(head_dim) / float(k @ k))
     q = q.to(dtype)
-    tiles = [(0, at, min(32, count - at)) for at in range(0, count, 32)]
+    tiles = ops.prefill_tiles([(0, 0, count)])
+    if dealt:
+        own = [tuple(t) for t in tiles.tolist() if t[2] > 0]
+        assert len(own) == 10
+        order = [0, 9, 1, 8, 7, 2, 3, 6, 5, 4]
+        tiles = torch.tensor([own[i] for i in order] + [(0, 0, 0)] * 2, dtype=torch.int32)
     out = torch.zeros((count, q_heads * head_dim), dtype=dtype, device=DEV)
     ops.attention_prefill(q.reshape(count, -1).to(DEV), out, k_pool.to(DEV), v_pool.to(DEV),
                           torch.tensor([p for _, p in rows], dtype=torch.int32, device=DEV),
-                          torch.tensor(tiles, dtype=torch.int32, device=DEV), table.to(DEV), q_heads,
-                          1.0 / math.sqrt(head_dim))
+                          tiles.to(DEV), table.to(DEV), q_heads, 1.0 / math.sqrt(head_dim))
     out = out.float().cpu().view(count, q_heads, head_dim)
     for i, j in enumerate(targets):
         want = values[0][j].repeat_interleave(2, dim=0)
