@@ -45,12 +45,17 @@ def _add_sampling(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--presence-penalty", type=float, default=0.0, help="Subtract once from any seen token")
     parser.add_argument("--frequency-penalty", type=float, default=0.0, help="Subtract once per earlier occurrence")
     parser.add_argument("--penalty-window", type=int, default=64, help="History the penalties count over; 0 disables")
+    parser.add_argument("--dry-multiplier", type=float, default=0.0, help="Enable the repeated-suffix penalty. 0.0 is off")
+    parser.add_argument("--dry-base", type=float, default=1.75, help="Growth per token of match. Default: 1.75")
+    parser.add_argument("--dry-allowed-length", type=int, default=2, help="Free match length. Default: 2")
+    parser.add_argument("--dry-window", type=int, default=64, help="Tokens of history searched. Default: 64")
 
 
 def _sampling_from(args):
     from .sampling.sampler import SamplingParams
     params = SamplingParams(args.temp, list(getattr(args, "truncations", None) or []), args.seed,
-                            args.repeat_penalty, args.presence_penalty, args.frequency_penalty, args.penalty_window)
+                            args.repeat_penalty, args.presence_penalty, args.frequency_penalty, args.penalty_window,
+                            args.dry_multiplier, args.dry_base, args.dry_allowed_length, args.dry_window)
     if params.truncations and params.temperature is None:
         raise SystemExit("error: truncation flags need --temp; without it generation is greedy")
     params.validate()

@@ -33,6 +33,11 @@ def test_truncation_flags_keep_their_order():
     greedy = cli.build_parser().parse_args(["generate", "-m", "x", "--prompt-tokens", "1", "-n", "2", "--top-k", "5"])
     with pytest.raises(SystemExit):
         cli._sampling_from(greedy)            # a truncation without a temperature
+    dry = cli._sampling_from(cli.build_parser().parse_args(
+        ["generate", "-m", "x", "--prompt-tokens", "1", "-n", "2", "--dry-multiplier", "0.8", "--dry-base", "2",
+         "--dry-allowed-length", "3", "--dry-window", "16"]))
+    assert (dry.dry_multiplier, dry.dry_base, dry.dry_allowed_length, dry.dry_window) == (0.8, 2.0, 3, 16)
+    assert dry.dry_active and not dry.device_eligible and not params.dry_active
 
 
 def test_bench_refuses_several_gpus(capsys):

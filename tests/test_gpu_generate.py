@@ -114,6 +114,36 @@ def test_mirostat_and_dry_generation_matches_oracle(folders):
         assert result.tokens == tokens[len(prompt):]
 
 
+def test_cycle_and_zero_models(tmp_path):
+    """Two models whose output is known without any arithmetic (the reference's fixtures,
+    crates/leone/src/runtime.rs:11567-11608 and crates/leone/tests/common/cpu_fixture.rs:67-105): one-hot
+    embedding, silent layers and a head shifted by one make token t answer t + 1; all-zero weights make
+    every logit 0, and the lowest id wins the tie."""
+    from leone_amd.api import Runtime
+    from leone_amd.weights.safetensors_io import write_file
+    size = 16
+    raw = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, hidden_size=size,
+               num_attention_heads=1, num_key_value_heads=1, head_dim=16, intermediate_size=8, vocab_size=size,
+               max_position_embeddings=64, rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False)
+    for kind in ("cycle", "zero"):
+        folder = make_model_dir(str(tmp_path / kind), raw, 1, torch.float32)
+        tensors = {name: torch.zeros_like(t) for name, t in read_weights(folder).items()}
+        if kind == "cycle":
+            for name in tensors:
+                if name.endswith("norm.weight") or name.endswith("layernorm.weight"):
+                    tensors[name] += 1.0
+            tensors["model.embed_tokens.weight"] = torch.eye(size)
+            tensors["lm_head.weight"] = torch.roll(torch.eye(size), 1, dims=0)       # row t + 1 reads column t
+        write_file(os.path.join(folder, "model.safetensors"), tensors)
+        for dtype in ("float32", "bfloat16"):
+            runtime = Runtime.load(folder, dtype, max_tokens=128, page_tokens=16, max_requests=2)
+            out = runtime.generate_tokens([[3], [14, 2, 9]], 6, eos_token_id=None)
+            if kind == "cycle":
+                assert out[0].tokens == [4, 5, 6, 7, 8, 9] and out[1].tokens == [10, 11, 12, 13, 14, 15]
+            else:
+                assert out[0].tokens == [0] * 6 and out[1].tokens == [0] * 6
+
+
 def test_eos_stops_generation(folders):
     from leone_amd.api import Runtime
     folder = folders["A"]

@@ -306,6 +306,187 @@ def test_toy_architecture_with_state_window_repeat_and_shared_cache(tmp_path, dt
         MIXERS.unregister("toy_decay")
 
 
+# ---- a second toy: a feed-forward that routes rows to experts, and another position encoding -------------
+
+SLOW = 4.0          # the second half of the rotary pairs turns this much slower
+TOY2 = dict(architectures=["ToyRoutedForCausalLM"], hidden=32, heads=2, kv_heads=2, head_dim=16, ffn=24, experts=3,
+            vocab=97, eps=1e-5, max_positions=128)
+
+
+def register_routed_toy():
+    from leone_amd.architectures import register_architecture
+    from leone_amd.config.base import FieldReader
+    from leone_amd.parts import FEED_FORWARDS, POSITIONS, Part, PartSpec
+    from leone_amd.parts.model import ModelSpec, default_schedule
+    from leone_amd.weights.loader import MATRIX, TensorSpec
+
+    class TopOneExperts(Part):
+        """Every row goes to the expert with the highest router logit (float32; the lowest index on a tie):
+        out = down_e(relu(up_e y)).  Rows are grouped by expert inside; nothing outside knows."""
+
+        def __init__(self, spec, **_):
+            self.hidden, self.ffn, self.experts, self.prefix = spec["hidden"], spec["ffn"], spec["experts"], spec["prefix"]
+
+        def tensor_specs(self):
+            specs = [TensorSpec(f"{self.prefix}.router", (self.experts, self.hidden), MATRIX)]
+            for e in range(self.experts):
+                specs += [TensorSpec(f"{self.prefix}.up{e}", (self.ffn, self.hidden), MATRIX),
+                          TensorSpec(f"{self.prefix}.down{e}", (self.hidden, self.ffn), MATRIX)]
+            return specs
+
+        def bind(self, tensors):
+            self.router = tensors.pop(f"{self.prefix}.router").float()
+            self.up = [tensors.pop(f"{self.prefix}.up{e}") for e in range(self.experts)]
+            self.down = [tensors.pop(f"{self.prefix}.down{e}") for e in range(self.experts)]
+
+        def forward(self, y, step):
+            choice = (y.float() @ self.router.t()).argmax(dim=1)          # first of equal maxima
+            out = torch.zeros((y.shape[0], self.hidden), dtype=y.dtype, device=y.device)
+            for e in range(self.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    hidden = torch.relu(torch.nn.functional.linear(y[rows], self.up[e]))
+                    out[rows] = torch.nn.functional.linear(hidden, self.down[e])
+            return out
+
+    class TwoSpeedRotary(Part):
+        """Half-split rotary pairs whose second half turns SLOW times slower (a per-pair frequency factor,
+        the reference's hook at crates/leone/src/cpu.rs:1739-1742).  It hands the mixer tables like the
+        framework's own rotary part."""
+        graph_safe = True
+
+        def __init__(self, spec, **_):
+            self.dim, self.theta = spec["rotary_dim"], spec["theta"]
+
+        def prepare(self, max_positions, device):
+            half = self.dim // 2
+            inv = torch.tensor([self.theta ** (-2.0 * i / self.dim) / (SLOW if i >= half // 2 else 1.0)
+                                for i in range(half)], dtype=torch.float64)
+            angles = torch.arange(max_positions, dtype=torch.float64)[:, None] * inv[None, :]
+            self.cos, self.sin = angles.cos().float().to(device), angles.sin().float().to(device)
+
+        def tables(self):
+            return self.cos, self.sin
+
+    if "toy_top_one" not in FEED_FORWARDS.kinds():
+        FEED_FORWARDS.register("toy_top_one", TopOneExperts)
+    if "toy_two_speed" not in POSITIONS.kinds():
+        POSITIONS.register("toy_two_speed", TwoSpeedRotary)
+
+    @dataclass(frozen=True)
+    class Config:
+        architecture: str
+        raw: tuple
+
+        @classmethod
+        def from_dict(cls, raw):
+            r = FieldReader(raw)
+            keys = ("hidden", "heads", "kv_heads", "head_dim", "ffn", "experts", "vocab", "max_positions")
+            return cls("ToyRoutedForCausalLM", tuple((k, r.positive_int(k)) for k in keys) + (("eps", r.positive_float("eps")),))
+
+    def spec(config):
+        c = dict(config.raw)
+
+        def norm(name):
+            return PartSpec("rmsnorm", {"size": c["hidden"], "eps": c["eps"], "weight": name})
+
+        layers = []
+        for l in range(2):
+            attention = PartSpec("gqa_attention", dict(
+                hidden=c["hidden"], q_heads=c["heads"], kv_heads=c["kv_heads"], head_dim=c["head_dim"], qk_norm_eps=None,
+                window=None, position="slow", q=f"l{l}.q", k=f"l{l}.k", v=f"l{l}.v", o=f"l{l}.o"))
+            experts = PartSpec("toy_top_one", dict(hidden=c["hidden"], ffn=c["ffn"], experts=c["experts"], prefix=f"l{l}.moe"))
+            layers.append(PartSpec("prenorm", {"norm1": norm(f"l{l}.n1"), "mixer": attention, "norm2": norm(f"l{l}.n2"),
+                                               "feed_forward": experts}))
+        return ModelSpec(hidden_size=c["hidden"], vocab_size=c["vocab"], max_positions=c["max_positions"], embedding="emb",
+                         layers=layers, schedule=default_schedule(2), final_norm=norm("final"), head="head",
+                         positions={"slow": PartSpec("toy_two_speed", {"rotary_dim": c["head_dim"], "theta": 300.0})})
+
+    register_architecture("ToyRoutedForCausalLM", Config.from_dict, spec)
+
+
+def routed_plain(w, tokens):
+    c, n = TOY2, len(tokens)
+    x = plain.embedding(w["emb"], tokens)
+
+    def rotate(t):                                                     # [n, heads, D], the toy's own angles
+        out, half = t.clone(), c["head_dim"] // 2
+        for pos in range(n):
+            for i in range(half):
+                angle = pos * 300.0 ** (-2.0 * i / c["head_dim"]) / (SLOW if i >= half // 2 else 1.0)
+                a, b = t[pos, :, i], t[pos, :, i + half]
+                out[pos, :, i] = a * math.cos(angle) - b * math.sin(angle)
+                out[pos, :, i + half] = a * math.sin(angle) + b * math.cos(angle)
+        return out
+
+    for l in range(2):
+        y = plain.rms_norm(x, w[f"l{l}.n1"], c["eps"])
+        q, k, v = (plain.linear(y, w[f"l{l}.{m}"]).view(n, 2, c["head_dim"]) for m in "qkv")
+        x = x + plain.linear(plain.causal_attention(rotate(q), rotate(k), v).reshape(n, -1), w[f"l{l}.o"])
+        y = plain.rms_norm(x, w[f"l{l}.n2"], c["eps"])
+        rows = []
+        for t in range(n):
+            logits = plain.linear(y[t:t + 1], w[f"l{l}.moe.router"])[0]
+            e = int(logits.argmax())
+            hidden = torch.clamp(plain.linear(y[t:t + 1], w[f"l{l}.moe.up{e}"]), min=0.0)
+            rows.append(plain.linear(hidden, w[f"l{l}.moe.down{e}"])[0])
+        x = x + torch.stack(rows)
+    return plain.linear(plain.rms_norm(x, w["final"], c["eps"]), w["head"])
+
+
+def test_toy_architecture_with_routed_feed_forward_and_another_position_encoding(tmp_path):
+    """Float32 only: a router's choice between two nearly equal experts is not stable under bfloat16
+    rounding, and a different choice is not a rounding difference."""
+    from leone_amd.architectures import config_from_dict, model_spec_for, unregister_architecture
+    from leone_amd.engine.engine import Engine, StepEntry
+    from leone_amd.parts import FEED_FORWARDS, POSITIONS
+    from leone_amd.parts.model import DecoderModel
+    from leone_amd.runtime import load_model
+    from leone_amd.weights.random_init import host_tensors
+    from leone_amd.weights.safetensors_io import write_file
+
+    register_routed_toy()
+    try:
+        folder = str(tmp_path / "routed")
+        os.makedirs(folder)
+        json.dump(TOY2, open(os.path.join(folder, "config.json"), "w"))
+        specs = DecoderModel(model_spec_for(config_from_dict(TOY2)), torch.float32, "cpu").tensor_specs()
+        tensors = host_tensors(specs, 5, torch.float32)
+        for name in tensors:
+            if name.endswith("router"):
+                tensors[name] = tensors[name] * 40.0                    # clear choices, all experts in use
+        write_file(os.path.join(folder, "model.safetensors"), tensors)
+        model = load_model(folder, "float32")
+        engine = Engine(model, num_pages=12, page_tokens=8, max_requests=3, poison_freed=True)
+        assert not engine.graphs                                        # the routed part does not claim to be graph-safe
+        requests = {f"r{i}": random_tokens(40 + i, n, TOY2["vocab"]) for i, n in enumerate([33, 21, 40])}
+        expected = {rid: routed_plain({k: v.double() for k, v in tensors.items()}, toks).numpy()
+                    for rid, toks in requests.items()}
+        used = set()
+        for toks in requests.values():
+            x = plain.rms_norm(plain.embedding(tensors["emb"].double(), toks), tensors["l0.n1"].double(), TOY2["eps"])
+            used |= set(plain.linear(x, tensors["l0.moe.router"].double()).argmax(dim=1).tolist())
+        assert len(used) >= 2
+        for mode in ("whole", "tail_decoded", "portions", "mixed"):
+            kwargs = {"max_live": 3} if mode == "mixed" else {"tail": 8} if mode == "tail_decoded" else {}
+            steps = getattr(schedules, mode)(requests, **kwargs)
+            outputs = {}
+            for s in steps:
+                out = engine.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+                if out.logits is not None:
+                    outputs[s["step"]] = out.logits.cpu().numpy()
+                for rid in s["end"]:
+                    engine.release(rid)
+            for rid, rows in schedules.collect(steps, outputs).items():
+                err = np.abs(np.stack(rows) - expected[rid]).max(axis=1)
+                assert np.isfinite(err).all() and err.max() <= 1e-4, (mode, rid, int(err.argmax()), float(err.max()))
+            assert engine.cache.free_pages(0) == 12
+    finally:
+        unregister_architecture("ToyRoutedForCausalLM")
+        FEED_FORWARDS.unregister("toy_top_one")
+        POSITIONS.unregister("toy_two_speed")
+
+
 def test_position_part():
     from leone_amd.parts import POSITIONS, PartSpec
     rope = POSITIONS.build(PartSpec("rope_half_split", {"rotary_dim": 48, "theta": 50000.0}))
