@@ -273,6 +273,196 @@ __global__ void qk_norm_rope_write_kernel(
     }
 }
 
+// The same work for head sizes that are multiples of 16, in runs of 8 elements: a head is shared by
+// head_dim / 16 neighbouring lanes, lane j of them owns elements 8j .. 8j+7 and their partners in the
+// other half, so a lane reads two runs, writes two runs of q or two runs of the key layout (a run of
+// the key layout is eight elements of one token), and the sum of squares crosses at most eight lanes.
+template <typename T>
+struct alignas(8 * sizeof(T)) HeadRun {
+    T v[8];
+};
+
+// Eight elements of a gain vector, from an offset that is a multiple of 8.
+__device__ inline void load_run(const AnyVec& v, int at, float out[8]) {
+    if (v.dtype == kF32) {
+        const HeadRun<float> r = *reinterpret_cast<const HeadRun<float>*>(static_cast<const float*>(v.ptr) + at);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = r.v[i];
+    } else {
+        const HeadRun<bf16_t> r = *reinterpret_cast<const HeadRun<bf16_t>*>(static_cast<const bf16_t*>(v.ptr) + at);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = to_float(r.v[i]);
+    }
+}
+
+template <typename T, int kD16>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_write_runs_kernel(
+    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_pool, T* __restrict__ v_pool,
+    AnyVec q_gain, AnyVec k_gain, float eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, int table_positions, const int* __restrict__ positions,
+    const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
+    int rows, int q_heads, int kv_heads, int page_tokens, int write_cache, int write_values) {
+    constexpr int kD = 16 * kD16;
+    constexpr int kHalf = kD / 2;
+    constexpr int kShare = kD16 <= 1 ? 1 : kD16 <= 2 ? 2 : kD16 <= 4 ? 4 : 8;   // lanes a head takes (a power of two)
+    const int heads_total = q_heads + (write_cache ? (write_values ? 2 : 1) * kv_heads : 0);
+    const long item = (static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x) / kShare;
+    const int j = threadIdx.x % kShare;
+    const bool mine = item < static_cast<long>(rows) * heads_total && j < kD16;
+    // Lanes without work still take part in the exchange below, with zeros.
+    const int row = mine ? static_cast<int>(item / heads_total) : 0;
+    const int head = mine ? static_cast<int>(item % heads_total) : 0;
+    const int qkv_width = (q_heads + 2 * kv_heads) * kD;
+    const T* src = qkv + static_cast<long>(row) * qkv_width + static_cast<long>(head) * kD + 8 * j;
+    const bool is_q = head < q_heads;
+    const bool is_k = !is_q && head < q_heads + kv_heads;
+
+    float a[8], b[8];
+    float ss = 0.f;
+    if (mine) {
+        const HeadRun<T> lo = *reinterpret_cast<const HeadRun<T>*>(src);
+        const HeadRun<T> hi = *reinterpret_cast<const HeadRun<T>*>(src + kHalf);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            a[i] = to_float(lo.v[i]);
+            b[i] = to_float(hi.v[i]);
+            ss = fmaf(a[i], a[i], ss);
+            ss = fmaf(b[i], b[i], ss);
+        }
+    }
+#pragma unroll
+    for (int off = kShare / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off, kWave);
+    if (!mine) return;
+
+    const int pos = positions[row];
+    T* page_base = nullptr;
+    int token = 0;
+    if (!is_q) {
+        const int kvh = is_k ? head - q_heads : head - q_heads - kv_heads;
+        const int page = block_table[static_cast<long>(row_entry[row]) * max_blocks + pos / page_tokens];
+        if (page < 0) return;  // host reserves pages before the launch
+        page_base = (is_k ? k_pool : v_pool) + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD;
+        token = pos % page_tokens;
+    }
+    if (!is_q && !is_k) {      // value head: copied as it is; eight elements of one token lie 16 bytes apart
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            page_base[value_offset(token, 8 * j + i, kD)] = from_float<T>(a[i]);
+            page_base[value_offset(token, kHalf + 8 * j + i, kD)] = from_float<T>(b[i]);
+        }
+        return;
+    }
+    const AnyVec gain = is_q ? q_gain : k_gain;
+    if (gain.ptr) {
+        const float inv = 1.0f / sqrtf(ss / static_cast<float>(kD) + eps);
+        float ga[8], gb[8];
+        load_run(gain, 8 * j, ga);
+        load_run(gain, kHalf + 8 * j, gb);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            a[i] = (a[i] * ga[i]) * inv;
+            b[i] = (b[i] * gb[i]) * inv;
+        }
+    }
+    if (cos_table != nullptr) {
+        const int tpos = pos < table_positions ? pos : table_positions - 1;  // host checks the bound
+        const HeadRun<float> cs = *reinterpret_cast<const HeadRun<float>*>(cos_table + static_cast<long>(tpos) * kHalf + 8 * j);
+        const HeadRun<float> sn = *reinterpret_cast<const HeadRun<float>*>(sin_table + static_cast<long>(tpos) * kHalf + 8 * j);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float ru = a[i] * cs.v[i] - b[i] * sn.v[i];
+            const float rv = a[i] * sn.v[i] + b[i] * cs.v[i];
+            a[i] = ru;
+            b[i] = rv;
+        }
+    }
+    HeadRun<T> lo, hi;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        lo.v[i] = from_float<T>(a[i]);
+        hi.v[i] = from_float<T>(b[i]);
+    }
+    if (is_q) {
+        T* dst = q_out + (static_cast<long>(row) * q_heads + head) * kD + 8 * j;
+        *reinterpret_cast<HeadRun<T>*>(dst) = lo;
+        *reinterpret_cast<HeadRun<T>*>(dst + kHalf) = hi;
+    } else {
+        *reinterpret_cast<HeadRun<T>*>(page_base + key_offset(token, 8 * j, page_tokens)) = lo;
+        *reinterpret_cast<HeadRun<T>*>(page_base + key_offset(token, kHalf + 8 * j, page_tokens)) = hi;
+    }
+}
+
+// Values of many rows at once.  A run of the value layout is one element of eight consecutive tokens,
+// so eight rows that are the consecutive positions 8n .. 8n+7 of one request fill whole runs: a
+// workgroup takes eight rows of the step and one kv head, reads the rows in runs of eight elements,
+// turns them in shared memory and writes head_dim runs that lie side by side.  Rows that do not line
+// up like that (the first and last rows of a portion, single decoded tokens) are written one element
+// at a time.  One thread an element of the head.
+template <typename T>
+__global__ void __launch_bounds__(512)
+value_write_kernel(const T* __restrict__ qkv, T* __restrict__ v_pool, const int* __restrict__ positions,
+                   const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
+                   int rows, int q_heads, int kv_heads, int head_dim, int page_tokens) {
+    extern __shared__ __align__(32) unsigned char turned_raw[];
+    T* turned = reinterpret_cast<T*>(turned_raw);                       // [8][head_dim]
+    const int row0 = blockIdx.x * 8;
+    const int kvh = blockIdx.y;
+    const int d = threadIdx.x;                                          // blockDim.x == head_dim
+    const int qkv_width = (q_heads + 2 * kv_heads) * head_dim;
+    const long head_at = static_cast<long>(q_heads + kv_heads + kvh) * head_dim;
+    const int n = rows - row0 < 8 ? rows - row0 : 8;
+    const int p0 = positions[row0], e0 = row_entry[row0];
+    bool lined_up = n == 8 && (p0 & 7) == 0;
+    for (int i = 1; i < n && lined_up; ++i) lined_up = positions[row0 + i] == p0 + i && row_entry[row0 + i] == e0;
+    // rows in, a run of eight elements a thread
+    for (int idx = threadIdx.x; idx < n * (head_dim / 8); idx += blockDim.x) {
+        const int r = idx / (head_dim / 8), chunk = idx % (head_dim / 8);
+        *reinterpret_cast<HeadRun<T>*>(turned + r * head_dim + 8 * chunk) =
+            *reinterpret_cast<const HeadRun<T>*>(qkv + static_cast<long>(row0 + r) * qkv_width + head_at + 8 * chunk);
+    }
+    __syncthreads();
+    if (lined_up) {
+        const int page = block_table[static_cast<long>(e0) * max_blocks + p0 / page_tokens];
+        if (page < 0) return;  // host reserves pages before the launch
+        HeadRun<T> run;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) run.v[i] = turned[i * head_dim + d];
+        T* base = v_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * head_dim;
+        *reinterpret_cast<HeadRun<T>*>(base + value_offset(p0 % page_tokens, d, head_dim)) = run;
+        return;
+    }
+    for (int i = 0; i < n; ++i) {
+        const int pos = positions[row0 + i];
+        const int page = block_table[static_cast<long>(row_entry[row0 + i]) * max_blocks + pos / page_tokens];
+        if (page < 0) continue;
+        T* base = v_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * head_dim;
+        base[value_offset(pos % page_tokens, d, head_dim)] = turned[i * head_dim + d];
+    }
+}
+
+template <typename T, int kD16>
+static void launch_runs(const void* qkv, void* q_out, void* k_pool, void* v_pool, AnyVec qg, AnyVec kg, float eps,
+                        const float* cos_table, const float* sin_table, int table_positions, const int* positions,
+                        const int* row_entry, const int* block_table, int max_blocks, int rows, int q_heads,
+                        int kv_heads, int page_tokens, int write_cache, hipStream_t stream) {
+    constexpr int kShare = kD16 <= 1 ? 1 : kD16 <= 2 ? 2 : kD16 <= 4 ? 4 : 8;
+    // Many rows are mostly prompt portions: their values go through the kernel that writes whole runs.
+    const bool values_apart = write_cache && rows >= 64 && ceil_div(rows, 8) <= 0x7fffffff && kv_heads <= 65535;
+    const long items = static_cast<long>(rows) * (q_heads + (write_cache ? (values_apart ? 1 : 2) * kv_heads : 0));
+    const int blocks = ceil_div(items * kShare, 256);
+    qk_norm_rope_write_runs_kernel<T, kD16><<<blocks, 256, 0, stream>>>(
+        static_cast<const T*>(qkv), static_cast<T*>(q_out), static_cast<T*>(k_pool), static_cast<T*>(v_pool), qg, kg, eps,
+        cos_table, sin_table, table_positions, positions, row_entry, block_table, max_blocks, rows, q_heads, kv_heads,
+        page_tokens, write_cache, values_apart ? 0 : 1);
+    if (values_apart) {
+        constexpr int kD = 16 * kD16;
+        value_write_kernel<T><<<dim3(ceil_div(rows, 8), kv_heads), kD, 8 * kD * sizeof(T), stream>>>(
+            static_cast<const T*>(qkv), static_cast<T*>(v_pool), positions, row_entry, block_table, max_blocks, rows,
+            q_heads, kv_heads, kD, page_tokens);
+    }
+}
+
 static int check_dtype(int dtype, const char* what) {
     if (dtype != kF32 && dtype != kBF16) {
         set_error("%s: unknown element type %d", what, dtype);
@@ -402,10 +592,35 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, void* q_out, void* k_po
                   "qk_norm_rope_write: head_dim %d must be even and at most %d", head_dim, 2 * kWave * kMaxPairsPerLane);
     LEONE_REQUIRE(!write_cache || (head_dim % 8 == 0 && page_tokens % 8 == 0),
                   "qk_norm_rope_write: the cache needs head_dim %d and page_tokens %d to be multiples of 8", head_dim, page_tokens);
+    AnyVec qg{q_gain, gain_dtype}, kg{k_gain, gain_dtype};
+    const uintptr_t run_bytes = 8 * (dtype == kF32 ? sizeof(float) : sizeof(bf16_t));
+    const bool aligned = reinterpret_cast<uintptr_t>(qkv) % run_bytes == 0 && reinterpret_cast<uintptr_t>(q_out) % run_bytes == 0 &&
+                         (!write_cache || (reinterpret_cast<uintptr_t>(k_pool) % run_bytes == 0 && page_tokens % 8 == 0));
+    const bool tables_aligned = (!q_gain || (reinterpret_cast<uintptr_t>(q_gain) % 32 == 0 && reinterpret_cast<uintptr_t>(k_gain) % 32 == 0)) &&
+                                (!cos_table || (reinterpret_cast<uintptr_t>(cos_table) % 32 == 0 && reinterpret_cast<uintptr_t>(sin_table) % 32 == 0));
+    if (head_dim % 16 == 0 && head_dim <= 128 && aligned && tables_aligned && static_cast<long>(rows) * (q_heads + 2 * kv_heads) * 8 < 0x7fffffffL * 256) {
+#define LEONE_RUNS_CASE(N)                                                                                          \
+    case N:                                                                                                         \
+        if (dtype == kF32)                                                                                          \
+            launch_runs<float, N>(qkv, q_out, k_pool, v_pool, qg, kg, eps, cos_table, sin_table, table_positions,   \
+                                  positions, row_entry, block_table, max_blocks, rows, q_heads, kv_heads,           \
+                                  page_tokens, write_cache, stream);                                                \
+        else                                                                                                        \
+            launch_runs<bf16_t, N>(qkv, q_out, k_pool, v_pool, qg, kg, eps, cos_table, sin_table, table_positions,  \
+                                   positions, row_entry, block_table, max_blocks, rows, q_heads, kv_heads,          \
+                                   page_tokens, write_cache, stream);                                               \
+        break;
+        switch (head_dim / 16) {
+            LEONE_RUNS_CASE(1) LEONE_RUNS_CASE(2) LEONE_RUNS_CASE(3) LEONE_RUNS_CASE(4)
+            LEONE_RUNS_CASE(5) LEONE_RUNS_CASE(6) LEONE_RUNS_CASE(7) LEONE_RUNS_CASE(8)
+        }
+#undef LEONE_RUNS_CASE
+        LEONE_LAUNCH_CHECK("qk_norm_rope_write");
+        return 0;
+    }
     const int heads_total = q_heads + (write_cache ? 2 * kv_heads : 0);
     const int waves_per_block = 4;
     dim3 grid(rows, ceil_div(heads_total, waves_per_block));
-    AnyVec qg{q_gain, gain_dtype}, kg{k_gain, gain_dtype};
     if (dtype == kF32)
         qk_norm_rope_write_kernel<float><<<grid, waves_per_block * kWave, 0, stream>>>(
             static_cast<const float*>(qkv), static_cast<float*>(q_out), static_cast<float*>(k_pool),
