@@ -247,6 +247,52 @@ def test_qk_norm_rope_write(dtype, shape):
     assert torch.equal(q3.cpu().view(n, q_heads, head_dim), q.to(dtype))
 
 
+@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (5, 5, 48, 16), (3, 1, 112, 32), (8, 2, 128, 64)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_qk_norm_rope_write_many_rows(dtype, shape):
+    """Enough rows for the values to go through the kernel that writes whole runs: a portion whose rows do not
+    line up with runs of eight tokens, one that does, and page edges inside both."""
+    from leone_amd import ops
+    q_heads, kv_heads, head_dim, page_tokens = shape
+    torch.manual_seed(6)
+    portions = [(0, 5, 70), (1, 16, 34), (2, 64, 48)]               # (entry, first position, rows); the third lines up
+    rows_meta = [(e, start + i) for e, start, count in portions for i in range(count)]
+    n = len(rows_meta)
+    assert n >= 64 and sum(c for _, _, c in portions[:2]) % 8 == 0
+    qkv = torch.randn(n, (q_heads + 2 * kv_heads) * head_dim).to(dtype)
+    q_gain, k_gain = 1 + 0.1 * torch.randn(head_dim), 1 + 0.1 * torch.randn(head_dim)
+    eps, theta = 1e-5, 1e4
+    max_blocks = 128 // page_tokens
+    n_pages = 3 * max_blocks + 1
+    order = torch.randperm(n_pages - 1)[:3 * max_blocks].view(3, max_blocks).int() + 1     # page 0 stays unused
+    k_pool = torch.full((n_pages, kv_heads, head_dim // 8, page_tokens, 8), 7.0).to(dtype)
+    v_pool = torch.full((n_pages, kv_heads, page_tokens // 8, head_dim, 8), 7.0).to(dtype)
+    cos, sin = ops.rope_table(theta, head_dim, 256, DEV)
+    positions = torch.tensor([p for _, p in rows_meta], dtype=torch.int32)
+    row_entry = torch.tensor([e for e, _ in rows_meta], dtype=torch.int32)
+    kp, vp = k_pool.to(DEV), v_pool.to(DEV)
+    q_out = ops.qk_norm_rope_write(qkv.to(DEV), q_heads, kv_heads, head_dim, q_gain.to(DEV), k_gain.to(DEV), eps,
+                                   cos, sin, positions.to(DEV), row_entry.to(DEV), order.to(DEV), kp, vp)
+    x = qkv.float()
+    q = x[:, :q_heads * head_dim].view(n, q_heads, head_dim)
+    k = x[:, q_heads * head_dim:(q_heads + kv_heads) * head_dim].view(n, kv_heads, head_dim)
+    v = x[:, (q_heads + kv_heads) * head_dim:].view(n, kv_heads, head_dim)
+    atol, rtol = (5e-6, 2e-5) if dtype == torch.float32 else (2e-2, 1e-2)
+    close(q_out.view(n, q_heads, head_dim), plain.rope_half_split(plain.rms_norm(q, q_gain, eps), positions, theta),
+          atol, rtol, "q")
+    want_k = plain.rope_half_split(plain.rms_norm(k, k_gain, eps), positions, theta)
+    k_plain = kp.cpu().transpose(2, 3).reshape(n_pages, kv_heads, page_tokens, head_dim)
+    v_plain = vp.cpu().transpose(3, 4).reshape(n_pages, kv_heads, page_tokens, head_dim)
+    touched = torch.zeros(n_pages, page_tokens, dtype=torch.bool)
+    for i, (e, p) in enumerate(rows_meta):
+        page, off = int(order[e, p // page_tokens]), p % page_tokens
+        touched[page, off] = True
+        close(k_plain[page, :, off], want_k[i], atol, rtol, f"k row {i}")
+        assert torch.equal(v_plain[page, :, off], v[i].to(dtype)), (i, e, p)
+    untouched = ~touched[:, None, :].expand(-1, kv_heads, -1)
+    assert (k_plain[untouched] == 7.0).all() and (v_plain[untouched] == 7.0).all()
+
+
 @pytest.mark.parametrize("mnk", [(1, 777, 80), (5, 64, 64), (130, 192, 96), (67, 1000, 333), (300, 130, 1029)])
 def test_gemm_f32(mnk):
     from leone_amd import ops
