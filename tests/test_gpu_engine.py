@@ -150,3 +150,40 @@ def test_forked_requests_share_prefix_pages_and_agree_with_plain(cases, dtype_na
     engine.release("b")
     engine.cache.check()
     assert engine.cache.free_pages(0) == 16
+
+
+def drawn_config(seed: int) -> dict:
+    """A configuration drawn at random: head sizes in steps of 16, any number of heads and groups, widths
+    and vocabularies that are multiples of nothing in particular."""
+    gen = np.random.default_rng(seed)
+    kv_heads = int(gen.integers(1, 5))
+    group = int(gen.integers(1, 8))
+    head_dim = int(gen.choice([16, 32, 48, 64, 80, 96, 112, 128, 144, 256]))
+    return dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=int(gen.integers(1, 4)),
+                hidden_size=int(gen.integers(5, 40)) * int(gen.choice([2, 4, 8])), num_attention_heads=kv_heads * group,
+                num_key_value_heads=kv_heads, head_dim=head_dim, intermediate_size=int(gen.integers(9, 200)),
+                vocab_size=int(gen.integers(40, 1500)), max_position_embeddings=512,
+                rope_theta=float(gen.choice([1e4, 5e5, 1e6, 123456.0])), rms_norm_eps=float(gen.choice([1e-6, 1e-5, 3e-5])),
+                tie_word_embeddings=bool(gen.integers(0, 2)))
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+@pytest.mark.parametrize("seed", range(10))
+def test_drawn_configurations(tmp_path, seed, dtype_name):
+    """Whatever sizes a configuration allows run, whole and cut up, and agree with the plain implementation."""
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+    raw = drawn_config(1000 + seed)
+    folder = make_model_dir(str(tmp_path / "m"), raw, seed=seed, dtype=DTYPES[dtype_name],
+                            sharpen=2.0 if dtype_name == "float32" else 1.0)
+    config, weights = read_config(folder), read_weights(folder)
+    gen = np.random.default_rng(seed)
+    requests = {f"r{i}": random_tokens(50 * seed + i, int(n), config["vocab_size"])
+                for i, n in enumerate(gen.integers(1, 160, size=3))}
+    expected = {rid: qwen3_plain.forward(weights, config, toks).numpy() for rid, toks in requests.items()}
+    plans = {name: SCHEDULES[name](requests, **({"max_live": 3} if name == "mixed" else {}))
+             for name in ("whole", "portions", "mixed")}
+    engine = Engine(load_model(folder, dtype_name), page_tokens=16, max_requests=4, poison_freed=True,
+                    max_tokens=max(schedules.max_live_tokens(steps, 16) for steps in plans.values()))
+    for name, steps in plans.items():
+        compare(steps, run_steps(engine, steps), expected, tolerance(dtype_name), f"{raw} {name}")
