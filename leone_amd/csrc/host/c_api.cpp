@@ -187,19 +187,12 @@ int leone_scheduler_has_work(void* scheduler) {
     return guarded([&]() -> long { return scheduler_of(scheduler).has_work() ? 1 : 0; });
 }
 
-namespace {
-thread_local std::vector<PlannedEntry> last_plan;
-}
-
 int leone_scheduler_plan(void* scheduler) {
-    return guarded([&]() -> long {
-        last_plan = scheduler_of(scheduler).plan();
-        return static_cast<long>(last_plan.size());
-    });
+    return guarded([&]() -> long { return static_cast<long>(scheduler_of(scheduler).plan().size()); });
 }
 int leone_scheduler_planned(void* scheduler, int64_t* requests, int* starts, int* counts, int* samples, int capacity) {
     return guarded([&]() -> long {
-        scheduler_of(scheduler);
+        const std::vector<PlannedEntry>& last_plan = scheduler_of(scheduler).planned();
         const int n = static_cast<int>(last_plan.size());
         for (int i = 0; i < std::min(n, capacity); ++i) {
             requests[i] = last_plan[i].request;

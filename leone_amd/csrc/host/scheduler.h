@@ -107,6 +107,8 @@ public:
     // The planned step failed: every request in it ends as aborted and gives back what it holds.
     int abort();
 
+    // The entries of the step that is planned and not yet completed or aborted (empty otherwise).
+    const std::vector<PlannedEntry>& planned() const { return planned_; }
     const std::vector<Finished>& finished() const { return finished_; }
     const std::vector<Event>& events() const { return events_; }
     const SchedulerStats& stats() const { return stats_; }
