@@ -6,6 +6,7 @@
 #include <unordered_map>
 
 #include "cache_manager.h"
+#include "sampler.h"
 #include "scheduler.h"
 #include "step_layout.h"
 
@@ -37,6 +38,9 @@ long guarded(Body&& body) {
     } catch (const StepRefused& e) {
         last_error = e.what();
         return LEONE_HOST_STEP_REFUSED;
+    } catch (const SamplerFault& e) {
+        last_error = e.what();
+        return LEONE_HOST_SAMPLER;
     } catch (const std::exception& e) {
         last_error = e.what();
         return LEONE_HOST_INVALID;
@@ -323,6 +327,27 @@ long leone_step_pack(void* cache, int n_entries, const int64_t* requests, const 
                 placed[5 * i + 4] = where[i].start;
             }
         return layout.total();
+    });
+}
+
+int leone_sample_rows(const float* logits, int rows, int vocab, const double* temperature, const int* stage_counts,
+                      const int* stage_kinds, const double* stage_values, const double* uniform, int* tokens) {
+    return guarded([&]() -> long {
+        if (!logits || !temperature || !stage_counts || !uniform || !tokens || rows <= 0 || vocab <= 0)
+            throw std::invalid_argument("sample_rows: missing argument");
+        int total = 0;
+        for (int r = 0; r < rows; ++r) {
+            if (stage_counts[r] < 0) throw std::invalid_argument("sample_rows: negative stage count");
+            total += stage_counts[r];
+        }
+        if (total > 0 && (!stage_kinds || !stage_values)) throw std::invalid_argument("sample_rows: stages are missing");
+        std::vector<StageSpec> stages(total);
+        for (int i = 0; i < total; ++i) {
+            if (stage_kinds[i] < 0 || stage_kinds[i] > 2) throw std::invalid_argument("sample_rows: unknown stage kind");
+            stages[i] = {static_cast<Stage>(stage_kinds[i]), stage_values[i]};
+        }
+        sample_rows(logits, rows, vocab, temperature, stage_counts, stages.data(), uniform, tokens);
+        return 0;
     });
 }
 

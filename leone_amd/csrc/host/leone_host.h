@@ -16,6 +16,7 @@ enum {
     LEONE_HOST_SCHEDULER = -4,
     LEONE_HOST_STEP_REFUSED = -5,
     LEONE_HOST_INVALID = -6,
+    LEONE_HOST_SAMPLER = -7,
 };
 
 const char* leone_host_last_error(void);
@@ -87,6 +88,13 @@ void leone_scheduler_stats(void* scheduler, int64_t* out15);
 long leone_step_pack(void* cache, int n_entries, const int64_t* requests, const int* counts, const int* want_counts,
                      const int32_t* tokens, const int32_t* wants, const int* shape, int32_t* out, long capacity,
                      long* sections, int* summary, int* placed);
+
+// ---- sampling on the host, in double.  `rows` rows of `vocab` float logits; row r is drawn at
+// temperature[r] after its stage_counts[r] truncation stages (kinds 0 top-k, 1 top-p, 2 min-p with
+// their values, one row's stages after the other's) with the uniform value uniform[r]; tokens[r] is the
+// token, -1 for a row without a finite logit.
+int leone_sample_rows(const float* logits, int rows, int vocab, const double* temperature, const int* stage_counts,
+                      const int* stage_kinds, const double* stage_values, const double* uniform, int* tokens);
 
 #ifdef __cplusplus
 }

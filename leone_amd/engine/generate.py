@@ -15,7 +15,8 @@ import torch
 
 from .. import ops
 from ..sampling import rng
-from ..sampling.sampler import MirostatState, SamplerError, SamplingParams, sample as host_sample
+from ..sampling.sampler import (MirostatState, SamplerError, SamplingParams, apply_penalties, native_eligible,
+                                sample as host_sample, sample_rows_native)
 from .engine import Engine, StepEntry
 from .scheduler import Finished, PlannedEntry, Reject, Request, Scheduler, SchedulerPolicy
 
@@ -88,7 +89,22 @@ def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params:
     if host_rows:
         index = torch.tensor(host_rows, dtype=torch.long, device=logits.device)
         copied = logits.index_select(0, index).cpu().numpy()
+        # Rows whose stages the host library knows are drawn there together, after their penalties;
+        # the others go through the general sampler one by one.
+        together = [k for k, i in enumerate(host_rows)
+                    if native_eligible(policies[i]) and rows[i].request not in (controllers or {})]
+        for k in together:
+            i = host_rows[k]
+            if policies[i].penalties_active:
+                copied[k] = apply_penalties(copied[k], history(rows[i].request), policies[i])
+        if together:
+            drawn = sample_rows_native(copied[together], [policies[host_rows[k]] for k in together],
+                                       [rows[host_rows[k]].sample_position for k in together])
+            for k, token in zip(together, drawn):
+                out[rows[host_rows[k]].request] = token
         for k, i in enumerate(host_rows):
+            if k in together:
+                continue
             e = rows[i]
             out[e.request] = host_sample(copied[k], policies[i], e.sample_position, history(e.request),
                                          (controllers or {}).get(e.request))

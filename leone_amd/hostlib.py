@@ -6,11 +6,11 @@ from __future__ import annotations
 
 import ctypes
 import threading
-from ctypes import POINTER, c_char_p, c_int, c_int32, c_int64, c_long, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64, c_long, c_void_p
 
 from .csrc import build as _build
 
-MISUSE, OUT_OF_PAGES, OUT_OF_SLOTS, SCHEDULER, STEP_REFUSED, INVALID = -1, -2, -3, -4, -5, -6
+MISUSE, OUT_OF_PAGES, OUT_OF_SLOTS, SCHEDULER, STEP_REFUSED, INVALID, SAMPLER = -1, -2, -3, -4, -5, -6, -7
 
 _lock = threading.Lock()
 _lib: ctypes.CDLL | None = None
@@ -20,6 +20,8 @@ PI = POINTER(c_int)
 PI32 = POINTER(c_int32)
 PI64 = POINTER(c_int64)
 PL = POINTER(c_long)
+PF = POINTER(c_float)
+PD = POINTER(c_double)
 
 _PROTOTYPES = {
     "leone_cache_create": (H, [PI, c_int, c_int, c_int]),
@@ -67,6 +69,7 @@ _PROTOTYPES = {
     "leone_scheduler_event_count": (c_int, [H]),
     "leone_scheduler_events": (c_int, [H, c_int, c_int, PI, PI64, PI, PI, PI]),
     "leone_scheduler_stats": (None, [H, PI64]),
+    "leone_sample_rows": (c_int, [PF, c_int, c_int, PD, PI, PI, PD, PD, PI]),
     "leone_step_pack": (c_long, [H, c_int, PI64, PI, PI, PI32, PI32, PI, PI32, c_long, PL, PI, PI]),
 }
 

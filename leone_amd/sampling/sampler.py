@@ -325,6 +325,38 @@ def select(probabilities: np.ndarray, u: float) -> int:
     return int(eligible[hit[0]] if hit.size else eligible[-1])
 
 
+_NATIVE_STAGES = {"top_k": 0, "top_p": 1, "min_p": 2}
+
+
+def native_eligible(params: SamplingParams) -> bool:
+    """Temperature with no stages other than top-k, top-p and min-p: the host library draws such rows
+    without sorting the whole vocabulary (``csrc/host/sampler.cpp``, the same rules)."""
+    return not params.greedy and all(stage in _NATIVE_STAGES for stage, _ in params.truncations)
+
+
+def sample_rows_native(logits: np.ndarray, params: Sequence[SamplingParams], positions: Sequence[int]) -> List[int]:
+    """One token for each row of ``logits`` (float32 [rows, vocab], penalties already applied); every row's
+    policy must be ``native_eligible``."""
+    import ctypes
+    from .. import hostlib
+    lib = hostlib.library()
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    rows, vocab = logits.shape
+    temperature = np.array([p.temperature for p in params], dtype=np.float64)
+    counts = np.array([len(p.truncations) for p in params], dtype=np.int32)
+    kinds = np.array([_NATIVE_STAGES[s] for p in params for s, _ in p.truncations] or [0], dtype=np.int32)
+    values = np.array([float(v) for p in params for _, v in p.truncations] or [0.0], dtype=np.float64)
+    draws = np.array([rng.uniform(p.seed, int(at)) for p, at in zip(params, positions)], dtype=np.float64)
+    tokens = np.empty(rows, dtype=np.int32)
+    as_ptr = lambda a, t: a.ctypes.data_as(t)
+    code = lib.leone_sample_rows(as_ptr(logits, hostlib.PF), rows, vocab, as_ptr(temperature, hostlib.PD),
+                                 as_ptr(counts, hostlib.PI), as_ptr(kinds, hostlib.PI), as_ptr(values, hostlib.PD),
+                                 as_ptr(draws, hostlib.PD), as_ptr(tokens, hostlib.PI))
+    if code < 0:
+        raise SamplerError(hostlib.last_error())
+    return tokens.tolist()
+
+
 def sample(logits: np.ndarray, params: SamplingParams, position: int, history: Sequence[int] = (),
            mirostat: Optional[MirostatState] = None) -> int:
     """One token for one row.  ``position`` is the absolute index of the token whose logits these are."""
@@ -337,4 +369,10 @@ def sample(logits: np.ndarray, params: SamplingParams, position: int, history: S
         if best < 0:
             raise SamplerError("no finite logit")
         return best
+    if native_eligible(params):
+        params.validate()
+        token = sample_rows_native(logits[None, :], [params], [position])[0]
+        if token < 0:
+            raise SamplerError("no finite logit")
+        return token
     return select(distribution(logits, params), rng.uniform(params.seed, position))

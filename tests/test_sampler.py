@@ -160,3 +160,46 @@ def test_mirostat_controller():
         token, bound = oracle.mirostat(p.tolist(), bound, 2.0, 0.3, u)
         assert state.select(p, u) == token
         assert state.maximum_surprise == pytest.approx(bound, rel=1e-12)
+
+
+def test_native_rows_against_the_general_sampler_and_the_oracle():
+    """The host library's sampler (selection instead of a full sort) draws what the general sampler draws:
+    small rows against the slow oracle, full-vocabulary rows (peaked, flat, with ties, NaN and infinities)
+    against the general sampler, and top-p 1.0, which has to look at everything."""
+    from leone_amd.sampling.sampler import native_eligible, sample_rows_native
+    gen = np.random.default_rng(4321)
+    for case in range(300):
+        n = int(gen.integers(1, 60))
+        logits = (gen.standard_normal(n) * gen.choice([0.1, 1.0, 5.0, 30.0])).astype(np.float32)
+        if gen.random() < 0.3:
+            logits[gen.integers(0, n)] = gen.choice([np.nan, np.inf, -np.inf])
+        if gen.random() < 0.2 and n > 2:
+            logits[1] = logits[0]
+        if not np.isfinite(logits).any():
+            continue
+        t = float(gen.choice([0.05, 0.5, 0.8, 1.0, 1.7, 10.0]))
+        stages = [(str(name), float(gen.integers(1, 8)) if name == "top_k" else float(gen.uniform(0.05, 1.0)))
+                  for name in gen.permutation(["top_k", "top_p", "min_p"])[:int(gen.integers(0, 4))]]
+        params = SamplingParams(temperature=t, truncations=stages, seed=int(gen.integers(0, 2**62)))
+        assert native_eligible(params)
+        position = int(gen.integers(0, 10000))
+        want = oracle.select(oracle.distribution(logits.tolist(), t, stages), oracle.uniform(params.seed, position))
+        assert sample_rows_native(logits[None, :], [params], [position]) == [want], (case, stages)
+    for vocab, spread in ((50000, 6.0), (151936, 3.0), (30000, 0.01)):
+        rows = 5
+        logits = (gen.standard_normal((rows, vocab)) * spread).astype(np.float32)
+        logits[1, 17] = np.nan
+        logits[2, :200] = logits[2, 0]                               # ties at the top
+        logits[3, 5] = np.inf
+        policies = [SamplingParams(temperature=0.8, truncations=[("top_k", 40), ("top_p", 0.9)], seed=3),
+                    SamplingParams(temperature=1.3, truncations=[("top_p", 0.95)], seed=4),
+                    SamplingParams(temperature=0.7, truncations=[("min_p", 0.02), ("top_k", 2000)], seed=5),
+                    SamplingParams(temperature=1.0, truncations=[("top_p", 1.0)], seed=6),
+                    SamplingParams(temperature=0.5, truncations=[("top_k", 100000)], seed=7)]
+        positions = [11, 12, 13, 14, 15]
+        got = sample_rows_native(logits, policies, positions)
+        for r in range(rows):
+            u = rng.uniform(policies[r].seed, positions[r])
+            assert got[r] == select(distribution(logits[r], policies[r]), u), (vocab, r)
+    assert not native_eligible(SamplingParams(temperature=1.0, truncations=[("tfs", 0.9)]))
+    assert sample_rows_native(np.full((1, 7), np.nan, dtype=np.float32), [SamplingParams(temperature=1.0)], [0]) == [-1]
