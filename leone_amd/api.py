@@ -15,6 +15,7 @@ import torch
 from .engine.engine import Engine
 from .engine.generate import GenerationResult, GenerationStats, generate_tokens
 from .engine.scheduler import SchedulerPolicy
+from .ops.profile import Recorder, StepProfile
 from .runtime import load_model, random_model
 from .sampling.sampler import SamplingParams
 
@@ -71,6 +72,7 @@ class Runtime:
         self.policy = policy or SchedulerPolicy(max_live_requests=max_requests)
         self.tokenizer = tokenizer
         self.last_stats: Optional[GenerationStats] = None
+        self.last_decode_profile: Optional[StepProfile] = None
 
     @classmethod
     def load(cls, model_dir: str, dtype: Union[str, torch.dtype] = "bfloat16", device: Optional[str] = None,
@@ -95,12 +97,17 @@ class Runtime:
     def generate_tokens(self, prompts: Sequence[Sequence[int]], max_new_tokens: int,
                         sampling: Optional[SamplingParams] = None, eos_token_id: Union[int, None, str] = "config",
                         on_token: Optional[Callable[[Hashable, int], None]] = None,
-                        logit_observer: Optional[Callable] = None) -> List[GenerationResult]:
-        """Token ids in, token ids out, one result per prompt in order."""
+                        logit_observer: Optional[Callable] = None,
+                        profile_decode_steps: int = 0) -> List[GenerationResult]:
+        """Token ids in, token ids out, one result per prompt in order.  ``profile_decode_steps``: time
+        that many decode steps operation by operation (they run without graph replay); the result is
+        left in ``last_decode_profile``."""
         eos = self.eos_token_id if eos_token_id == "config" else eos_token_id
+        recorder = Recorder(profile_decode_steps) if profile_decode_steps > 0 else None
         results, stats = generate_tokens(self.engine, prompts, max_new_tokens, sampling, eos, self.policy, on_token,
-                                         logit_observer)
+                                         logit_observer, recorder)
         self.last_stats = stats
+        self.last_decode_profile = recorder.profile if recorder is not None else None
         return results
 
     def encode(self, text: str) -> List[int]:

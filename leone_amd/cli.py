@@ -15,6 +15,9 @@ import sys
 import time
 from typing import List, Optional
 
+# Decode steps that --profile-decode times (the reference's figure, crates/leone-cli/src/main.rs:2828-2830).
+PROFILE_DECODE_STEPS = 64
+
 _STAGE_FLAGS = {"--top-k": "top_k", "--top-p": "top_p", "--min-p": "min_p", "--top-a": "top_a", "--tfs": "tfs",
                 "--typical": "typical", "--epsilon": "epsilon", "--eta": "eta", "--min-k": "min_k",
                 "--top-n-sigma": "top_n_sigma"}
@@ -73,6 +76,8 @@ def build_parser() -> argparse.ArgumentParser:
     g.add_argument("-n", "--tokens", type=int, required=True, help="Number of tokens to generate")
     g.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"], help="Weights, activations and cache")
     g.add_argument("--eager-decode", action="store_true", help="Disable decode graph replay")
+    g.add_argument("--profile-decode", action="store_true",
+                   help=f"Time the first {PROFILE_DECODE_STEPS} decode steps operation by operation")
     g.add_argument("--prefill-chunk", type=int, default=2048, help="Longest prompt portion per step")
     g.add_argument("--max-context", type=int, default=None, help="Context the cache is sized for")
     g.add_argument("--debug-tokens", help="Write generated token IDs as JSON")
@@ -146,7 +151,8 @@ def cmd_generate(args) -> int:
 
     eos = None if args.ignore_eos else "config"
     results = runtime.generate_tokens([prompt], args.tokens, sampling, eos_token_id=eos, on_token=on_token,
-                                      logit_observer=observe)
+                                      logit_observer=observe,
+                                      profile_decode_steps=PROFILE_DECODE_STEPS if args.profile_decode else 0)
     stats = runtime.last_stats
     sys.stdout.write("\n")
     if args.debug_tokens:
@@ -160,6 +166,8 @@ def cmd_generate(args) -> int:
     print(f"prefill: {stats.prefill_rate:.2f} tok/s", file=sys.stderr)
     print(f"tokens emitted: {stats.emitted_tokens}", file=sys.stderr)
     print(f"finish: {results[0].finish_reason}", file=sys.stderr)
+    if runtime.last_decode_profile is not None:
+        print("\n".join(runtime.last_decode_profile.lines()), file=sys.stderr)
     return 0
 
 

@@ -21,6 +21,7 @@ import numpy as np
 import torch
 
 from .. import hostlib, ops
+from ..ops import profile
 from ..cache.manager import CacheManager, OutOfPages
 from ..cache.pools import DevicePools
 from ..parts.context import EntryInfo, StepContext
@@ -240,7 +241,8 @@ class Engine:
             for e in entries:
                 if self.cache.length(e.request) == 0:
                     self.pools.zero_state(self.cache.slot(e.request))   # a request's state starts from zero
-            if self.graphs and all(len(e.tokens) == 1 for e in entries):
+            # A step that is being profiled runs call by call: a replayed recording has no calls to time.
+            if self.graphs and not profile.recording() and all(len(e.tokens) == 1 for e in entries):
                 logits, rows = self._run_decode_graph(entries)
             else:
                 tokens, context, rows = self._build_context(entries)

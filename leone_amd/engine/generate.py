@@ -14,6 +14,7 @@ import numpy as np
 import torch
 
 from .. import ops
+from ..ops.profile import Recorder
 from ..sampling import rng
 from ..sampling.sampler import (MirostatState, SamplerError, SamplingParams, apply_penalties, native_eligible,
                                 sample as host_sample, sample_rows_native)
@@ -127,6 +128,8 @@ class Generator:
         self.stats = GenerationStats()
         # Called with (request, position, float32 logits row on the device) for every sampled row.
         self.logit_observer: Optional[Callable[[Hashable, int, torch.Tensor], None]] = None
+        # When set, the decode-only steps are timed operation by operation until it has its fill.
+        self.decode_profile: Optional[Recorder] = None
 
     def submit(self, request_id: Hashable, prompt: Sequence[int], max_new_tokens: int,
                sampling: Optional[SamplingParams] = None, eos_token_id: Optional[int] = None) -> None:
@@ -150,20 +153,30 @@ class Generator:
         plan = scheduler.plan()
         if not plan:
             return []
+        decoding = all(len(e.tokens) == 1 and e.start > 0 for e in plan)
+        recorder = self.decode_profile if decoding and self.decode_profile is not None \
+            and not self.decode_profile.done else None
         started = time.perf_counter()
         try:
             entries = [StepEntry(e.request, e.tokens, [len(e.tokens) - 1] if e.sample else []) for e in plan]
+            if recorder is not None:
+                recorder.begin_step()
             output = self.engine.run_reserved(entries)
-            sampled = choose_tokens(output.logits, plan, self.params, scheduler.history, self.controllers) if output.logits is not None else {}
+            sampled = choose_tokens(output.logits, plan, self.params, scheduler.history, self.controllers) \
+                if output.logits is not None else {}
+            if recorder is not None:
+                recorder.end_step(len(plan))
             if self.logit_observer is not None and output.logits is not None:
                 for row, e in enumerate([e for e in plan if e.sample]):
                     self.logit_observer(e.request, e.sample_position, output.logits[row])
         except Exception:
+            if recorder is not None:
+                recorder.abandon_step()
             scheduler.abort()
             raise
         elapsed = time.perf_counter() - started
         rows = sum(len(e.tokens) for e in plan)
-        if all(len(e.tokens) == 1 and e.start > 0 for e in plan):
+        if decoding:
             self.stats.decode_seconds += elapsed
             self.stats.decode_tokens += rows
         else:
@@ -199,10 +212,12 @@ def generate_tokens(engine: Engine, prompts: Sequence[Sequence[int]], max_new_to
                     sampling: Optional[SamplingParams] = None, eos_token_id: Optional[int] = None,
                     policy: Optional[SchedulerPolicy] = None,
                     on_token: Optional[Callable[[Hashable, int], None]] = None,
-                    logit_observer: Optional[Callable[[Hashable, int, torch.Tensor], None]] = None):
+                    logit_observer: Optional[Callable[[Hashable, int, torch.Tensor], None]] = None,
+                    decode_profile: Optional[Recorder] = None):
     """Generates for every prompt (token ids); returns results in prompt order and the run's statistics."""
     generator = Generator(engine, policy)
     generator.logit_observer = logit_observer
+    generator.decode_profile = decode_profile
     for i, prompt in enumerate(prompts):
         generator.submit(i, prompt, max_new_tokens, sampling, eos_token_id)
     finished = {f.id: f for f in generator.run(on_token)}

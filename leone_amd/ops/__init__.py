@@ -10,6 +10,7 @@ from typing import Optional
 
 import torch
 
+from . import profile
 from .library import KernelError, call, library
 
 F32, BF16 = 0, 1
@@ -271,8 +272,9 @@ def gemm_f32(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = Non
         raise KernelError(f"gemm_f32: inner sizes {k} and {k2} differ")
     if out is None:
         out = torch.empty((m, n), dtype=torch.float32, device=a.device)
-    call("leone_gemm_f32", _dev(a, "gemm a", torch.float32), _dev(b, "gemm b", torch.float32),
-         _dev(out, "gemm out", torch.float32, (m, n)), m, n, k, _stream())
+    with profile.span("gemm f32", b):
+        call("leone_gemm_f32", _dev(a, "gemm a", torch.float32), _dev(b, "gemm b", torch.float32),
+             _dev(out, "gemm out", torch.float32, (m, n)), m, n, k, _stream())
     return out
 
 
@@ -316,8 +318,9 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,
         raise KernelError(f"gemm_skinny: inner sizes {k} and {k2} differ")
     if out is None:
         out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-    call("leone_gemm_skinny_bf16", _dev(x, "gemm x", torch.bfloat16), _dev(weight, "gemm weight", torch.bfloat16),
-         _dev(out, "gemm out", out_dtype, (m, n)), _CODES[out_dtype], m, n, k, _stream())
+    with profile.span("gemv", weight):
+        call("leone_gemm_skinny_bf16", _dev(x, "gemm x", torch.bfloat16), _dev(weight, "gemm weight", torch.bfloat16),
+             _dev(out, "gemm out", out_dtype, (m, n)), _CODES[out_dtype], m, n, k, _stream())
     return out
 
 
@@ -339,12 +342,14 @@ def gemm_fused(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
         out, mode, out_dtype = torch.empty((m, n // 2), dtype=torch.bfloat16, device=weight.device), 2, torch.bfloat16
     else:
         out, mode = torch.empty((m, n), dtype=out_dtype, device=weight.device), 0
-    call("leone_gemm_fused_bf16",
-         _dev(x.x, "stream", torch.float32) if normed else _dev(x, "gemm x", torch.bfloat16, (m, k)),
-         1 if normed else 0, _dev(x.rows, "rows", torch.int32) if normed else 0,
-         _dev(x.gain, "gain", None, (k,)) if normed else 0, _code(x.gain, "gain") if normed else 0,
-         x.eps if normed else 0.0, _dev(weight, "gemm weight", torch.bfloat16),
-         _dev(out, "gemm out", out_dtype, (m, n // 2 if gated else n)), mode, _CODES[out_dtype], m, n, k, _stream())
+    with profile.span("gemv fused", weight):
+        call("leone_gemm_fused_bf16",
+             _dev(x.x, "stream", torch.float32) if normed else _dev(x, "gemm x", torch.bfloat16, (m, k)),
+             1 if normed else 0, _dev(x.rows, "rows", torch.int32) if normed else 0,
+             _dev(x.gain, "gain", None, (k,)) if normed else 0, _code(x.gain, "gain") if normed else 0,
+             x.eps if normed else 0.0, _dev(weight, "gemm weight", torch.bfloat16),
+             _dev(out, "gemm out", out_dtype, (m, n // 2 if gated else n)), mode, _CODES[out_dtype], m, n, k,
+             _stream())
     return None if residual is not None else out
 
 
@@ -382,9 +387,11 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         raise KernelError("linear: tensor is not on the GPU")
     elif out_dtype == torch.float32:
         # float32 results (logits) for many rows: the library's product with float output
-        y = torch.mm(x, weight.t(), out_dtype=torch.float32)
+        with profile.span(profile.LIBRARY_PRODUCT, weight):
+            y = torch.mm(x, weight.t(), out_dtype=torch.float32)
     else:
-        y = torch.nn.functional.linear(x, weight)  # library matrix product, float accumulation
+        with profile.span(profile.LIBRARY_PRODUCT, weight):
+            y = torch.nn.functional.linear(x, weight)  # library matrix product, float accumulation
         if out_dtype != y.dtype:
             y = y.to(out_dtype)
     return swiglu(y) if gated else y

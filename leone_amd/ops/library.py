@@ -10,6 +10,7 @@ import threading
 from ctypes import c_char_p, c_double, c_float, c_int, c_void_p
 
 from ..csrc import build as _build
+from . import profile
 
 
 class KernelError(RuntimeError):
@@ -68,6 +69,10 @@ def library() -> ctypes.CDLL:
 
 def call(name: str, *args) -> None:
     lib = library()
-    status = getattr(lib, name)(*args)
+    if profile.recording():
+        with profile.span(profile.OPERATIONS.get(name, name)):
+            status = getattr(lib, name)(*args)
+    else:
+        status = getattr(lib, name)(*args)
     if status != 0:
         raise KernelError(lib.leone_last_error().decode("utf-8", "replace"))

@@ -188,15 +188,45 @@ def test_command_line_generate(folders, tmp_path):
     tokens_file, logits_file = tmp_path / "tokens.json", tmp_path / "logits.txt"
     run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "leone"), "generate", "-m", folder,
                           "--prompt-tokens", ",".join(map(str, prompt)), "-n", "8", "--dtype", "float32",
-                          "--debug-tokens", str(tokens_file), "--debug-logits", str(logits_file)],
+                          "--debug-tokens", str(tokens_file), "--debug-logits", str(logits_file),
+                          "--profile-decode"],
                          capture_output=True, text=True, timeout=300)
     assert run.returncode == 0, run.stderr
+    assert "decode profile: 7 evaluations" in run.stderr
     expect = plain_greedy(weights, config, prompt, 8)
     assert json.load(open(tokens_file)) == expect
     assert [int(t) for t in run.stdout.split()] == expect
     assert "decode:" in run.stderr and "prefill:" in run.stderr and "tokens emitted: 8" in run.stderr
     lines = open(logits_file).read().strip().splitlines()
     assert len(lines) == 8 and int(lines[0].split()[0].split(":")[0]) == expect[0]
+
+
+def test_decode_profile_counts_operations_and_keeps_tokens(folders):
+    """Profiled decode steps run call by call between replayed ones: same tokens, and what was counted is
+    what one decode step of this model launches."""
+    from leone_amd.api import Runtime
+    folder = folders["B"]
+    config = read_config(folder)
+    prompt = random_tokens(77, 19, config["vocab_size"])
+    for dtype in ("float32", "bfloat16"):
+        runtime = Runtime.load(folder, dtype, max_tokens=128, page_tokens=16, max_requests=1)
+        expect = runtime.generate_tokens([prompt], 12, eos_token_id=None)[0].tokens
+        assert runtime.last_decode_profile is None
+        assert runtime.generate_tokens([prompt], 12, eos_token_id=None, profile_decode_steps=5)[0].tokens == expect
+        profile = runtime.last_decode_profile
+        layers = config["num_hidden_layers"]
+        assert profile.steps == 5 and profile.tokens == 5
+        assert profile.launches % 5 == 0 and profile.launches // 5 >= 5 * layers
+        assert 0 < profile.gpu_seconds <= profile.wall_seconds
+        assert {"embed", "attention", "qknorm rope kv", "argmax"} <= set(profile.seconds_by_operation)
+        # every layer's four products and the head, five times each
+        assert sum(t.calls for t in profile.products.values()) == 5 * (4 * layers + 1)
+        head = [t for (name, rows, columns, size), t in profile.products.items() if rows == config["vocab_size"]]
+        assert sum(t.calls for t in head) == 5
+        text = "\n".join(profile.lines())
+        assert "decode profile: 5 evaluations" in text and "host gap" in text and "weight GB/s" in text
+        from leone_amd.ops import profile as recording
+        assert not recording.recording()
 
 
 def test_command_line_eval_and_doctor(folders, tmp_path):
