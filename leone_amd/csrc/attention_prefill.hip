@@ -20,6 +20,11 @@
 // lanes; p stays below 2^8 and the quotient of accumulator and sum does not depend on m.  The sum
 // of a query's p is one more row of the second product (a row of ones in V^T), so that numerator
 // and denominator are sums of the same rounded values.
+//
+// Few rows over many keys (a late portion of a long prompt) would leave most of the chip idle: then
+// the keys of a workgroup are cut into `splits` ranges of whole 64-key stages, one workgroup a range
+// (blockIdx.y), each writes its reference, sum and unnormalised accumulator per (row, head, range),
+// and a second kernel merges the ranges in order.
 #include "common.h"
 #include "leone_hip.h"
 
@@ -50,7 +55,8 @@ __global__ void __launch_bounds__(kPrefillThreads, 2)
 attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_pool,
                          const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
                          const int* __restrict__ tiles, int n_groups, const int* __restrict__ block_table,
-                         int max_blocks, int q_heads, int kv_heads, int page_shift, float scale, int window) {
+                         int max_blocks, int q_heads, int kv_heads, int page_shift, float scale, int window,
+                         float* __restrict__ part_acc, float* __restrict__ part_ml, int splits) {
     constexpr int kD = kD16 * 16;
     constexpr int kRuns = kD / 8;                      // 16-byte runs of one key
     constexpr int kSteps = (kD16 + 1) / 2;             // 32-element steps of the first product
@@ -115,6 +121,29 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         group_hi = wave_hi[w] > group_hi ? wave_hi[w] : group_hi;
     }
     if (group_hi <= group_lo) return;                            // a group without rows (every wave agrees)
+    if (splits > 1) {
+        // This workgroup's share of the group's stages; what is outside it is treated like keys outside
+        // the group's range.
+        const int s_begin = group_lo / kStageKeys, s_end = (group_hi + kStageKeys - 1) / kStageKeys;
+        const int share = (s_end - s_begin + splits - 1) / splits;
+        const int mine_lo = (s_begin + static_cast<int>(blockIdx.y) * share) * kStageKeys;
+        const int mine_hi = mine_lo + share * kStageKeys;
+        group_lo = mine_lo > group_lo ? mine_lo : group_lo;
+        group_hi = mine_hi < group_hi ? mine_hi : group_hi;
+        if (group_hi <= group_lo) {                              // more ranges than stages: this one is empty
+            if (g == 0) {
+#pragma unroll
+                for (int j = 0; j < kColsPerWave; ++j) {
+                    const int r = 16 * j + c;
+                    if (r >= wave_rows) continue;
+                    const long slot = (static_cast<long>(tile_row0 + r) * q_heads + head) * splits + blockIdx.y;
+                    part_ml[2 * slot] = -INFINITY;
+                    part_ml[2 * slot + 1] = 0.f;
+                }
+            }
+            return;
+        }
+    }
 
     // The page ids of the keys the group reads go to shared memory first, so that no load of keys or
     // values waits on a read of the block table.
@@ -345,6 +374,23 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     }
 
     const bool poisoned = unmapped_seen != 0;                    // every write to it came before the last barrier
+    if (splits > 1) {
+#pragma unroll
+        for (int j = 0; j < kColsPerWave; ++j) {
+            const int r = 16 * j + c;
+            if (r >= wave_rows) continue;
+            const long slot = (static_cast<long>(tile_row0 + r) * q_heads + head) * splits + blockIdx.y;
+            if (g == 0) {
+                part_ml[2 * slot] = m_ref[j];
+                part_ml[2 * slot + 1] = poisoned ? __builtin_nanf("") : acc_sum[j][0];
+            }
+            if (m_ref[j] == -INFINITY) continue;                 // no key of this range for the row: nothing to merge
+#pragma unroll
+            for (int dt = 0; dt < kD16; ++dt)
+                *reinterpret_cast<floatx4*>(part_acc + slot * kD + 16 * dt + 4 * g) = acc[j][dt];
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < kColsPerWave; ++j) {
         const int r = 16 * j + c;
@@ -364,10 +410,60 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     }
 }
 
+// Merges the key ranges of one row and query head: out = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M),
+// the sums taken in range order; a range that held no key for the row (m_s = -inf) counts as nothing,
+// whatever its accumulator holds.  One wave a (row, head): lane s takes the reference and sum of range s,
+// then all lanes walk the accumulators together.  blockIdx.x is a tile and a quarter of its rows.
+constexpr int kMergeWaves = 4;
+constexpr int kMergeThreads = kMergeWaves * kWave;
+constexpr int kMergeBlocksPerTile = kRowsPerWave / kMergeWaves / 2;   // a wave takes two rows, one after the other
+constexpr int kMaxPrefillSplits = 32;
+
+__global__ void __launch_bounds__(kMergeThreads)
+attention_prefill_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                               bf16_t* __restrict__ out, const int* __restrict__ tiles, int q_heads, int head_dim,
+                               int splits) {
+    const int* tile = tiles + 3 * static_cast<long>(blockIdx.x / kMergeBlocksPerTile);
+    const int row0 = tile[1], rows = tile[2], head = blockIdx.y;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    for (int r = (blockIdx.x % kMergeBlocksPerTile) * kMergeWaves + wave; r < rows; r += kMergeWaves * kMergeBlocksPerTile) {
+        const long rh = static_cast<long>(row0 + r) * q_heads + head;
+        const float2 ml = lane < splits ? reinterpret_cast<const float2*>(part_ml)[rh * splits + lane]
+                                        : float2{-INFINITY, 0.f};
+        const float top = wave_max(ml.x);
+        const bool counts = ml.x != -INFINITY;
+        const float my_weight = counts ? __builtin_amdgcn_exp2f(ml.x - top) : 0.f;
+        // A range without keys for this row has sum 0; a sum that is NaN (a key without a page) still shows.
+        const float my_share = counts || ml.y != ml.y ? ml.y * (counts ? my_weight : 1.f) : 0.f;
+        float den = 0.f;
+        float num[4] = {0.f, 0.f, 0.f, 0.f};                     // head_dim <= 256: at most four elements a lane
+        const float* acc = part_acc + rh * splits * head_dim;
+#pragma unroll 4
+        for (int s = 0; s < splits; ++s) {
+            const float weight = __shfl(my_weight, s, kWave);
+            den += __shfl(my_share, s, kWave);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int d = lane + kWave * i;
+                if (d < head_dim) {
+                    const float value = acc[static_cast<long>(s) * head_dim + d];   // may be anything where weight is 0
+                    num[i] += weight != 0.f ? value * weight : 0.f;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int d = lane + kWave * i;
+            if (d < head_dim) out[rh * head_dim + d] = from_float<bf16_t>(num[i] / den);
+        }
+    }
+}
+
 template <int kD16>
 static int launch_prefill(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
                           const int* tiles, int n_groups, const int* block_table, int max_blocks, int q_heads,
-                          int kv_heads, int page_shift, float scale, int window, hipStream_t stream) {
+                          int kv_heads, int page_shift, float scale, int window, float* part_acc, float* part_ml,
+                          int splits, hipStream_t stream) {
     const size_t shared = 2 * static_cast<size_t>(stage_runs(16 * kD16)) * sizeof(uint4) + static_cast<size_t>(max_blocks) * sizeof(int);
     static size_t allowed = 48 * 1024;                 // what a kernel may use without asking
     if (shared > allowed) {
@@ -379,10 +475,10 @@ static int launch_prefill(const void* q, void* out, const void* k_pool, const vo
         }
         allowed = shared;
     }
-    attention_prefill_kernel<kD16><<<n_groups * q_heads, kPrefillThreads, shared, stream>>>(
+    attention_prefill_kernel<kD16><<<dim3(n_groups * q_heads, splits), kPrefillThreads, shared, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), positions, tiles, n_groups, block_table, max_blocks, q_heads, kv_heads,
-        page_shift, scale, window);
+        page_shift, scale, window, part_acc, part_ml, splits);
     return 0;
 }
 
@@ -393,11 +489,17 @@ using namespace leone;
 extern "C" int leone_attention_prefill_tile_rows() { return kRowsPerWave; }
 extern "C" int leone_attention_prefill_group_tiles() { return kPrefillWaves; }
 
+extern "C" int leone_attention_prefill_max_splits() { return kMaxPrefillSplits; }
+
 // tiles holds n_groups * leone_attention_prefill_group_tiles() entries of (entry, first row, rows).
+// splits > 1 cuts every workgroup's keys into that many ranges and needs the workspace: part_acc of
+// rows * q_heads * splits * head_dim floats and part_ml of rows * q_heads * splits * 2, `rows` being one
+// more than the last row any tile names; with splits == 1 both may be null.
 extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_pool, const void* v_pool,
                                        const int* positions, const int* tiles, int n_groups, const int* block_table,
                                        int max_blocks, int q_heads, int kv_heads, int head_dim, int page_tokens,
-                                       float scale, int window, hipStream_t stream) {
+                                       float scale, int window, float* part_acc, float* part_ml, int splits,
+                                       hipStream_t stream) {
     LEONE_REQUIRE(q && out && k_pool && v_pool && positions && tiles && block_table, "attention_prefill: null pointer");
     LEONE_REQUIRE(n_groups > 0 && q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
                   "attention_prefill: %d tile groups, %d query heads over %d kv heads", n_groups, q_heads, kv_heads);
@@ -408,6 +510,10 @@ extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_p
                   "attention_prefill: page_tokens %d must be a power of two, at least 16", page_tokens);
     LEONE_REQUIRE(window >= 0 && max_blocks > 0, "attention_prefill: bad window or block table");
     LEONE_REQUIRE(scale > 0.f, "attention_prefill: the score scale must be positive");
+    LEONE_REQUIRE(splits >= 1 && splits <= kMaxPrefillSplits, "attention_prefill: splits %d must be in 1..%d", splits,
+                  kMaxPrefillSplits);
+    LEONE_REQUIRE(splits == 1 || (part_acc && part_ml), "attention_prefill: %d key ranges need the workspace", splits);
+    LEONE_REQUIRE(q_heads <= 65535, "attention_prefill: too many heads for one launch");
     LEONE_REQUIRE(static_cast<size_t>(max_blocks) * sizeof(int) <= 16 * 1024,
                   "attention_prefill: a block table of %d entries does not fit shared memory", max_blocks);
     int page_shift = 0;
@@ -416,7 +522,8 @@ extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_p
 #define LEONE_PREFILL_CASE(N)                                                                                      \
     case N:                                                                                                        \
         status = launch_prefill<N>(q, out, k_pool, v_pool, positions, tiles, n_groups, block_table, max_blocks,    \
-                                   q_heads, kv_heads, page_shift, scale, window, stream);                          \
+                                   q_heads, kv_heads, page_shift, scale, window, part_acc, part_ml, splits,        \
+                                   stream);                                                                        \
         break;
     switch (head_dim / 16) {
         LEONE_PREFILL_CASE(1) LEONE_PREFILL_CASE(2) LEONE_PREFILL_CASE(3) LEONE_PREFILL_CASE(4)
@@ -428,5 +535,11 @@ extern "C" int leone_attention_prefill(const void* q, void* out, const void* k_p
 #undef LEONE_PREFILL_CASE
     if (status) return status;
     LEONE_LAUNCH_CHECK("attention_prefill");
+    if (splits > 1) {
+        attention_prefill_merge_kernel<<<dim3(n_groups * kPrefillWaves * kMergeBlocksPerTile, q_heads), kMergeThreads, 0,
+                                         stream>>>(
+            part_acc, part_ml, static_cast<bf16_t*>(out), tiles, q_heads, head_dim, splits);
+        LEONE_LAUNCH_CHECK("attention_prefill_merge");
+    }
     return 0;
 }

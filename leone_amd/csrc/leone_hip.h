@@ -53,11 +53,18 @@ int leone_attention_decode(const void* q, void* out, const void* k_pool, const v
 
 // Causal attention of prompt portions on the matrix cores for bfloat16.  `tiles` lists (entry, first
 // row, rows) for runs of at most leone_attention_prefill_tile_rows() consecutive rows of one request;
-// the rows of a tile sit at consecutive positions.  head_dim a multiple of 16 up to 128.
+// the rows of a tile sit at consecutive positions; leone_attention_prefill_group_tiles() tiles of one
+// request make a group (a workgroup), unused places have 0 rows.  head_dim a multiple of 16 up to 128.
+// splits > 1 (at most leone_attention_prefill_max_splits()) cuts each group's keys into that many ranges,
+// one workgroup each, merged by a second kernel; it needs part_acc (rows * q_heads * splits * head_dim
+// floats) and part_ml (rows * q_heads * splits * 2), rows being one more than the last row a tile names.
 int leone_attention_prefill_tile_rows();
+int leone_attention_prefill_group_tiles();
+int leone_attention_prefill_max_splits();
 int leone_attention_prefill(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
-                            const int* tiles, int n_tiles, const int* block_table, int max_blocks, int q_heads,
-                            int kv_heads, int head_dim, int page_tokens, float scale, int window, hipStream_t stream);
+                            const int* tiles, int n_groups, const int* block_table, int max_blocks, int q_heads,
+                            int kv_heads, int head_dim, int page_tokens, float scale, int window, float* part_acc,
+                            float* part_ml, int splits, hipStream_t stream);
 
 // C[M,N] = A[M,K] . B[N,K]^T in float.
 int leone_gemm_f32(const float* a, const float* b, float* c, int m, int n, int k, hipStream_t stream);

@@ -307,10 +307,13 @@ class Engine:
                  for given, slot, first_row, count, start in packed.placed]
         rows_map = [(e.request, int(w)) for e in entries for w in e.want]
         n_groups = len(self.cache.groups)
+        tiled = [(count, start) for _, _, first_row, count, start in packed.placed if first_row < packed.prefill_rows]
+        mean_keys = sum(count * (start + (count + 1) // 2) for count, start in tiled) // max(1, sum(c for c, _ in tiled))
         context = StepContext(
             rows=packed.rows, dtype=self.dtype, device=self.device, positions=pieces[1], row_entry=pieces[2],
             entries=infos, entry_slots=pieces[3], want_rows=pieces[4] if packed.wanted else None,
             block_tables={g: pieces[6 + g].view(len(entries), -1) for g in range(n_groups)},
             max_position=packed.max_position, decode_only=packed.decode_only,
-            prefill_rows=packed.prefill_rows, q_tiles=pieces[5].view(-1, 3) if packed.tiles else None)
+            prefill_rows=packed.prefill_rows, q_tiles=pieces[5].view(-1, 3) if packed.tiles else None,
+            prefill_mean_keys=mean_keys)
         return pieces[0], context, rows_map

@@ -219,6 +219,8 @@ def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
 PREFILL_TILE_ROWS = 32       # rows of one request a wave of the prompt kernel takes (checked against the library)
 PREFILL_GROUP_TILES = 4      # tiles of one request a workgroup of the prompt kernel takes (likewise)
 PREFILL_MIN_ROWS = 16        # shorter portions go through the split-KV kernel row by row
+PREFILL_SPLIT_MIN_STAGES = 8 # a key range of the prompt kernel is worth a workgroup from this many 64-key stages
+PREFILL_MAX_SPLITS = 32      # most key ranges the prompt kernel takes (checked against the library)
 
 
 def prefill_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int, max_blocks: int = 0) -> bool:
@@ -227,16 +229,30 @@ def prefill_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: 
             and page_tokens >= 16 and page_tokens & (page_tokens - 1) == 0)
 
 
+def choose_prefill_splits(groups: int, q_heads: int, mean_keys: int, window: int = 0) -> int:
+    """How many ranges the keys of a prompt workgroup are cut into: enough for about two workgroups on each
+    of the 256 CUs, as long as a range keeps PREFILL_SPLIT_MIN_STAGES stages of 64 keys where a row sees
+    ``mean_keys`` keys.  (A prompt from position 0 gains nothing: its early rows see few keys.)"""
+    reach = PREFILL_GROUP_TILES * PREFILL_TILE_ROWS
+    keys = min(mean_keys, window + reach) if window > 0 else mean_keys
+    stages = -(-keys // 64)
+    return max(1, min(512 // max(1, groups * q_heads), stages // PREFILL_SPLIT_MIN_STAGES, PREFILL_MAX_SPLITS))
+
+
 def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                       positions: torch.Tensor, tiles: torch.Tensor, block_table: torch.Tensor, q_heads: int,
-                      scale: float, window: int = 0) -> torch.Tensor:
+                      scale: float, window: int = 0, mean_keys: int = 1, splits: Optional[int] = None,
+                      covered_rows: Optional[int] = None) -> torch.Tensor:
     """Attention for the rows that ``tiles`` covers; writes into ``out``.
 
     ``tiles`` is int32 [n, 3]: (entry, first row, rows) with at most PREFILL_TILE_ROWS consecutive rows of one
     request each, PREFILL_GROUP_TILES to a group, all tiles of a group of the same entry, unused places with
-    0 rows (``prefill_tiles`` builds such a list)."""
+    0 rows (``prefill_tiles`` builds such a list).  ``mean_keys`` (keys a row sees on average) only steers
+    the number of key ranges (``splits``); ``covered_rows``: one more than the last row a tile names, if the
+    caller knows it."""
     if (library().leone_attention_prefill_tile_rows() != PREFILL_TILE_ROWS
-            or library().leone_attention_prefill_group_tiles() != PREFILL_GROUP_TILES):
+            or library().leone_attention_prefill_group_tiles() != PREFILL_GROUP_TILES
+            or library().leone_attention_prefill_max_splits() != PREFILL_MAX_SPLITS):
         raise KernelError("the kernel library was built for another prompt tile size")
     rows = q.shape[0]
     pages, kv_heads, page_tokens, head_dim = cache_dims(k_pool, v_pool)
@@ -244,12 +260,22 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, 
         raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
     if tiles.dim() != 2 or tiles.shape[1] != 3 or tiles.shape[0] % PREFILL_GROUP_TILES:
         raise KernelError(f"attention_prefill: tiles must be int32 [n, 3] with n a multiple of {PREFILL_GROUP_TILES}")
+    groups = tiles.shape[0] // PREFILL_GROUP_TILES
+    if splits is None:
+        splits = choose_prefill_splits(groups, q_heads, mean_keys, window)
+    part_acc = part_ml = None
+    if splits > 1:
+        covered = rows if covered_rows is None else covered_rows
+        if not 0 < covered <= rows:
+            raise KernelError(f"attention_prefill: {covered} covered rows of {rows}")
+        part_acc = torch.empty((covered * q_heads * splits * head_dim,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((covered * q_heads * splits * 2,), dtype=torch.float32, device=q.device)
     call("leone_attention_prefill", _dev(q, "attention q", torch.bfloat16),
          _dev(out, "attention out", torch.bfloat16, q.shape), _dev(k_pool, "k pool", torch.bfloat16),
          _dev(v_pool, "v pool", torch.bfloat16), _dev(positions, "positions", torch.int32, (rows,)),
-         _dev(tiles, "tiles", torch.int32), tiles.shape[0] // PREFILL_GROUP_TILES,
-         _dev(block_table, "block table", torch.int32),
-         block_table.shape[1], q_heads, kv_heads, head_dim, page_tokens, float(scale), int(window), _stream())
+         _dev(tiles, "tiles", torch.int32), groups, _dev(block_table, "block table", torch.int32),
+         block_table.shape[1], q_heads, kv_heads, head_dim, page_tokens, float(scale), int(window),
+         _dev(part_acc, "partials"), _dev(part_ml, "partial sums"), int(splits), _stream())
     return out
 
 

@@ -32,7 +32,8 @@ _PROTOTYPES = {
                              c_int, P],
     "leone_attention_decode": [P, P, P, P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                c_int, P],
-    "leone_attention_prefill": [P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
+    "leone_attention_prefill": [P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P, P,
+                                c_int, P],
     "leone_gemm_f32": [P, P, P, c_int, c_int, c_int, P],
     "leone_gemm_skinny_bf16": [P, P, P, c_int, c_int, c_int, c_int, P],
     "leone_gemm_fused_bf16": [P, c_int, P, P, c_int, c_float, P, P, c_int, c_int, c_int, c_int, c_int, P],
@@ -57,6 +58,8 @@ def library() -> ctypes.CDLL:
             lib.leone_attention_prefill_tile_rows.argtypes = []
             lib.leone_attention_prefill_group_tiles.restype = c_int
             lib.leone_attention_prefill_group_tiles.argtypes = []
+            lib.leone_attention_prefill_max_splits.restype = c_int
+            lib.leone_attention_prefill_max_splits.argtypes = []
             lib.leone_argmax_chunk.restype = c_int
             lib.leone_argmax_chunk.argtypes = []
             for name, argtypes in _PROTOTYPES.items():

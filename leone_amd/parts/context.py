@@ -41,6 +41,7 @@ class StepContext:
     # the prompt-attention kernel takes; places of no rows fill a group up).
     prefill_rows: int = 0
     q_tiles: Optional[torch.Tensor] = None
+    prefill_mean_keys: int = 0         # keys a row of these portions sees on average (steers the kernel's grid only)
 
 
 @dataclass

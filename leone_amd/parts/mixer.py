@@ -105,7 +105,9 @@ class GqaAttention(Part):
         if (step.prefill_rows and step.q_tiles is not None
                 and ops.prefill_attention_supported(q.dtype, self.head_dim, cache.page_tokens, max_blocks)):
             ops.attention_prefill(q, out, cache.k_pool, cache.v_pool, step.positions, step.q_tiles,
-                                  cache.block_table, self.q_heads, self.scale, window)
+                                  cache.block_table, self.q_heads, self.scale, window,
+                                  mean_keys=step.prefill_mean_keys or step.max_position + 1,
+                                  covered_rows=step.prefill_rows)
             first = step.prefill_rows
         if first < step.rows:
             ops.attention_decode(q[first:], cache.k_pool, cache.v_pool, step.positions[first:],

@@ -96,6 +96,34 @@ def test_engine_matches_plain(cases, name, dtype_name, schedule, page_tokens):
     assert all(engine.cache.free_pages(g) == engine.cache.groups[g].num_pages for g in range(len(engine.cache.groups)))
 
 
+@pytest.mark.parametrize("schedule", ["whole", "portions", "mixed"])
+@pytest.mark.parametrize("name", ["M", "C"])
+def test_prompt_key_ranges_agree_with_plain(cases, monkeypatch, name, schedule):
+    """The prompt kernel cuts a workgroup's keys into ranges when rows are few and keys many; here every
+    64-key stage may be a range of its own, so that the tiny prompts go that way too."""
+    from leone_amd import ops
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+
+    chosen = []
+    choose = ops.choose_prefill_splits
+
+    def recording(*args, **kwargs):
+        chosen.append(choose(*args, **kwargs))
+        return chosen[-1]
+
+    monkeypatch.setattr(ops, "PREFILL_SPLIT_MIN_STAGES", 1)
+    monkeypatch.setattr(ops, "choose_prefill_splits", recording)
+    folder, requests, expected = cases(name, "bfloat16")
+    steps = SCHEDULES[schedule](requests)
+    model = load_model(folder, "bfloat16")
+    engine = Engine(model, num_pages=schedules.max_live_tokens(steps, round_to=16) // 16, page_tokens=16,
+                    max_requests=4, poison_freed=True)
+    outputs = run_steps(engine, steps)
+    assert max(chosen) >= 2, "no step took the key-range path"
+    compare(steps, outputs, expected, tolerance("bfloat16"), f"{name}/key ranges/{schedule}")
+
+
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 def test_rerun_is_bitwise_identical(cases, dtype_name):
     from leone_amd.engine.engine import Engine

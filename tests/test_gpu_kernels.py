@@ -398,11 +398,13 @@ def test_gemm_skinny(mnk, out_dtype):
     assert torch.equal(ops.gemm_skinny(x[m - 1:m].contiguous(), w, out_dtype)[0], out[m - 1])
 
 
+@pytest.mark.parametrize("splits", [1, 2, 5, 32])
 @pytest.mark.parametrize("window", [0, 5, 37])
 @pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 1, 32, 64), (5, 5, 48, 16), (32, 8, 128, 64), (3, 3, 112, 32)])
-def test_attention_prefill(shape, window):
+def test_attention_prefill(shape, window, splits):
     """Portions that start at position 0 and in the middle of a request, longer and shorter than a
-    128-row tile, over scattered pages; rows of the step that belong to no tile stay untouched."""
+    128-row tile, over scattered pages; rows of the step that belong to no tile stay untouched.  The keys
+    of a workgroup in one range or cut into several, down to ranges of one 64-key stage and empty ones."""
     from leone_amd import ops
     q_heads, kv_heads, head_dim, page_tokens = shape
     dtype = torch.bfloat16
@@ -422,7 +424,7 @@ def test_attention_prefill(shape, window):
     scale = 1.0 / math.sqrt(head_dim)
     out = torch.full((len(rows), q_heads * head_dim), 5.0, dtype=dtype, device=DEV)
     ops.attention_prefill(q.reshape(len(rows), -1).to(DEV), out, k_pool.to(DEV), v_pool.to(DEV), positions.to(DEV),
-                          tiles.to(DEV), table.to(DEV), q_heads, scale, window)
+                          tiles.to(DEV), table.to(DEV), q_heads, scale, window, splits=splits)
     assert torch.isfinite(out.float()).all()
     assert (out[-1] == 5.0).all()
     want = torch.stack([plain.attend_one(q[i].float(), keys[r][:p + 1], values[r][:p + 1], window or None)
@@ -430,8 +432,9 @@ def test_attention_prefill(shape, window):
     close(out[:-1].reshape(len(rows) - 1, q_heads, head_dim), want, 2e-2, 2e-2, "attention_prefill")
 
 
+@pytest.mark.parametrize("splits", [1, 3])
 @pytest.mark.parametrize("dealt", [False, True])
-def test_attention_prefill_finds_the_one_key_that_matters(dealt):
+def test_attention_prefill_finds_the_one_key_that_matters(dealt, splits):
     """``dealt``: the tiles of the portion stand in another order, first and last tiles together in a group;
     the kernel takes the tiles of a group as they come."""
     from leone_amd import ops
@@ -462,7 +465,7 @@ def test_attention_prefill_finds_the_one_key_that_matters(dealt):
     out = torch.zeros((count, q_heads * head_dim), dtype=dtype, device=DEV)
     ops.attention_prefill(q.reshape(count, -1).to(DEV), out, k_pool.to(DEV), v_pool.to(DEV),
                           torch.tensor([p for _, p in rows], dtype=torch.int32, device=DEV),
-                          tiles.to(DEV), table.to(DEV), q_heads, 1.0 / math.sqrt(head_dim))
+                          tiles.to(DEV), table.to(DEV), q_heads, 1.0 / math.sqrt(head_dim), splits=splits)
     out = out.float().cpu().view(count, q_heads, head_dim)
     for i, j in enumerate(targets):
         want = values[0][j].repeat_interleave(2, dim=0)
