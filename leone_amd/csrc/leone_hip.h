@@ -88,4 +88,12 @@ int leone_argmax(const float* logits, int* out, float* part_value, int* part_ind
                  hipStream_t stream);
 int leone_sample_temperature(const float* logits, const double* temperature, const double* uniform, int* out,
                              int rows, int vocab, hipStream_t stream);
+
+// The wanted[row] best finite logits of each row (higher first, lower id on a tie), best first, for a
+// sampler that truncates to the k best before anything else.  out_values and out_ids have
+// leone_top_candidates_max() places a row; out_count[row] is the number filled, or -1 for a row that has
+// to be selected another way.  max_wanted: the largest of wanted[], checked against the limit.
+int leone_top_candidates_max();
+int leone_top_candidates(const float* logits, const int* wanted, float* out_values, int* out_ids, int* out_count,
+                         int rows, int vocab, int max_wanted, hipStream_t stream);
 }

@@ -160,9 +160,116 @@ sample_temperature_kernel(const float* __restrict__ logits, const double* __rest
     }
 }
 
+// ---- the best k logits of a row, for the host sampler ---------------------------------------------------
+//
+// The sampler's order (crates/leone/src/sampler.rs:502-534): finite logits only, the higher first, the
+// lower id on a tie.  A logit and its id become one 64-bit key whose unsigned order is that order
+// (0 for a value that is not finite, behind every finite one), so that selection is a sort of integers.
+//
+// One workgroup a row.  Every thread finds the best key among the ids it owns (t, t + 1024, ...); the
+// k-th best of these 1024 keys is a bound that the row's k-th best key cannot lie behind.  A second walk
+// collects every key not behind the bound (for k <= 256 and a vocabulary of 150,000 a few hundred), the
+// collection is sorted and its first k keys are the result.  A row whose collection would not fit
+// (values arranged against the deal) reports -1 and is left to the host.
+constexpr int kCandidateMaxK = 256;
+constexpr int kCandidateRoom = 4096;
+
+__device__ inline unsigned long long candidate_key(float v, int id) {
+    v += 0.0f;                                              // -0 and +0 are one value
+    const unsigned bits = __float_as_uint(v);
+    if ((bits & 0x7f800000u) == 0x7f800000u) return 0ull;   // infinity or NaN
+    const unsigned ordered = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+    return (static_cast<unsigned long long>(ordered) << 32) | (0xffffffffu - static_cast<unsigned>(id));
+}
+
+// Sorts keys[0, n) (n a power of two) so that the greatest comes first; every thread of the workgroup calls it.
+__device__ inline void sort_keys_descending(unsigned long long* keys, int n) {
+    for (int width = 2; width <= n; width <<= 1) {
+        for (int stride = width >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int i = threadIdx.x; i < n; i += kSampleThreads) {
+                const int partner = i ^ stride;
+                if (partner > i) {
+                    const unsigned long long a = keys[i], b = keys[partner];
+                    const bool descending = (i & width) == 0;
+                    if (descending ? a < b : a > b) {
+                        keys[i] = b;
+                        keys[partner] = a;
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+}
+
+__global__ void __launch_bounds__(kSampleThreads)
+top_candidates_kernel(const float* __restrict__ logits, const int* __restrict__ wanted, float* __restrict__ out_values,
+                      int* __restrict__ out_ids, int* __restrict__ out_count, int vocab) {
+    __shared__ unsigned long long keys[kCandidateRoom];
+    __shared__ int collected;
+    const float* row = logits + static_cast<long>(blockIdx.x) * vocab;
+    int k = wanted[blockIdx.x];
+    k = k < 1 ? 1 : (k > kCandidateMaxK ? kCandidateMaxK : k);   // the host checks; no index may depend on it
+
+    unsigned long long best = 0ull;
+    for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
+        const unsigned long long key = candidate_key(row[i], i);
+        best = key > best ? key : best;
+    }
+    keys[threadIdx.x] = best;
+    if (threadIdx.x == 0) collected = 0;
+    sort_keys_descending(keys, kSampleThreads);
+    // 0 if fewer than k threads own a finite value: then every finite value is collected.
+    const unsigned long long bound = keys[k - 1];
+    __syncthreads();
+
+    for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
+        const unsigned long long key = candidate_key(row[i], i);
+        if (key != 0ull && key >= bound) {
+            const int at = atomicAdd(&collected, 1);
+            if (at < kCandidateRoom) keys[at] = key;
+        }
+    }
+    __syncthreads();
+    const int found = collected;
+    if (found > kCandidateRoom) {
+        if (threadIdx.x == 0) out_count[blockIdx.x] = -1;
+        return;
+    }
+    int room = 1;
+    while (room < found) room <<= 1;
+    for (int i = found + threadIdx.x; i < room; i += kSampleThreads) keys[i] = 0ull;
+    sort_keys_descending(keys, room);
+    const int kept = found < k ? found : k;
+    for (int i = threadIdx.x; i < kept; i += kSampleThreads) {
+        const int id = static_cast<int>(0xffffffffu - static_cast<unsigned>(keys[i] & 0xffffffffull));
+        out_ids[static_cast<long>(blockIdx.x) * kCandidateMaxK + i] = id;
+        out_values[static_cast<long>(blockIdx.x) * kCandidateMaxK + i] = row[id];
+    }
+    if (threadIdx.x == 0) out_count[blockIdx.x] = kept;
+}
+
 }  // namespace leone
 
 using namespace leone;
+
+extern "C" int leone_top_candidates_max() { return kCandidateMaxK; }
+
+// For each row the wanted[row] (1..leone_top_candidates_max()) best finite logits in the sampler's order,
+// best first: out_values and out_ids hold leone_top_candidates_max() places a row, out_count[row] says how
+// many are filled (fewer than wanted if the row has fewer finite logits), or is -1 if the row's values are
+// laid out so that the selection did not fit: such a row must be selected another way.
+extern "C" int leone_top_candidates(const float* logits, const int* wanted, float* out_values, int* out_ids,
+                                    int* out_count, int rows, int vocab, int max_wanted, hipStream_t stream) {
+    LEONE_REQUIRE(logits && wanted && out_values && out_ids && out_count, "top_candidates: null pointer");
+    LEONE_REQUIRE(rows > 0 && vocab > 0, "top_candidates: rows %d vocab %d must be positive", rows, vocab);
+    LEONE_REQUIRE(max_wanted >= 1 && max_wanted <= kCandidateMaxK,
+                  "top_candidates: %d wanted, at most %d can be selected", max_wanted, kCandidateMaxK);
+    top_candidates_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, wanted, out_values, out_ids, out_count, vocab);
+    LEONE_LAUNCH_CHECK("top_candidates");
+    return 0;
+}
 
 extern "C" int leone_argmax_chunk() { return kArgmaxChunk; }
 

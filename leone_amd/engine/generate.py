@@ -17,6 +17,7 @@ from .. import ops
 from ..ops.profile import Recorder
 from ..sampling import rng
 from ..sampling.sampler import (MirostatState, SamplerError, SamplingParams, apply_penalties, native_eligible,
+                                preselect_count, sample_candidates_native,
                                 sample as host_sample, sample_rows_native)
 from .engine import Engine, StepEntry
 from .scheduler import Finished, PlannedEntry, Reject, Request, Scheduler, SchedulerPolicy
@@ -87,6 +88,23 @@ def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params:
         for i in scaled:
             out[rows[i].request] = picked[i]
     host_rows = [i for i in range(len(rows)) if i not in on_device]
+    # Rows that keep their k best logits before anything else: the device selects those, and only they
+    # come to the host.  A row the selection could not serve goes the long way with the others.
+    narrow = [i for i in host_rows if preselect_count(policies[i], ops.TOP_CANDIDATES_MAX)
+              and rows[i].request not in (controllers or {})]
+    if narrow:
+        index = torch.tensor(narrow, dtype=torch.long, device=logits.device)
+        values, ids, counts = ops.top_candidates(logits.index_select(0, index),
+                                                 [preselect_count(policies[i], ops.TOP_CANDIDATES_MAX) for i in narrow])
+        served = [k for k in range(len(narrow)) if counts[k] >= 0]
+        if served:
+            drawn = sample_candidates_native(values[served], ids[served], counts[served],
+                                             [policies[narrow[k]] for k in served],
+                                             [rows[narrow[k]].sample_position for k in served])
+            for k, token in zip(served, drawn):
+                out[rows[narrow[k]].request] = token
+        done = {narrow[k] for k in served}
+        host_rows = [i for i in host_rows if i not in done]
     if host_rows:
         index = torch.tensor(host_rows, dtype=torch.long, device=logits.device)
         copied = logits.index_select(0, index).cpu().numpy()

@@ -444,4 +444,31 @@ def sample_temperature(logits: torch.Tensor, temperature: torch.Tensor, uniform:
     return out
 
 
+TOP_CANDIDATES_MAX = 256     # most candidates a row the selection kernel gives (checked against the library)
+
+
+def top_candidates(logits: torch.Tensor, wanted) -> tuple:
+    """The ``wanted[row]`` best finite logits of every row in the sampler's order (higher first, the lower
+    id on a tie), selected on the device and brought to the host in one copy.
+
+    Returns numpy arrays: values float32 [rows, TOP_CANDIDATES_MAX], ids int32 likewise, counts int32
+    [rows]; row r is filled up to counts[r], and counts[r] is -1 for a row whose values are laid out so
+    that the selection did not fit, which the caller has to select from the whole row."""
+    if library().leone_top_candidates_max() != TOP_CANDIDATES_MAX:
+        raise KernelError("the kernel library was built for another number of candidates")
+    rows, vocab = logits.shape
+    wanted = [int(k) for k in wanted]
+    if len(wanted) != rows or not all(1 <= k <= TOP_CANDIDATES_MAX for k in wanted):
+        raise KernelError(f"top_candidates: one count in 1..{TOP_CANDIDATES_MAX} for each of {rows} rows, found {wanted}")
+    want = torch.tensor(wanted, dtype=torch.int32, device=logits.device)
+    room = rows * TOP_CANDIDATES_MAX
+    flat = torch.empty((rows + 2 * room,), dtype=torch.int32, device=logits.device)   # counts | values | ids
+    call("leone_top_candidates", _dev(logits, "candidate logits", torch.float32), _dev(want, "wanted"),
+         _dev(flat[rows:rows + room], "candidate values"), _dev(flat[rows + room:], "candidate ids"),
+         _dev(flat[:rows], "candidate counts"), rows, vocab, max(wanted), _stream())
+    host = flat.cpu().numpy()
+    return (host[rows:rows + room].view("float32").reshape(rows, TOP_CANDIDATES_MAX),
+            host[rows + room:].reshape(rows, TOP_CANDIDATES_MAX), host[:rows])
+
+
 __all__ = [name for name in dir() if not name.startswith("_")]

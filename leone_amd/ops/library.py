@@ -39,6 +39,7 @@ _PROTOTYPES = {
     "leone_gemm_fused_bf16": [P, c_int, P, P, c_int, c_float, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "leone_argmax": [P, P, P, P, c_int, c_int, P],
     "leone_sample_temperature": [P, P, P, P, c_int, c_int, P],
+    "leone_top_candidates": [P, P, P, P, P, c_int, c_int, c_int, P],
 }
 
 
@@ -60,6 +61,8 @@ def library() -> ctypes.CDLL:
             lib.leone_attention_prefill_group_tiles.argtypes = []
             lib.leone_attention_prefill_max_splits.restype = c_int
             lib.leone_attention_prefill_max_splits.argtypes = []
+            lib.leone_top_candidates_max.restype = c_int
+            lib.leone_top_candidates_max.argtypes = []
             lib.leone_argmax_chunk.restype = c_int
             lib.leone_argmax_chunk.argtypes = []
             for name, argtypes in _PROTOTYPES.items():

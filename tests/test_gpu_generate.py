@@ -181,6 +181,78 @@ def test_device_sampling_kernels_against_the_double_precision_sampler():
                                   torch.zeros(1, dtype=torch.float64, device="cuda")).tolist() == [-1]
 
 
+def best_in_sampler_order(row, k):
+    """Ids of the k best finite logits: the higher first, the lower id on a tie."""
+    ids = [i for i in range(len(row)) if np.isfinite(row[i])]
+    ids.sort(key=lambda i: (-float(row[i]), i))
+    return ids[:k]
+
+
+def test_top_candidates_kernel():
+    """The device's selection of a row's k best logits against a plain sort: ties, values that are not
+    finite, fewer finite values than k, vocabularies smaller and larger than a workgroup, and a row laid
+    out against the deal of ids to threads, which the kernel hands back."""
+    from leone_amd import ops
+    gen = np.random.default_rng(11)
+    for vocab in (1, 5, 300, 1024, 4097, 151936):
+        rows = 7
+        logits = (gen.standard_normal((rows, vocab)) * 3).astype(np.float32)
+        logits[1] = np.round(logits[1])                                  # many ties
+        logits[2, ::3] = np.nan
+        logits[2, 1::7] = -np.inf
+        logits[3] = 0.0                                                  # all equal, +0 and -0 alike: the lowest ids win
+        logits[3, ::2] = -0.0
+        logits[4, vocab // 3:] = np.inf                                  # few finite values
+        logits[5] = np.sort(logits[5])                                   # ascending: the best come last
+        logits[6] = -np.sort(-logits[6])
+        wanted = [40, 256, 17, 9, 50, 1, 255]
+        values, ids, counts = ops.top_candidates(torch.from_numpy(logits).cuda(), wanted)
+        for r in range(rows):
+            want = best_in_sampler_order(logits[r], wanted[r])
+            assert counts[r] == len(want), (vocab, r, counts[r], len(want))
+            assert ids[r, :counts[r]].tolist() == want, (vocab, r)
+            assert np.array_equal(values[r, :counts[r]], logits[r, want]), (vocab, r)
+    # 39 threads own nothing but large values: the bound falls among the small ones and the large ones
+    # (39 * 148) do not fit the kernel's room.
+    against = np.full((2, 151936), -5.0, dtype=np.float32)
+    against[0, :] = gen.standard_normal(151936).astype(np.float32)
+    for t in range(39):
+        against[1, t::1024] = 50.0 + t
+    values, ids, counts = ops.top_candidates(torch.from_numpy(against).cuda(), [40, 40])
+    assert counts[0] == 40 and counts[1] == -1
+    with pytest.raises(ops.KernelError):
+        ops.top_candidates(torch.from_numpy(against).cuda(), [40, 257])
+
+
+def test_truncated_sampling_takes_the_candidates_and_matches_the_whole_row(folders, monkeypatch):
+    """top-k first: the device selects, the host draws from the selection; the tokens are those of the
+    sampler over whole rows, alone or in a batch, and a row the selection hands back goes the long way."""
+    from leone_amd import ops
+    from leone_amd.api import Runtime, sampling_params
+    from leone_amd.engine import generate
+    folder = folders["B"]
+    config = read_config(folder)
+    prompts = [random_tokens(90 + i, n, config["vocab_size"]) for i, n in enumerate([9, 33, 70])]
+    params = sampling_params(temperature=0.9, seed=4321, top_k=12, top_p=0.85, min_p=0.02)
+    runtime = Runtime.load(folder, "float32", max_tokens=3 * 128, page_tokens=16, max_requests=3)
+    calls = []
+    real = ops.top_candidates
+    monkeypatch.setattr(ops, "top_candidates", lambda *a: calls.append(1) or real(*a))
+    narrow = [r.tokens for r in runtime.generate_tokens(prompts, 20, params, eos_token_id=None)]
+    assert len(calls) >= 20
+    monkeypatch.setattr(generate, "preselect_count", lambda policy, limit: 0)      # everything the long way
+    calls.clear()
+    whole = [r.tokens for r in runtime.generate_tokens(prompts, 20, params, eos_token_id=None)]
+    assert not calls and whole == narrow
+    monkeypatch.undo()
+    # every row handed back: the same tokens again
+    def refused(logits, wanted):
+        values, ids, counts = real(logits, wanted)
+        return values, ids, np.full_like(counts, -1)
+    monkeypatch.setattr(ops, "top_candidates", refused)
+    assert [r.tokens for r in runtime.generate_tokens(prompts, 20, params, eos_token_id=None)] == narrow
+
+
 def test_command_line_generate(folders, tmp_path):
     folder = folders["A"]
     weights, config = read_weights(folder), read_config(folder)
