@@ -124,6 +124,38 @@ def test_prompt_key_ranges_agree_with_plain(cases, monkeypatch, name, schedule):
     compare(steps, outputs, expected, tolerance("bfloat16"), f"{name}/key ranges/{schedule}")
 
 
+def test_late_portions_of_a_long_request(tmp_path):
+    """One request of 2,200 tokens at the large models' head shape: a long first portion, then portions of
+    changing size far into the context, where the prompt kernel cuts the keys into ranges by its own rule,
+    then single tokens."""
+    from leone_amd import ops
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+
+    folder = make_model_dir(str(tmp_path / "long"), dict(TINY["M"], max_position_embeddings=4096), seed=77,
+                            dtype=torch.bfloat16)
+    config, weights = read_config(folder), read_weights(folder)
+    tokens = random_tokens(4242, 2200, config["vocab_size"])
+    expected = {"long": qwen3_plain.forward(weights, config, tokens).numpy()}
+    cuts = [1200, 300, 150, 64, 40, 17, 200, 200] + [1] * 29
+    assert sum(cuts) == len(tokens)
+    steps, at = [], 0
+    for n, size in enumerate(cuts):
+        steps.append({"step": n, "entries": [{"id": "long", "tokens": tokens[at:at + size], "want": list(range(size))}],
+                      "end": ["long"] if at + size == len(tokens) else []})
+        at += size
+    chosen = []
+    choose = ops.choose_prefill_splits
+    ops.choose_prefill_splits = lambda *a, **k: chosen.append(choose(*a, **k)) or chosen[-1]
+    try:
+        engine = Engine(load_model(folder, "bfloat16"), max_tokens=2240, page_tokens=64, max_requests=1)
+        outputs = run_steps(engine, steps)
+    finally:
+        ops.choose_prefill_splits = choose
+    assert chosen[0] == 1 and max(chosen) >= 2, chosen
+    compare(steps, outputs, expected, tolerance("bfloat16"), "long request in late portions")
+
+
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 def test_rerun_is_bitwise_identical(cases, dtype_name):
     from leone_amd.engine.engine import Engine
