@@ -532,7 +532,7 @@ def test_gemm_fused_gated(mfk):
     inv = 1.0 / torch.sqrt((stream.double() ** 2).mean(dim=1, keepdim=True) + 1e-6)
     want = plain.swiglu((operand @ wg.double().T) * inv, (operand @ wu.double().T) * inv)
     close(out, want, 1e-2, 1e-2, "gated product")
-    # through linear(): the same call falls back to product + swiglu kernel beyond 16 rows
+    # through linear(): the same call falls back to product + swiglu kernel beyond ops.FUSED_ROWS rows
     many = torch.randn(40, k, device=DEV)
     lazy40 = ops.NormedRows(many, gain, 1e-6, torch.bfloat16)
     got = ops.linear(lazy40, w, gated=True)

@@ -511,6 +511,7 @@ def test_position_part():
 def test_block_part(dtype, rows):
     """One pre-norm block alone: x1 = x + attention(norm1 x), x2 = x1 + feed_forward(norm2 x1).  With few
     rows the bfloat16 products add into the stream themselves; with many the block hands back a delta."""
+    from leone_amd import ops
     from leone_amd.parts import BLOCKS, POSITIONS, PartSpec
     from leone_amd.parts.context import KvCacheView
     hidden, heads, kv, dim, ffn, page = 64, 4, 2, 16, 96, 16
@@ -541,7 +542,7 @@ def test_block_part(dtype, rows):
     pending = block.forward(x, None, step, cache)
     got = x.cpu().double() + (0 if pending is None else pending.cpu().double())
     if dtype == torch.bfloat16:
-        assert (pending is None) == (rows <= 16)
+        assert (pending is None) == (rows <= ops.FUSED_ROWS)
     wf = {k: v.float() for k, v in w.items()}
     cfg = dict(num_attention_heads=heads, num_key_value_heads=kv, head_dim=dim, rms_norm_eps=1e-5, rope_theta=1e4)
     x1 = x0.double() + plain.attention_block(plain.rms_norm(x0, wf["n1"], 1e-5), wf, "a", cfg, list(range(rows)))
