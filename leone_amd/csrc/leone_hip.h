@@ -86,14 +86,18 @@ int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const voi
 int leone_argmax_chunk();
 int leone_argmax(const float* logits, int* out, float* part_value, int* part_index, int rows, int vocab,
                  hipStream_t stream);
+// The token whose share of the weights exp(l / t - max / t), walked in id order, holds uniform[row]; -1 for a
+// row without a finite logit.  Workspace: part_value and part_index as for leone_argmax, best with one
+// entry a row, sums with rows * ceil(vocab / leone_argmax_chunk()) doubles.
 int leone_sample_temperature(const float* logits, const double* temperature, const double* uniform, int* out,
-                             int rows, int vocab, hipStream_t stream);
+                             float* part_value, int* part_index, int* best, double* sums, int rows, int vocab,
+                             hipStream_t stream);
 
-// The wanted[row] best finite logits of each row (higher first, lower id on a tie), best first, for a
-// sampler that truncates to the k best before anything else.  out_values and out_ids have
+// The `wanted` best finite logits of each row (higher first, lower id on a tie), best first, for a sampler
+// that truncates to the k best before anything else.  out_values and out_ids have
 // leone_top_candidates_max() places a row; out_count[row] is the number filled, or -1 for a row that has
-// to be selected another way.  max_wanted: the largest of wanted[], checked against the limit.
+// to be selected another way.
 int leone_top_candidates_max();
-int leone_top_candidates(const float* logits, const int* wanted, float* out_values, int* out_ids, int* out_count,
-                         int rows, int vocab, int max_wanted, hipStream_t stream);
+int leone_top_candidates(const float* logits, float* out_values, int* out_ids, int* out_count, int rows, int vocab,
+                         int wanted, hipStream_t stream);
 }

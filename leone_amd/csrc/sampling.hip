@@ -81,82 +81,117 @@ argmax_final_kernel(const float* __restrict__ part_value, const int* __restrict_
     if (threadIdx.x == 0) out[blockIdx.x] = total.index;
 }
 
-// Thread t owns the ids [t * chunk, (t + 1) * chunk): running sums follow id order.
-__global__ void __launch_bounds__(kSampleThreads)
-sample_temperature_kernel(const float* __restrict__ logits, const double* __restrict__ temperature,
-                          const double* __restrict__ uniform, int* __restrict__ out, int vocab) {
-    __shared__ Best scratch[kSampleThreads / kWave];
-    __shared__ double sums[kSampleThreads];
-    __shared__ int last_finite[kSampleThreads];
-    __shared__ int chosen_thread;
-    __shared__ double chosen_before, target;
-
-    const float* row = logits + static_cast<long>(blockIdx.x) * vocab;
-    const double t = temperature[blockIdx.x];
-    const int chunk = (vocab + kSampleThreads - 1) / kSampleThreads;
-    const int begin = threadIdx.x * chunk;
-    const int end = begin + chunk < vocab ? begin + chunk : vocab;
-
-    Best mine{0.f, -1};
-    int last = -1;
-    for (int i = begin; i < end; ++i) {
-        const float v = row[i];
-        if (!isfinite(v)) continue;
-        last = i;
-        if (mine.index < 0 || v > mine.value) mine = Best{v, i};
+// Temperature sampling, three steps: the row's highest logit (the two argmax kernels), then the sum of
+// the weights of every chunk of 4096 ids (one workgroup a chunk), then one workgroup a row walks the chunk
+// sums in id order to the chunk that holds the drawn value, and inside it the sums of its 16 waves, of the
+// wave's 64 threads and the thread's 4 ids.  Sums are always taken in the same order (ids of a thread, threads
+// of a wave, waves of a chunk, chunks of a row, each from the left), in both kernels, so that what the walk
+// adds up is what was summed.  Where rounding lets the walk end without crossing the drawn value, the last
+// token with a weight above zero is taken.
+__device__ inline void chunk_weights(const float* row, int vocab, int chunk, double t, double highest, double w[4]) {
+    const int base = chunk * kArgmaxChunk + 4 * static_cast<int>(threadIdx.x);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int id = base + i;
+        const float v = id < vocab ? row[id] : NAN;
+        w[i] = isfinite(v) ? exp(static_cast<double>(v) / t - highest) : 0.0;
     }
-    const Best top = block_best(mine, scratch);
-    if (top.index < 0) {
-        if (threadIdx.x == 0) out[blockIdx.x] = -1;
+}
+
+// thread_sum[t] = the weights of thread t's ids, wave_sum[v] = the thread sums of wave v from the left.
+__device__ inline void chunk_sums_in_order(const double w[4], double* thread_sum, double* wave_sum) {
+    thread_sum[threadIdx.x] = ((w[0] + w[1]) + w[2]) + w[3];
+    __syncthreads();
+    if (threadIdx.x % kWave == 0) {
+        double sum = 0.0;
+        for (int i = 0; i < kWave; ++i) sum += thread_sum[threadIdx.x + i];
+        wave_sum[threadIdx.x / kWave] = sum;
+    }
+    __syncthreads();
+}
+
+__global__ void __launch_bounds__(kSampleThreads)
+temperature_sums_kernel(const float* __restrict__ logits, const double* __restrict__ temperature,
+                        const int* __restrict__ best, double* __restrict__ sums, int vocab, int chunks) {
+    __shared__ double thread_sum[kSampleThreads];
+    __shared__ double wave_sum[kSampleThreads / kWave];
+    const int r = blockIdx.y, chunk = blockIdx.x;
+    const float* row = logits + static_cast<long>(r) * vocab;
+    const int top = best[r];
+    if (top < 0) return;                                    // no finite logit: the row's answer is -1
+    const double t = temperature[r];
+    double w[4];
+    chunk_weights(row, vocab, chunk, t, static_cast<double>(row[top]) / t, w);
+    chunk_sums_in_order(w, thread_sum, wave_sum);
+    if (threadIdx.x == 0) {
+        double sum = 0.0;
+        for (int v = 0; v < kSampleThreads / kWave; ++v) sum += wave_sum[v];
+        sums[static_cast<long>(r) * chunks + chunk] = sum;
+    }
+}
+
+// In `sum[0, n)`, walked from the left with `running` as the sum before: the first positive entry that takes
+// the running sum above `target`, or the last positive entry; `running` ends as the sum before that entry.
+__device__ inline int walk_to(const double* sum, int n, double target, double& running) {
+    int at = -1;
+    double before = running;
+    for (int i = 0; i < n; ++i) {
+        const double s = sum[i];
+        if (!(s > 0.0)) continue;
+        at = i;
+        before = running;
+        if (target < running + s) break;
+        running += s;
+    }
+    running = before;
+    return at;
+}
+
+__global__ void __launch_bounds__(kSampleThreads)
+temperature_pick_kernel(const float* __restrict__ logits, const double* __restrict__ temperature,
+                        const double* __restrict__ uniform, const int* __restrict__ best,
+                        const double* __restrict__ sums, int* __restrict__ out, int vocab, int chunks) {
+    __shared__ double thread_sum[kSampleThreads];
+    __shared__ double wave_sum[kSampleThreads / kWave];
+    __shared__ int chosen_chunk, chosen_thread;
+    __shared__ double chosen_before, target;
+    const int r = blockIdx.x;
+    const float* row = logits + static_cast<long>(r) * vocab;
+    const int top = best[r];
+    if (top < 0) {
+        if (threadIdx.x == 0) out[r] = -1;
         return;
     }
-    const double highest = static_cast<double>(top.value) / t;
-    double sum = 0.0;
-    for (int i = begin; i < end; ++i) {
-        const float v = row[i];
-        if (isfinite(v)) sum += exp(static_cast<double>(v) / t - highest);
-    }
-    sums[threadIdx.x] = sum;
-    last_finite[threadIdx.x] = last;
-    __syncthreads();
+    const double* mine = sums + static_cast<long>(r) * chunks;
     if (threadIdx.x == 0) {
         double total = 0.0;
-        for (int i = 0; i < kSampleThreads; ++i) total += sums[i];
-        target = uniform[blockIdx.x] * total;
+        for (int c = 0; c < chunks; ++c) total += mine[c];
+        target = uniform[r] * total;
         double running = 0.0;
-        int pick = -1;
-        for (int i = 0; i < kSampleThreads; ++i) {
-            if (sums[i] > 0.0 && target < running + sums[i]) {
-                pick = i;
-                break;
-            }
-            running += sums[i];
-        }
-        chosen_thread = pick;
+        chosen_chunk = walk_to(mine, chunks, target, running);   // the highest logit weighs 1: some chunk is positive
         chosen_before = running;
-        if (pick < 0) {  // rounding left the running sum short: the last eligible token
-            int fallback = -1;
-            for (int i = 0; i < kSampleThreads; ++i)
-                if (last_finite[i] > fallback) fallback = last_finite[i];
-            out[blockIdx.x] = fallback;
-        }
+        if (chosen_chunk < 0) out[r] = top;                      // sums that are not numbers (a temperature the host let through)
+    }
+    __syncthreads();
+    const int chunk = chosen_chunk;
+    if (chunk < 0) return;
+    const double t = temperature[r];
+    double w[4];
+    chunk_weights(row, vocab, chunk, t, static_cast<double>(row[top]) / t, w);
+    chunk_sums_in_order(w, thread_sum, wave_sum);
+    if (threadIdx.x == 0) {
+        double running = chosen_before;
+        const int wave = walk_to(wave_sum, kSampleThreads / kWave, target, running);
+        const int lane = wave < 0 ? -1 : walk_to(thread_sum + wave * kWave, kWave, target, running);
+        chosen_thread = lane < 0 ? -1 : wave * kWave + lane;
+        chosen_before = running;
+        if (lane < 0) out[r] = top;
     }
     __syncthreads();
     if (static_cast<int>(threadIdx.x) == chosen_thread) {
         double running = chosen_before;
-        int token = last;
-        for (int i = begin; i < end; ++i) {
-            const float v = row[i];
-            if (!isfinite(v)) continue;
-            const double w = exp(static_cast<double>(v) / t - highest);
-            if (w <= 0.0) continue;
-            running += w;
-            if (target < running) {
-                token = i;
-                break;
-            }
-        }
-        out[blockIdx.x] = token;
+        const int at = walk_to(w, 4, target, running);
+        out[r] = at < 0 ? top : chunk * kArgmaxChunk + 4 * static_cast<int>(threadIdx.x) + at;
     }
 }
 
@@ -204,13 +239,11 @@ __device__ inline void sort_keys_descending(unsigned long long* keys, int n) {
 }
 
 __global__ void __launch_bounds__(kSampleThreads)
-top_candidates_kernel(const float* __restrict__ logits, const int* __restrict__ wanted, float* __restrict__ out_values,
+top_candidates_kernel(const float* __restrict__ logits, int k, float* __restrict__ out_values,
                       int* __restrict__ out_ids, int* __restrict__ out_count, int vocab) {
     __shared__ unsigned long long keys[kCandidateRoom];
     __shared__ int collected;
     const float* row = logits + static_cast<long>(blockIdx.x) * vocab;
-    int k = wanted[blockIdx.x];
-    k = k < 1 ? 1 : (k > kCandidateMaxK ? kCandidateMaxK : k);   // the host checks; no index may depend on it
 
     unsigned long long best = 0ull;
     for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
@@ -256,16 +289,17 @@ using namespace leone;
 
 extern "C" int leone_top_candidates_max() { return kCandidateMaxK; }
 
-// For each row the wanted[row] (1..leone_top_candidates_max()) best finite logits in the sampler's order,
-// best first: out_values and out_ids hold leone_top_candidates_max() places a row, out_count[row] says how
-// many are filled (fewer than wanted if the row has fewer finite logits), or is -1 if the row's values are
-// laid out so that the selection did not fit: such a row must be selected another way.
-extern "C" int leone_top_candidates(const float* logits, const int* wanted, float* out_values, int* out_ids,
-                                    int* out_count, int rows, int vocab, int max_wanted, hipStream_t stream) {
-    LEONE_REQUIRE(logits && wanted && out_values && out_ids && out_count, "top_candidates: null pointer");
+// For each row the `wanted` (1..leone_top_candidates_max()) best finite logits in the sampler's order,
+// best first (so that the first j of them are the row's j best): out_values and out_ids hold
+// leone_top_candidates_max() places a row, out_count[row] says how many are filled (fewer than wanted if
+// the row has fewer finite logits), or is -1 if the row's values are laid out so that the selection did
+// not fit: such a row must be selected another way.
+extern "C" int leone_top_candidates(const float* logits, float* out_values, int* out_ids, int* out_count, int rows,
+                                    int vocab, int wanted, hipStream_t stream) {
+    LEONE_REQUIRE(logits && out_values && out_ids && out_count, "top_candidates: null pointer");
     LEONE_REQUIRE(rows > 0 && vocab > 0, "top_candidates: rows %d vocab %d must be positive", rows, vocab);
-    LEONE_REQUIRE(max_wanted >= 1 && max_wanted <= kCandidateMaxK,
-                  "top_candidates: %d wanted, at most %d can be selected", max_wanted, kCandidateMaxK);
+    LEONE_REQUIRE(wanted >= 1 && wanted <= kCandidateMaxK,
+                  "top_candidates: %d wanted, at most %d can be selected", wanted, kCandidateMaxK);
     top_candidates_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, wanted, out_values, out_ids, out_count, vocab);
     LEONE_LAUNCH_CHECK("top_candidates");
     return 0;
@@ -286,11 +320,22 @@ extern "C" int leone_argmax(const float* logits, int* out, float* part_value, in
     return 0;
 }
 
+// Workspace: part_value and part_index as for leone_argmax, best with one entry a row, sums with
+// rows * ceil(vocab / leone_argmax_chunk()) doubles.
 extern "C" int leone_sample_temperature(const float* logits, const double* temperature, const double* uniform,
-                                        int* out, int rows, int vocab, hipStream_t stream) {
-    LEONE_REQUIRE(logits && temperature && uniform && out, "sample_temperature: null pointer");
-    LEONE_REQUIRE(rows > 0 && vocab > 0, "sample_temperature: rows %d vocab %d must be positive", rows, vocab);
-    sample_temperature_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, temperature, uniform, out, vocab);
+                                        int* out, float* part_value, int* part_index, int* best, double* sums,
+                                        int rows, int vocab, hipStream_t stream) {
+    LEONE_REQUIRE(logits && temperature && uniform && out && part_value && part_index && best && sums,
+                  "sample_temperature: null pointer");
+    LEONE_REQUIRE(rows > 0 && rows <= 65535 && vocab > 0, "sample_temperature: rows %d vocab %d out of range", rows, vocab);
+    const int chunks = ceil_div(vocab, kArgmaxChunk);
+    argmax_partial_kernel<<<dim3(chunks, rows), kSampleThreads, 0, stream>>>(logits, part_value, part_index, vocab, chunks);
+    LEONE_LAUNCH_CHECK("sample_temperature");
+    argmax_final_kernel<<<rows, kSampleThreads, 0, stream>>>(part_value, part_index, best, chunks);
+    LEONE_LAUNCH_CHECK("sample_temperature");
+    temperature_sums_kernel<<<dim3(chunks, rows), kSampleThreads, 0, stream>>>(logits, temperature, best, sums, vocab, chunks);
+    LEONE_LAUNCH_CHECK("sample_temperature");
+    temperature_pick_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, temperature, uniform, best, sums, out, vocab, chunks);
     LEONE_LAUNCH_CHECK("sample_temperature");
     return 0;
 }

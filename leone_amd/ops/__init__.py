@@ -8,6 +8,7 @@ from __future__ import annotations
 
 from typing import Optional
 
+import numpy as np
 import torch
 
 from . import profile
@@ -440,11 +441,19 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 
 
 def sample_temperature(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor) -> torch.Tensor:
+    """One token a row by its temperature (float64 [rows], positive) and uniform value (float64 [rows] in
+    [0, 1)); -1 for a row without a finite logit."""
     rows, vocab = logits.shape
+    chunks = -(-vocab // library().leone_argmax_chunk())
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    part_value = torch.empty((rows * chunks,), dtype=torch.float32, device=logits.device)
+    part_index = torch.empty((rows * (chunks + 1),), dtype=torch.int32, device=logits.device)   # and the best of each row
+    sums = torch.empty((rows * chunks,), dtype=torch.float64, device=logits.device)
     call("leone_sample_temperature", _dev(logits, "sample logits", torch.float32),
          _dev(temperature, "sample temperature", torch.float64, (rows,)),
-         _dev(uniform, "sample uniform", torch.float64, (rows,)), _dev(out, "sample out"), rows, vocab, _stream())
+         _dev(uniform, "sample uniform", torch.float64, (rows,)), _dev(out, "sample out"),
+         _dev(part_value, "sample partial values"), _dev(part_index[:rows * chunks], "sample partial indices"),
+         _dev(part_index[rows * chunks:], "sample best"), _dev(sums, "sample sums"), rows, vocab, _stream())
     return out
 
 
@@ -464,15 +473,16 @@ def top_candidates(logits: torch.Tensor, wanted) -> tuple:
     wanted = [int(k) for k in wanted]
     if len(wanted) != rows or not all(1 <= k <= TOP_CANDIDATES_MAX for k in wanted):
         raise KernelError(f"top_candidates: one count in 1..{TOP_CANDIDATES_MAX} for each of {rows} rows, found {wanted}")
-    want = torch.tensor(wanted, dtype=torch.int32, device=logits.device)
     room = rows * TOP_CANDIDATES_MAX
     flat = torch.empty((rows + 2 * room,), dtype=torch.int32, device=logits.device)   # counts | values | ids
-    call("leone_top_candidates", _dev(logits, "candidate logits", torch.float32), _dev(want, "wanted"),
+    # The kernel selects the largest count for every row, best first: a row that wants fewer takes the first.
+    call("leone_top_candidates", _dev(logits, "candidate logits", torch.float32),
          _dev(flat[rows:rows + room], "candidate values"), _dev(flat[rows + room:], "candidate ids"),
          _dev(flat[:rows], "candidate counts"), rows, vocab, max(wanted), _stream())
     host = flat.cpu().numpy()
+    counts = np.where(host[:rows] < 0, -1, np.minimum(host[:rows], np.asarray(wanted, dtype=np.int32)))
     return (host[rows:rows + room].view("float32").reshape(rows, TOP_CANDIDATES_MAX),
-            host[rows + room:].reshape(rows, TOP_CANDIDATES_MAX), host[:rows])
+            host[rows + room:].reshape(rows, TOP_CANDIDATES_MAX), counts)
 
 
 __all__ = [name for name in dir() if not name.startswith("_")]

@@ -38,8 +38,8 @@ _PROTOTYPES = {
     "leone_gemm_skinny_bf16": [P, P, P, c_int, c_int, c_int, c_int, P],
     "leone_gemm_fused_bf16": [P, c_int, P, P, c_int, c_float, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "leone_argmax": [P, P, P, P, c_int, c_int, P],
-    "leone_sample_temperature": [P, P, P, P, c_int, c_int, P],
-    "leone_top_candidates": [P, P, P, P, P, c_int, c_int, c_int, P],
+    "leone_sample_temperature": [P, P, P, P, P, P, P, P, c_int, c_int, P],
+    "leone_top_candidates": [P, P, P, P, c_int, c_int, c_int, P],
 }
 
 
