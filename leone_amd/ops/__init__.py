@@ -40,7 +40,14 @@ def _dev(t: Optional[torch.Tensor], what: str, dtype=None, shape=None) -> int:
     return t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """The current stream's handle.  Asked for before every launch, so the short way is taken where this
+    torch has it (a tenth of the time of building a Stream object)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
