@@ -11,8 +11,14 @@
 //           gated    : W holds, in every block of 16 rows, 8 gate rows then the 8 up rows that belong to
 //                      them; Y[M,N/2] = silu(gate) * up (crates/leone/src/cpu.rs:892-907)
 //
-// Structure and operand layout are those of gemm_skinny.hip: a workgroup owns 16 rows of W, its waves
-// split K in steps of 64 elements, partial tiles are added in wave order in shared memory.
+// The weight matrix is streamed once; this is the place of the reference's row-per-block matrix-vector
+// kernels (crates/leone-cuda/cuda/ie_cuda.cu:1719, launch shape :6178-6205).  A workgroup owns 16 rows of W
+// and splits K between its waves in steps of 64 elements; a wave computes Y^T tiles (16 rows of W x 16 rows
+// of X) with v_mfma_f32_16x16x32_bf16, W as the A operand, X as the B operand.  Lane (c, g) reads 32
+// contiguous bytes of weight row c per step (elements 16g .. 16g+15 of the step), so a row's four lanes take
+// a whole 128-byte line; both operands use the same assignment of elements to k-slots, which is all the
+// instruction needs.  The partial tiles are added in wave order in shared memory, so a launch repeats bit
+// for bit.
 #include "common.h"
 #include "leone_hip.h"
 
@@ -191,7 +197,7 @@ static void launch_fused(const FusedArgs& a, hipStream_t stream) {
     const int tiles = ceil_div(a.n, 16);
     const int steps = ceil_div(a.k, 64);
     const bool tail = a.k % 64 != 0;
-    const bool many = tiles * 4 >= 4096 || steps < 16;    // as in gemm_skinny: few rows of W split K further
+    const bool many = tiles * 4 >= 4096 || steps < 16;    // matrices with few rows split K over eight waves, so that the chip is filled
 #define LEONE_FUSED(TAIL, WAVES) \
     gemm_fused_kernel<kIn, kOut, TAIL, WAVES, TOut><<<tiles, WAVES * kWave, 0, stream>>>(a)
     if (many) {

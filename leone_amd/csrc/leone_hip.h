@@ -69,11 +69,7 @@ int leone_attention_prefill(const void* q, void* out, const void* k_pool, const 
 // C[M,N] = A[M,K] . B[N,K]^T in float.
 int leone_gemm_f32(const float* a, const float* b, float* c, int m, int n, int k, hipStream_t stream);
 
-// Y[M,N] = X[M,K] . W[N,K]^T for bfloat16 X and W, M <= 64, K a multiple of 8; Y float or bfloat16.
-int leone_gemm_skinny_bf16(const void* x, const void* w, void* y, int out_dtype, int m, int n, int k,
-                           hipStream_t stream);
-
-// The same product for M <= 16 with row-wise neighbours folded in.  in_mode 0: x is bfloat16 [M,K];
+// Y[M,N] = X[M,K] . W[N,K]^T for bfloat16 W, M <= 16, K a multiple of 8, with row-wise neighbours folded in.  in_mode 0: x is bfloat16 [M,K];
 // 1: x is the float32 stream (row r reads rows[r] if rows is given), the operand is x * gain and the
 // result is scaled by 1/sqrt(mean(x^2) + eps).  out_mode 0: y[M,N] of out_dtype; 1: y float32 [M,N] +=
 // product; 2: W interleaves 8 gate rows with their 8 up rows, y bfloat16 [M,N/2] = silu(gate) * up.

@@ -312,7 +312,6 @@ def gemm_f32(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = Non
     return out
 
 
-SKINNY_ROWS = 64           # most rows one launch of the weight-streaming kernel takes
 # Up to here norm, gate and residual are folded into the weight-streaming kernel (which takes up to 16 rows).
 # Beyond, its reads of X weigh as much as those of W and the library's product with separate row-wise kernels
 # is faster (measured at the 8B shape: 6.02 against 6.38 ms a step at 8 rows, 6.71 : 6.82 at 10, 7.57 : 7.36 at 12,
@@ -345,21 +344,6 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     if ffn % 8 or up.shape != gate.shape:
         raise KernelError(f"gate and up must both be [F, H] with F a multiple of 8, found {tuple(gate.shape)}")
     return torch.stack([gate.view(ffn // 8, 8, hidden), up.view(ffn // 8, 8, hidden)], dim=1).reshape(2 * ffn, hidden)
-
-
-def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,
-                out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x[M,K] . weight[N,K]^T on the matrix cores for M <= 64 (bfloat16 in, float accumulation)."""
-    m, k = x.shape
-    n, k2 = weight.shape
-    if k != k2:
-        raise KernelError(f"gemm_skinny: inner sizes {k} and {k2} differ")
-    if out is None:
-        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-    with profile.span("gemv", weight):
-        call("leone_gemm_skinny_bf16", _dev(x, "gemm x", torch.bfloat16), _dev(weight, "gemm weight", torch.bfloat16),
-             _dev(out, "gemm out", out_dtype, (m, n)), _CODES[out_dtype], m, n, k, _stream())
-    return out
 
 
 def gemm_fused(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,

@@ -28,14 +28,13 @@ OPERATIONS = {
     "leone_attention_rows": "attention",
     "leone_attention_prefill": "attention",
     "leone_gemm_fused_bf16": "gemv fused",
-    "leone_gemm_skinny_bf16": "gemv",
     "leone_gemm_f32": "gemm f32",
     "leone_swiglu": "swiglu",
     "leone_argmax": "argmax",
     "leone_sample_temperature": "sample",
 }
 LIBRARY_PRODUCT = "gemm library"
-ORDER = ["embed", "norm", "gemv fused", "gemv", LIBRARY_PRODUCT, "gemm f32", "qknorm rope kv", "attention", "swiglu",
+ORDER = ["embed", "norm", "gemv fused", LIBRARY_PRODUCT, "gemm f32", "qknorm rope kv", "attention", "swiglu",
          "argmax", "sample"]
 
 

@@ -378,24 +378,25 @@ def test_attention_finds_the_one_key_that_matters(kernel):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("mnk", [(1, 777, 80), (5, 64, 64), (8, 6144, 4096), (16, 1000, 96), (17, 130, 1032),
-                                 (33, 48, 176), (64, 4096, 12288), (1, 151936, 256), (3, 20, 8)])
-def test_gemm_skinny(mnk, out_dtype):
-    """Inputs rounded to bfloat16 as the kernel sees them, products summed in double
-    (the reference's way for its matrix-core product, crates/leone-cuda/tests/gpu.rs:287-386)."""
+@pytest.mark.parametrize("mnk", [(1, 777, 80), (5, 64, 64), (8, 6144, 4096), (16, 1000, 96), (13, 130, 1032),
+                                 (9, 48, 176), (16, 4096, 12288), (1, 151936, 256), (3, 20, 8)])
+def test_gemm_fused_plain(mnk, out_dtype):
+    """The weight-streaming product with nothing folded in.  Inputs rounded to bfloat16 as the kernel sees
+    them, products summed in double (the reference's way for its matrix-core product,
+    crates/leone-cuda/tests/gpu.rs:287-386)."""
     from leone_amd import ops
     m, n, k = mnk
     torch.manual_seed(8)
     x, w = torch.randn(m, k, device=DEV).bfloat16(), (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
-    out = ops.gemm_skinny(x, w, out_dtype)
+    out = ops.gemm_fused(x, w, out_dtype)
     want = x.double() @ w.double().T
     if out_dtype == torch.float32:
-        close(out, want, 2e-6 * k, 1e-5, "gemm_skinny")
+        close(out, want, 2e-6 * k, 1e-5, "gemm_fused")
     else:
-        close(out, want, 2e-6 * k + 1e-3, 8e-3, "gemm_skinny bf16")
-    assert torch.equal(out, ops.gemm_skinny(x, w, out_dtype))
+        close(out, want, 2e-6 * k + 1e-3, 8e-3, "gemm_fused bf16")
+    assert torch.equal(out, ops.gemm_fused(x, w, out_dtype))
     # a row alone gives the same bits as the row inside a batch (crates/leone-cuda/tests/gpu.rs:770)
-    assert torch.equal(ops.gemm_skinny(x[m - 1:m].contiguous(), w, out_dtype)[0], out[m - 1])
+    assert torch.equal(ops.gemm_fused(x[m - 1:m].contiguous(), w, out_dtype)[0], out[m - 1])
 
 
 @pytest.mark.parametrize("splits", [1, 2, 5, 32])
@@ -496,7 +497,7 @@ def test_gemm_fused_norm_and_store(mnk, gain_dtype):
         close(out, want, 2e-6 * k, 2e-5, "norm + product")
         assert torch.equal(out, ops.gemm_fused(lazy, w, torch.float32))
         # and it agrees with the unfused pair within bfloat16 rounding of the normalised rows
-        unfused = ops.gemm_skinny(lazy.materialize(), w, torch.float32)
+        unfused = ops.gemm_fused(lazy.materialize(), w, torch.float32)
         close(out, unfused.double(), 2e-2 * math.sqrt(k) * 0.05 * 3, 2e-2, "fused against unfused")
 
 
