@@ -55,3 +55,37 @@ def test_bench_arithmetic():
     assert abs(benchmark.decode_bytes(c, 1, 0, 2) / 1e9 - 15.14) < 0.01
     assert benchmark.decode_bytes(c, 8, 100, 2) - benchmark.decode_bytes(c, 8, 0, 2) == 8 * 100 * 147456
     assert abs(benchmark.prefill_flops(c, 2048) / 2.97e13 - 1) < 0.01
+
+
+def test_decode_profile_report():
+    """The table of `generate --profile-decode`: totals, shares, the host gap, and weight GB/s by shape."""
+    from leone_amd.ops.profile import ProductTiming, StepProfile
+    profile = StepProfile(steps=4, tokens=4, wall_seconds=0.010, launches=40,
+                          seconds_by_operation={"attention": 0.002, "gemv fused": 0.006, "zeta": 0.001},
+                          products={("gemv fused", 1000, 500, 2): ProductTiming(calls=8, seconds=0.004)})
+    assert abs(profile.gpu_seconds - 0.009) < 1e-12 and abs(profile.host_gap_seconds - 0.001) < 1e-12
+    assert profile.operations() == ["gemv fused", "attention", "zeta"]          # known ones in their order, then the rest
+    lines = profile.lines()
+    assert "decode profile: 4 evaluations" in lines[1]
+    fused = next(line for line in lines if line.strip().startswith("gemv fused") and "%" in line).split()
+    assert fused[-3:] == ["6.000", "1500.000", "66.67%"]
+    gap = next(line for line in lines if "host gap" in line).split()
+    assert gap[-2:] == ["1.000", "250.000"]
+    traffic = lines[-1].split()
+    assert traffic[-5:] == ["1000", "500", "8", "4.000", "2.0"]                 # 8 calls x 1 MB in 4 ms
+
+
+def test_key_ranges_of_the_prompt_kernel_are_chosen_by_rows_and_keys():
+    from leone_amd import ops
+    heads = 32
+    assert ops.choose_prefill_splits(16, heads, 1024) == 1                       # 2,048 rows fill the chip by themselves
+    assert ops.choose_prefill_splits(4, heads, 256) == 1                         # a prompt's first portion: few keys a row
+    assert ops.choose_prefill_splits(4, heads, 30720 + 256) == 4                 # 512 rows far into a long prompt
+    assert ops.choose_prefill_splits(1, heads, 8192) == 16
+    assert ops.choose_prefill_splits(1, 1, 10**6) == ops.PREFILL_MAX_SPLITS
+    assert ops.choose_prefill_splits(1, heads, 100000, window=128) == 1          # a window bounds the keys a row sees
+    for groups in (1, 2, 3, 7, 16, 40):
+        for keys in (1, 63, 64, 1000, 5000, 200000):
+            splits = ops.choose_prefill_splits(groups, heads, keys)
+            assert 1 <= splits <= ops.PREFILL_MAX_SPLITS
+            assert splits == 1 or (splits * groups * heads <= 512 and -(-keys // 64) // splits >= ops.PREFILL_SPLIT_MIN_STAGES)
