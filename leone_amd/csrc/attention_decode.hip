@@ -12,7 +12,9 @@
 // query heads of its group.  The waves' partial results are
 // merged in shared memory, the splits' by a second kernel, both in a fixed
 // order (the reference's partial + reduce pair:
-// crates/leone-cuda/cuda/ie_cuda.cu:4465, 4769).
+// crates/leone-cuda/cuda/ie_cuda.cu:4465, 4769).  (Letting the workgroup that
+// finishes last do the merge was measured: the device-wide fences it needs
+// cost far more than the second launch, 8.8 against 6.0 ms a step.)
 //
 // Operand layouts of the 16x16x32 instruction (lane l, c = l % 16, g = l / 16):
 //   A: row c,    k-slots 8g .. 8g+7        B: column c, k-slots 8g .. 8g+7
@@ -50,8 +52,8 @@ __global__ void __launch_bounds__(kDecodeThreads)
 attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
                         const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
                         const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
-                        float* __restrict__ part_acc, float* __restrict__ part_ml, int q_heads, int kv_heads,
-                        int page_shift, float scale, int window, int splits) {
+                        float* __restrict__ part_acc, float* __restrict__ part_ml, bf16_t* __restrict__ out,
+                        int q_heads, int kv_heads, int page_shift, float scale, int window, int splits) {
     constexpr int kD = kD16 * 16;
     constexpr int kSteps = (kD16 + 1) / 2;           // 32-element steps of the q.k product
     extern __shared__ float smem[];                   // [waves][columns][kD] accumulators, then m and l
@@ -250,7 +252,12 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                 den += sm_l[w * cols + col] * wgt;
             }
         }
-        const long slot = (static_cast<long>(row) * q_heads + kvh * group + col0 + col) * splits + split;
+        const long rh = static_cast<long>(row) * q_heads + kvh * group + col0 + col;
+        if (splits == 1) {                            // nothing to merge with: this is the result
+            out[rh * kD + d] = from_float<bf16_t>(num / den);
+            continue;
+        }
+        const long slot = rh * splits + split;
         part_acc[slot * kD + d] = num;
         if (d == 0) {
             part_ml[slot * 2] = top;
@@ -299,29 +306,30 @@ static size_t decode_smem_bytes(int head_dim, int group, int max_blocks) {
 template <int kD16>
 static void launch_decode(const void* q, const void* k_pool, const void* v_pool, const int* positions,
                           const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
-                          float* part_ml, int rows, int q_heads, int kv_heads, int page_shift, float scale,
+                          float* part_ml, void* out, int rows, int q_heads, int kv_heads, int page_shift, float scale,
                           int window, int splits, hipStream_t stream) {
     const int group = q_heads / kv_heads;
     dim3 grid(rows, kv_heads * ((group + 15) / 16), splits);
     const size_t smem = decode_smem_bytes(kD16 * 16, group, max_blocks);
     attention_decode_kernel<kD16><<<grid, kDecodeThreads, smem, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
-        positions, row_entry, block_table, max_blocks, part_acc, part_ml, q_heads, kv_heads, page_shift, scale, window,
-        splits);
+        positions, row_entry, block_table, max_blocks, part_acc, part_ml, static_cast<bf16_t*>(out), q_heads, kv_heads,
+        page_shift, scale, window, splits);
 }
 
 }  // namespace leone
 
 using namespace leone;
 
-// Workspace: part_acc holds rows*q_heads*splits*head_dim floats, part_ml rows*q_heads*splits*2.
+// Workspace for splits > 1: part_acc holds rows*q_heads*splits*head_dim floats, part_ml rows*q_heads*splits*2.
 extern "C" int leone_attention_decode(const void* q, void* out, const void* k_pool, const void* v_pool,
                                       const int* positions, const int* row_entry, const int* block_table,
                                       int max_blocks, float* part_acc, float* part_ml, int rows, int q_heads,
                                       int kv_heads, int head_dim, int page_tokens, float scale, int window,
                                       int splits, hipStream_t stream) {
-    LEONE_REQUIRE(q && out && k_pool && v_pool && positions && row_entry && block_table && part_acc && part_ml,
+    LEONE_REQUIRE(q && out && k_pool && v_pool && positions && row_entry && block_table,
                   "attention_decode: null pointer");
+    LEONE_REQUIRE(splits == 1 || (part_acc && part_ml), "attention_decode: %d splits need the workspace", splits);
     LEONE_REQUIRE(rows > 0 && q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
                   "attention_decode: rows %d, %d query heads over %d kv heads", rows, q_heads, kv_heads);
     LEONE_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
@@ -339,7 +347,7 @@ extern "C" int leone_attention_decode(const void* q, void* out, const void* k_po
 #define LEONE_DECODE_CASE(N)                                                                                      \
     case N:                                                                                                       \
         launch_decode<N>(q, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml,     \
-                         rows, q_heads, kv_heads, page_shift, scale, window, splits, stream);                     \
+                         out, rows, q_heads, kv_heads, page_shift, scale, window, splits, stream);                \
         break;
     switch (head_dim / 16) {
         LEONE_DECODE_CASE(1) LEONE_DECODE_CASE(2) LEONE_DECODE_CASE(3) LEONE_DECODE_CASE(4)
@@ -352,8 +360,10 @@ extern "C" int leone_attention_decode(const void* q, void* out, const void* k_po
     }
 #undef LEONE_DECODE_CASE
     LEONE_LAUNCH_CHECK("attention_decode");
-    attention_reduce_kernel<<<rows * q_heads, kReduceThreads, 0, stream>>>(
-        part_acc, part_ml, static_cast<bf16_t*>(out), head_dim, splits);
-    LEONE_LAUNCH_CHECK("attention_reduce");
+    if (splits > 1) {                                 // a single split has written the result itself
+        attention_reduce_kernel<<<rows * q_heads, kReduceThreads, 0, stream>>>(
+            part_acc, part_ml, static_cast<bf16_t*>(out), head_dim, splits);
+        LEONE_LAUNCH_CHECK("attention_reduce");
+    }
     return 0;
 }

@@ -213,8 +213,10 @@ def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
         splits = choose_splits(rows, kv_heads, q_heads // kv_heads, max_context)
     if out is None:
         out = torch.empty_like(q)
-    part_acc = torch.empty((rows * q_heads * splits * head_dim,), dtype=torch.float32, device=q.device)
-    part_ml = torch.empty((rows * q_heads * splits * 2,), dtype=torch.float32, device=q.device)
+    part_acc = part_ml = None
+    if splits > 1:
+        part_acc = torch.empty((rows * q_heads * splits * head_dim,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((rows * q_heads * splits * 2,), dtype=torch.float32, device=q.device)
     call("leone_attention_decode", _dev(q, "attention q", torch.bfloat16),
          _dev(out, "attention out", torch.bfloat16, q.shape), _dev(k_pool, "k pool", torch.bfloat16),
          _dev(v_pool, "v pool", torch.bfloat16), _dev(positions, "positions", torch.int32, (rows,)),
