@@ -10,6 +10,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import signal
 import struct
 import sys
 import time
@@ -66,7 +67,11 @@ def _sampling_from(args):
 
 
 def build_parser() -> argparse.ArgumentParser:
+    from . import __version__
     parser = argparse.ArgumentParser(prog="leone", description="Qwen3 dense inference on MI355X")
+    parser.add_argument("-V", "--version", action="version", version=f"leone {__version__}")
+    parser.add_argument("--build-info", action="store_true",
+                        help="Print where the two native libraries come from, as JSON")
     sub = parser.add_subparsers(dest="command")
 
     g = sub.add_parser("generate", help="Generate text", usage="leone generate -m <model> -p <prompt> -n <tokens> [options]")
@@ -150,9 +155,16 @@ def cmd_generate(args) -> int:
         sys.stdout.flush()
 
     eos = None if args.ignore_eos else "config"
-    results = runtime.generate_tokens([prompt], args.tokens, sampling, eos_token_id=eos, on_token=on_token,
-                                      logit_observer=observe,
-                                      profile_decode_steps=PROFILE_DECODE_STEPS if args.profile_decode else 0)
+    # Ctrl-C asks the run to stop after the step in hand; what was generated is still reported.
+    interrupted = []
+    earlier = signal.signal(signal.SIGINT, lambda *_: interrupted.append(True))
+    try:
+        results = runtime.generate_tokens([prompt], args.tokens, sampling, eos_token_id=eos, on_token=on_token,
+                                          logit_observer=observe,
+                                          profile_decode_steps=PROFILE_DECODE_STEPS if args.profile_decode else 0,
+                                          cancelled=lambda: bool(interrupted))
+    finally:
+        signal.signal(signal.SIGINT, earlier)
     stats = runtime.last_stats
     sys.stdout.write("\n")
     if args.debug_tokens:
@@ -330,9 +342,12 @@ def cmd_random_model(args) -> int:
 def main(argv: Optional[List[str]] = None) -> int:
     parser = build_parser()
     args = parser.parse_args(argv)
+    if args.build_info:
+        from .csrc import build
+        print(json.dumps(build.build_info()))
+        return 0
     if args.command is None:
-        from . import __version__
-        print(f"leone-amd {__version__}")
+        parser.print_help()
         return 0
     if args.command == "generate":
         return cmd_generate(args)

@@ -203,6 +203,40 @@ def build(verbose: bool = True, force: bool = True) -> str:
     return lib
 
 
+def _tool_version(tool: str) -> str | None:
+    try:
+        out = subprocess.run([tool, "--version"], capture_output=True, text=True, timeout=30)
+    except (OSError, subprocess.TimeoutExpired):
+        return None
+    lines = [line.strip() for line in (out.stdout or out.stderr).splitlines() if line.strip()]
+    return lines[0] if lines else None
+
+
+def build_info() -> dict:
+    """Where the two native libraries come from: sources and flags (as digests), compilers, and whether the
+    built files match the present sources.  The reference prints the same kind of record for its
+    executable (crates/leone-cli/src/build_info.rs:37-75)."""
+    from .. import __version__
+
+    def one(name, names, flags, digest, path, compiler):
+        return {"library": name, "sources": names, "flags": flags, "source_digest": digest,
+                "built": path, "built_matches_sources": path is not None,
+                "compiler": compiler, "compiler_version": _tool_version(compiler) if compiler else None}
+
+    try:
+        device_compiler = hipcc()
+    except RuntimeError:
+        device_compiler = None
+    try:
+        cxx = host_compiler()
+    except RuntimeError:
+        cxx = None
+    return {"schema_version": "leone_amd.build-info.v1", "version": __version__, "target": ARCH,
+            "python": sys.version.split()[0],
+            "kernels": one(LIB_NAME, sources(), FLAGS, source_digest(), library_path(), device_compiler),
+            "host": one(HOST_LIB_NAME, host_sources(), HOST_FLAGS, host_digest(), host_library_path(), cxx)}
+
+
 if __name__ == "__main__":
     print(build_host())
     print(build())

@@ -231,14 +231,17 @@ def generate_tokens(engine: Engine, prompts: Sequence[Sequence[int]], max_new_to
                     policy: Optional[SchedulerPolicy] = None,
                     on_token: Optional[Callable[[Hashable, int], None]] = None,
                     logit_observer: Optional[Callable[[Hashable, int, torch.Tensor], None]] = None,
-                    decode_profile: Optional[Recorder] = None):
-    """Generates for every prompt (token ids); returns results in prompt order and the run's statistics."""
+                    decode_profile: Optional[Recorder] = None,
+                    cancelled: Optional[Callable[[], bool]] = None):
+    """Generates for every prompt (token ids); returns results in prompt order and the run's statistics.
+    ``cancelled`` is asked before every step; once it says yes, every request ends as "cancelled" with the
+    tokens it has."""
     generator = Generator(engine, policy)
     generator.logit_observer = logit_observer
     generator.decode_profile = decode_profile
     for i, prompt in enumerate(prompts):
         generator.submit(i, prompt, max_new_tokens, sampling, eos_token_id)
-    finished = {f.id: f for f in generator.run(on_token)}
+    finished = {f.id: f for f in generator.run(on_token, cancelled)}
     results = [GenerationResult(i, list(finished[i].prompt), list(finished[i].tokens), finished[i].reason)
                for i in range(len(prompts))]
     return results, generator.stats

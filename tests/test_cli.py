@@ -1,4 +1,6 @@
 """Command-line pieces that need no GPU."""
+import json
+
 import numpy as np
 import pytest
 
@@ -89,3 +91,25 @@ def test_key_ranges_of_the_prompt_kernel_are_chosen_by_rows_and_keys():
             splits = ops.choose_prefill_splits(groups, heads, keys)
             assert 1 <= splits <= ops.PREFILL_MAX_SPLITS
             assert splits == 1 or (splits * groups * heads <= 512 and -(-keys // 64) // splits >= ops.PREFILL_SPLIT_MIN_STAGES)
+
+
+def test_version_and_build_info(capsys):
+    from leone_amd import __version__, cli
+    from leone_amd.csrc import build
+    with pytest.raises(SystemExit) as stop:
+        cli.main(["--version"])
+    assert stop.value.code == 0 and capsys.readouterr().out.strip() == f"leone {__version__}"
+    assert cli.main(["--build-info"]) == 0
+    info = json.loads(capsys.readouterr().out)
+    assert info["schema_version"] == "leone_amd.build-info.v1" and info["target"] == "gfx950"
+    assert info["kernels"]["sources"] == build.sources() and "attention_decode.hip" in info["kernels"]["sources"]
+    assert info["kernels"]["source_digest"] == build.source_digest()
+    assert info["host"]["source_digest"] == build.host_digest() and "scheduler.cpp" in info["host"]["sources"]
+    assert "-packed-fp32-ops" in info["kernels"]["flags"]
+    # a change of a flag is a change of the digest: a library built otherwise does not pass for this one
+    flags = list(build.FLAGS)
+    try:
+        build.FLAGS.append("-DSOMETHING")
+        assert build.source_digest() != info["kernels"]["source_digest"]
+    finally:
+        build.FLAGS[:] = flags

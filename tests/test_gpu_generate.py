@@ -154,6 +154,27 @@ def test_eos_stops_generation(folders):
     assert stopped.tokens == free[:free.index(free[3]) + 1] and stopped.finish_reason == "eos"
 
 
+def test_cancellation_ends_every_request_with_what_it_has(folders):
+    """The cancellation flag (Ctrl-C on the command line) is looked at before every step: the requests end
+    as cancelled with the tokens generated so far, which are the tokens of an undisturbed run, and nothing
+    stays live."""
+    from leone_amd.api import Runtime
+    folder = folders["A"]
+    config = read_config(folder)
+    prompts = [random_tokens(300 + i, n, config["vocab_size"]) for i, n in enumerate([12, 30])]
+    runtime = Runtime.load(folder, "float32", max_tokens=256, page_tokens=16, max_requests=2)
+    whole = runtime.generate_tokens(prompts, 20, eos_token_id=None)
+    steps = []
+    cut = runtime.generate_tokens(prompts, 20, eos_token_id=None, on_token=lambda request, token: steps.append(request),
+                                  cancelled=lambda: len(steps) >= 10)
+    for full, part in zip(whole, cut):
+        assert part.finish_reason == "cancelled" and 0 < len(part.tokens) < 20
+        assert full.tokens[:len(part.tokens)] == part.tokens
+    assert not runtime.engine.cache.live_requests()
+    runtime.engine.cache.check()
+    assert runtime.generate_tokens(prompts, 20, eos_token_id=None)[0].tokens == whole[0].tokens
+
+
 def test_device_sampling_kernels_against_the_double_precision_sampler():
     from leone_amd import ops
     from leone_amd.sampling.sampler import SamplingParams, distribution, select
