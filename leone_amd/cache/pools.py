@@ -1,7 +1,7 @@
 """Device storage behind the cache manager: key/value pages per group, state per slot."""
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Union
+from typing import Dict, List, Union
 
 import torch
 

@@ -22,7 +22,7 @@ import torch
 
 from .. import hostlib, ops
 from ..ops import profile
-from ..cache.manager import CacheManager, OutOfPages
+from ..cache.manager import CacheManager
 from ..cache.pools import DevicePools
 from ..parts.context import EntryInfo, StepContext
 from ..parts.model import DecoderModel

@@ -7,10 +7,9 @@ tokens, why generation stopped and timing (crates/leone/src/runtime.rs:442-452, 
 from __future__ import annotations
 
 import time
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Callable, Dict, Hashable, List, Optional, Sequence
 
-import numpy as np
 import torch
 
 from .. import ops

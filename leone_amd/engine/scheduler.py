@@ -31,7 +31,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_int, c_int32, c_int64
-from dataclasses import dataclass, fields
+from dataclasses import dataclass
 from enum import Enum
 from typing import Dict, Hashable, List, Optional, Sequence
 

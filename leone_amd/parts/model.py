@@ -8,7 +8,7 @@ import torch
 
 from .. import ops
 from ..weights.loader import MATRIX, TensorSpec
-from .base import BLOCKS, NORMS, POSITIONS, KvNeed, PartSpec, StateNeed
+from .base import BLOCKS, NORMS, POSITIONS, PartSpec
 from .context import CacheView, StepContext
 
 
