@@ -438,7 +438,6 @@ attention_prefill_merge_kernel(const float* __restrict__ part_acc, const float* 
         float den = 0.f;
         float num[4] = {0.f, 0.f, 0.f, 0.f};                     // head_dim <= 256: at most four elements a lane
         const float* acc = part_acc + rh * splits * head_dim;
-#pragma unroll 4
         for (int s = 0; s < splits; ++s) {
             const float weight = __shfl(my_weight, s, kWave);
             den += __shfl(my_share, s, kWave);
