@@ -202,6 +202,8 @@ static void launch_fused(const FusedArgs& a, hipStream_t stream) {
     gemm_fused_kernel<kIn, kOut, TAIL, WAVES, TOut><<<tiles, WAVES * kWave, 0, stream>>>(a)
     if (many) {
         if (tail) LEONE_FUSED(true, 4); else LEONE_FUSED(false, 4);
+    } else if (tiles <= 384 && steps >= 64) {             // about one workgroup a compute unit: sixteen waves keep more loads in flight
+        if (tail) LEONE_FUSED(true, 16); else LEONE_FUSED(false, 16);
     } else {
         if (tail) LEONE_FUSED(true, 8); else LEONE_FUSED(false, 8);
     }
