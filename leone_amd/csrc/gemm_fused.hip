@@ -197,13 +197,16 @@ static void launch_fused(const FusedArgs& a, hipStream_t stream) {
     const int tiles = ceil_div(a.n, 16);
     const int steps = ceil_div(a.k, 64);
     const bool tail = a.k % 64 != 0;
-    const bool many = tiles * 4 >= 4096 || steps < 16;    // matrices with few rows split K over eight waves, so that the chip is filled
+    const bool many = tiles * 4 >= 4096 || steps < 16;    // workgroups enough to fill the chip, or too little of K to split further
 #define LEONE_FUSED(TAIL, WAVES) \
     gemm_fused_kernel<kIn, kOut, TAIL, WAVES, TOut><<<tiles, WAVES * kWave, 0, stream>>>(a)
-    if (many) {
-        if (tail) LEONE_FUSED(true, 4); else LEONE_FUSED(false, 4);
-    } else if (tiles <= 384 && steps >= 64) {             // about one workgroup a compute unit: sixteen waves keep more loads in flight
+    // Measured at the 8B shapes: about one workgroup a compute unit (output and down projections) wants
+    // sixteen waves to keep enough loads in flight; matrices with many rows want four waves when X has many
+    // rows and eight when it has few.
+    if (tiles <= 256 && steps >= 64) {
         if (tail) LEONE_FUSED(true, 16); else LEONE_FUSED(false, 16);
+    } else if (many && a.m > 4) {
+        if (tail) LEONE_FUSED(true, 4); else LEONE_FUSED(false, 4);
     } else {
         if (tail) LEONE_FUSED(true, 8); else LEONE_FUSED(false, 8);
     }
