@@ -119,6 +119,9 @@ SCENARIOS = {
     # 16 requests of 4096 tokens, 256 tokens at temperature 0.7, the page pool at 60 % of what all would need
     "pressure32b": dict(config=QWEN3_32B, requests=16, prompt=(4096, 4096), new_tokens=256, chunk=1024,
                         temperature=0.7, live=16, pool_fraction=0.6),
+    # one prompt of 32,768 tokens in portions of 512 (late portions: few rows over many keys), then 64 tokens
+    "long32k": dict(config=QWEN3_8B, requests=1, prompt=(32768, 32768), new_tokens=64, chunk=512, temperature=None,
+                    live=1, pool_fraction=1.0),
 }
 
 
