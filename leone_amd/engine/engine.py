@@ -50,7 +50,9 @@ class PackedStep:
     tokens, positions, row -> entry, state slots, wanted rows, query tiles, one block table per cache group."""
 
     def __init__(self, cache: CacheManager, vocab_size: int, entries: Sequence[StepEntry], all_rows_wanted: bool = False,
-                 host: Optional[torch.Tensor] = None):
+                 host=None):
+        """``host``: nothing (a buffer is made), a buffer to write into (it must be large enough), or a
+        callable that is given the number of words and returns one."""
         n = len(entries)
         lib = hostlib.library()
         requests = (c_int64 * max(1, n))()
@@ -85,6 +87,8 @@ class PackedStep:
         if total >= 0:
             if host is None:
                 host = torch.empty(max(1, total), dtype=torch.int32)
+            elif callable(host):
+                host = host(max(1, total))                  # the caller hands out a buffer of that many words
             elif host.numel() < total:
                 raise StepError("the step does not fit the recorded layout")
             total = lib.leone_step_pack(*args, ctypes.cast(host.data_ptr(), hostlib.PI32), host.numel(), sections,
@@ -165,6 +169,8 @@ class Engine:
         # Steps of single decoded tokens are recorded once per batch size and replayed.
         self.graphs = bool(graphs) and model.graph_safe
         self._decode_graphs: Dict[int, _DecodeGraph] = {}
+        self._staging: List[Optional[tuple]] = [None, None]
+        self._staging_turn = 0
 
     # ---- requests -----------------------------------------------------------------
     def admit(self, request: Hashable) -> int:
@@ -298,10 +304,25 @@ class Engine:
         index = torch.tensor(wanted, dtype=torch.long, device=self.device)
         return logits.index_select(0, index), rows_map
 
+    def _staging_buffer(self, words: int) -> torch.Tensor:
+        """A pinned host buffer for one step's metadata.  Two take turns, each guarded by an event, so that
+        the upload need not be waited for and the host can prepare the next step while this one runs."""
+        self._staging_turn ^= 1
+        held = self._staging[self._staging_turn]
+        if held is None or held[0].numel() < words:
+            grown = max(words, 4096, 2 * held[0].numel() if held is not None else 0)
+            held = (torch.empty(grown, dtype=torch.int32).pin_memory(), torch.cuda.Event())
+            self._staging[self._staging_turn] = held
+        else:
+            held[1].synchronize()                       # its last upload has left the buffer
+        return held[0]
+
     def _build_context(self, entries: Sequence[StepEntry]):
         """The step's metadata, laid out by the native routine and uploaded in one copy."""
-        packed = PackedStep(self.cache, self.vocab_size, entries)
-        device = packed.host[:max(1, packed.total)].to(self.device)
+        packed = PackedStep(self.cache, self.vocab_size, entries, host=self._staging_buffer)
+        device = torch.empty(max(1, packed.total), dtype=torch.int32, device=self.device)
+        device.copy_(packed.host[:max(1, packed.total)], non_blocking=True)
+        self._staging[self._staging_turn][1].record()
         pieces = packed.pieces(device)
         infos = [EntryInfo(entries[given].request, slot, first_row, count, start)
                  for given, slot, first_row, count, start in packed.placed]
