@@ -201,6 +201,13 @@ def cmd_doctor(args) -> int:
     except Exception as error:  # noqa: BLE001 - doctor reports, it does not raise
         print(f"kernel library: FAILED: {error}")
         ok = False
+    try:
+        from .csrc import build
+        path = build.host_library_path() or build.build_host(verbose=True)
+        print(f"host library: {path}")
+    except Exception as error:  # noqa: BLE001
+        print(f"host library: FAILED: {error}")
+        ok = False
     if args.model:
         from .architectures import config_from_dir, model_spec_for
         from .parts.model import DecoderModel

@@ -32,6 +32,7 @@ OPERATIONS = {
     "leone_swiglu": "swiglu",
     "leone_argmax": "argmax",
     "leone_sample_temperature": "sample",
+    "leone_top_candidates": "sample",
 }
 LIBRARY_PRODUCT = "gemm library"
 ORDER = ["embed", "norm", "gemv fused", LIBRARY_PRODUCT, "gemm f32", "qknorm rope kv", "attention", "swiglu",
