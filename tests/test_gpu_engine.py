@@ -156,6 +156,38 @@ def test_late_portions_of_a_long_request(tmp_path):
     compare(steps, outputs, expected, tolerance("bfloat16"), "long request in late portions")
 
 
+def test_a_hundred_thousand_tokens_cut_three_ways(tmp_path):
+    """A context far beyond what the plain implementation can check: block tables of 1,500 pages, key
+    ranges in both attention kernels.  The last prompt token's logits and those of eight decoded tokens
+    must not depend on how the prompt was cut."""
+    from leone_amd.engine.engine import Engine, StepEntry
+    from leone_amd.runtime import load_model
+
+    config = dict(TINY["M"], max_position_embeddings=131072)
+    folder = make_model_dir(str(tmp_path / "far"), config, seed=9, dtype=torch.bfloat16)
+    model = load_model(folder, "bfloat16")
+    n = 100_000
+    tokens = random_tokens(5, n + 8, config["vocab_size"])
+    results = []
+    for chunk in (2048, 1000, 333):
+        engine = Engine(model, max_tokens=n + 64, page_tokens=64, max_requests=1, max_context=n + 64)
+        at = 0
+        while at < n:
+            size = min(chunk, n - at)
+            out = engine.step([StepEntry("r", tokens[at:at + size], [size - 1] if at + size == n else [])])
+            at += size
+        rows = [out.logits[0].float().cpu()]
+        for i in range(8):
+            rows.append(engine.step([StepEntry("r", [tokens[n + i]], [0])]).logits[0].float().cpu())
+        results.append(torch.stack(rows))
+        engine.release("r")
+        engine.cache.check()
+    assert all(torch.isfinite(r).all() for r in results)
+    assert float(results[0].abs().max()) > 0.5                    # the logits are not all alike
+    for other in results[1:]:
+        assert float((other - results[0]).abs().max()) <= tolerance("bfloat16")
+
+
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 def test_rerun_is_bitwise_identical(cases, dtype_name):
     from leone_amd.engine.engine import Engine
