@@ -377,6 +377,45 @@ def test_attention_finds_the_one_key_that_matters(kernel):
         assert (out[i] - want).abs().max() < 0.25, (i, r, p, j)       # nearly all the weight is on key j
 
 
+@pytest.mark.parametrize("kernel", ["decode", "prefill"])
+def test_attention_finds_one_key_among_seventy_thousand(kernel):
+    """The same far into a long request: more than a thousand pages, key ranges in both kernels, targets at
+    the edges of pages, of 4,096 and of 65,536 keys."""
+    from leone_amd import ops
+    q_heads, kv_heads, head_dim, page_tokens = 8, 2, 64, 64
+    dtype = torch.bfloat16
+    n = 70_000
+    table, k_pool, v_pool, keys, values = paged_setup([n], kv_heads, head_dim, page_tokens, dtype, seed=61)
+    edges = [0, 63, 64, 4095, 4096, 32767, 32768, 65535, 65536, 69839]
+    count = 160 if kernel == "prefill" else 24
+    first = n - count if kernel == "prefill" else n - 1
+    g = torch.Generator().manual_seed(62)
+    targets = [edges[i] if i < len(edges) else int(torch.randint(0, n - count, (1,), generator=g)) for i in range(count)]
+    positions = [first + i if kernel == "prefill" else n - 1 for i in range(count)]
+    targets[-1] = positions[-1]                                   # the last row looks at itself
+    q = torch.zeros(count, q_heads, head_dim)
+    for i, j in enumerate(targets):
+        for h in range(q_heads):
+            k = keys[0][j, h // (q_heads // kv_heads)]
+            q[i, h] = k * (60.0 * math.sqrt(head_dim) / float(k @ k))
+    q = q.to(dtype).reshape(count, -1).to(DEV)
+    where = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    scale = 1.0 / math.sqrt(head_dim)
+    if kernel == "prefill":
+        out = torch.zeros((count, q_heads * head_dim), dtype=dtype, device=DEV)
+        tiles = ops.prefill_tiles([(0, 0, count)])
+        assert ops.choose_prefill_splits(tiles.shape[0] // ops.PREFILL_GROUP_TILES, q_heads, n) > 1
+        ops.attention_prefill(q, out, k_pool.to(DEV), v_pool.to(DEV), where, tiles.to(DEV), table.to(DEV), q_heads, scale,
+                              mean_keys=n)
+    else:
+        out = ops.attention_decode(q, k_pool.to(DEV), v_pool.to(DEV), where, torch.zeros(count, dtype=torch.int32, device=DEV),
+                                   table.to(DEV), q_heads, scale, max_context=n)
+    out = out.float().cpu().view(count, q_heads, head_dim)
+    for i, j in enumerate(targets):
+        want = values[0][j].repeat_interleave(q_heads // kv_heads, dim=0)
+        assert (out[i] - want).abs().max() < 0.25, (i, positions[i], j)
+
+
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("mnk", [(1, 777, 80), (5, 64, 64), (8, 6144, 4096), (16, 1000, 96), (13, 130, 1032),
                                  (9, 48, 176), (16, 4096, 12288), (1, 151936, 256), (3, 20, 8)])
