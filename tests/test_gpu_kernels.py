@@ -377,7 +377,7 @@ def test_attention_finds_the_one_key_that_matters(kernel):
         assert (out[i] - want).abs().max() < 0.25, (i, r, p, j)       # nearly all the weight is on key j
 
 
-@pytest.mark.parametrize("kernel", ["decode", "prefill"])
+@pytest.mark.parametrize("kernel", ["rows", "decode", "prefill"])
 def test_attention_finds_one_key_among_seventy_thousand(kernel):
     """The same far into a long request: more than a thousand pages, key ranges in both kernels, targets at
     the edges of pages, of 4,096 and of 65,536 keys."""
@@ -407,9 +407,12 @@ def test_attention_finds_one_key_among_seventy_thousand(kernel):
         assert ops.choose_prefill_splits(tiles.shape[0] // ops.PREFILL_GROUP_TILES, q_heads, n) > 1
         ops.attention_prefill(q, out, k_pool.to(DEV), v_pool.to(DEV), where, tiles.to(DEV), table.to(DEV), q_heads, scale,
                               mean_keys=n)
-    else:
+    elif kernel == "decode":
         out = ops.attention_decode(q, k_pool.to(DEV), v_pool.to(DEV), where, torch.zeros(count, dtype=torch.int32, device=DEV),
                                    table.to(DEV), q_heads, scale, max_context=n)
+    else:
+        out = ops.attention_rows(q, k_pool.to(DEV), v_pool.to(DEV), where, torch.zeros(count, dtype=torch.int32, device=DEV),
+                                 table.to(DEV), q_heads, scale)
     out = out.float().cpu().view(count, q_heads, head_dim)
     for i, j in enumerate(targets):
         want = values[0][j].repeat_interleave(q_heads // kv_heads, dim=0)
