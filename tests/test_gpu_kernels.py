@@ -102,6 +102,13 @@ def test_rope_table():
             angle = pos * (1e6 ** (-2.0 * i / 128))
             assert abs(float(cos[pos, i]) - math.cos(angle)) < 5e-7
             assert abs(float(sin[pos, i]) - math.sin(angle)) < 5e-7
+    # far positions and a small base: angles of 10^5 radians, which single precision could not reduce
+    cos, sin = ops.rope_table(1e4, 48, 131072, DEV)
+    for pos in (65535, 100000, 131071):
+        for i in (0, 1, 7, 23):
+            angle = pos * (1e4 ** (-2.0 * i / 48))
+            assert abs(float(cos[pos, i]) - math.cos(angle)) < 5e-7
+            assert abs(float(sin[pos, i]) - math.sin(angle)) < 5e-7
 
 
 def paged_setup(lengths, kv_heads, head_dim, page_tokens, dtype, seed, extra_pages=3):
