@@ -3,9 +3,10 @@
 // A portion's rows are cut into tiles of 32 consecutive rows; a wave takes one tile and one query
 // head, its rows as two 16-column operands.  A workgroup is four waves whose tiles belong to the
 // same request (the host lists them: entry, first row, row count, four to a workgroup).  The
-// workgroup walks the keys its tiles can see once, 64 at a time: all threads copy the next 64
-// keys and values from the cache to shared memory while the waves work on the present 64, and
-// every wave takes from shared memory the 32-key halves its own rows can see.  A wave keeps the
+// workgroup walks the keys its tiles can see once, 64 at a time: the next 64 keys and values travel
+// from the cache to shared memory while the waves work on the present 64 (by loads that write to
+// shared memory themselves; a stage at the edge of the keys or across pages goes through registers,
+// where it is masked), and every wave takes from shared memory the 32-key halves its own rows can see.  A wave keeps the
 // running reference, sum and accumulator of the reference's recurrence
 // (crates/leone/src/cpu.rs:2359-2421) per query in registers; nothing of size rows x keys is ever
 // stored (the reference's prefill materialises the scores, crates/leone-cuda/cuda/ie_cuda.cu:5124-5220).
@@ -190,18 +191,30 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     const long head_elems = static_cast<long>(kvh) * page_elems;
     const long pool_stride = static_cast<long>(kv_heads) * page_elems;
     uint4 held_k[kCopies], held_v[kCopies];
-    // A stage that lies inside one page and inside the group's keys needs one page id and no masks:
-    // its loads are issued back to back.
-    auto fetch_plain = [&](int key_base, int page) {
+    // A stage that lies inside one page and inside the group's keys needs one page id and no masks: its
+    // runs go from the cache straight into shared memory, no register in between.  Such a load puts the 64
+    // runs of a wave one after the other from a place in shared memory that is the same for the wave, each
+    // lane naming the address it reads: so the lane that fills place L of the stage reads the run that
+    // belongs there (for the keys, the order the first product's operand wants, see `deposit`).
+    constexpr int kGroups = kKeyRuns / kWave;                       // loads of 64 runs that make up the keys of a stage
+    constexpr int kDirect = (kGroups + kPrefillWaves - 1) / kPrefillWaves;
+    auto fetch_direct = [&](int key_base, int page, uint4* to) {
         const int in_page = key_base & page_mask;
         const bf16_t* kp = k_pool + page * pool_stride + head_elems + static_cast<long>(in_page) * 8;
         const bf16_t* vp = v_pool + page * pool_stride + head_elems + static_cast<long>(in_page >> 3) * kD * 8;
+        // place -> key of the 32-key half: the inverse of `deposit`'s order
+        const int place = lane & 31;
+        const int kk = ((place >> 2) & 3) * 8 + (place >> 4) * 4 + (place & 3);
 #pragma unroll
-        for (int i = 0; i < kCopies; ++i) {
-            const int idx = i * kPrefillThreads + tid;
-            if (kKeyRuns % kPrefillThreads != 0 && idx >= kKeyRuns) continue;
-            held_k[i] = *reinterpret_cast<const uint4*>(kp + (static_cast<long>(idx / kStageKeys) * page_tokens + idx % kStageKeys) * 8);
-            held_v[i] = *reinterpret_cast<const uint4*>(vp + static_cast<long>(idx) * 8);   // (8 tg / 8 * kD + d) * 8 with idx = tg * kD + d
+        for (int i = 0; i < kDirect; ++i) {
+            const int group = i * kPrefillWaves + wave;               // the same for the whole wave
+            if (kGroups % kPrefillWaves != 0 && group >= kGroups) continue;
+            const int q = 2 * group + (lane >> 5);                    // (half, run) of this lane's place
+            const int half = q / kRuns, run = q % kRuns;
+            const bf16_t* k_from = kp + (static_cast<long>(run) * page_tokens + 32 * half + kk) * 8;
+            const bf16_t* v_from = vp + (static_cast<long>(group) * kWave + lane) * 8;
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(k_from), to + group * kWave, 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint4*>(v_from), to + kKeyRuns + group * kWave, 16, 0, 0);
         }
     };
     auto fetch_any = [&](int key_base) {
@@ -249,17 +262,21 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             }
         }
     };
-    auto fetch = [&](int t) {
+    // Starts bringing stage t to `to`.  True: the runs are on their way to shared memory by themselves and
+    // only have to be waited for; false: they are on their way to registers and `deposit` has to follow.
+    auto fetch = [&](int t, uint4* to) -> bool {
         const int key_base = t * kStageKeys;
         if (page_shift >= 6 && key_base >= group_lo && key_base + kStageKeys <= group_hi) {
             const int page = __builtin_amdgcn_readfirstlane(pages[(key_base >> page_shift) - first_page]);
             if (page >= 0) {
-                fetch_plain(key_base, page);
-                return;
+                fetch_direct(key_base, page, to);
+                return true;
             }
         }
         fetch_any(key_base);
+        return false;
     };
+    auto arrived = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
     auto deposit = [&](uint4* to) {
 #pragma unroll
         for (int i = 0; i < kCopies; ++i) {
@@ -355,20 +372,30 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     };
 
     const int t_begin = group_lo / kStageKeys, t_end = (group_hi + kStageKeys - 1) / kStageKeys;
-    fetch(t_begin);
-    deposit(shared);
+    if (!fetch(t_begin, shared)) deposit(shared);
+    arrived();
     __syncthreads();
-    int cur = 0;
-    for (int t = t_begin; t < t_end; ++t) {
-        const bool more = t + 1 < t_end;
-        if (more) fetch(t + 1);                                  // in flight while the waves work
+    // One round: start bringing the next stage to `writing`, work on the present one in `reading`.  The two
+    // are told apart for the compiler (they never overlap), so that it does not wait for the runs on their way
+    // to `writing` before it reads `reading`.
+    auto round = [&](const uint4* __restrict__ reading, uint4* __restrict__ writing, int t, bool more) {
+        // `writing` was last read before the barrier that ended the round before: it is free.  The next
+        // stage is sent for between the two halves (measured: better than before the first half, where its
+        // arrival in shared memory gets in the way of the reads of both halves).
+        bool direct = false;
 #pragma unroll
         for (int half = 0; half < kStageKeys / kKeysPerPass; ++half) {
             const int key0 = t * kStageKeys + half * kKeysPerPass;
+            if (half == kStageKeys / kKeysPerPass - 1) direct = more && fetch(t + 1, writing);
             if (key0 >= key_hi || key0 + kKeysPerPass <= key_lo) continue;      // nothing of it for this wave
-            pass(shared + cur * kStageRuns, key0, half, key0 >= full_lo && key0 + kKeysPerPass <= full_hi);
+            pass(reading, key0, half, key0 >= full_lo && key0 + kKeysPerPass <= full_hi);
         }
-        if (more) deposit(shared + (cur ^ 1) * kStageRuns);      // the other stage was last read before the barrier below
+        if (more && !direct) deposit(writing);
+    };
+    int cur = 0;
+    for (int t = t_begin; t < t_end; ++t) {
+        round(shared + cur * kStageRuns, shared + (cur ^ 1) * kStageRuns, t, t + 1 < t_end);
+        arrived();
         __syncthreads();
         cur ^= 1;
     }
