@@ -215,8 +215,13 @@ class Engine:
             seen.add(e.request)
             if len(e.tokens) == 0:
                 raise StepError(f"request {e.request!r} brings no tokens")
-            tokens = np.asarray(e.tokens)
-            if tokens.dtype.kind not in "iu" or tokens.min() < 0 or tokens.max() >= self.vocab_size:
+            if len(e.tokens) <= 4:                      # decoded tokens: not worth an array
+                fine = all(isinstance(t, (int, np.integer)) and not isinstance(t, bool) and 0 <= t < self.vocab_size
+                           for t in e.tokens)
+            else:
+                tokens = np.asarray(e.tokens)
+                fine = tokens.dtype.kind in "iu" and tokens.min() >= 0 and tokens.max() < self.vocab_size
+            if not fine:
                 raise StepError(f"request {e.request!r}: a token is outside the vocabulary of {self.vocab_size}")
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):

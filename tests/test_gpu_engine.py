@@ -188,6 +188,30 @@ def test_a_hundred_thousand_tokens_cut_three_ways(tmp_path):
         assert float((other - results[0]).abs().max()) <= tolerance("bfloat16")
 
 
+def test_a_malformed_step_is_refused_and_changes_nothing(cases):
+    from leone_amd.engine.engine import Engine, StepEntry, StepError
+    from leone_amd.runtime import load_model
+
+    folder, requests, expected = cases("A", "float32")
+    engine = Engine(load_model(folder, "float32"), max_tokens=256, page_tokens=16, max_requests=4)
+    vocab = TINY["A"]["vocab_size"]
+    tokens = requests["r3"]
+    engine.step([StepEntry("kept", tokens[:10], [])])
+    free = engine.cache.free_pages(0)
+    bad = [[], [StepEntry("a", [1, 2], []), StepEntry("a", [3], [])], [StepEntry("a", [], [])],
+           [StepEntry("a", [vocab], [0])], [StepEntry("a", [-1], [0])], [StepEntry("a", [1, 2, 3, 4, 5, vocab], [0])],
+           [StepEntry("a", [True], [0])], [StepEntry("a", [1.5], [0])], [StepEntry("a", [1, 2], [2])],
+           [StepEntry("a", [1, 2], [-1])], [StepEntry("kept", [5], [0]), StepEntry("b", [1, vocab + 7], [])]]
+    for entries in bad:
+        with pytest.raises(StepError):
+            engine.step(entries)
+        assert engine.cache.free_pages(0) == free and engine.cache.length("kept") == 10
+        assert not engine.cache.has("a") and not engine.cache.has("b")
+        engine.cache.check()
+    out = engine.step([StepEntry("kept", tokens[10:20], list(range(10)))])
+    assert np.abs(out.logits.float().cpu().numpy() - expected["r3"][10:20]).max() <= tolerance("float32")
+
+
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 def test_rerun_is_bitwise_identical(cases, dtype_name):
     from leone_amd.engine.engine import Engine
