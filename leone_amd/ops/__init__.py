@@ -409,8 +409,9 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         y = gemm_f32(x, weight)
     elif not x.is_cuda:
         raise KernelError("linear: tensor is not on the GPU")
-    elif out_dtype == torch.float32:
-        # float32 results (logits) for many rows: the library's product with float output
+    elif out_dtype == torch.float32 or (residual is not None and not gated):
+        # float32 results for many rows, from the library's product with float output: logits, and what is
+        # to be added into the float32 stream, which the kernel for few rows adds unrounded as well
         with profile.span(profile.LIBRARY_PRODUCT, weight):
             y = torch.mm(x, weight.t(), out_dtype=torch.float32)
     else:
