@@ -31,9 +31,11 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
 // ---- residual add + RMSNorm -------------------------------------------------
 // One block per output row.  With `rows` == nullptr row r of `x` is updated in
 // place (x += delta) and normalised into y[r].  With `rows` given, output row r
-// reads x[rows[r]] (+ delta[rows[r]]) and x is left untouched.
+// reads x[rows[r]] (+ delta[rows[r]]) and x is left untouched.  `delta` may come in
+// several planes, `plane` elements apart, whose sum (taken in order) is meant: the
+// parts of a product whose inner dimension was cut.
 template <typename TD, typename TY, int kThreads>
-__global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int planes, long plane,
                                    AnyVec gain, float eps, TY* __restrict__ y,
                                    const int* __restrict__ rows, int hidden) {
     __shared__ float scratch[kThreads / kWave];
@@ -46,7 +48,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__
     for (int c = threadIdx.x; c < hidden; c += kThreads) {
         float v = xr[c];
         if (dr) {
-            v += to_float(dr[c]);
+            for (int p = 0; p < planes; ++p) v += to_float(dr[p * plane + c]);
             if (!rows) xr[c] = v;
         }
         ss = fmaf(v, v, ss);
@@ -55,7 +57,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__
     const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
     for (int c = threadIdx.x; c < hidden; c += kThreads) {
         float v = xr[c];
-        if (dr && rows) v += to_float(dr[c]);
+        if (dr && rows)
+            for (int p = 0; p < planes; ++p) v += to_float(dr[p * plane + c]);
         yr[c] = from_float<TY>((v * load_any(gain, c)) * inv);
     }
 }
@@ -84,8 +87,9 @@ __device__ inline void store4(bf16_t* p, const float v[4]) {
 
 template <typename TD, typename TG, typename TY, int kThreads, int kChunks>
 __global__ void __launch_bounds__(kThreads)
-add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, const TG* __restrict__ gain, float eps,
-                       TY* __restrict__ y, const int* __restrict__ rows, int hidden) {
+add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, int planes, long plane,
+                       const TG* __restrict__ gain, float eps, TY* __restrict__ y, const int* __restrict__ rows,
+                       int hidden) {
     __shared__ float scratch[kThreads / kWave];
     const int out_row = blockIdx.x;
     const long in_row = rows ? rows[out_row] : out_row;
@@ -101,10 +105,12 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, cons
             load4(xr + c, v[i]);
             load4(gain + c, gv[i]);
             if (dr) {
-                float d[4];
-                load4(dr + c, d);
+                for (int p = 0; p < planes; ++p) {
+                    float d[4];
+                    load4(dr + p * plane + c, d);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) v[i][j] += d[j];
+                    for (int j = 0; j < 4; ++j) v[i][j] += d[j];
+                }
                 if (!rows) store4(xr + c, v[i]);
             }
 #pragma unroll
@@ -490,39 +496,39 @@ extern "C" int leone_embed(const void* table, int dtype, const int* tokens, floa
 }
 
 template <typename TD, typename TG, typename TY>
-static void launch_add_rmsnorm_vec(float* x, const void* delta, const void* gain, float eps, void* y,
-                                   const int* rows, int n_rows, int hidden, hipStream_t stream) {
+static void launch_add_rmsnorm_vec(float* x, const void* delta, int planes, long plane, const void* gain, float eps,
+                                   void* y, const int* rows, int n_rows, int hidden, hipStream_t stream) {
     const TD* d = static_cast<const TD*>(delta);
     const TG* g = static_cast<const TG*>(gain);
     TY* out = static_cast<TY*>(y);
     if (hidden <= 4 * 64 * 2)
-        add_rmsnorm_vec_kernel<TD, TG, TY, 64, 2><<<n_rows, 64, 0, stream>>>(x, d, g, eps, out, rows, hidden);
+        add_rmsnorm_vec_kernel<TD, TG, TY, 64, 2><<<n_rows, 64, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden);
     else if (hidden <= 4 * 256 * 2)
-        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 2><<<n_rows, 256, 0, stream>>>(x, d, g, eps, out, rows, hidden);
+        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 2><<<n_rows, 256, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden);
     else if (hidden <= 4 * 256 * 4)
-        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 4><<<n_rows, 256, 0, stream>>>(x, d, g, eps, out, rows, hidden);
+        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 4><<<n_rows, 256, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden);
     else
-        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 8><<<n_rows, 256, 0, stream>>>(x, d, g, eps, out, rows, hidden);
+        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 8><<<n_rows, 256, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden);
 }
 
 template <typename TD, typename TY>
-static void launch_add_rmsnorm(float* x, const void* delta, AnyVec gain, float eps, void* y,
+static void launch_add_rmsnorm(float* x, const void* delta, int planes, long plane, AnyVec gain, float eps, void* y,
                                const int* rows, int n_rows, int hidden, hipStream_t stream) {
     if (hidden % 4 == 0 && hidden <= 4 * 256 * 8) {
         if (gain.dtype == kF32)
-            launch_add_rmsnorm_vec<TD, float, TY>(x, delta, gain.ptr, eps, y, rows, n_rows, hidden, stream);
+            launch_add_rmsnorm_vec<TD, float, TY>(x, delta, planes, plane, gain.ptr, eps, y, rows, n_rows, hidden, stream);
         else
-            launch_add_rmsnorm_vec<TD, bf16_t, TY>(x, delta, gain.ptr, eps, y, rows, n_rows, hidden, stream);
+            launch_add_rmsnorm_vec<TD, bf16_t, TY>(x, delta, planes, plane, gain.ptr, eps, y, rows, n_rows, hidden, stream);
         return;
     }
     if (hidden > 512)
-        add_rmsnorm_kernel<TD, TY, 256><<<n_rows, 256, 0, stream>>>(x, static_cast<const TD*>(delta), gain, eps, static_cast<TY*>(y), rows, hidden);
+        add_rmsnorm_kernel<TD, TY, 256><<<n_rows, 256, 0, stream>>>(x, static_cast<const TD*>(delta), planes, plane, gain, eps, static_cast<TY*>(y), rows, hidden);
     else
-        add_rmsnorm_kernel<TD, TY, 64><<<n_rows, 64, 0, stream>>>(x, static_cast<const TD*>(delta), gain, eps, static_cast<TY*>(y), rows, hidden);
+        add_rmsnorm_kernel<TD, TY, 64><<<n_rows, 64, 0, stream>>>(x, static_cast<const TD*>(delta), planes, plane, gain, eps, static_cast<TY*>(y), rows, hidden);
 }
 
-extern "C" int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, const void* gain,
-                                 int gain_dtype, float eps, void* y, int y_dtype, const int* rows,
+extern "C" int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, int delta_planes, long delta_plane,
+                                 const void* gain, int gain_dtype, float eps, void* y, int y_dtype, const int* rows,
                                  int n_rows, int hidden, hipStream_t stream) {
     if (check_dtype(delta_dtype, "add_rmsnorm delta") || check_dtype(gain_dtype, "add_rmsnorm gain") ||
         check_dtype(y_dtype, "add_rmsnorm output"))
@@ -530,15 +536,19 @@ extern "C" int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, c
     LEONE_REQUIRE(x && gain && y, "add_rmsnorm: null pointer");
     LEONE_REQUIRE(n_rows > 0 && hidden > 0, "add_rmsnorm: rows %d hidden %d must be positive", n_rows, hidden);
     LEONE_REQUIRE(eps > 0.f && eps == eps, "add_rmsnorm: eps must be positive");
+    LEONE_REQUIRE(!delta || (delta_planes >= 1 && delta_planes <= 16 && delta_plane >= 0),
+                  "add_rmsnorm: %d planes of what is to be added", delta_planes);
+    const int planes = delta_planes;
+    const long plane = delta_plane;
     AnyVec g{gain, gain_dtype};
     if (delta_dtype == kF32 && y_dtype == kF32)
-        launch_add_rmsnorm<float, float>(x, delta, g, eps, y, rows, n_rows, hidden, stream);
+        launch_add_rmsnorm<float, float>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, stream);
     else if (delta_dtype == kBF16 && y_dtype == kBF16)
-        launch_add_rmsnorm<bf16_t, bf16_t>(x, delta, g, eps, y, rows, n_rows, hidden, stream);
+        launch_add_rmsnorm<bf16_t, bf16_t>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, stream);
     else if (delta_dtype == kF32 && y_dtype == kBF16)
-        launch_add_rmsnorm<float, bf16_t>(x, delta, g, eps, y, rows, n_rows, hidden, stream);
+        launch_add_rmsnorm<float, bf16_t>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, stream);
     else
-        launch_add_rmsnorm<bf16_t, float>(x, delta, g, eps, y, rows, n_rows, hidden, stream);
+        launch_add_rmsnorm<bf16_t, float>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, stream);
     LEONE_LAUNCH_CHECK("add_rmsnorm");
     return 0;
 }

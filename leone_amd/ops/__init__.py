@@ -90,14 +90,21 @@ def embed(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor]
 def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x += delta, then y = rmsnorm(x) * gain; with ``rows``, y[i] comes from row rows[i] and x is not written."""
+    """x += delta, then y = rmsnorm(x) * gain; with ``rows``, y[i] comes from row rows[i] and x is not written.
+    ``delta`` is [n, hidden] or a stack of planes [p, n, hidden] whose sum, taken in order, is meant (the
+    parts of a product whose inner dimension was cut, see ``linear``)."""
     n, hidden = x.shape
     n_out = n if rows is None else rows.numel()
     if out is None:
         out = torch.empty((n_out, hidden), dtype=out_dtype, device=x.device)
     delta_code = _code(delta, "add_rmsnorm delta") if delta is not None else _CODES[out_dtype]
+    stacked = delta is not None and delta.dim() == 3
+    planes = delta.shape[0] if stacked else 1
+    if not 1 <= planes <= 16:
+        raise KernelError(f"add_rmsnorm: {planes} planes of what is to be added")
     call("leone_add_rmsnorm", _dev(x, "add_rmsnorm x", torch.float32),
-         _dev(delta, "add_rmsnorm delta", None, (n, hidden)), delta_code,
+         _dev(delta, "add_rmsnorm delta", None, (planes, n, hidden) if stacked else (n, hidden)), delta_code, planes,
+         n * hidden,
          _dev(gain, "add_rmsnorm gain", None, (hidden,)), _code(gain, "add_rmsnorm gain"), float(eps),
          _dev(out, "add_rmsnorm out", out_dtype, (n_out, hidden)), _CODES[out_dtype],
          _dev(rows, "add_rmsnorm rows", torch.int32), n_out, hidden, _stream())
@@ -377,6 +384,19 @@ def gemm_fused(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
     return None if residual is not None else out
 
 
+def inner_parts(rows: int, n: int, k: int) -> int:
+    """Into how many parts the inner dimension of x[rows, k] . w[n, k]^T is cut when the result goes into the
+    float32 stream.  The library's product does badly with a few hundred rows, few columns and a long inner
+    dimension (the down projection of a prompt portion: 81 us whole against 64 in four parts for 512 x 4096 x
+    12288, 171 against 97 for 512 x 5120 x 17408); beyond 1,024 rows and below 128 it is best left whole."""
+    if not (128 <= rows <= 1024 and k >= 8192 and k >= 2 * n):
+        return 1
+    for parts in ((4, 2) if rows <= 512 else (2,)):
+        if k % (64 * parts) == 0:
+            return parts
+    return 1
+
+
 def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
            residual: Optional[torch.Tensor] = None, gated: bool = False) -> Optional[torch.Tensor]:
     """x[R,K] . weight[N,K]^T, with optional neighbours.
@@ -384,7 +404,8 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     ``x`` is a tensor or ``NormedRows`` (a norm still to be done).  ``gated``: the weight is an
     interleaved gate/up weight and the result is silu(gate) * up, ``[R, N/2]``.  ``residual``: the caller
     wants the product added into this float32 tensor; if the kernel in use can do that, it does and None
-    is returned, otherwise the product is returned for the caller to add later.
+    is returned, otherwise the product is returned for the caller to add later, as float32 ``[R, N]`` or
+    as a stack of planes ``[p, R, N]`` whose sum is meant (``add_rmsnorm`` takes either).
 
     float32 runs the single-precision kernel.  bfloat16 accumulates in float: up to FUSED_ROWS rows on the
     weight-streaming kernel with everything folded in, more rows through the library's matrix product;
@@ -412,8 +433,14 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     elif out_dtype == torch.float32 or (residual is not None and not gated):
         # float32 results for many rows, from the library's product with float output: logits, and what is
         # to be added into the float32 stream, which the kernel for few rows adds unrounded as well
+        parts = inner_parts(rows, weight.shape[0], k) if residual is not None else 1
         with profile.span(profile.LIBRARY_PRODUCT, weight):
-            y = torch.mm(x, weight.t(), out_dtype=torch.float32)
+            if parts > 1:
+                # [parts, rows, N]: the planes are summed, in order, by the norm kernel that adds them
+                y = torch.bmm(x.view(rows, parts, k // parts).transpose(0, 1),
+                              weight.view(weight.shape[0], parts, k // parts).permute(1, 2, 0), out_dtype=torch.float32)
+            else:
+                y = torch.mm(x, weight.t(), out_dtype=torch.float32)
     else:
         with profile.span(profile.LIBRARY_PRODUCT, weight):
             y = torch.nn.functional.linear(x, weight)  # library matrix product, float accumulation

@@ -24,6 +24,9 @@ block         ``tensor_specs()``, ``bind(tensors)``, ``cache_need()``,
 
 ``x`` is the residual stream, float32 ``[rows, hidden]``; ``pending`` is a delta
 not yet added to it (the next norm adds it, so add and norm are one kernel).
+A delta is ``[rows, hidden]`` or a stack of planes ``[p, rows, hidden]`` whose sum
+is meant (what ``ops.linear`` returns when it cut a product's inner dimension);
+``ops.add_rmsnorm`` takes either, and a norm of another kind can sum the planes first.
 """
 from __future__ import annotations
 

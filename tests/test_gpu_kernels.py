@@ -62,6 +62,52 @@ def test_add_rmsnorm(dtype, hidden):
     close(y3, plain.rms_norm((x1.double() + delta.double())[rows.long()].cpu(), gain.cpu(), eps), 2e-5, 2e-5, "gather")
 
 
+@pytest.mark.parametrize("hidden", [80, 4096, 9000])
+def test_add_rmsnorm_takes_what_is_added_in_planes(hidden):
+    """The parts of a product whose inner dimension was cut come as planes; their sum in order is added."""
+    from leone_amd import ops
+    torch.manual_seed(3)
+    rows = 7
+    x = torch.randn(rows, hidden, device=DEV)
+    planes = torch.randn(3, rows, hidden, device=DEV)
+    gain = 1 + 0.1 * torch.randn(hidden, device=DEV)
+    whole = ((x + planes[0]) + planes[1]) + planes[2]                 # the planes are added one after the other
+    want_y = ops.add_rmsnorm(whole.clone(), None, gain, 1e-5, torch.float32)
+    mine = x.clone()
+    got_y = ops.add_rmsnorm(mine, planes, gain, 1e-5, torch.float32)
+    assert torch.equal(mine, whole) and torch.equal(got_y, want_y)
+    picked = torch.tensor([5, 0, 5, 2], dtype=torch.int32, device=DEV)
+    untouched = x.clone()
+    got = ops.add_rmsnorm(untouched, planes, gain, 1e-5, torch.bfloat16, picked)
+    assert torch.equal(untouched, x)
+    assert torch.equal(got, ops.add_rmsnorm(whole.clone(), None, gain, 1e-5, torch.bfloat16, picked))
+    with pytest.raises(ops.KernelError):
+        ops.add_rmsnorm(x.clone(), torch.zeros(17, rows, hidden, device=DEV), gain, 1e-5, torch.float32)
+
+
+def test_linear_cuts_a_long_inner_dimension_for_a_few_hundred_rows():
+    """A product that goes into the stream with a few hundred rows, few columns and a long inner dimension
+    comes back in planes, which the next norm adds up: the same stream as with the product whole."""
+    from leone_amd import ops
+    torch.manual_seed(4)
+    rows, n, k = 300, 64, 8192
+    assert ops.inner_parts(rows, n, k) == 4 and ops.inner_parts(1000, n, k) == 2
+    assert ops.inner_parts(2048, n, k) == 1 and ops.inner_parts(64, n, k) == 1 and ops.inner_parts(rows, 8192, 8192) == 1
+    assert ops.inner_parts(rows, n, 8192 + 64) == 1          # no part would be whole steps of 64
+    x = (torch.randn(rows, k, device=DEV) * 0.5).bfloat16()
+    w = (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    stream = torch.randn(rows, n, device=DEV)
+    delta = ops.linear(x, w, residual=stream)
+    assert delta.shape == (4, rows, n) and delta.dtype == torch.float32
+    gain = torch.ones(n, device=DEV)
+    after = stream.clone()
+    ops.add_rmsnorm(after, delta, gain, 1e-6, torch.bfloat16)
+    want = stream.double() + x.double() @ w.double().T
+    close(after, want, 2e-6 * k, 1e-5, "stream after a product in parts")
+    # without a stream to go into, the product stays whole and bfloat16
+    assert ops.linear(x, w).shape == (rows, n)
+
+
 def test_rmsnorm_reference_vector():
     """rows [1,2],[3,4], gain [1,0.5], eps 1e-6: the largest of the four outputs is index 2
     (crates/leone/src/cpu.rs:2781-2807)."""
