@@ -388,8 +388,9 @@ def inner_parts(rows: int, n: int, k: int) -> int:
     """Into how many parts the inner dimension of x[rows, k] . w[n, k]^T is cut when the result goes into the
     float32 stream.  The library's product does badly with a few hundred rows, few columns and a long inner
     dimension (the down projection of a prompt portion: 81 us whole against 64 in four parts for 512 x 4096 x
-    12288, 171 against 97 for 512 x 5120 x 17408); beyond 1,024 rows and below 128 it is best left whole."""
-    if not (128 <= rows <= 1024 and k >= 8192 and k >= 2 * n):
+    12288, 171 against 97 for 512 x 5120 x 17408, 55 against 32 for 96 x 4096 x 12288); beyond 1,024 rows
+    and up to 64 it is best left whole."""
+    if not (64 < rows <= 1024 and k >= 8192 and k >= 2 * n):
         return 1
     for parts in ((4, 2) if rows <= 512 else (2,)):
         if k % (64 * parts) == 0:

@@ -93,6 +93,7 @@ def test_linear_cuts_a_long_inner_dimension_for_a_few_hundred_rows():
     rows, n, k = 300, 64, 8192
     assert ops.inner_parts(rows, n, k) == 4 and ops.inner_parts(1000, n, k) == 2
     assert ops.inner_parts(2048, n, k) == 1 and ops.inner_parts(64, n, k) == 1 and ops.inner_parts(rows, 8192, 8192) == 1
+    assert ops.inner_parts(65, n, k) == 4
     assert ops.inner_parts(rows, n, 8192 + 64) == 1          # no part would be whole steps of 64
     x = (torch.randn(rows, k, device=DEV) * 0.5).bfloat16()
     w = (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
