@@ -188,6 +188,34 @@ def test_a_hundred_thousand_tokens_cut_three_ways(tmp_path):
         assert float((other - results[0]).abs().max()) <= tolerance("bfloat16")
 
 
+@pytest.mark.parametrize("schedule", ["whole", "portions", "mixed"])
+def test_a_wide_feed_forward_whose_down_projection_is_cut(tmp_path, schedule):
+    """An intermediate size of 8,192 over a width of 64: for portions of 65 rows and more the down projection
+    runs in parts whose planes the next norm adds up; the last block's planes go to the final norm."""
+    from leone_amd import ops
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+
+    config = dict(TINY["A"], intermediate_size=8192, max_position_embeddings=512)
+    folder = make_model_dir(str(tmp_path / "wide"), config, seed=23, dtype=torch.bfloat16)
+    weights = read_weights(folder)
+    requests = {f"w{i}": random_tokens(900 + i, n, config["vocab_size"]) for i, n in enumerate([230, 90, 70, 140])}
+    expected = {rid: qwen3_plain.forward(weights, read_config(folder), toks).numpy() for rid, toks in requests.items()}
+    steps = (schedules.portions(requests, sizes=(100, 66, 7, 130)) if schedule == "portions"
+             else schedules.mixed(requests, sizes=(70, 3, 120)) if schedule == "mixed" else schedules.whole(requests))
+    taken = []
+    real = ops.inner_parts
+    ops.inner_parts = lambda *a: taken.append(real(*a)) or taken[-1]
+    try:
+        engine = Engine(load_model(folder, "bfloat16"), num_pages=schedules.max_live_tokens(steps, round_to=16) // 16,
+                        page_tokens=16, max_requests=4, poison_freed=True)
+        outputs = run_steps(engine, steps)
+    finally:
+        ops.inner_parts = real
+    assert max(taken) == 4 and min(taken) == 1
+    compare(steps, outputs, expected, tolerance("bfloat16"), f"wide feed-forward/{schedule}")
+
+
 def test_a_malformed_step_is_refused_and_changes_nothing(cases):
     from leone_amd.engine.engine import Engine, StepEntry, StepError
     from leone_amd.runtime import load_model
