@@ -34,25 +34,25 @@ class _Stage(argparse.Action):
 
 
 def _add_sampling(parser: argparse.ArgumentParser) -> None:
-    parser.add_argument("--seed", type=int, default=0, help="Seed the sampler. Default: 0")
+    parser.add_argument("--seed", type=int, default=0, help="Number the random draws are derived from (0 unless given)")
     parser.add_argument("--temp", "--temperature", dest="temp", type=float, default=None,
-                        help="Scale logits by 1/t (without it: greedy)")
-    helps = {"--top-k": "Keep the n highest-probability tokens", "--top-p": "Keep the smallest set covering mass p",
-             "--min-p": "Keep tokens with at least p times the highest probability",
-             "--top-a": "Keep tokens with at least a times the highest probability squared",
-             "--tfs": "Tail-free sampling with share z", "--typical": "Locally typical sampling with mass p",
-             "--epsilon": "Keep tokens with probability at least e", "--eta": "Eta sampling with floor e",
-             "--min-k": "Min-k on raw logits with fallback tau", "--top-n-sigma": "Keep raw logits within n deviations"}
+                        help="Sample at temperature t; left out, the best token is always taken")
+    helps = {"--top-k": "Only the n likeliest tokens stay in the draw", "--top-p": "Likeliest tokens first, until their probabilities add up to p",
+             "--min-p": "Drop what is less than p times as likely as the best token",
+             "--top-a": "Drop what falls below a times the square of the best probability",
+             "--tfs": "Cut the tail where the sorted probabilities flatten out (share z of the curvature kept)", "--typical": "Tokens whose surprise is nearest the entropy, up to mass p",
+             "--epsilon": "Drop tokens whose probability is under e", "--eta": "Like --epsilon, with a bound that shrinks as the entropy grows (base e)",
+             "--min-k": "Cut on the unscaled logits at their steepest drop; tau is the bound when none is found", "--top-n-sigma": "Unscaled logits no further than n standard deviations under the best"}
     for flag, text in helps.items():
         parser.add_argument(flag, action=_Stage, help=text)
-    parser.add_argument("--repeat-penalty", type=float, default=1.0, help="Apply sign-aware scaling to seen logits")
-    parser.add_argument("--presence-penalty", type=float, default=0.0, help="Subtract once from any seen token")
-    parser.add_argument("--frequency-penalty", type=float, default=0.0, help="Subtract once per earlier occurrence")
-    parser.add_argument("--penalty-window", type=int, default=64, help="History the penalties count over; 0 disables")
-    parser.add_argument("--dry-multiplier", type=float, default=0.0, help="Enable the repeated-suffix penalty. 0.0 is off")
-    parser.add_argument("--dry-base", type=float, default=1.75, help="Growth per token of match. Default: 1.75")
-    parser.add_argument("--dry-allowed-length", type=int, default=2, help="Free match length. Default: 2")
-    parser.add_argument("--dry-window", type=int, default=64, help="Tokens of history searched. Default: 64")
+    parser.add_argument("--repeat-penalty", type=float, default=1.0, help="Tokens already seen: a positive logit is divided by r, a negative one multiplied (1.0 does nothing)")
+    parser.add_argument("--presence-penalty", type=float, default=0.0, help="Amount taken off the logit of every token already seen")
+    parser.add_argument("--frequency-penalty", type=float, default=0.0, help="Amount taken off a logit for each time its token was seen")
+    parser.add_argument("--penalty-window", type=int, default=64, help="How many of the latest tokens the three penalties look at (0: none)")
+    parser.add_argument("--dry-multiplier", type=float, default=0.0, help="Strength of the penalty on continuing a repeated run of tokens (0.0: no such penalty)")
+    parser.add_argument("--dry-base", type=float, default=1.75, help="Factor by which that penalty grows with every further matching token (1.75)")
+    parser.add_argument("--dry-allowed-length", type=int, default=2, help="Matching tokens that go unpunished (2)")
+    parser.add_argument("--dry-window", type=int, default=64, help="How far back repeated runs are looked for, in tokens (64)")
 
 
 def _sampling_from(args):
@@ -74,19 +74,19 @@ def build_parser() -> argparse.ArgumentParser:
                         help="Print where the two native libraries come from, as JSON")
     sub = parser.add_subparsers(dest="command")
 
-    g = sub.add_parser("generate", help="Generate text", usage="leone generate -m <model> -p <prompt> -n <tokens> [options]")
+    g = sub.add_parser("generate", help="Continue a prompt", usage="leone generate -m <model> -p <prompt> -n <tokens> [options]")
     g.add_argument("-m", "--model", required=True, help="Model folder (config.json, model.safetensors)")
     g.add_argument("-p", "--prompt", help="Prompt text (needs tokenizer.json in the model folder)")
     g.add_argument("--prompt-tokens", help="Prompt as comma-separated token ids")
-    g.add_argument("-n", "--tokens", type=int, required=True, help="Number of tokens to generate")
+    g.add_argument("-n", "--tokens", type=int, required=True, help="How many tokens to produce")
     g.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"], help="Weights, activations and cache")
-    g.add_argument("--eager-decode", action="store_true", help="Disable decode graph replay")
+    g.add_argument("--eager-decode", action="store_true", help="Launch every decode step kernel by kernel instead of replaying its recording")
     g.add_argument("--profile-decode", action="store_true",
                    help=f"Time the first {PROFILE_DECODE_STEPS} decode steps operation by operation")
     g.add_argument("--prefill-chunk", type=int, default=2048, help="Longest prompt portion per step")
     g.add_argument("--max-context", type=int, default=None, help="Context the cache is sized for")
-    g.add_argument("--debug-tokens", help="Write generated token IDs as JSON")
-    g.add_argument("--debug-logits", help="Write the top five logits for each token")
+    g.add_argument("--debug-tokens", help="File that receives the generated ids as a JSON list")
+    g.add_argument("--debug-logits", help="File that receives, step by step, the five largest logits with their bits")
     g.add_argument("--ignore-eos", action="store_true", help="Do not stop at the end token")
     _add_sampling(g)
 
@@ -95,14 +95,14 @@ def build_parser() -> argparse.ArgumentParser:
     d.add_argument("--probe", action="store_true", help="Also load the weights onto the GPU")
     d.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
 
-    e = sub.add_parser("eval", help="Evaluate model logits for given token ids")
+    e = sub.add_parser("eval", help="Feed given token ids and write the logits of every position")
     e.add_argument("-m", "--model", required=True)
-    e.add_argument("--tokens", required=True, help="Token ids as little-endian u32")
-    e.add_argument("--logits", required=True, help="Output: row-major little-endian f32 logits")
-    e.add_argument("--metadata", help="Write execution metadata as JSON")
-    e.add_argument("--window", type=int, default=512, help="Overlapping evaluation window. Default: 512")
-    e.add_argument("--position-limit", type=int, default=None, help="Score only the first n positions")
-    e.add_argument("--prefill-chunk", type=int, default=None, help="Feed windows in chunks of n tokens")
+    e.add_argument("--tokens", required=True, help="Input file: token ids, 32-bit unsigned, little-endian")
+    e.add_argument("--logits", required=True, help="Output file: one row of 32-bit float logits per position, little-endian")
+    e.add_argument("--metadata", help="Also write a JSON record of model, type, schedule and file digests")
+    e.add_argument("--window", type=int, default=512, help="Tokens per window; a window starts on the last token of the one before, with an empty cache (512)")
+    e.add_argument("--position-limit", type=int, default=None, help="Stop after n positions")
+    e.add_argument("--prefill-chunk", type=int, default=None, help="Cut every window into portions of n tokens")
     e.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
 
     r = sub.add_parser("random-model", help="Write a model folder with seeded random weights")
@@ -117,7 +117,7 @@ def build_parser() -> argparse.ArgumentParser:
     q.add_argument("--vocab", type=int, help="Vocabulary size (or give -m)")
     q.add_argument("-m", "--model", help="Model folder to take the vocabulary size from")
 
-    b = sub.add_parser("bench", help="Measure decode and prefill throughput")
+    b = sub.add_parser("bench", help="Time decoding and prompt processing")
     b.add_argument("rest", nargs=argparse.REMAINDER)
     return parser
 

@@ -28,6 +28,7 @@
 // and a second kernel merges the ranges in order.
 #include "common.h"
 #include "leone_hip.h"
+#include "prefill_order.h"
 
 #include <math.h>
 
@@ -70,25 +71,9 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     const int tid = threadIdx.x;
     const int c = lane & 15, g = lane >> 4;
 
-    // Workgroups go round the chip's eight dies in turn, each die has a cache of its own, and a compute
-    // unit holds two workgroups.  Work is numbered with a key/value head's query heads and tile groups
-    // together; a die gets a run of neighbouring numbers (few key/value heads, whose keys its cache then
-    // keeps), and within a die the second half of the workgroups takes the groups in falling order, so
-    // that a compute unit tends to hold a group that sees few keys beside one that sees many.
-    constexpr int kDies = 8;
-    const int launched = gridDim.x;
-    int head, group;
-    if (launched % (2 * kDies) == 0 && n_groups % 2 == 0) {
-        const int per_die = launched / kDies, spot = blockIdx.x / kDies;
-        const int heads_here = per_die / n_groups;                     // per_die = heads_here * n_groups
-        const int late = spot / (per_die / 2), r = spot % (per_die / 2);
-        const int pair = r / heads_here;
-        head = (blockIdx.x % kDies) * heads_here + r % heads_here;
-        group = late ? n_groups - 1 - pair : pair;
-    } else {
-        head = blockIdx.x / n_groups;
-        group = blockIdx.x % n_groups;
-    }
+    // Which head and tile group this workgroup takes (an order that suits the dies' caches: prefill_order.h).
+    const PrefillWork work = prefill_work(static_cast<int>(blockIdx.x), q_heads, n_groups);
+    const int head = work.head, group = work.group;
     const int kvh = head / (q_heads / kv_heads);
     const int page_tokens = 1 << page_shift, page_mask = page_tokens - 1;
 

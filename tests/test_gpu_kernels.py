@@ -529,6 +529,43 @@ def test_attention_prefill(shape, window, splits):
     close(out[:-1].reshape(len(rows) - 1, q_heads, head_dim), want, 2e-2, 2e-2, "attention_prefill")
 
 
+@pytest.mark.parametrize("portions", [[(0, 0, 200)], [(0, 0, 40), (1, 10, 20), (2, 0, 100), (3, 5, 16)],
+                                      [(0, 0, 500)], [(0, 3, 900)], [(0, 0, 130), (1, 0, 385)]],
+                         ids=["2groups", "4groups", "4groups-one", "8groups", "6groups"])
+@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 1, 32, 64), (12, 4, 64, 16), (20, 4, 32, 32), (32, 8, 128, 64),
+                                   (2, 1, 16, 16), (8, 8, 48, 16)])
+def test_attention_prefill_every_head_of_every_group(shape, portions):
+    """Head counts that are no multiple of eight with 2, 4, 6 and 8 tile groups in one launch: every
+    (head, group) pair must be computed (a numbering of workgroups by dies once left some out).  The
+    output starts as NaN, so a pair that nobody takes shows."""
+    from leone_amd import ops
+    q_heads, kv_heads, head_dim, page_tokens = shape
+    dtype = torch.bfloat16
+    lengths = {}
+    for r, start, count in portions:
+        lengths[r] = max(lengths.get(r, 0), start + count)
+    table, k_pool, v_pool, keys, values = paged_setup([lengths[r] for r in sorted(lengths)], kv_heads, head_dim,
+                                                      page_tokens, dtype, seed=71)
+    rows, listed = [], []
+    for entry, (r, start, count) in enumerate(portions):
+        listed.append((entry, len(rows), count))
+        rows += [(r, start + i) for i in range(count)]
+    tiles = ops.prefill_tiles(listed)
+    # an entry's block table is its request's
+    entry_table = table[[r for r, _, _ in portions]].contiguous()
+    g = torch.Generator().manual_seed(72)
+    q = torch.randn(len(rows), q_heads, head_dim, generator=g).to(dtype)
+    positions = torch.tensor([p for _, p in rows], dtype=torch.int32)
+    out = torch.full((len(rows), q_heads * head_dim), float("nan"), dtype=dtype, device=DEV)
+    ops.attention_prefill(q.reshape(len(rows), -1).to(DEV), out, k_pool.to(DEV), v_pool.to(DEV), positions.to(DEV),
+                          tiles.to(DEV), entry_table.to(DEV), q_heads, 1.0 / math.sqrt(head_dim), splits=1)
+    assert torch.isfinite(out.float()).all(), "some (head, group) pair was not computed"
+    picked = list(range(0, len(rows), 7)) + [len(rows) - 1]
+    want = torch.stack([plain.attend_one(q[i].float(), keys[rows[i][0]][:rows[i][1] + 1], values[rows[i][0]][:rows[i][1] + 1], None)
+                        for i in picked])
+    close(out[picked].reshape(len(picked), q_heads, head_dim), want, 2e-2, 2e-2, "attention_prefill")
+
+
 @pytest.mark.parametrize("splits", [1, 3])
 @pytest.mark.parametrize("dealt", [False, True])
 def test_attention_prefill_finds_the_one_key_that_matters(dealt, splits):

@@ -26,3 +26,18 @@ def test_random_workload_is_clean_under_sanitizers(tmp_path):
                UBSAN_OPTIONS="halt_on_error=1")
     run = subprocess.run([binary], capture_output=True, text=True, env=env, timeout=300)
     assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout + run.stderr
+
+
+def test_prompt_attention_workgroup_numbering_covers_every_pair_once(tmp_path):
+    """Every (head, tile group) pair belongs to exactly one workgroup, for 1..64 heads and 1..32 groups
+    (head counts that are no multiple of the eight dies once left heads out)."""
+    compiler = shutil.which("g++") or shutil.which("clang++")
+    if compiler is None:
+        pytest.skip("no C++ compiler")
+    binary = str(tmp_path / "prefill_order_check")
+    build = subprocess.run([compiler, "-std=c++17", "-O1", "-I", os.path.join(ROOT, "leone_amd", "csrc"),
+                            os.path.join(ROOT, "tests", "native", "prefill_order_check.cpp"), "-o", binary],
+                           capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr
+    run = subprocess.run([binary], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0 and run.stdout.strip().endswith("ok"), run.stdout + run.stderr
