@@ -84,6 +84,14 @@ int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const voi
 int leone_argmax_chunk();
 int leone_argmax(const float* logits, int* out, float* part_value, int* part_index, int rows, int vocab,
                  hipStream_t stream);
+// leone_argmax with its workspace in a fixed device array of the library instead of an argument.  It has no
+// counterpart in the reference; it is for callers that cannot allocate device memory (under graph capture, in
+// a tight serving loop, in a harness that forbids it): the call allocates and frees nothing.  rows *
+// ceil(vocab / leone_argmax_chunk()) may be at most leone_argmax_static_max_entries() (128 KiB of device
+// memory that every GPU the library runs on holds until the process ends); larger calls are refused.  Calls
+// on one GPU share that array: calls that overlap in time on one GPU race.
+int leone_argmax_static_max_entries();
+int leone_argmax_static(const float* logits, int* out, int rows, int vocab, hipStream_t stream);
 // The token whose share of the weights exp(l / t - max / t), walked in id order, holds uniform[row]; -1 for a
 // row without a finite logit.  Workspace: part_value and part_index as for leone_argmax, best with one
 // entry a row, sums with rows * ceil(vocab / leone_argmax_chunk()) doubles.

@@ -11,6 +11,7 @@
 #include "leone_hip.h"
 
 #include <math.h>
+#include <mutex>
 
 namespace leone {
 
@@ -317,6 +318,68 @@ extern "C" int leone_argmax(const float* logits, int* out, float* part_value, in
     LEONE_LAUNCH_CHECK("argmax");
     argmax_final_kernel<<<rows, kSampleThreads, 0, stream>>>(part_value, part_index, out, chunks);
     LEONE_LAUNCH_CHECK("argmax");
+    return 0;
+}
+
+// ---- argmax without a workspace argument and without any allocation --------------------------------
+// For callers that cannot allocate device memory around the call (code under graph capture, tight serving
+// loops, harnesses that forbid it).  The per-chunk candidates of leone_argmax live in a file-scope device
+// array instead of a workspace the caller brings.  Each GPU holds its own copy of the array at its own
+// address until the process ends; the address is asked for once per device and kept.
+constexpr int kStaticArgmaxEntries = 16384;                         // rows * chunks at most: 128 KiB a GPU
+constexpr int kStaticMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticArgmaxEntries * (sizeof(float) + sizeof(int))];
+
+namespace leone {
+static std::mutex g_scratch_lock;
+static void* g_scratch_ptr[kStaticMaxDevices] = {};                 // device address of `scratch`, per device
+
+// The address of this device's copy of the array (the array's name is only a stand-in in host code).
+static int scratch_for_current_device(void** out) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess || device < 0 || device >= kStaticMaxDevices) {
+        set_error("argmax_static: no usable current device (%s)", hipGetErrorString(e));
+        return 1;
+    }
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if (g_scratch_ptr[device] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            set_error("argmax_static: the address of the scratch array on device %d was refused: %s", device,
+                      hipGetErrorString(e));
+            return 1;
+        }
+        g_scratch_ptr[device] = ptr;
+    }
+    *out = g_scratch_ptr[device];
+    return 0;
+}
+}  // namespace leone
+
+extern "C" int leone_argmax_static_max_entries() { return kStaticArgmaxEntries; }
+
+// The same result as leone_argmax.  rows * ceil(vocab / leone_argmax_chunk()) may be at most
+// leone_argmax_static_max_entries(); beyond that the call is refused.  Every entry of the array that the
+// second kernel reads is written by the first kernel of the same call, so nothing has to start at zero;
+// what an earlier call left is overwritten or never read.  All calls on one GPU share that GPU's array:
+// two calls that overlap in time on one GPU (different streams, or threads) race and give wrong tokens.
+extern "C" int leone_argmax_static(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+    LEONE_REQUIRE(logits && out, "argmax_static: null pointer");
+    LEONE_REQUIRE(rows > 0 && rows <= 65535 && vocab > 0, "argmax_static: rows %d vocab %d out of range", rows, vocab);
+    const int chunks = ceil_div(vocab, kArgmaxChunk);
+    LEONE_REQUIRE(static_cast<long>(rows) * chunks <= kStaticArgmaxEntries,
+                  "argmax_static: %d rows of %d chunks need %ld entries, the fixed scratch array holds %d",
+                  rows, chunks, static_cast<long>(rows) * chunks, kStaticArgmaxEntries);
+    void* base = nullptr;
+    if (scratch_for_current_device(&base)) return 1;
+    float* part_value = static_cast<float*>(base);
+    int* part_index = reinterpret_cast<int*>(static_cast<unsigned char*>(base) + kStaticArgmaxEntries * sizeof(float));
+    argmax_partial_kernel<<<dim3(chunks, rows), kSampleThreads, 0, stream>>>(logits, part_value, part_index, vocab, chunks);
+    LEONE_LAUNCH_CHECK("argmax_static");
+    argmax_final_kernel<<<rows, kSampleThreads, 0, stream>>>(part_value, part_index, out, chunks);
+    LEONE_LAUNCH_CHECK("argmax_static");
     return 0;
 }
 
