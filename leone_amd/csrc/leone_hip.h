@@ -31,8 +31,10 @@ int leone_rope_table(float* cos_out, float* sin_out, double theta, int rotary_di
                      hipStream_t stream);
 
 // Per-head RMSNorm (gains may be null), half-split rotation (tables may be
-// null), q to q_out, k and v into the paged cache.
-int leone_qk_norm_rope_write(const void* qkv, void* q_out, void* k_pool, void* v_pool, int dtype,
+// null), q to q_out, k and v into the paged cache.  The input is of the outputs' type, or float32 in
+// qkv_planes planes (qkv_plane elements apart) that are added up in order: a product cut along K.
+int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_planes, long qkv_plane, void* q_out,
+                             void* k_pool, void* v_pool, int dtype,
                              const void* q_gain, const void* k_gain, int gain_dtype, float eps,
                              const float* cos_table, const float* sin_table, int table_positions,
                              const int* positions, const int* row_entry, const int* block_table, int max_blocks,
@@ -78,6 +80,18 @@ int leone_gemm_f32(const float* a, const float* b, float* c, int m, int n, int k
 int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const void* gain, int gain_dtype, float eps,
                           const void* w, void* y, int out_mode, int out_dtype, int m, int n, int k,
                           hipStream_t stream);
+
+// Y[M,N] = X[M,K] . W[N,K]^T for bfloat16 X and W, M in 1..leone_gemm_rows_max_rows(), K a multiple of 8: W is
+// streamed once, X goes through shared memory.  out_mode 0: y[M,N] of out_dtype; 1: y float32 [M,N] += product;
+// 2: W interleaves 8 gate rows with their 8 up rows, y bfloat16 [M,N/2] = silu(gate) * up; 3: y float32
+// [splits][M,N], planes `plane` elements apart, plane s holding the product over the s-th range of K (whole
+// chunks of leone_gemm_rows_chunk(M) elements, ceil(chunks / splits) a range, no range empty).  splits > 1 only
+// with out_mode 3.  waves (4, 6 or 8; 16 rows of W each) is a tuning choice: it changes the result only through
+// the order of the sum over K.
+int leone_gemm_rows_max_rows();
+int leone_gemm_rows_chunk(int m);
+int leone_gemm_rows_bf16(const void* x, const void* w, void* y, int out_mode, int out_dtype, int m, int n, int k,
+                         int splits, long plane, int waves, hipStream_t stream);
 
 // Highest finite logit of each row, lowest index on ties, -1 if none.  Workspace: part_value and
 // part_index with rows * ceil(vocab / leone_argmax_chunk()) entries each.

@@ -8,6 +8,8 @@
 // (crates/leone/src/cpu.rs:892-907).  Sums of squares, gains and rotations are
 // computed in float whatever the storage type; rotary angles in double.
 #include "common.h"
+
+#include <type_traits>
 #include "leone_hip.h"
 
 namespace leone {
@@ -188,9 +190,9 @@ __global__ void rope_table_kernel(float* __restrict__ cos_out, float* __restrict
 // another layer's cache).
 constexpr int kMaxPairsPerLane = 4;  // head_dim up to 512
 
-template <typename T>
+template <typename TIn, typename T>
 __global__ void qk_norm_rope_write_kernel(
-    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_pool, T* __restrict__ v_pool,
+    const TIn* __restrict__ qkv, int planes, long plane, T* __restrict__ q_out, T* __restrict__ k_pool, T* __restrict__ v_pool,
     AnyVec q_gain, AnyVec k_gain, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int table_positions, const int* __restrict__ positions,
     const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
@@ -202,7 +204,7 @@ __global__ void qk_norm_rope_write_kernel(
     if (head >= heads_total) return;
     const int half = head_dim / 2;
     const int qkv_width = (q_heads + 2 * kv_heads) * head_dim;
-    const T* src = qkv + static_cast<long>(row) * qkv_width + static_cast<long>(head) * head_dim;
+    const TIn* src = qkv + static_cast<long>(row) * qkv_width + static_cast<long>(head) * head_dim;
     const int pos = positions[row];
 
     const bool is_q = head < q_heads;
@@ -233,6 +235,10 @@ __global__ void qk_norm_rope_write_kernel(
         if (p < half) {
             a[i] = to_float(src[p]);
             b[i] = to_float(src[p + half]);
+            for (int s = 1; s < planes; ++s) {       // planes of a product cut along K: added in order
+                a[i] += to_float(src[s * plane + p]);
+                b[i] += to_float(src[s * plane + p + half]);
+            }
             ss = fmaf(a[i], a[i], ss);
             ss = fmaf(b[i], b[i], ss);
         }
@@ -301,10 +307,10 @@ __device__ inline void load_run(const AnyVec& v, int at, float out[8]) {
     }
 }
 
-template <typename T, int kD16>
+template <typename TIn, typename T, int kD16>
 __global__ void __launch_bounds__(256)
 qk_norm_rope_write_runs_kernel(
-    const T* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_pool, T* __restrict__ v_pool,
+    const TIn* __restrict__ qkv, int planes, long plane, T* __restrict__ q_out, T* __restrict__ k_pool, T* __restrict__ v_pool,
     AnyVec q_gain, AnyVec k_gain, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int table_positions, const int* __restrict__ positions,
     const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
@@ -320,19 +326,31 @@ qk_norm_rope_write_runs_kernel(
     const int row = mine ? static_cast<int>(item / heads_total) : 0;
     const int head = mine ? static_cast<int>(item % heads_total) : 0;
     const int qkv_width = (q_heads + 2 * kv_heads) * kD;
-    const T* src = qkv + static_cast<long>(row) * qkv_width + static_cast<long>(head) * kD + 8 * j;
+    const TIn* src = qkv + static_cast<long>(row) * qkv_width + static_cast<long>(head) * kD + 8 * j;
     const bool is_q = head < q_heads;
     const bool is_k = !is_q && head < q_heads + kv_heads;
 
     float a[8], b[8];
     float ss = 0.f;
     if (mine) {
-        const HeadRun<T> lo = *reinterpret_cast<const HeadRun<T>*>(src);
-        const HeadRun<T> hi = *reinterpret_cast<const HeadRun<T>*>(src + kHalf);
+        const HeadRun<TIn> lo = *reinterpret_cast<const HeadRun<TIn>*>(src);
+        const HeadRun<TIn> hi = *reinterpret_cast<const HeadRun<TIn>*>(src + kHalf);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             a[i] = to_float(lo.v[i]);
             b[i] = to_float(hi.v[i]);
+        }
+        for (int s = 1; s < planes; ++s) {           // planes of a product cut along K: added in order
+            const HeadRun<TIn> lo_s = *reinterpret_cast<const HeadRun<TIn>*>(src + s * plane);
+            const HeadRun<TIn> hi_s = *reinterpret_cast<const HeadRun<TIn>*>(src + s * plane + kHalf);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                a[i] += to_float(lo_s.v[i]);
+                b[i] += to_float(hi_s.v[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
             ss = fmaf(a[i], a[i], ss);
             ss = fmaf(b[i], b[i], ss);
         }
@@ -447,24 +465,25 @@ value_write_kernel(const T* __restrict__ qkv, T* __restrict__ v_pool, const int*
     }
 }
 
-template <typename T, int kD16>
-static void launch_runs(const void* qkv, void* q_out, void* k_pool, void* v_pool, AnyVec qg, AnyVec kg, float eps,
+template <typename TIn, typename T, int kD16>
+static void launch_runs(const void* qkv, int planes, long plane, void* q_out, void* k_pool, void* v_pool, AnyVec qg, AnyVec kg, float eps,
                         const float* cos_table, const float* sin_table, int table_positions, const int* positions,
                         const int* row_entry, const int* block_table, int max_blocks, int rows, int q_heads,
                         int kv_heads, int page_tokens, int write_cache, hipStream_t stream) {
     constexpr int kShare = kD16 <= 1 ? 1 : kD16 <= 2 ? 2 : kD16 <= 4 ? 4 : 8;
     // Many rows are mostly prompt portions: their values go through the kernel that writes whole runs.
-    const bool values_apart = write_cache && rows >= 64 && ceil_div(rows, 8) <= 0x7fffffff && kv_heads <= 65535;
+    const bool values_apart = write_cache && rows >= 64 && ceil_div(rows, 8) <= 0x7fffffff && kv_heads <= 65535 &&
+                              std::is_same<TIn, T>::value && planes == 1;
     const long items = static_cast<long>(rows) * (q_heads + (write_cache ? (values_apart ? 1 : 2) * kv_heads : 0));
     const int blocks = ceil_div(items * kShare, 256);
-    qk_norm_rope_write_runs_kernel<T, kD16><<<blocks, 256, 0, stream>>>(
-        static_cast<const T*>(qkv), static_cast<T*>(q_out), static_cast<T*>(k_pool), static_cast<T*>(v_pool), qg, kg, eps,
+    qk_norm_rope_write_runs_kernel<TIn, T, kD16><<<blocks, 256, 0, stream>>>(
+        static_cast<const TIn*>(qkv), planes, plane, static_cast<T*>(q_out), static_cast<T*>(k_pool), static_cast<T*>(v_pool), qg, kg, eps,
         cos_table, sin_table, table_positions, positions, row_entry, block_table, max_blocks, rows, q_heads, kv_heads,
         page_tokens, write_cache, values_apart ? 0 : 1);
     if (values_apart) {
         constexpr int kD = 16 * kD16;
         value_write_kernel<T><<<dim3(ceil_div(rows, 8), kv_heads), kD, 8 * kD * sizeof(T), stream>>>(
-            static_cast<const T*>(qkv), static_cast<T*>(v_pool), positions, row_entry, block_table, max_blocks, rows,
+            reinterpret_cast<const T*>(qkv), static_cast<T*>(v_pool), positions, row_entry, block_table, max_blocks, rows,
             q_heads, kv_heads, kD, page_tokens);
     }
 }
@@ -584,14 +603,20 @@ extern "C" int leone_rope_table(float* cos_out, float* sin_out, double theta, in
     return 0;
 }
 
-extern "C" int leone_qk_norm_rope_write(const void* qkv, void* q_out, void* k_pool, void* v_pool, int dtype,
+extern "C" int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_planes, long qkv_plane, void* q_out,
+                                        void* k_pool, void* v_pool, int dtype,
                                         const void* q_gain, const void* k_gain, int gain_dtype, float eps,
                                         const float* cos_table, const float* sin_table, int table_positions,
                                         const int* positions, const int* row_entry, const int* block_table,
                                         int max_blocks, int rows, int q_heads, int kv_heads, int head_dim,
                                         int page_tokens, int write_cache, hipStream_t stream) {
-    if (check_dtype(dtype, "qk_norm_rope_write") || check_dtype(gain_dtype, "qk_norm_rope_write gain")) return 1;
+    if (check_dtype(dtype, "qk_norm_rope_write") || check_dtype(gain_dtype, "qk_norm_rope_write gain") ||
+        check_dtype(qkv_dtype, "qk_norm_rope_write input"))
+        return 1;
     LEONE_REQUIRE(qkv && q_out && positions, "qk_norm_rope_write: null pointer");
+    LEONE_REQUIRE(qkv_dtype == dtype || qkv_dtype == kF32, "qk_norm_rope_write: the input is of the output's type or float32");
+    LEONE_REQUIRE(qkv_planes >= 1 && qkv_planes <= 64 && (qkv_planes == 1 || qkv_plane % 8 == 0),
+                  "qk_norm_rope_write: %d planes of input", qkv_planes);
     LEONE_REQUIRE(!write_cache || (k_pool && v_pool && row_entry && block_table && max_blocks > 0 && page_tokens > 0),
                   "qk_norm_rope_write: cache write needs pools, row map and block table");
     LEONE_REQUIRE((q_gain == nullptr) == (k_gain == nullptr), "qk_norm_rope_write: q and k gains come together");
@@ -604,43 +629,42 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, void* q_out, void* k_po
                   "qk_norm_rope_write: the cache needs head_dim %d and page_tokens %d to be multiples of 8", head_dim, page_tokens);
     AnyVec qg{q_gain, gain_dtype}, kg{k_gain, gain_dtype};
     const uintptr_t run_bytes = 8 * (dtype == kF32 ? sizeof(float) : sizeof(bf16_t));
-    const bool aligned = reinterpret_cast<uintptr_t>(qkv) % run_bytes == 0 && reinterpret_cast<uintptr_t>(q_out) % run_bytes == 0 &&
+    const uintptr_t in_run_bytes = 8 * (qkv_dtype == kF32 ? sizeof(float) : sizeof(bf16_t));
+    const bool aligned = reinterpret_cast<uintptr_t>(qkv) % in_run_bytes == 0 && reinterpret_cast<uintptr_t>(q_out) % run_bytes == 0 &&
                          (!write_cache || (reinterpret_cast<uintptr_t>(k_pool) % run_bytes == 0 && page_tokens % 8 == 0));
     const bool tables_aligned = (!q_gain || (reinterpret_cast<uintptr_t>(q_gain) % 32 == 0 && reinterpret_cast<uintptr_t>(k_gain) % 32 == 0)) &&
                                 (!cos_table || (reinterpret_cast<uintptr_t>(cos_table) % 32 == 0 && reinterpret_cast<uintptr_t>(sin_table) % 32 == 0));
     if (head_dim % 16 == 0 && head_dim <= 128 && aligned && tables_aligned && static_cast<long>(rows) * (q_heads + 2 * kv_heads) * 8 < 0x7fffffffL * 256) {
-#define LEONE_RUNS_CASE(N)                                                                                          \
-    case N:                                                                                                         \
-        if (dtype == kF32)                                                                                          \
-            launch_runs<float, N>(qkv, q_out, k_pool, v_pool, qg, kg, eps, cos_table, sin_table, table_positions,   \
-                                  positions, row_entry, block_table, max_blocks, rows, q_heads, kv_heads,           \
-                                  page_tokens, write_cache, stream);                                                \
-        else                                                                                                        \
-            launch_runs<bf16_t, N>(qkv, q_out, k_pool, v_pool, qg, kg, eps, cos_table, sin_table, table_positions,  \
-                                   positions, row_entry, block_table, max_blocks, rows, q_heads, kv_heads,          \
-                                   page_tokens, write_cache, stream);                                               \
+#define LEONE_RUNS_ARGS                                                                                             \
+    qkv, qkv_planes, qkv_plane, q_out, k_pool, v_pool, qg, kg, eps, cos_table, sin_table, table_positions, positions, \
+        row_entry, block_table, max_blocks, rows, q_heads, kv_heads, page_tokens, write_cache, stream
+#define LEONE_RUNS_CASE(N)                                                     \
+    case N:                                                                    \
+        if (dtype == kF32) launch_runs<float, float, N>(LEONE_RUNS_ARGS);      \
+        else if (qkv_dtype == kF32) launch_runs<float, bf16_t, N>(LEONE_RUNS_ARGS); \
+        else launch_runs<bf16_t, bf16_t, N>(LEONE_RUNS_ARGS);                  \
         break;
         switch (head_dim / 16) {
             LEONE_RUNS_CASE(1) LEONE_RUNS_CASE(2) LEONE_RUNS_CASE(3) LEONE_RUNS_CASE(4)
             LEONE_RUNS_CASE(5) LEONE_RUNS_CASE(6) LEONE_RUNS_CASE(7) LEONE_RUNS_CASE(8)
         }
 #undef LEONE_RUNS_CASE
+#undef LEONE_RUNS_ARGS
         LEONE_LAUNCH_CHECK("qk_norm_rope_write");
         return 0;
     }
     const int heads_total = q_heads + (write_cache ? 2 * kv_heads : 0);
     const int waves_per_block = 4;
     dim3 grid(rows, ceil_div(heads_total, waves_per_block));
-    if (dtype == kF32)
-        qk_norm_rope_write_kernel<float><<<grid, waves_per_block * kWave, 0, stream>>>(
-            static_cast<const float*>(qkv), static_cast<float*>(q_out), static_cast<float*>(k_pool),
-            static_cast<float*>(v_pool), qg, kg, eps, cos_table, sin_table, table_positions, positions, row_entry,
-            block_table, max_blocks, q_heads, kv_heads, head_dim, page_tokens, write_cache);
-    else
-        qk_norm_rope_write_kernel<bf16_t><<<grid, waves_per_block * kWave, 0, stream>>>(
-            static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(q_out), static_cast<bf16_t*>(k_pool),
-            static_cast<bf16_t*>(v_pool), qg, kg, eps, cos_table, sin_table, table_positions, positions, row_entry,
-            block_table, max_blocks, q_heads, kv_heads, head_dim, page_tokens, write_cache);
+#define LEONE_QK_ANY(TIN, T)                                                                                        \
+    qk_norm_rope_write_kernel<TIN, T><<<grid, waves_per_block * kWave, 0, stream>>>(                                \
+        static_cast<const TIN*>(qkv), qkv_planes, qkv_plane, static_cast<T*>(q_out), static_cast<T*>(k_pool),       \
+        static_cast<T*>(v_pool), qg, kg, eps, cos_table, sin_table, table_positions, positions, row_entry,          \
+        block_table, max_blocks, q_heads, kv_heads, head_dim, page_tokens, write_cache)
+    if (dtype == kF32) LEONE_QK_ANY(float, float);
+    else if (qkv_dtype == kF32) LEONE_QK_ANY(float, bf16_t);
+    else LEONE_QK_ANY(bf16_t, bf16_t);
+#undef LEONE_QK_ANY
     LEONE_LAUNCH_CHECK("qk_norm_rope_write");
     return 0;
 }

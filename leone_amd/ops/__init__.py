@@ -136,13 +136,19 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim:
                        cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
                        row_entry: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                        k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor], write_cache: bool = True,
-                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Splits the fused projection, normalises and rotates q and k heads, writes k and v into the cache."""
-    rows, width = qkv.shape
+                       out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Splits the fused projection, normalises and rotates q and k heads, writes k and v into the cache.
+    ``qkv`` is ``[rows, width]`` of the cache's type, or float32 (also as planes ``[p, rows, width]`` whose
+    sum, in order, is meant: a product cut along K) with ``out_dtype`` naming the type of q and the cache."""
+    planes = qkv.shape[0] if qkv.dim() == 3 else 1
+    rows, width = qkv.shape[-2:]
+    kind = out_dtype or qkv.dtype
+    if qkv.dtype != kind and qkv.dtype != torch.float32:
+        raise KernelError(f"qk_norm_rope_write: input {qkv.dtype} for outputs of {kind}")
     if width != (q_heads + 2 * kv_heads) * head_dim:
         raise KernelError(f"qk_norm_rope_write: width {width} is not ({q_heads}+2*{kv_heads})*{head_dim}")
     if out is None:
-        out = torch.empty((rows, q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+        out = torch.empty((rows, q_heads * head_dim), dtype=kind, device=qkv.device)
     max_blocks = page_tokens = 0
     if write_cache:
         if k_pool is None or v_pool is None or block_table is None or row_entry is None:
@@ -160,9 +166,10 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim:
     gain_code = _code(q_gain, "q gain") if q_gain is not None else F32
     if q_gain is not None and (k_gain is None or k_gain.dtype != q_gain.dtype):
         raise KernelError("qk_norm_rope_write: q and k gains must come together in one type")
-    call("leone_qk_norm_rope_write", _dev(qkv, "qkv"), _dev(out, "q out", qkv.dtype),
-         _dev(k_pool if write_cache else None, "k pool", qkv.dtype),
-         _dev(v_pool if write_cache else None, "v pool", qkv.dtype), _code(qkv, "qkv"),
+    call("leone_qk_norm_rope_write", _dev(qkv, "qkv"), _code(qkv, "qkv"), planes, rows * width,
+         _dev(out, "q out", kind),
+         _dev(k_pool if write_cache else None, "k pool", kind),
+         _dev(v_pool if write_cache else None, "v pool", kind), _CODES[kind],
          _dev(q_gain, "q gain", None, (head_dim,)), _dev(k_gain, "k gain", None, (head_dim,)), gain_code,
          float(eps), _dev(cos, "rope cos", torch.float32), _dev(sin, "rope sin", torch.float32), table_positions,
          _dev(positions, "positions", torch.int32, (rows,)),
@@ -384,6 +391,92 @@ def gemm_fused(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
     return None if residual is not None else out
 
 
+ROWS_MAX = 128               # most rows the multi-row weight-streaming product takes (checked against the library)
+ROWS_WAVES = (4, 6, 8)       # workgroup sizes it is built for, in waves (16 weight rows each)
+_UNITS = {}
+
+
+def compute_units(device) -> int:
+    index = torch.device(device).index or 0
+    if index not in _UNITS:
+        _UNITS[index] = torch.cuda.get_device_properties(index).multi_processor_count if torch.cuda.is_available() else 256
+    return _UNITS[index]
+
+
+def rows_plan(m: int, n: int, k: int, may_split: bool, units: int = 256) -> tuple[int, int]:
+    """(waves, splits) for ``gemm_rows``: how many waves (tiles of 16 weight rows) a workgroup gets and into
+    how many ranges K is cut.  The kernel is fastest with one workgroup on every compute unit and none
+    waiting for a second round (6,144 x 4,096 at 64 rows: 18 us with 256 workgroups, 22 with 480, 24 with
+    288), so the plan minimises rounds x the longest workgroup's traffic, where a chunk of K costs a
+    workgroup its waves' weight tiles plus half of X's tiles (those come from the cache) and starting up
+    costs as much as 768 elements of K; ties go to fewer ranges, then fewer waves.  Matrices with rows for many rounds (a vocabulary) take the workgroup size by
+    the rows of X alone."""
+    chunk = library().leone_gemm_rows_chunk(m)
+    chunks = -(-k // chunk)
+    tiles = -(-n // 16)
+    x_tiles = -(-m // 16)
+    if tiles >= 8 * units:
+        return (4 if m <= 32 else 6 if m <= 80 else 8), 1
+    best = None
+    for waves in ROWS_WAVES:
+        groups = -(-tiles // waves)
+        for splits in range(1, (min(chunks, 16) if may_split else 1) + 1):
+            per = -(-chunks // splits)
+            if per * (splits - 1) >= chunks:            # a range would be empty
+                continue
+            rounds = -(-groups * splits // units)
+            cost = (rounds * (per + 768 // chunk) * (waves + 0.5 * x_tiles), splits, waves)
+            if best is None or cost < best:
+                best = cost
+    return best[2], best[1]
+
+
+def gemm_rows(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+              residual: Optional[torch.Tensor] = None, gated: bool = False, splits: Optional[int] = None,
+              waves: Optional[int] = None, may_split: bool = True) -> Optional[torch.Tensor]:
+    """The weight-streaming product for up to ROWS_MAX rows of bfloat16 ``x``.  With ``residual`` and one
+    range of K the product is added into that float32 tensor (None returned); with ``gated`` the weight is
+    an interleaved gate/up weight and silu(gate) * up comes out.  With more than one range of K (``splits``;
+    by default what ``rows_plan`` finds best, one if ``may_split`` is false or the product is gated) float32
+    planes ``[splits, M, N]`` are returned whose sum, in order, is the product (with ``residual``: for the
+    caller to add)."""
+    m, k = x.shape
+    n, k2 = weight.shape
+    if k != k2:
+        raise KernelError(f"gemm_rows: inner sizes {k} and {k2} differ")
+    if library().leone_gemm_rows_max_rows() != ROWS_MAX:
+        raise KernelError("the kernel library was built for another number of rows")
+    if not 1 <= m <= ROWS_MAX:
+        raise KernelError(f"gemm_rows: {m} rows, the kernel takes 1..{ROWS_MAX}")
+    if residual is not None and gated:
+        raise KernelError("gemm_rows: a gated product cannot also be added into the stream")
+    if splits is None or waves is None:
+        plan = rows_plan(m, n, k, may_split and not gated, compute_units(weight.device))
+        waves = plan[0] if waves is None else waves
+        splits = plan[1] if splits is None else splits
+    chunks = -(-k // library().leone_gemm_rows_chunk(m))
+    splits = max(1, min(int(splits), chunks))
+    splits = -(-chunks // -(-chunks // splits))        # no range of K may be empty
+    if gated:
+        splits = 1
+    plane = 0
+    if splits > 1:
+        out, mode, kind = torch.empty((splits, m, n), dtype=torch.float32, device=weight.device), 3, torch.float32
+        plane = m * n
+    elif residual is not None:
+        out, mode, kind = residual, 1, torch.float32
+        _dev(out, "gemm_rows stream", torch.float32, (m, n))
+    elif gated:
+        out, mode, kind = torch.empty((m, n // 2), dtype=torch.bfloat16, device=weight.device), 2, torch.bfloat16
+    else:
+        out, mode, kind = torch.empty((m, n), dtype=out_dtype, device=weight.device), 0, out_dtype
+    with profile.span("gemm rows", weight):
+        call("leone_gemm_rows_bf16", _dev(x, "gemm x", torch.bfloat16, (m, k)),
+             _dev(weight, "gemm weight", torch.bfloat16), _dev(out, "gemm out", kind), mode, _CODES[kind], m, n, k,
+             splits, plane, int(waves), _stream())
+    return None if (residual is not None and splits == 1) else out
+
+
 def inner_parts(rows: int, n: int, k: int) -> int:
     """Into how many parts the inner dimension of x[rows, k] . w[n, k]^T is cut when the result goes into the
     float32 stream.  The library's product does badly with a few hundred rows, few columns and a long inner
@@ -399,7 +492,8 @@ def inner_parts(rows: int, n: int, k: int) -> int:
 
 
 def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-           residual: Optional[torch.Tensor] = None, gated: bool = False) -> Optional[torch.Tensor]:
+           residual: Optional[torch.Tensor] = None, gated: bool = False,
+           planes_ok: bool = False) -> Optional[torch.Tensor]:
     """x[R,K] . weight[N,K]^T, with optional neighbours.
 
     ``x`` is a tensor or ``NormedRows`` (a norm still to be done).  ``gated``: the weight is an
@@ -408,9 +502,13 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     is returned, otherwise the product is returned for the caller to add later, as float32 ``[R, N]`` or
     as a stack of planes ``[p, R, N]`` whose sum is meant (``add_rmsnorm`` takes either).
 
+    ``planes_ok``: the caller also takes a plain product as float32 planes ``[p, R, N]`` whose sum, in
+    order, is meant (``qk_norm_rope_write`` does).
+
     float32 runs the single-precision kernel.  bfloat16 accumulates in float: up to FUSED_ROWS rows on the
-    weight-streaming kernel with everything folded in, more rows through the library's matrix product;
-    float32 results (logits) always come from the weight-streaming kernel.
+    weight-streaming kernel with everything folded in, up to ROWS_MAX rows (a decode step of many requests)
+    on the multi-row weight-streaming kernel, more rows (prompt portions) through the library's matrix
+    product, with float32 output for logits and for what goes into the stream.
     """
     dtype = x.dtype if isinstance(x, NormedRows) else x.dtype
     if dtype != weight.dtype:
@@ -425,6 +523,9 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
             x = x.materialize()
         return gemm_fused(x, weight, out_dtype, residual, gated)
     x = materialize(x)
+    if dtype == torch.bfloat16 and weight.is_cuda and k % 8 == 0 and rows <= ROWS_MAX \
+            and (not gated or weight.shape[0] % 16 == 0):
+        return gemm_rows(x, weight, out_dtype, residual, gated, may_split=planes_ok or residual is not None)
     if dtype == torch.float32:
         if out_dtype != torch.float32:
             raise KernelError("linear: the float32 path produces float32")

@@ -26,7 +26,7 @@ _PROTOTYPES = {
     "leone_add_rmsnorm": [P, P, c_int, c_int, ctypes.c_long, P, c_int, c_float, P, c_int, P, c_int, c_int, P],
     "leone_swiglu": [P, P, c_int, c_int, c_int, P],
     "leone_rope_table": [P, P, c_double, c_int, c_int, P],
-    "leone_qk_norm_rope_write": [P, P, P, P, c_int, P, P, c_int, c_float, P, P, c_int, P, P, P, c_int,
+    "leone_qk_norm_rope_write": [P, c_int, c_int, ctypes.c_long, P, P, P, c_int, P, P, c_int, c_float, P, P, c_int, P, P, P, c_int,
                                  c_int, c_int, c_int, c_int, c_int, c_int, P],
     "leone_attention_rows": [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                              c_int, P],
@@ -36,6 +36,7 @@ _PROTOTYPES = {
                                 c_int, P],
     "leone_gemm_f32": [P, P, P, c_int, c_int, c_int, P],
     "leone_gemm_fused_bf16": [P, c_int, P, P, c_int, c_float, P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "leone_gemm_rows_bf16": [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, ctypes.c_long, c_int, P],
     "leone_argmax": [P, P, P, P, c_int, c_int, P],
     "leone_sample_temperature": [P, P, P, P, P, P, P, P, c_int, c_int, P],
     "leone_top_candidates": [P, P, P, P, c_int, c_int, c_int, P],
@@ -64,6 +65,10 @@ def library() -> ctypes.CDLL:
             lib.leone_top_candidates_max.argtypes = []
             lib.leone_argmax_chunk.restype = c_int
             lib.leone_argmax_chunk.argtypes = []
+            lib.leone_gemm_rows_max_rows.restype = c_int
+            lib.leone_gemm_rows_max_rows.argtypes = []
+            lib.leone_gemm_rows_chunk.restype = c_int
+            lib.leone_gemm_rows_chunk.argtypes = [c_int]
             for name, argtypes in _PROTOTYPES.items():
                 fn = getattr(lib, name)
                 fn.argtypes = argtypes

@@ -80,14 +80,14 @@ class GqaAttention(Part):
     def forward(self, y, step: StepContext, cache: KvCacheView,
                 residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned)."""
-        qkv = ops.linear(y, self.w_qkv)
+        qkv = ops.linear(y, self.w_qkv, planes_ok=True)
         cos, sin = self.position.tables() if self.position is not None else (None, None)
         if cos is not None and step.max_position >= cos.shape[0]:
             raise ValueError(f"position {step.max_position} is beyond the rotary table of {cos.shape[0]} positions")
         q = ops.qk_norm_rope_write(qkv, self.q_heads, self.kv_heads, self.head_dim, self.q_gain, self.k_gain,
                                    self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin,
                                    step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
-                                   write_cache=cache.writes)
+                                   write_cache=cache.writes, out_dtype=step.dtype)
         attended = self._attend(q, step, cache)
         return ops.linear(attended, self.w_o, residual=residual)
 

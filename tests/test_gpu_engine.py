@@ -190,8 +190,9 @@ def test_a_hundred_thousand_tokens_cut_three_ways(tmp_path):
 
 @pytest.mark.parametrize("schedule", ["whole", "portions", "mixed"])
 def test_a_wide_feed_forward_whose_down_projection_is_cut(tmp_path, schedule):
-    """An intermediate size of 8,192 over a width of 64: for portions of 65 rows and more the down projection
-    runs in parts whose planes the next norm adds up; the last block's planes go to the final norm."""
+    """An intermediate size of 8,192 over a width of 64: for steps of more than 128 rows the down projection
+    runs in parts on the library, for 11 to 128 on the multi-row weight-streaming kernel with K cut into
+    ranges; either way the next norm adds up the planes, and the last block's planes go to the final norm."""
     from leone_amd import ops
     from leone_amd.engine.engine import Engine
     from leone_amd.runtime import load_model
@@ -199,9 +200,9 @@ def test_a_wide_feed_forward_whose_down_projection_is_cut(tmp_path, schedule):
     config = dict(TINY["A"], intermediate_size=8192, max_position_embeddings=512)
     folder = make_model_dir(str(tmp_path / "wide"), config, seed=23, dtype=torch.bfloat16)
     weights = read_weights(folder)
-    requests = {f"w{i}": random_tokens(900 + i, n, config["vocab_size"]) for i, n in enumerate([230, 90, 70, 140])}
+    requests = {f"w{i}": random_tokens(900 + i, n, config["vocab_size"]) for i, n in enumerate([330, 90, 70, 200])}
     expected = {rid: qwen3_plain.forward(weights, read_config(folder), toks).numpy() for rid, toks in requests.items()}
-    steps = (schedules.portions(requests, sizes=(100, 66, 7, 130)) if schedule == "portions"
+    steps = (schedules.portions(requests, sizes=(100, 66, 7, 157)) if schedule == "portions"
              else schedules.mixed(requests, sizes=(70, 3, 120)) if schedule == "mixed" else schedules.whole(requests))
     taken = []
     real = ops.inner_parts

@@ -299,6 +299,26 @@ def test_qk_norm_rope_write(dtype, shape):
     q3 = ops.qk_norm_rope_write(qkv.to(DEV), q_heads, kv_heads, head_dim, None, None, eps, None, None,
                                 positions.to(DEV), row_entry.to(DEV), table.to(DEV), kp2, vp2)
     assert torch.equal(q3.cpu().view(n, q_heads, head_dim), q.to(dtype))
+    # float32 input in planes (a product cut along K): the planes are added up in order, then the same work
+    if dtype == torch.bfloat16:
+        parts = torch.randn(3, n, width) * torch.tensor([1.0, 0.01, 1e-4]).view(3, 1, 1)
+        total = (parts[0] + parts[1]) + parts[2]
+        kp3, vp3 = k_pool.to(DEV), v_pool.to(DEV)
+        q4 = ops.qk_norm_rope_write(parts.to(DEV), q_heads, kv_heads, head_dim, q_gain.to(DEV), k_gain.to(DEV), eps,
+                                    cos, sin, positions.to(DEV), row_entry.to(DEV), table.to(DEV), kp3, vp3,
+                                    out_dtype=dtype)
+        tq = total[:, :q_heads * head_dim].view(n, q_heads, head_dim)
+        tk = total[:, q_heads * head_dim:(q_heads + kv_heads) * head_dim].view(n, kv_heads, head_dim)
+        tv = total[:, (q_heads + kv_heads) * head_dim:].view(n, kv_heads, head_dim)
+        close(q4.view(n, q_heads, head_dim), plain.rope_half_split(plain.rms_norm(tq, q_gain, eps), positions, theta),
+              atol, rtol, "q from planes")
+        k4, v4 = unpack(kp3, vp3)
+        for i, (e, p) in enumerate(rows_meta):
+            page, off = int(table[e, p // page_tokens]), p % page_tokens
+            close(k4[page, :, off], plain.rope_half_split(plain.rms_norm(tk, k_gain, eps), positions, theta)[i],
+                  atol, rtol, f"k row {i} from planes")
+            assert torch.equal(v4[page, :, off], tv[i].to(dtype))
+        assert (k4[untouched] == 7.0).all() and (v4[untouched] == 7.0).all()
 
 
 @pytest.mark.parametrize("shape", [(4, 2, 16, 16), (5, 5, 48, 16), (3, 1, 112, 32), (8, 2, 128, 64)])
@@ -672,3 +692,93 @@ def test_gemm_fused_gated(mfk):
     got = ops.linear(lazy40, w, gated=True)
     y = lazy40.materialize().double().cpu()
     close(got, plain.swiglu(y @ wg.double().cpu().T, y @ wu.double().cpu().T), 3e-2, 3e-2, "unfused gated")
+
+
+ROWS_SHAPES = [(16, 6144, 4096), (17, 777, 264), (33, 130, 1032), (64, 4096, 4096), (100, 1000, 96), (128, 4096, 12288),
+               (48, 24576, 4096), (11, 20, 8), (128, 333, 72), (96, 151936, 4096), (1, 4096, 4096)]
+
+
+@pytest.mark.parametrize("mnk", ROWS_SHAPES)
+def test_gemm_rows_plain(mnk):
+    """The multi-row weight-streaming product (crates/leone/src/runtime.rs:7865-7906 is the reference's place
+    for it) against double sums of the bfloat16 inputs (crates/leone-cuda/tests/gpu.rs:287-386), for every
+    workgroup size and several cuts of K, and as the plan would run it."""
+    from leone_amd import ops
+    m, n, k = mnk
+    torch.manual_seed(21)
+    x, w = torch.randn(m, k, device=DEV).bfloat16(), (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    want = x.double() @ w.double().T
+    big = n * k > 1 << 27
+    for waves in ((6,) if big else ops.ROWS_WAVES):
+        for splits in ((1,) if big else (1, 2, 5)):
+            out = ops.gemm_rows(x, w, torch.float32, splits=splits, waves=waves)
+            if out.dim() == 3:
+                assert out.shape[1:] == (m, n)
+                out = out.double().sum(0)
+            close(out, want, 2e-6 * k, 1e-5, f"gemm_rows waves {waves} splits {splits}")
+    planned = ops.gemm_rows(x, w, torch.float32)
+    assert torch.equal(planned, ops.gemm_rows(x, w, torch.float32))            # a launch repeats bit for bit
+    close(planned.double().sum(0) if planned.dim() == 3 else planned, want, 2e-6 * k, 1e-5, "gemm_rows as planned")
+    rounded = ops.gemm_rows(x, w, torch.bfloat16, may_split=False)
+    assert rounded.shape == (m, n) and rounded.dtype == torch.bfloat16
+    close(rounded, want, 2e-6 * k + 1e-3, 8e-3, "gemm_rows bf16")
+    # a row gives the same bits whatever the other rows are (crates/leone-cuda/tests/gpu.rs:770)
+    waves, splits = ops.rows_plan(m, n, k, False)
+    whole = ops.gemm_rows(x, w, torch.float32, splits=1, waves=waves)
+    other = x.clone()
+    other[:m - 1] = torch.randn(m - 1, k, device=DEV).bfloat16()
+    assert torch.equal(ops.gemm_rows(other, w, torch.float32, splits=1, waves=waves)[m - 1], whole[m - 1])
+
+
+def test_gemm_rows_plan_fills_the_compute_units():
+    """The plan at the shapes it was measured on, and that it never names an empty range of K."""
+    from leone_amd import ops
+    assert ops.rows_plan(64, 6144, 4096, True) == (6, 4)
+    assert ops.rows_plan(64, 4096, 4096, True) == (4, 4)
+    assert ops.rows_plan(64, 24576, 4096, False) == (6, 1)
+    assert ops.rows_plan(64, 4096, 12288, True) == (4, 4)
+    assert ops.rows_plan(128, 151936, 4096, False) == (8, 1)
+    assert ops.rows_plan(128, 4096, 4096, True) == (4, 4)
+    for m, n, k in [(16, 40, 8), (128, 100000, 72), (33, 5120, 25600), (90, 51200, 5120), (20, 7168, 5120)]:
+        for may in (False, True):
+            waves, splits = ops.rows_plan(m, n, k, may)
+            chunks = -(-k // (256 if m <= 64 else 128))
+            assert waves in ops.ROWS_WAVES and 1 <= splits <= (16 if may else 1)
+            assert -(-chunks // splits) * (splits - 1) < chunks
+
+
+@pytest.mark.parametrize("mnk", [(16, 4096, 4096), (37, 80, 176), (128, 777, 64), (64, 4096, 12288)])
+def test_gemm_rows_residual(mnk):
+    from leone_amd import ops
+    m, n, k = mnk
+    torch.manual_seed(22)
+    x = torch.randn(m, k, device=DEV).bfloat16()
+    w = (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    stream = torch.randn(m, n, device=DEV)
+    before = stream.clone()
+    assert ops.gemm_rows(x, w, residual=stream, splits=1, waves=4) is None
+    want = before.double() + x.double() @ w.double().T
+    close(stream, want, 2e-6 * k, 1e-5, "product added into the stream")
+    assert torch.equal(stream, before + ops.gemm_rows(x, w, torch.float32, splits=1, waves=4))
+    # as the engine runs it: what comes back (planes, if K was cut) is added by the next norm's kernel
+    stream2 = before.clone()
+    delta = ops.linear(x, w, residual=stream2)
+    gain = torch.ones(n, device=DEV)
+    ops.add_rmsnorm(stream2, delta, gain, 1e-6, torch.bfloat16)
+    close(stream2, want, 2e-6 * k, 1e-5, "planes added by the norm")
+
+
+@pytest.mark.parametrize("mfk", [(16, 12288, 4096), (36, 88, 80), (128, 256, 96), (64, 17408, 5120)])
+def test_gemm_rows_gated(mfk):
+    from leone_amd import ops
+    m, f, k = mfk
+    torch.manual_seed(23)
+    x = torch.randn(m, k, device=DEV).bfloat16()
+    wg, wu = (torch.randn(f, k, device=DEV) * 0.05).bfloat16(), (torch.randn(f, k, device=DEV) * 0.05).bfloat16()
+    w = ops.interleave_gate_up(wg, wu).contiguous()
+    for waves in ops.ROWS_WAVES:
+        out = ops.gemm_rows(x, w, gated=True, waves=waves)
+        assert out.shape == (m, f) and out.dtype == torch.bfloat16
+        want = plain.swiglu(x.double() @ wg.double().T, x.double() @ wu.double().T)
+        close(out, want, 1e-2, 1e-2, "gated product")
+    assert torch.equal(ops.linear(x, w, gated=True), ops.gemm_rows(x, w, gated=True))

@@ -540,9 +540,12 @@ def test_block_part(dtype, rows):
     step = step_context([(0, i) for i in range(rows)], dtype, {0: table})
     x = x0.to(DEV)
     pending = block.forward(x, None, step, cache)
+    if pending is not None and pending.dim() == 3:
+        pending = pending.double().sum(0)
     got = x.cpu().double() + (0 if pending is None else pending.cpu().double())
     if dtype == torch.bfloat16:
-        assert (pending is None) == (rows <= ops.FUSED_ROWS)
+        # the weight-streaming kernels add into the stream themselves (the inner sizes here are one chunk of K)
+        assert (pending is None) == (rows <= ops.ROWS_MAX)
     wf = {k: v.float() for k, v in w.items()}
     cfg = dict(num_attention_heads=heads, num_key_value_heads=kv, head_dim=dim, rms_norm_eps=1e-5, rope_theta=1e4)
     x1 = x0.double() + plain.attention_block(plain.rms_norm(x0, wf["n1"], 1e-5), wf, "a", cfg, list(range(rows)))
