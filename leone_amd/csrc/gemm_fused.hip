@@ -5,9 +5,16 @@
 //           norm  : X is the float32 residual stream; the operand is bf16(x * gain) and the result is
 //                   scaled by 1/sqrt(mean(x^2) + eps) per row afterwards, which is the same RMSNorm
 //                   (crates/leone/src/cpu.rs:1642-1663) because that factor is constant along a row
+//           prepared : X is bfloat16 [M,K] = bf16(x * gain), written by a product before (see `prepare`
+//                   below) together with partial sums of x^2, one for every 16 columns of a row; the
+//                   result is scaled by 1/sqrt(sum / K + eps) as for `norm`, and no kernel runs in between
 //   output  store    : Y[M,N] in bfloat16 or float32
 //           residual : Y is the float32 stream, Y += product (the reference's fused
 //                      matrix-vector + residual, crates/leone/src/runtime.rs:9151-9157, 9311)
+//           prepare  : as residual, and from the new stream values the operand of the norm that comes
+//                      next: T[M,N] = bf16(y * next_gain) and, for this workgroup's 16 columns, the
+//                      sum of y^2 of every row (the reference's fused norm + residual store,
+//                      crates/leone/src/backend.rs:2371-2390)
 //           gated    : W holds, in every block of 16 rows, 8 gate rows then the 8 up rows that belong to
 //                      them; Y[M,N/2] = silu(gate) * up (crates/leone/src/cpu.rs:892-907)
 //
@@ -29,8 +36,8 @@ namespace leone {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
-enum FusedIn : int { kInPlain = 0, kInNorm = 1 };
-enum FusedOut : int { kOutStore = 0, kOutResidual = 1, kOutGated = 2 };
+enum FusedIn : int { kInPlain = 0, kInNorm = 1, kInPrepared = 2 };
+enum FusedOut : int { kOutStore = 0, kOutResidual = 1, kOutGated = 2, kOutPrepare = 3 };
 
 struct FusedArgs {
     const void* x;       // plain: bfloat16 [M,K]; norm: float [*, K]
@@ -41,6 +48,11 @@ struct FusedArgs {
     const bf16_t* w;     // [N,K]
     void* y;
     int m, n, k;
+    const float* squares_in;   // prepared: [M, ceil(K / 16)] partial sums of squares
+    bf16_t* operand_out;       // prepare: [M,N]
+    float* squares_out;        // prepare: [M, ceil(N / 16)]
+    const void* next_gain;     // prepare: [N]
+    int next_gain_dtype;
 };
 
 __device__ inline bf16x8 fz8() {
@@ -80,12 +92,21 @@ gemm_fused_kernel(FusedArgs a) {
     // Rows past the end are clamped: they only feed output rows and columns that are never stored.
     const long wr = n0 + c < n ? n0 + c : n - 1;
     const bf16_t* wrow = a.w + wr * k + 16 * g;
+    float ss = 0.f;
     const int xr = c < m ? c : m - 1;
     const long xrow_index = (kIn == kInNorm && a.rows) ? a.rows[xr] : xr;
+    if (kIn == kInPrepared) {
+        // The partial sums of squares of row c, a contiguous share for every (wave, g), summed in index order.
+        const int parts = (k + 15) / 16;
+        const int share = (parts + 4 * kWaves - 1) / (4 * kWaves);
+        const int begin = (wave * 4 + g) * share;
+        const int end = begin + share < parts ? begin + share : parts;
+        const float* from = a.squares_in + static_cast<long>(xr) * parts;
+        for (int i = begin; i < end; ++i) ss += from[i];
+    }
     const bf16_t* xb = static_cast<const bf16_t*>(a.x) + xrow_index * k + 16 * g;   // plain
     const float* xf = static_cast<const float*>(a.x) + xrow_index * k + 16 * g;     // norm
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-    float ss = 0.f;
 
     // One step: 64 elements of K; this lane's run is elements at + 16g .. + 15, `left` of which exist.
     auto step = [&](int s, bf16x8 a0, bf16x8 a1, bool tail) {
@@ -96,7 +117,7 @@ gemm_fused_kernel(FusedArgs a) {
         for (int h = 0; h < 2; ++h) {
             if (left < 8 * (h + 1)) {
                 b[h] = fz8();
-            } else if (kIn == kInPlain) {
+            } else if (kIn != kInNorm) {
                 b[h] = fld8(xb + at + 8 * h);
             } else {
                 const float4 lo = *reinterpret_cast<const float4*>(xf + at + 8 * h);
@@ -138,7 +159,7 @@ gemm_fused_kernel(FusedArgs a) {
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) partial[wave][lane][r] = acc[r];
-    if (kIn == kInNorm) {
+    if (kIn != kInPlain) {
         ss += __shfl_xor(ss, 16, kWave);             // the four lanes that share X row c
         ss += __shfl_xor(ss, 32, kWave);
         if (g == 0) squares[wave][c] = ss;
@@ -152,7 +173,7 @@ gemm_fused_kernel(FusedArgs a) {
     for (int v = 0; v < kWaves; ++v)
 #pragma unroll
         for (int r = 0; r < 4; ++r) sum[r] += partial[v][lane][r];
-    if (kIn == kInNorm) {
+    if (kIn != kInPlain) {
         float total = 0.f;
 #pragma unroll
         for (int v = 0; v < kWaves; ++v) total += squares[v][c];
@@ -177,8 +198,27 @@ gemm_fused_kernel(FusedArgs a) {
         }
         return;
     }
-    if (row >= m) return;
     const long col = n0 + 4 * g;
+    if (kOut == kOutPrepare) {
+        // every lane takes part in the exchange; rows and columns past the end count as zero
+        float* out = static_cast<float*>(a.y) + static_cast<long>(row) * n + col;
+        const AnyVec gain{a.next_gain, a.next_gain_dtype};
+        float squares = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            if (row < m && col + r < n) {
+                const float v = out[r] + sum[r];
+                out[r] = v;
+                squares = fmaf(v, v, squares);
+                a.operand_out[static_cast<long>(row) * n + col + r] = from_float<bf16_t>(v * load_any(gain, col + r));
+            }
+        }
+        squares += __shfl_xor(squares, 16, kWave);
+        squares += __shfl_xor(squares, 32, kWave);
+        if (g == 0 && row < m) a.squares_out[static_cast<long>(row) * gridDim.x + blockIdx.x] = squares;
+        return;
+    }
+    if (row >= m) return;
     if (kOut == kOutResidual) {
         float* out = static_cast<float*>(a.y) + static_cast<long>(row) * n + col;
 #pragma unroll
@@ -217,21 +257,30 @@ static void launch_fused(const FusedArgs& a, hipStream_t stream) {
 
 using namespace leone;
 
-// in_mode: 0 plain (x bfloat16 [m,k]), 1 norm (x float32 stream, optional rows, gain, eps).
-// out_mode: 0 store (y of out_dtype [m,n]), 1 residual (y float32 [m,n] += product), 2 gated (y bfloat16 [m,n/2]).
+// in_mode: 0 plain (x bfloat16 [m,k]), 1 norm (x float32 stream, optional rows, gain, eps), 2 prepared (x bfloat16
+// [m,k] and squares_in float32 [m, ceil(k / 16)] as an earlier call's out_mode 3 wrote them, eps).
+// out_mode: 0 store (y of out_dtype [m,n]), 1 residual (y float32 [m,n] += product), 2 gated (y bfloat16 [m,n/2]),
+// 3 prepare (as 1, and operand_out bfloat16 [m,n] = bf16(y * next_gain), squares_out float32 [m, ceil(n / 16)]).
 extern "C" int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const void* gain, int gain_dtype,
                                      float eps, const void* w, void* y, int out_mode, int out_dtype, int m, int n,
-                                     int k, hipStream_t stream) {
+                                     int k, const float* squares_in, void* operand_out, float* squares_out,
+                                     const void* next_gain, int next_gain_dtype, hipStream_t stream) {
     LEONE_REQUIRE(x && w && y, "gemm_fused: null pointer");
     LEONE_REQUIRE(m > 0 && m <= 16, "gemm_fused: rows %d must be in 1..16", m);
     LEONE_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_fused: sizes %d x %d: K must be a positive multiple of 8", n, k);
-    LEONE_REQUIRE(in_mode == kInPlain || in_mode == kInNorm, "gemm_fused: unknown input mode %d", in_mode);
-    LEONE_REQUIRE(in_mode == kInPlain || (gain && eps > 0.f && (gain_dtype == kF32 || gain_dtype == kBF16)),
+    LEONE_REQUIRE(in_mode >= kInPlain && in_mode <= kInPrepared, "gemm_fused: unknown input mode %d", in_mode);
+    LEONE_REQUIRE(in_mode != kInNorm || (gain && eps > 0.f && (gain_dtype == kF32 || gain_dtype == kBF16)),
                   "gemm_fused: the norm input needs a gain and a positive eps");
-    LEONE_REQUIRE(out_mode >= kOutStore && out_mode <= kOutGated, "gemm_fused: unknown output mode %d", out_mode);
+    LEONE_REQUIRE(in_mode != kInPrepared || (squares_in && eps > 0.f),
+                  "gemm_fused: the prepared input needs the sums of squares and a positive eps");
+    LEONE_REQUIRE(out_mode >= kOutStore && out_mode <= kOutPrepare, "gemm_fused: unknown output mode %d", out_mode);
     LEONE_REQUIRE(out_mode != kOutGated || n % 16 == 0, "gemm_fused: gated output needs N %d to be a multiple of 16", n);
     LEONE_REQUIRE(out_mode != kOutStore || out_dtype == kF32 || out_dtype == kBF16, "gemm_fused: unknown output type");
-    FusedArgs a{x, rows, gain, gain_dtype, eps, static_cast<const bf16_t*>(w), y, m, n, k};
+    LEONE_REQUIRE(out_mode != kOutPrepare || (operand_out && squares_out && next_gain &&
+                                              (next_gain_dtype == kF32 || next_gain_dtype == kBF16)),
+                  "gemm_fused: the prepare output needs room for the operand and the sums, and the next gain");
+    FusedArgs a{x, rows, gain, gain_dtype, eps, static_cast<const bf16_t*>(w), y, m, n, k,
+                squares_in, static_cast<bf16_t*>(operand_out), squares_out, next_gain, next_gain_dtype};
 #define LEONE_FUSED_OUT(IN)                                                                  \
     switch (out_mode) {                                                                      \
         case kOutStore:                                                                      \
@@ -239,12 +288,15 @@ extern "C" int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows
             else launch_fused<IN, kOutStore, bf16_t>(a, stream);                             \
             break;                                                                           \
         case kOutResidual: launch_fused<IN, kOutResidual, float>(a, stream); break;          \
+        case kOutPrepare: launch_fused<IN, kOutPrepare, float>(a, stream); break;            \
         default: launch_fused<IN, kOutGated, bf16_t>(a, stream); break;                      \
     }
     if (in_mode == kInPlain) {
         LEONE_FUSED_OUT(kInPlain)
-    } else {
+    } else if (in_mode == kInNorm) {
         LEONE_FUSED_OUT(kInNorm)
+    } else {
+        LEONE_FUSED_OUT(kInPrepared)
     }
 #undef LEONE_FUSED_OUT
     LEONE_LAUNCH_CHECK("gemm_fused");

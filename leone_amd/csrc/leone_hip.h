@@ -73,13 +73,18 @@ int leone_attention_prefill(const void* q, void* out, const void* k_pool, const 
 // C[M,N] = A[M,K] . B[N,K]^T in float.
 int leone_gemm_f32(const float* a, const float* b, float* c, int m, int n, int k, hipStream_t stream);
 
-// Y[M,N] = X[M,K] . W[N,K]^T for bfloat16 W, M <= 16, K a multiple of 8, with row-wise neighbours folded in.  in_mode 0: x is bfloat16 [M,K];
-// 1: x is the float32 stream (row r reads rows[r] if rows is given), the operand is x * gain and the
-// result is scaled by 1/sqrt(mean(x^2) + eps).  out_mode 0: y[M,N] of out_dtype; 1: y float32 [M,N] +=
-// product; 2: W interleaves 8 gate rows with their 8 up rows, y bfloat16 [M,N/2] = silu(gate) * up.
+// Y[M,N] = X[M,K] . W[N,K]^T for bfloat16 W, M <= 16, K a multiple of 8, with row-wise neighbours folded in.
+// in_mode 0: x is bfloat16 [M,K]; 1: x is the float32 stream (row r reads rows[r] if rows is given), the
+// operand is x * gain and the result is scaled by 1/sqrt(mean(x^2) + eps); 2: x is bfloat16 [M,K] = bf16(stream *
+// gain) and squares_in float32 [M, ceil(K / 16)] partial sums of stream^2, as a call with out_mode 3 leaves
+// them; the result is scaled as for 1.  out_mode 0: y[M,N] of out_dtype; 1: y float32 [M,N] += product; 2: W
+// interleaves 8 gate rows with their 8 up rows, y bfloat16 [M,N/2] = silu(gate) * up; 3: as 1, and from the new
+// y: operand_out bfloat16 [M,N] = bf16(y * next_gain), squares_out float32 [M, ceil(N / 16)] sums of y^2 over
+// 16 columns each.
 int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const void* gain, int gain_dtype, float eps,
                           const void* w, void* y, int out_mode, int out_dtype, int m, int n, int k,
-                          hipStream_t stream);
+                          const float* squares_in, void* operand_out, float* squares_out, const void* next_gain,
+                          int next_gain_dtype, hipStream_t stream);
 
 // Y[M,N] = X[M,K] . W[N,K]^T for bfloat16 X and W, M in 1..leone_gemm_rows_max_rows(), K a multiple of 8: W is
 // streamed once, X goes through shared memory.  out_mode 0: y[M,N] of out_dtype; 1: y float32 [M,N] += product;

@@ -349,6 +349,18 @@ class NormedRows:
         return add_rmsnorm(self.x, None, self.gain, self.eps, self.dtype, self.rows)
 
 
+class PreparedRows(NormedRows):
+    """A norm of the whole stream ``x`` whose operand the product before has left behind: ``operand`` is
+    bf16(x * gain), ``squares`` float32 ``[rows, ceil(hidden / 16)]`` partial sums of x^2, so that the
+    product that consumes it needs no norm kernel and no second read of the stream.  The stream itself is
+    up to date: any other consumer normalises it in the usual way (``materialize``)."""
+
+    def __init__(self, x: torch.Tensor, gain: torch.Tensor, eps: float, dtype: torch.dtype,
+                 operand: torch.Tensor, squares: torch.Tensor):
+        super().__init__(x, gain, eps, dtype, None)
+        self.operand, self.squares = operand, squares
+
+
 def materialize(x) -> torch.Tensor:
     return x.materialize() if isinstance(x, NormedRows) else x
 
@@ -363,31 +375,50 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
 
 
 def gemm_fused(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
-               residual: Optional[torch.Tensor] = None, gated: bool = False) -> Optional[torch.Tensor]:
-    """The product for at most 16 rows with its neighbours folded in: ``x`` may be ``NormedRows``;
-    with ``residual`` the product is added into that float32 tensor and None is returned; with ``gated``
-    the weight is an interleaved gate/up weight and silu(gate) * up comes out."""
+               residual: Optional[torch.Tensor] = None, gated: bool = False, next_norm=None):
+    """The product for at most 16 rows with its neighbours folded in: ``x`` may be ``NormedRows`` or
+    ``PreparedRows``; with ``residual`` the product is added into that float32 tensor and None is returned;
+    with ``gated`` the weight is an interleaved gate/up weight and silu(gate) * up comes out.  With
+    ``residual`` and ``next_norm = (gain, eps, dtype)`` the kernel also leaves the operand of that norm
+    behind and ``PreparedRows`` is returned (the residual has been added)."""
     m, k = x.shape
     n, k2 = weight.shape
     if k != k2:
         raise KernelError(f"gemm_fused: inner sizes {k} and {k2} differ")
-    normed = isinstance(x, NormedRows)
+    prepared = isinstance(x, PreparedRows)
+    normed = isinstance(x, NormedRows) and not prepared
     if residual is not None and gated:
         raise KernelError("gemm_fused: a gated product cannot also be added into the stream")
+    if next_norm is not None and residual is None:
+        raise KernelError("gemm_fused: the next norm can only be prepared from the stream the product is added into")
+    operand = squares = None
     if residual is not None:
         out, mode, out_dtype = residual, 1, torch.float32
+        if next_norm is not None:
+            mode = 3
+            operand = torch.empty((m, n), dtype=torch.bfloat16, device=weight.device)
+            squares = torch.empty((m, -(-n // 16)), dtype=torch.float32, device=weight.device)
     elif gated:
         out, mode, out_dtype = torch.empty((m, n // 2), dtype=torch.bfloat16, device=weight.device), 2, torch.bfloat16
     else:
         out, mode = torch.empty((m, n), dtype=out_dtype, device=weight.device), 0
+    if prepared:
+        source, in_mode = _dev(x.operand, "prepared operand", torch.bfloat16, (m, k)), 2
+        _dev(x.squares, "prepared sums", torch.float32, (m, -(-k // 16)))
+    elif normed:
+        source, in_mode = _dev(x.x, "stream", torch.float32), 1
+    else:
+        source, in_mode = _dev(x, "gemm x", torch.bfloat16, (m, k)), 0
     with profile.span("gemv fused", weight):
-        call("leone_gemm_fused_bf16",
-             _dev(x.x, "stream", torch.float32) if normed else _dev(x, "gemm x", torch.bfloat16, (m, k)),
-             1 if normed else 0, _dev(x.rows, "rows", torch.int32) if normed else 0,
+        call("leone_gemm_fused_bf16", source, in_mode, _dev(x.rows, "rows", torch.int32) if normed else 0,
              _dev(x.gain, "gain", None, (k,)) if normed else 0, _code(x.gain, "gain") if normed else 0,
-             x.eps if normed else 0.0, _dev(weight, "gemm weight", torch.bfloat16),
+             x.eps if (normed or prepared) else 0.0, _dev(weight, "gemm weight", torch.bfloat16),
              _dev(out, "gemm out", out_dtype, (m, n // 2 if gated else n)), mode, _CODES[out_dtype], m, n, k,
-             _stream())
+             x.squares.data_ptr() if prepared else 0, _dev(operand, "operand out"), _dev(squares, "sums out"),
+             _dev(next_norm[0], "next gain", None, (n,)) if next_norm is not None else 0,
+             _code(next_norm[0], "next gain") if next_norm is not None else 0, _stream())
+    if next_norm is not None:
+        return PreparedRows(residual, next_norm[0], next_norm[1], next_norm[2], operand, squares)
     return None if residual is not None else out
 
 
@@ -493,7 +524,7 @@ def inner_parts(rows: int, n: int, k: int) -> int:
 
 def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
            residual: Optional[torch.Tensor] = None, gated: bool = False,
-           planes_ok: bool = False) -> Optional[torch.Tensor]:
+           planes_ok: bool = False, next_norm=None):
     """x[R,K] . weight[N,K]^T, with optional neighbours.
 
     ``x`` is a tensor or ``NormedRows`` (a norm still to be done).  ``gated``: the weight is an
@@ -502,7 +533,9 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
     is returned, otherwise the product is returned for the caller to add later, as float32 ``[R, N]`` or
     as a stack of planes ``[p, R, N]`` whose sum is meant (``add_rmsnorm`` takes either).
 
-    ``planes_ok``: the caller also takes a plain product as float32 planes ``[p, R, N]`` whose sum, in
+    ``next_norm`` = (gain, eps, dtype) with ``residual``: the caller will normalise the stream with this
+    gain next; the kernel may leave that norm's operand behind, and then ``PreparedRows`` is returned
+    instead of None.  ``planes_ok``: the caller also takes a plain product as float32 planes ``[p, R, N]`` whose sum, in
     order, is meant (``qk_norm_rope_write`` does).
 
     float32 runs the single-precision kernel.  bfloat16 accumulates in float: up to FUSED_ROWS rows on the
@@ -519,9 +552,11 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
             and (not gated or weight.shape[0] % 16 == 0):
         # Every workgroup (16 weight rows) would redo a folded norm for its own use: that pays only for
         # matrices with few rows; for the others the norm kernel runs once and the product reads its result.
-        if isinstance(x, NormedRows) and weight.shape[0] > FUSED_NORM_WEIGHT_ROWS:
+        if isinstance(x, NormedRows) and not isinstance(x, PreparedRows) and weight.shape[0] > FUSED_NORM_WEIGHT_ROWS:
             x = x.materialize()
-        return gemm_fused(x, weight, out_dtype, residual, gated)
+        if next_norm is not None and (residual is None or weight.shape[0] % 8 or next_norm[2] != torch.bfloat16):
+            next_norm = None
+        return gemm_fused(x, weight, out_dtype, residual, gated, next_norm)
     x = materialize(x)
     if dtype == torch.bfloat16 and weight.is_cuda and k % 8 == 0 and rows <= ROWS_MAX \
             and (not gated or weight.shape[0] % 16 == 0):

@@ -43,16 +43,32 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
-    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], step: StepContext,
-                cache: Optional[CacheView]) -> Optional[torch.Tensor]:
-        """Returns the delta that is still to be added to ``x``, or None if everything has been added."""
+    prepares_next = True
+
+    def entry_norm(self, out_dtype):
+        """What the block before may prepare for this block's first norm (``RmsNorm.folded``), or None."""
+        if getattr(self.mixer, "fused_io", False) and hasattr(self.norm1, "folded"):
+            return self.norm1.folded(out_dtype)
+        return None
+
+    def forward(self, x: torch.Tensor, pending, step: StepContext, cache: Optional[CacheView], next_norm=None):
+        """Returns the delta that is still to be added to ``x``, None if everything has been added, or, if
+        ``next_norm`` (the next block's ``entry_norm``) was given and the last product could do it, that
+        norm's operand (``ops.PreparedRows``; everything has been added then)."""
         y = self._normed(self.norm1, x, pending, step, self.mixer)
         if getattr(self.mixer, "fused_io", False):
-            delta = self.mixer.forward(y, step, cache, residual=x)
+            inner = None
+            if getattr(self.mixer, "prepares_next", False) and getattr(self.feed_forward, "fused_io", False) \
+                    and hasattr(self.norm2, "folded"):
+                inner = self.norm2.folded(step.dtype)
+            delta = (self.mixer.forward(y, step, cache, residual=x, next_norm=inner) if inner is not None
+                     else self.mixer.forward(y, step, cache, residual=x))
         else:
             delta = self.mixer.forward(y, step, cache)
         y = self._normed(self.norm2, x, delta, step, self.feed_forward)
         if getattr(self.feed_forward, "fused_io", False):
+            if next_norm is not None and getattr(self.feed_forward, "prepares_next", False):
+                return self.feed_forward.forward(y, step, residual=x, next_norm=next_norm)
             return self.feed_forward.forward(y, step, residual=x)
         return self.feed_forward.forward(y, step)
 

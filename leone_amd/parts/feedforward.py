@@ -34,6 +34,7 @@ class SwiGluMlp(Part):
                 TensorSpec(self.names["down"], (self.hidden, self.intermediate), MATRIX)]
 
     fused_io = True
+    prepares_next = True
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         # One product for gate and up: 8 gate rows, their 8 up rows, and so on (a pure re-layout), which
@@ -49,7 +50,8 @@ class SwiGluMlp(Part):
         self.w_gate_up = ops.interleave_gate_up(gate, up).contiguous()
         self.w_down = down.contiguous()
 
-    def forward(self, y, step: StepContext, residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-        """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned)."""
+    def forward(self, y, step: StepContext, residual: Optional[torch.Tensor] = None, next_norm=None):
+        """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned),
+        and with ``next_norm`` the norm that follows may come back prepared (see ``ops.linear``)."""
         activated = ops.linear(y, self.w_gate_up, gated=True)
-        return ops.linear(activated, self.w_down, residual=residual)
+        return ops.linear(activated, self.w_down, residual=residual, next_norm=next_norm)

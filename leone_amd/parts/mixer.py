@@ -76,10 +76,12 @@ class GqaAttention(Part):
                 self.q_gain, self.k_gain = self.q_gain.float(), self.k_gain.float()
 
     fused_io = True
+    prepares_next = True
 
     def forward(self, y, step: StepContext, cache: KvCacheView,
-                residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-        """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned)."""
+                residual: Optional[torch.Tensor] = None, next_norm=None):
+        """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned),
+        and with ``next_norm`` the norm that follows may come back prepared (see ``ops.linear``)."""
         qkv = ops.linear(y, self.w_qkv, planes_ok=True)
         cos, sin = self.position.tables() if self.position is not None else (None, None)
         if cos is not None and step.max_position >= cos.shape[0]:
@@ -89,7 +91,7 @@ class GqaAttention(Part):
                                    step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
                                    write_cache=cache.writes, out_dtype=step.dtype)
         attended = self._attend(q, step, cache)
-        return ops.linear(attended, self.w_o, residual=residual)
+        return ops.linear(attended, self.w_o, residual=residual, next_norm=next_norm)
 
     def _attend(self, q: torch.Tensor, step: StepContext, cache: KvCacheView) -> torch.Tensor:
         """Long prompt portions through the prompt kernel, the other rows through the split-KV kernel; the

@@ -116,15 +116,24 @@ class DecoderModel:
         """Runs the step's rows through every scheduled layer; returns float32 logits of the wanted rows."""
         x = ops.embed(self.embedding, tokens)
         pending = None
-        for run in self.schedule:
+        for at, run in enumerate(self.schedule):
             cache = caches.get(run.cache) if run.cache is not None else None
             if cache is not None and cache.writes != run.writes:
                 cache = type(cache)(**{**cache.__dict__, "writes": run.writes})
-            pending = self.layers[run.layer].forward(x, pending, step, cache)
+            layer = self.layers[run.layer]
+            # A block that can do so leaves the first norm of the block that runs next prepared.
+            after = self.layers[self.schedule[at + 1].layer] if at + 1 < len(self.schedule) else None
+            next_norm = after.entry_norm(step.dtype) if hasattr(after, "entry_norm") else None
+            if next_norm is not None and getattr(layer, "prepares_next", False):
+                pending = layer.forward(x, pending, step, cache, next_norm=next_norm)
+            else:
+                pending = layer.forward(x, pending, step, cache)
         if step.want_rows is None or step.want_rows.numel() == 0:
             if pending is not None:
                 pass  # nothing reads the last delta when no logits are wanted
             return None
+        if isinstance(pending, ops.PreparedRows):
+            pending = None                    # prepared for a norm that never ran: the stream is up to date
         if hasattr(self.final_norm, "lazy"):
             y = self.final_norm.lazy(x, pending, self.dtype, rows=step.want_rows)
         else:

@@ -33,12 +33,23 @@ class RmsNorm(Part):
 
     def add_norm(self, x: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype,
                  rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if isinstance(delta, ops.PreparedRows):
+            delta = None                      # the product that made it has added into the stream already
         return ops.add_rmsnorm(x, delta, self.gain, self.eps, out_dtype, rows)
+
+    def folded(self, out_dtype: torch.dtype):
+        """(gain, eps, type) for a product that can leave this norm's operand behind when it adds into the
+        stream (``ops.linear(..., next_norm=)``)."""
+        return (self.gain, self.eps, out_dtype)
 
     def lazy(self, x: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype,
              rows: Optional[torch.Tensor] = None):
         """The same, but if there is nothing to add the norm is only described (``ops.NormedRows``), so
         that the product that consumes it can carry it out itself."""
+        if isinstance(delta, ops.PreparedRows):
+            if rows is None and delta.gain is self.gain and delta.eps == self.eps and delta.dtype == out_dtype:
+                return delta
+            delta = None                      # made for another norm: the stream itself is up to date
         if delta is not None:
             return self.add_norm(x, delta, out_dtype, rows)
         return ops.NormedRows(x, self.gain, self.eps, out_dtype, rows)

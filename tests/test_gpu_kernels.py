@@ -782,3 +782,47 @@ def test_gemm_rows_gated(mfk):
         want = plain.swiglu(x.double() @ wg.double().T, x.double() @ wu.double().T)
         close(out, want, 1e-2, 1e-2, "gated product")
     assert torch.equal(ops.linear(x, w, gated=True), ops.gemm_rows(x, w, gated=True))
+
+
+@pytest.mark.parametrize("gain_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mnk", [(1, 4096, 4096), (7, 80, 176), (10, 1000, 64), (16, 4096, 12288)])
+def test_gemm_fused_prepares_the_next_norm(mnk, gain_dtype):
+    """The product that adds into the stream leaves bf16(stream * gain) and partial sums of squares behind;
+    the next product takes them in place of a norm kernel (the reference's fused norm + residual store,
+    crates/leone/src/backend.rs:2371-2390).  Both halves against double, and against the kernels they replace."""
+    from leone_amd import ops
+    m, n, k = mnk
+    torch.manual_seed(31)
+    x = torch.randn(m, k, device=DEV).bfloat16()
+    w = (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    gain = (1 + 0.1 * torch.randn(n, device=DEV)).to(gain_dtype)
+    eps = 1e-5
+    stream = torch.randn(m, n, device=DEV) * 2
+    plain_stream = stream.clone()
+    assert ops.gemm_fused(x, w, residual=plain_stream) is None
+    prepared = ops.gemm_fused(x, w, residual=stream, next_norm=(gain, eps, torch.bfloat16))
+    assert isinstance(prepared, ops.PreparedRows) and prepared.x is stream
+    assert torch.equal(stream, plain_stream)                                    # the same sum, the same bits
+    assert torch.equal(prepared.operand, (stream * gain.float()).bfloat16())
+    assert prepared.squares.shape == (m, -(-n // 16))
+    close(prepared.squares.double().sum(1), (stream.double() ** 2).sum(1), 1e-4, 1e-5, "sums of squares")
+    # the consumer: scaled by 1/rms of the stream, like the folded norm and like norm, then product
+    n2 = 96
+    w2 = (torch.randn(n2, n, device=DEV) * 0.05).bfloat16()
+    out = ops.gemm_fused(prepared, w2, torch.float32)
+    inv = 1.0 / torch.sqrt((stream.double() ** 2).mean(dim=1, keepdim=True) + eps)
+    want = (prepared.operand.double() @ w2.double().T) * inv
+    close(out, want, 2e-6 * n, 2e-5, "prepared operand, then product")
+    folded = ops.gemm_fused(ops.NormedRows(stream, gain, eps, torch.bfloat16), w2, torch.float32)
+    close(out, folded.double(), 1e-5, 1e-5, "prepared against folded")
+    assert torch.equal(out, ops.gemm_fused(prepared, w2, torch.float32))
+    # anyone else normalises the stream in the usual way
+    assert torch.equal(prepared.materialize(), ops.add_rmsnorm(stream, None, gain, eps, torch.bfloat16))
+    # and linear() takes the prepared rows for a gated product as well (beyond FUSED_ROWS rows it normalises
+    # the stream itself and rounds in another place)
+    if m > ops.FUSED_ROWS:
+        return
+    wg, wu = (torch.randn(40, n, device=DEV) * 0.1).bfloat16(), (torch.randn(40, n, device=DEV) * 0.1).bfloat16()
+    got = ops.linear(prepared, ops.interleave_gate_up(wg, wu).contiguous(), gated=True)
+    operand = prepared.operand.double()
+    close(got, plain.swiglu((operand @ wg.double().T) * inv, (operand @ wu.double().T) * inv), 1e-2, 1e-2, "gated")
