@@ -19,6 +19,7 @@ QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidd
                 tie_word_embeddings=False)
 CONTEXT = 8192
 PREFILL_TOKENS = 2048
+STATED_PROMPT, STATED_NEW = 2048, 256     # the decode workload the configuration states
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
@@ -37,12 +38,57 @@ def prefill_flops(c, tokens: int, start: int = 0) -> float:
     return gemm + attention
 
 
-def decode_bytes(c, batch: int, context: float, size: int) -> float:
-    """Bytes one decode step has to read: every weight it uses once, and the cache of the live requests."""
-    norms = c.num_hidden_layers * (2 * c.hidden_size + 2 * c.head_dim) + c.hidden_size
-    weights = (matmul_params(c) + c.vocab_size * c.hidden_size + norms + batch * c.hidden_size) * size
-    cache = batch * context * 2 * c.num_hidden_layers * c.num_key_value_heads * c.head_dim * size
-    return weights + cache
+def cache_bytes_per_token(model) -> int:
+    """Bytes of keys and values one cached token takes over all cache slots of the model."""
+    size = 2 if str(model.dtype).endswith("bfloat16") else 4
+    return sum(2 * need.kv_heads * need.head_dim * size for need in model.cache_needs().values()
+               if hasattr(need, "kv_heads"))
+
+
+def decode_bytes(model, batch: int, context: float) -> float:
+    """Bytes one decode step has to read: every weight it uses once (the model's own accounting), the rows
+    of the stream, and the cache of the live requests."""
+    size = 2 if str(model.dtype).endswith("bfloat16") else 4
+    return (model.decode_step_weight_bytes(rows=batch) + batch * model.spec.hidden_size * size
+            + batch * context * cache_bytes_per_token(model))
+
+
+def measure_peaks(device: str = "cuda:0", megabytes: int = 1024, repeats: int = 5) -> dict:
+    """What this GPU gives with nothing else going on: GB/s of a read and of a copy of a buffer several times
+    the size of the caches, and TFLOP/s of a register-only loop of bfloat16 matrix instructions (own kernels,
+    ``csrc/peaks.hip``; the reference's bench measures its stream rate the same way,
+    crates/leone-cli/src/main.rs:4655-4802).  The best of ``repeats`` runs each."""
+    import torch
+    from .ops.library import call, library
+    from . import ops
+    count = megabytes * (1 << 20)
+    src = torch.empty(count, dtype=torch.uint8, device=device)
+    src.random_(0, 255)
+    dst = torch.empty_like(src)
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+    units = ops.compute_units(device)
+    first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def best_ms(launch):
+        launch()
+        found = None
+        for _ in range(repeats):
+            first.record()
+            launch()
+            last.record()
+            torch.cuda.synchronize()
+            ms = first.elapsed_time(last)
+            found = ms if found is None else min(found, ms)
+        return found
+
+    stream = ops._stream()
+    read_ms = best_ms(lambda: call("leone_peak_read", src.data_ptr(), count, sink.data_ptr(), 8 * units, stream))
+    copy_ms = best_ms(lambda: call("leone_peak_copy", src.data_ptr(), dst.data_ptr(), count, 8 * units, stream))
+    blocks, iterations = 8 * units, 4000
+    mfma_ms = best_ms(lambda: call("leone_peak_mfma", blocks, iterations, sink.data_ptr(), stream))
+    flops = library().leone_peak_mfma_flops(blocks, iterations)
+    return {"hbm_read_gbs": round(count / read_ms / 1e6, 1), "hbm_copy_gbs": round(2 * count / copy_ms / 1e6, 1),
+            "mfma_bf16_tflops": round(flops / mfma_ms / 1e9, 1), "buffer_mb": megabytes}
 
 
 def fill_cache(engine, batch: int, tokens: int, seed: int = 0):
@@ -51,19 +97,22 @@ def fill_cache(engine, batch: int, tokens: int, seed: int = 0):
     import torch
     gen = torch.Generator(device=engine.device)
     gen.manual_seed(seed)
-    for k_pool, v_pool in engine.pools.kv.values():
+    for k_pool, v_pool in ([] if getattr(engine, "_bench_filled", False) else engine.pools.kv.values()):
         for pool in (k_pool, v_pool):
             flat = pool.view(-1)
             for at in range(0, flat.numel(), 1 << 28):
                 part = flat[at:at + (1 << 28)]
                 part.copy_(torch.randn(part.numel(), generator=gen, device=engine.device, dtype=torch.float32) * 0.5)
+    engine._bench_filled = True
     for b in range(batch):
         engine.admit(("bench", b))
         engine.cache.reserve(("bench", b), tokens)
         engine.cache.commit(("bench", b))
 
 
-def time_decode(engine, batch: int, start_context: int, steps: int, warmup: int, seed: int = 1):
+def time_decode(engine, batch: int, start_context: int, steps: int, warmup: int, seed: int = 1,
+                profile_steps: int = 0):
+    """(seconds of ``steps`` decode steps, mean context over them[, per-operation profile of further steps])."""
     import torch
     from .engine.engine import StepEntry
     from . import ops
@@ -83,10 +132,36 @@ def time_decode(engine, batch: int, start_context: int, steps: int, warmup: int,
         tokens = one_step(tokens)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
+    profiled = None
+    if profile_steps:
+        from .ops.profile import Recorder
+        recorder = Recorder(profile_steps)
+        for _ in range(profile_steps):
+            recorder.begin_step()
+            tokens = one_step(tokens)
+            recorder.end_step(batch)
+        profiled = recorder.profile
     for b in range(batch):
         engine.release(("bench", b))
     mean_context = start_context + warmup + (steps + 1) / 2.0
-    return elapsed, mean_context
+    return (elapsed, mean_context, profiled) if profile_steps else (elapsed, mean_context)
+
+
+def kernel_table(profiled, model, batch: int, context: float) -> dict:
+    """Per operation of a decode step: microseconds a step and, where the operation streams something, the
+    GB/s it reached (products: their weight bytes; attention: the cache of the live requests)."""
+    steps = max(profiled.steps, 1)
+    table = {}
+    for name in profiled.operations():
+        table[name] = {"us": round(profiled.seconds_by_operation[name] * 1e6 / steps, 1)}
+    for (name, rows, columns, size), timing in sorted(profiled.products.items()):
+        key = f"{name} {rows}x{columns}"
+        table[key] = {"us": round(timing.seconds * 1e6 / steps, 1), "calls": timing.calls // steps,
+                      "gbs": round(rows * columns * size * timing.calls / timing.seconds / 1e9, 1)}
+    if "attention" in table:
+        seconds = profiled.seconds_by_operation["attention"] / steps
+        table["attention"]["gbs"] = round(batch * context * cache_bytes_per_token(model) / seconds / 1e9, 1)
+    return table
 
 
 def time_prefill(engine, tokens: int, repeats: int = 3, seed: int = 2):
@@ -187,6 +262,9 @@ def main(argv: Optional[List[str]] = None) -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--no-kernels", action="store_true", help="skip the per-operation table of the decode step")
+    parser.add_argument("--no-peaks", action="store_true", help="skip the measurement of this GPU's own peaks")
+    parser.add_argument("--peaks", action="store_true", help="only measure this GPU's own peaks and print them")
     parser.add_argument("--scenario", choices=sorted(SCENARIOS), help="run a serving scenario instead of the headline figure")
     args = parser.parse_args(argv)
     if args.gpus != 1:
@@ -195,6 +273,9 @@ def main(argv: Optional[List[str]] = None) -> int:
 
     if args.scenario:
         print(json.dumps(run_scenario(args.scenario, args.dtype, args.layers)), flush=True)
+        return 0
+    if args.peaks:
+        print(json.dumps({"metric": "measured peaks", **measure_peaks()}), flush=True)
         return 0
 
     import torch
@@ -217,11 +298,14 @@ def main(argv: Optional[List[str]] = None) -> int:
     engine = Engine(model, num_pages=pages, page_tokens=page_tokens, max_requests=largest + 1,
                     max_context=args.context)
 
-    start = args.context - args.steps - args.warmup - 1
-    elapsed, mean_context = time_decode(engine, args.batch, start, args.steps, args.warmup)
+    peaks = None if args.no_peaks else measure_peaks()
+    profile_steps = 0 if args.no_kernels else 4
+    start = args.context - args.steps - args.warmup - 1 - profile_steps
+    timed = time_decode(engine, args.batch, start, args.steps, args.warmup, profile_steps=profile_steps)
+    elapsed, mean_context = timed[0], timed[1]
     ms_per_step = elapsed / args.steps * 1e3
     value = args.batch * args.steps / elapsed
-    step_bytes = decode_bytes(config, args.batch, mean_context, size)
+    step_bytes = decode_bytes(model, args.batch, mean_context)
     achieved = step_bytes / (elapsed / args.steps) / 1e9
     record = {
         "metric": "decode tok/s (Qwen3-8B shape)", "value": round(value, 2), "unit": "tok/s", "n_gpus": 1,
@@ -237,17 +321,33 @@ def main(argv: Optional[List[str]] = None) -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
     }
+    weights = model.weight_accounting(rows=args.batch)
+    record["bytes"] = {"weights_resident": weights["tensor_bytes"], "weights_a_step": sum(weights["decode"].values()),
+                       "cache_a_token": cache_bytes_per_token(model), "a_step": int(step_bytes)}
+    if peaks is not None:
+        record["peaks_measured"] = peaks
+        record["roofline"]["frac_of_measured"] = round(achieved / peaks["hbm_read_gbs"], 4)
+    if profile_steps:
+        record["kernels"] = kernel_table(timed[2], model, args.batch, start + args.warmup + args.steps + 2)
     if not args.no_prefill:
         seconds = time_prefill(engine, PREFILL_TOKENS)
         flops = prefill_flops(config, PREFILL_TOKENS)
         record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
                              "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[dtype_name], 4)}
+        if peaks is not None and dtype_name == "bf16":
+            record["prefill"]["frac_of_measured"] = round(flops / seconds / (peaks["mfma_bf16_tflops"] * 1e12), 4)
     points = {}
     for batch in points_batches:
         steps = max(8, args.steps // 2)
         warm = max(2, args.warmup // 2)
         e, _ = time_decode(engine, batch, args.context - steps - warm - 1, steps, warm)
         points[f"decode_b{batch}"] = round(batch * steps / e, 2)
+    # The workload the configuration states: prompts of 2,048 tokens, 256 new tokens each.
+    for batch in ([] if args.no_points else sorted({1, args.batch, 64})):
+        if STATED_PROMPT + STATED_NEW + 1 > args.context:
+            break
+        e, _ = time_decode(engine, batch, STATED_PROMPT, STATED_NEW - 8, 8)
+        points[f"decode_b{batch}_prompt{STATED_PROMPT}_new{STATED_NEW}"] = round(batch * (STATED_NEW - 8) / e, 2)
     if points:
         record["points"] = points
     print(json.dumps(record), flush=True)

@@ -228,6 +228,13 @@ def cmd_doctor(args) -> int:
         found = {n: (e.shape, e.dtype) for n, e in files.entries.items()}
         loader.check(model.tensor_specs(), found, args.model, model.spec.ignore_tensors)
         print("tensor names and shapes: ok")
+        # bytes by class as the file stores them: in memory, and as one decode step reads them
+        accounting = model.weight_accounting(lambda spec: files.entries[spec.name].nbytes)
+        for family in sorted(accounting["resident"]):
+            print(f"  {family:<13} resident {accounting['resident'][family] / 2**20:10.1f} MiB   "
+                  f"a decode step {accounting['decode'][family] / 2**20:10.1f} MiB")
+        print(f"weights a decode step reads: {sum(accounting['decode'].values()) / 2**20:.1f} MiB of "
+              f"{accounting['tensor_bytes'] / 2**20:.1f} MiB")
         size = 2 if args.dtype == "bfloat16" else 4
         per_token = sum(2 * need.kv_heads * need.head_dim * size for need in model.cache_needs().values()
                         if hasattr(need, "kv_heads"))

@@ -39,7 +39,8 @@ Reject Scheduler::submit(RequestKey request, const std::int32_t* prompt, int pro
     state->order = ++order_;
     queue_.push_back(std::move(state));
     stats_.max_queue_depth = std::max<std::int64_t>(stats_.max_queue_depth, queue_.size());
-    events_.push_back({EventKind::Submit, request, 0, 0, 0});
+    events_.push_back({EventKind::Submit, request, prompt_tokens,
+                       static_cast<int>(std::min<std::int64_t>(max_new_tokens, 0x7fffffff)), 0});
     return Reject::None;
 }
 

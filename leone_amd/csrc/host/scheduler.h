@@ -81,7 +81,9 @@ struct SchedulerStats {
 };
 
 // One record of the decision log.  A step is a StepBegin record (a = number of entries) followed by
-// that many StepEntry records (a = start, b = count, c = sample).
+// that many StepEntry records (a = start, b = count, c = sample).  Submit: a = prompt tokens, b = most new
+// tokens; Reject: a = reason; Preempt: a = tokens known; Token: a = position of the row that gave it,
+// b = token; Finish: a = reason.
 enum class EventKind : int { Reject = 0, Submit, StepBegin, StepEntry, Admit, Preempt, Token, Finish };
 struct Event {
     EventKind kind;

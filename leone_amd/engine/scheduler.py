@@ -251,7 +251,8 @@ class Scheduler:
 
     @property
     def events(self) -> List[tuple]:
-        """The decision log: ("reject", id, reason), ("submit", id), ("step", [(id, start, tokens, sample)]),
+        """The decision log: ("reject", id, reason), ("submit", id, prompt tokens, most new tokens),
+        ("step", [(id, start, tokens, sample)]),
         ("admit", id), ("preempt", id, tokens known), ("token", id, position, token), ("finish", id, reason)."""
         n = self._checked(self._lib.leone_scheduler_event_count(self.handle))
         kinds, a, b, c = (c_int * max(1, n))(), (c_int * max(1, n))(), (c_int * max(1, n))(), (c_int * max(1, n))()
@@ -265,7 +266,7 @@ class Scheduler:
             if kind == 0:
                 out.append(("reject", name, _REJECTS[a[i]].value))
             elif kind == 1:
-                out.append(("submit", name))
+                out.append(("submit", name, a[i], b[i]))
             elif kind == 2:
                 rows = [(self._names[keys[j]], a[j], b[j], bool(c[j])) for j in range(i + 1, i + 1 + a[i])]
                 out.append(("step", rows))

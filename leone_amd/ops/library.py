@@ -39,6 +39,9 @@ _PROTOTYPES = {
                               c_int, P],
     "leone_gemm_rows_bf16": [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, ctypes.c_long, c_int, P],
     "leone_argmax": [P, P, P, P, c_int, c_int, P],
+    "leone_peak_read": [P, ctypes.c_long, P, c_int, P],
+    "leone_peak_copy": [P, P, ctypes.c_long, c_int, P],
+    "leone_peak_mfma": [c_int, c_int, P, P],
     "leone_sample_temperature": [P, P, P, P, P, P, P, P, c_int, c_int, P],
     "leone_top_candidates": [P, P, P, P, c_int, c_int, c_int, P],
 }
@@ -66,6 +69,8 @@ def library() -> ctypes.CDLL:
             lib.leone_top_candidates_max.argtypes = []
             lib.leone_argmax_chunk.restype = c_int
             lib.leone_argmax_chunk.argtypes = []
+            lib.leone_peak_mfma_flops.restype = ctypes.c_double
+            lib.leone_peak_mfma_flops.argtypes = [c_int, c_int]
             lib.leone_gemm_rows_max_rows.restype = c_int
             lib.leone_gemm_rows_max_rows.argtypes = []
             lib.leone_gemm_rows_chunk.restype = c_int

@@ -28,6 +28,7 @@ OPERATIONS = {
     "leone_attention_rows": "attention",
     "leone_attention_prefill": "attention",
     "leone_gemm_fused_bf16": "gemv fused",
+    "leone_gemm_rows_bf16": "gemm rows",
     "leone_gemm_f32": "gemm f32",
     "leone_swiglu": "swiglu",
     "leone_argmax": "argmax",
@@ -35,7 +36,7 @@ OPERATIONS = {
     "leone_top_candidates": "sample",
 }
 LIBRARY_PRODUCT = "gemm library"
-ORDER = ["embed", "norm", "gemv fused", LIBRARY_PRODUCT, "gemm f32", "qknorm rope kv", "attention", "swiglu",
+ORDER = ["embed", "norm", "gemv fused", "gemm rows", LIBRARY_PRODUCT, "gemm f32", "qknorm rope kv", "attention", "swiglu",
          "argmax", "sample"]
 
 

@@ -18,9 +18,14 @@ feed_forward  ``tensor_specs()``, ``bind(tensors)``, ``forward(y, step)`` -> del
               A mixer or feed-forward that sets ``fused_io = True`` is instead called with
               ``forward(y, step[, cache], residual=x)``: ``y`` may then be an ``ops.NormedRows`` (a norm
               not yet carried out, which ``ops.linear`` folds into the product), and the part may add its
-              result into the float32 stream ``residual`` itself and return None.
+              result into the float32 stream ``residual`` itself and return None.  One that also sets
+              ``prepares_next = True`` takes ``next_norm=`` (what ``RmsNorm.folded`` gives for the norm
+              that runs next) and may then return ``ops.PreparedRows``: the result has been added and
+              that norm's operand lies ready, so no norm kernel runs between the two products.
 block         ``tensor_specs()``, ``bind(tensors)``, ``cache_need()``,
-              ``forward(x, pending, step, cache)`` -> new pending delta.
+              ``forward(x, pending, step, cache)`` -> new pending delta.  Optional: ``entry_norm(dtype)``
+              (what the block before may prepare) and ``prepares_next = True`` with
+              ``forward(..., next_norm=)``, as above.
 
 ``x`` is the residual stream, float32 ``[rows, hidden]``; ``pending`` is a delta
 not yet added to it (the next norm adds it, so add and norm are one kernel).
@@ -89,7 +94,12 @@ class Registry:
         except KeyError:
             raise ValueError(
                 f"unknown {self.family} kind {spec.kind!r}; registered: {', '.join(sorted(self._classes))}") from None
-        return cls(spec, **context)
+        part = cls(spec, **context)
+        try:
+            part.family = self.family            # what the model's byte accounting files its tensors under
+        except AttributeError:
+            pass
+        return part
 
     def kinds(self) -> List[str]:
         return sorted(self._classes)

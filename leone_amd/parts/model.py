@@ -89,6 +89,44 @@ class DecoderModel:
         for position in self.positions.values():
             position.prepare(self.spec.max_positions, self.device)
 
+    # ---- bytes ---------------------------------------------------------------
+    def weight_accounting(self, nbytes=None, rows: int = 1) -> Dict[str, object]:
+        """Bytes of the model's tensors by class, as they lie in memory (``resident``) and as a decode step
+        of ``rows`` rows reads them (``decode``): of the token table only the rows' own rows, and the whole
+        table once more as the head if the head is tied to it (the reference's accounting,
+        crates/leone/src/model.rs:306-366).  ``nbytes(spec)`` gives a tensor's size; by default its element
+        count in this model's type."""
+        size = 2 if self.dtype == torch.bfloat16 else 4
+        if nbytes is None:
+            def nbytes(spec):
+                count = 1
+                for extent in spec.shape:
+                    count *= extent
+                return count * size
+        resident: Dict[str, int] = {"embed": 0, "head": 0}
+        table = TensorSpec(self.spec.embedding, (self.spec.vocab_size, self.spec.hidden_size), MATRIX)
+        resident["embed"] = nbytes(table)
+        if self.spec.head is not None:
+            resident["head"] = nbytes(TensorSpec(self.spec.head, (self.spec.vocab_size, self.spec.hidden_size), MATRIX))
+        for layer in self.layers:
+            for part in (layer.parts() if hasattr(layer, "parts") else (layer,)):
+                family = getattr(part, "family", "layer")
+                resident[family] = resident.get(family, 0) + sum(nbytes(s) for s in part.tensor_specs())
+        resident["norm"] = resident.get("norm", 0) + sum(nbytes(s) for s in self.final_norm.tensor_specs())
+        decode = dict(resident)
+        decode["embed"] = resident["embed"] // self.spec.vocab_size * rows
+        if self.spec.head is None:
+            decode["head"] = resident["embed"]
+        return {"tensor_bytes": sum(resident.values()), "resident": resident, "decode": decode}
+
+    def weight_bytes(self) -> int:
+        """Bytes of all tensors of the model."""
+        return self.weight_accounting()["tensor_bytes"]
+
+    def decode_step_weight_bytes(self, rows: int = 1) -> int:
+        """Weight bytes a decode step of ``rows`` rows has to read: every weight it uses, once."""
+        return sum(self.weight_accounting(rows=rows)["decode"].values())
+
     # ---- cache ---------------------------------------------------------------
     def cache_needs(self) -> Dict[int, object]:
         """Cache slot -> what the layer runs on it need (one need per slot)."""

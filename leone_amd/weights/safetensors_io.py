@@ -144,6 +144,28 @@ class ModelFiles:
         self._maps.clear()
 
 
+def file_digests(model_dir: str, whole_up_to: int = 1 << 30) -> list:
+    """What identifies the weight files of a model folder: name, size and SHA-256 of the header (names,
+    types, shapes and offsets) of each; of the whole file too if it has at most ``whole_up_to`` bytes."""
+    import hashlib
+    files = sorted({entry.file for entry in ModelFiles(model_dir).entries.values()})
+    out = []
+    for path in files:
+        size = os.path.getsize(path)
+        with open(path, "rb") as handle:
+            length = int.from_bytes(handle.read(8), "little")
+            record = {"file": os.path.basename(path), "bytes": size,
+                      "header_sha256": hashlib.sha256(handle.read(length)).hexdigest()}
+            if size <= whole_up_to:
+                handle.seek(0)
+                digest = hashlib.sha256()
+                for block in iter(lambda: handle.read(1 << 22), b""):
+                    digest.update(block)
+                record["sha256"] = digest.hexdigest()
+        out.append(record)
+    return out
+
+
 def write_file(path: str, tensors: Mapping[str, torch.Tensor], metadata: Mapping[str, str] | None = None) -> None:
     """Writes CPU tensors as one safetensors file, names in sorted order."""
     header: dict = {}

@@ -53,9 +53,26 @@ def test_bench_arithmetic():
     from leone_amd.architectures import config_from_dict
     c = config_from_dict(benchmark.QWEN3_8B)
     assert benchmark.matmul_params(c) == 36 * (4096 * 6144 + 4096 * 4096 + 3 * 4096 * 12288)
-    # weights 15.14 GB a step, cache 147,456 bytes a token of context
-    assert abs(benchmark.decode_bytes(c, 1, 0, 2) / 1e9 - 15.14) < 0.01
-    assert benchmark.decode_bytes(c, 8, 100, 2) - benchmark.decode_bytes(c, 8, 0, 2) == 8 * 100 * 147456
+    # weights 15.14 GB a step, cache 147,456 bytes a token of context: from the model's own accounting
+    import torch
+    from leone_amd.architectures import model_spec_for
+    from leone_amd.parts.model import DecoderModel
+    model = DecoderModel(model_spec_for(c), torch.bfloat16, "cpu")
+    assert abs(benchmark.decode_bytes(model, 1, 0) / 1e9 - 15.14) < 0.01
+    assert benchmark.decode_bytes(model, 8, 100) - benchmark.decode_bytes(model, 8, 0) == 8 * 100 * 147456
+    assert benchmark.cache_bytes_per_token(model) == 147456
+    accounting = model.weight_accounting(rows=8)
+    table = 151936 * 4096 * 2
+    assert accounting["resident"]["embed"] == table and accounting["resident"]["head"] == table
+    assert accounting["decode"]["embed"] == 8 * 4096 * 2 and accounting["decode"]["head"] == table
+    assert accounting["resident"]["feed_forward"] == 36 * 3 * 4096 * 12288 * 2
+    assert accounting["resident"]["mixer"] == 36 * (4096 * 6144 + 4096 * 4096 + 2 * 128) * 2
+    assert accounting["resident"]["norm"] == (36 * 2 + 1) * 4096 * 2
+    assert model.weight_bytes() == sum(accounting["resident"].values())
+    assert model.decode_step_weight_bytes(8) == model.weight_bytes() - table + 8 * 4096 * 2
+    tied = DecoderModel(model_spec_for(config_from_dict(dict(benchmark.QWEN3_8B, tie_word_embeddings=True))),
+                        torch.bfloat16, "cpu")
+    assert tied.weight_accounting()["resident"]["head"] == 0 and tied.weight_accounting()["decode"]["head"] == table
     assert abs(benchmark.prefill_flops(c, 2048) / 2.97e13 - 1) < 0.01
 
 

@@ -16,9 +16,9 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def replay(folder, dtype_name, steps, out_dir, max_tokens):
+def replay(folder, dtype_name, steps, out_dir, max_tokens, *flags):
     process = subprocess.Popen([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype",
-                                dtype_name, "--out", out_dir, "--max-tokens", str(max_tokens)],
+                                dtype_name, "--out", out_dir, "--max-tokens", str(max_tokens), *flags],
                                stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
     outputs = {}
     vocab = read_config(folder)["vocab_size"]
@@ -68,3 +68,42 @@ def test_replay_modes_agree_with_plain(tmp_path, name, dtype_name):
                         f"{mode}: request {e['id']} position {at[e['id']] + w}: {err:.3e}"
                     row += 1
                 at[e["id"]] += len(e["tokens"])
+
+
+def test_sidecar_ties_the_logits_to_what_made_them(tmp_path):
+    """--sidecar: model and build identity, the schedule and digests of input and outputs; --poison-freed: pages
+    given back are filled with NaN and the logits of a run that reuses them are the same bits as without."""
+    import hashlib
+    folder = make_model_dir(str(tmp_path / "model"), TINY["A"], 33, torch.bfloat16)
+    config = read_config(folder)
+    requests = {f"q{i}": random_tokens(700 + i, n, config["vocab_size"]) for i, n in enumerate([90, 70, 40, 120, 64, 33])}
+    steps = schedules.mixed(requests)
+    room = schedules.max_live_tokens(steps, 64)
+    plain_out, poisoned_out = str(tmp_path / "plain"), str(tmp_path / "poisoned")
+    first = replay(folder, "bfloat16", steps, plain_out, room)
+    second = replay(folder, "bfloat16", steps, poisoned_out, room, "--sidecar", "--poison-freed")
+    assert not os.path.exists(os.path.join(plain_out, "sidecar.json"))
+    for step, block in first.items():
+        assert np.isfinite(block).all() and np.array_equal(block, second[step])
+    with open(os.path.join(poisoned_out, "sidecar.json")) as handle:
+        sidecar = json.load(handle)
+    assert sidecar["schema"] == "leone-amd.trace.v1" and sidecar["dtype"] == "bfloat16" and sidecar["poison_freed"]
+    assert sidecar["architecture"] == config["architectures"][0] and sidecar["vocab"] == config["vocab_size"]
+    with open(os.path.join(folder, "config.json"), "rb") as handle:
+        assert sidecar["config_sha256"] == hashlib.sha256(handle.read()).hexdigest()
+    with open(os.path.join(folder, "model.safetensors"), "rb") as handle:
+        assert sidecar["weights"] == [{"file": "model.safetensors", "bytes": os.path.getsize(handle.name),
+                                       "header_sha256": sidecar["weights"][0]["header_sha256"],
+                                       "sha256": hashlib.sha256(handle.read()).hexdigest()}]
+    assert sidecar["input_sha256"] == hashlib.sha256("".join(json.dumps(s) + "\n" for s in steps).encode()).hexdigest()
+    assert len(sidecar["build"]["kernels"]) == 16 and len(sidecar["build"]["host"]) == 16
+    assert [s["step"] for s in sidecar["steps"]] == [s["step"] for s in steps]
+    for noted, s in zip(sidecar["steps"], steps):
+        assert noted["end"] == s["end"]
+        assert noted["entries"] == [{"id": e["id"], "tokens": len(e["tokens"]), "want": e["want"]} for e in s["entries"]]
+        if any(e["want"] for e in s["entries"]):
+            with open(os.path.join(poisoned_out, noted["file"]), "rb") as handle:
+                assert noted["sha256"] == hashlib.sha256(handle.read()).hexdigest()
+            assert noted["rows"] == sum(len(e["want"]) for e in s["entries"])
+        else:
+            assert "file" not in noted

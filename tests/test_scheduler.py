@@ -217,3 +217,84 @@ def test_random_load_under_page_pressure(seed):
             for rid, start, count, _ in event[1]:
                 assert fed.get(rid, 0) == start
                 fed[rid] = start + count
+
+
+# ---- the checker that works from the decision log alone ------------------------------------------
+
+def _loaded(seed, window=None):
+    from leone_amd.engine import trace_check
+    rng = random.Random(500 + seed)
+    page_tokens = rng.choice([4, 8])
+    groups = [GroupSpec(rng.choice([12, 16, 24]), page_tokens)]
+    if window:
+        groups.append(GroupSpec(12, page_tokens, window))
+    cache = CacheManager(groups, 8, 4096)
+    s = Scheduler(SchedulerPolicy(max_live_requests=4, prefill_chunk_tokens=rng.choice([3, 16, 64]),
+                                  max_step_tokens=rng.choice([8, 24, 200])), cache)
+    wanted = {}
+    for i in range(20):
+        prompt = [rng.randrange(97) for _ in range(rng.randrange(1, 40))]
+        n = rng.randrange(1, 30)
+        if s.submit(Request(i, prompt, n, eos_token_id=rng.choice([None, 5]))) is None:
+            wanted[i] = (prompt, n)
+    if seed % 2:
+        s.cancel(3)
+    run(s, fail_at_step=7 if seed == 2 else None)
+    return s, wanted, trace_check
+
+
+@pytest.mark.parametrize("window", [None, 9])
+@pytest.mark.parametrize("seed", range(4))
+def test_the_log_alone_shows_a_sound_run(seed, window):
+    """Page conservation, budgets, one step in flight and contiguous positions are re-derived from the
+    events by a checker that shares nothing with the scheduler, and the transcript it reads off the events
+    equals every request run alone (crates/leone/src/scheduler.rs:1349-1655)."""
+    s, wanted, trace_check = _loaded(seed, window)
+    figures = trace_check.figures_of(s)
+    report = trace_check.verify_events(s.events, figures)
+    assert report.steps == s.stats.steps and report.peak_live <= 4
+    assert report.peak_pages == s.cache.pages_high_water
+    assert report.peak_step_tokens <= s.policy.max_step_tokens
+    finished = {f.id: f for f in s.finished}
+    assert set(report.requests) == set(wanted)
+    for rid, trace in report.requests.items():
+        assert trace.state == "finished" and trace.reason == finished[rid].reason
+        assert trace.tokens == finished[rid].tokens and trace.preemptions == finished[rid].preemptions
+        if trace.reason in ("eos", "length"):
+            prompt, n = wanted[rid]
+            assert trace.tokens == isolated(prompt, n, eos=5 if trace.reason == "eos" else None)[:len(trace.tokens)]
+            assert trace.fed >= len(prompt) + len(trace.tokens) - 1
+
+
+def test_the_checker_refuses_a_log_that_breaks_a_rule():
+    s, wanted, trace_check = _loaded(0)
+    figures = trace_check.figures_of(s)
+    events = s.events
+    trace_check.verify_events(events, figures)
+
+    def broken(change):
+        changed = [list(e) if e[0] != "step" else ["step", [list(r) for r in e[1]]] for e in events]
+        change(changed)
+        with pytest.raises(trace_check.TraceError):
+            trace_check.verify_events([tuple(e) for e in changed], figures)
+
+    first_step = next(i for i, e in enumerate(events) if e[0] == "step")
+    first_token = next(i for i, e in enumerate(events) if e[0] == "token")
+    later_step = next(i for i, e in enumerate(events) if e[0] == "step" and i > first_token and e[1][0][1] > 0)
+    broken(lambda ev: ev.pop(first_token))                                   # a row's token never arrives
+    broken(lambda ev: ev.insert(first_token, ev[first_token]))               # a token twice
+    broken(lambda ev: ev[later_step][1][0].__setitem__(1, ev[later_step][1][0][1] + 1))   # a position skipped
+    broken(lambda ev: ev[later_step][1][0].__setitem__(1, ev[later_step][1][0][1] - 1))   # a position fed twice
+    broken(lambda ev: ev[first_step][1].append(list(ev[first_step][1][0])))  # a request twice in a step
+    broken(lambda ev: ev.insert(first_step, ev[first_step]))                 # two steps in flight
+    broken(lambda ev: ev.append(("token", 0, 5, 1)))                         # something after the end
+    broken(lambda ev: ev.pop(next(i for i, e in enumerate(ev) if e[0] == "admit")))   # a step for a queued request
+    import dataclasses
+    with pytest.raises(trace_check.TraceError, match="pages"):
+        small = dataclasses.replace(figures, pools=[trace_check.PoolFigures(figures.pools[0].num_pages // 3,
+                                                                             figures.pools[0].page_tokens)])
+        trace_check.verify_events(events, small)
+    with pytest.raises(trace_check.TraceError, match="budget"):
+        trace_check.verify_events(events, dataclasses.replace(figures, max_step_tokens=1))
+    with pytest.raises(trace_check.TraceError, match="live requests"):
+        trace_check.verify_events(events, dataclasses.replace(figures, max_live_requests=1))
