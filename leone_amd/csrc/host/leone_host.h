@@ -96,6 +96,26 @@ long leone_step_pack(void* cache, int n_entries, const int64_t* requests, const 
 int leone_sample_rows(const float* logits, int rows, int vocab, const double* temperature, const int* stage_counts,
                       const int* stage_kinds, const double* stage_values, const double* uniform, int* tokens);
 
+// ---- scalar single-precision reference of the kernel entry points, on host memory (scalar_reference.cpp).
+// Arguments as the kernels', float32 only, no stream; for comparison, never on the product path.
+int leone_ref_embed(const float* table, const int* tokens, float* out, int rows, int hidden, int vocab);
+int leone_ref_add_rmsnorm(float* x, const float* delta, int planes, long plane, const float* gain, float eps,
+                          float* y, const int* rows, int n_rows, int hidden);
+int leone_ref_rope_table(float* cos_out, float* sin_out, double theta, int rotary_dim, int positions);
+int leone_ref_qk_norm_rope_write(const float* qkv, int planes, long plane, float* q_out, float* k_pool, float* v_pool,
+                                 const float* q_gain, const float* k_gain, float eps, const float* cos_table,
+                                 const float* sin_table, int table_positions, const int* positions,
+                                 const int* row_entry, const int* block_table, int max_blocks, int rows, int q_heads,
+                                 int kv_heads, int head_dim, int page_tokens, int write_cache);
+int leone_ref_attention(const float* q, float* out, const float* k_pool, const float* v_pool, const int* positions,
+                        const int* row_entry, const int* block_table, int max_blocks, int rows, int q_heads,
+                        int kv_heads, int head_dim, int page_tokens, float scale, int window);
+int leone_ref_gemm(const float* a, const float* b, float* c, int m, int n, int k);
+int leone_ref_swiglu(const float* gate_up, float* out, int rows, int ffn);
+int leone_ref_argmax(const float* logits, int* out, int rows, int vocab);
+int leone_ref_sample_temperature(const float* logits, const double* temperature, const double* uniform, int* out,
+                                 int rows, int vocab);
+
 #ifdef __cplusplus
 }
 #endif
