@@ -5,7 +5,14 @@
 // tile a wave computes S^T = K . Q^T (keys x heads) with
 // v_mfma_f32_16x16x32_bf16, runs the running-maximum softmax of the reference
 // (crates/leone/src/cpu.rs:2299-2357) in float on the accumulator registers,
-// and adds O^T += V^T . P^T with the same instruction.  The cache packs keys
+// and adds O^T += V^T . P^T with the same instruction.  The softmax works in
+// powers of two against a reference that is a whole number (the running
+// maximum rounded up): the weights 2^(s - reference) that are rounded to
+// bfloat16 for the second product then have the same significant bits
+// whatever the reference, so they do not depend on how the keys are cut
+// into tiles, waves and splits, and changes of the reference rescale the
+// sums by exact powers of two.  The row sum is taken over the rounded
+// weights, the ones the values are weighted with.  The cache packs keys
 // as [element / 8][token][8] and values as [token / 8][element][8], so that
 // both operands are 16-byte loads straight from the cache with the 16 lanes of
 // a quarter wave on neighbouring runs, a key or value being read once for all
@@ -55,7 +62,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                         const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
                         const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
                         float* __restrict__ part_acc, float* __restrict__ part_ml, bf16_t* __restrict__ out,
-                        int q_heads, int kv_heads, int page_shift, float scale, int window, int splits) {
+                        int q_heads, int kv_heads, int page_shift, float to_log2, int window, int splits) {
     constexpr int kD = kD16 * 16;
     constexpr int kSteps = (kD16 + 1) / 2;           // 32-element steps of the q.k product
     extern __shared__ float smem[];                   // [waves][columns][kD] accumulators, then m and l
@@ -171,20 +178,19 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         for (int j = 0; j < 8; ++j) {
             const int key = run0 + j;
             const float raw = j < 4 ? sa[j & 3] : sb[j & 3];
-            sc[j] = (kFull || (key >= lo && key < n)) ? raw * scale : -INFINITY;
+            sc[j] = (kFull || (key >= lo && key < n)) ? raw * to_log2 : -INFINITY;
             tile_max = fmaxf(tile_max, sc[j]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
-        const float m_new = fmaxf(m_run, tile_max);      // finite: every tile of the range holds a key in reach
-        const float alpha = __expf(m_run - m_new);
+        const float m_new = fmaxf(m_run, ceilf(tile_max));   // finite: every tile of the range holds a key in reach
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);   // an exact power of two (0 from -inf)
         float psum = 0.f;
         bf16x8 pt;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const float p = __expf(sc[j] - m_new);
-            psum += p;
-            pt[j] = static_cast<__bf16>(p);
+            pt[j] = static_cast<__bf16>(__builtin_amdgcn_exp2f(sc[j] - m_new));
+            psum += static_cast<float>(pt[j]);
         }
         psum += __shfl_xor(psum, 16, kWave);
         psum += __shfl_xor(psum, 32, kWave);
@@ -249,7 +255,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
 #pragma unroll
             for (int w = 0; w < kDecodeWaves; ++w) {
                 const float mw = sm_m[w * cols + col];
-                const float wgt = mw == -INFINITY ? 0.f : __expf(mw - top);
+                const float wgt = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - top);
                 num += sm_acc[(w * cols + col) * kD + d] * wgt;
                 den += sm_l[w * cols + col] * wgt;
             }
@@ -268,8 +274,8 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     }
 }
 
-// Merges the splits of one (row, query head): out = sum_s acc_s e^(m_s - M) / sum_s l_s e^(m_s - M),
-// the sums taken in split order.  The weights e^(m_s - M) are computed once, one thread a split.
+// Merges the splits of one (row, query head): out = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M),
+// the sums taken in split order.  The weights 2^(m_s - M) are computed once, one thread a split.
 constexpr int kReduceThreads = 128;
 constexpr int kMaxSplits = 256;
 
@@ -287,7 +293,7 @@ attention_reduce_kernel(const float* __restrict__ part_acc, const float* __restr
     __syncthreads();
     top = fmaxf(wave_top[0], wave_top[1]);
     for (int s = threadIdx.x; s < splits; s += kReduceThreads)
-        weight[s] = ml[2 * s] == -INFINITY ? 0.f : __expf(ml[2 * s] - top);
+        weight[s] = ml[2 * s] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ml[2 * s] - top);
     __syncthreads();
     float den = 0.f;
     for (int s = 0; s < splits; ++s) den += ml[2 * s + 1] * weight[s];
@@ -316,7 +322,7 @@ static void launch_decode(const void* q, const void* k_pool, const void* v_pool,
     attention_decode_kernel<kD16><<<grid, kDecodeThreads, smem, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
         positions, row_entry, block_table, max_blocks, part_acc, part_ml, static_cast<bf16_t*>(out), q_heads, kv_heads,
-        page_shift, scale, window, splits);
+        page_shift, scale * 1.4426950408889634f, window, splits);
 }
 
 }  // namespace leone

@@ -18,7 +18,10 @@
 // The recurrence is kept in base-2 units: t = score * scale * log2(e), p = 2^(t - m).  m is a
 // reference, not always the maximum: it is raised (and sums and accumulators rescaled) only when
 // a score exceeds it by more than 8, so that in the common case a pass needs no exchange between
-// lanes; p stays below 2^8 and the quotient of accumulator and sum does not depend on m.  The sum
+// lanes; p stays below 2^8 and the quotient of accumulator and sum does not depend on m.  m is
+// always a whole number (the maximum rounded up), so that the bfloat16 rounding of p gives the same
+// significant bits whatever m is: the weights do not depend on how the keys are cut into passes,
+// stages and ranges, and a raised reference rescales by an exact power of two.  The sum
 // of a query's p is one more row of the second product (a row of ones in V^T), so that numerator
 // and denominator are sums of the same rounded values.
 //
@@ -327,7 +330,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             for (int j = 0; j < kColsPerWave; ++j) {
                 float col_top = fmaxf(top[j], __shfl_xor(top[j], 16, kWave));
                 col_top = fmaxf(col_top, __shfl_xor(col_top, 32, kWave));
-                const float m_new = fmaxf(m_ref[j], col_top);
+                const float m_new = fmaxf(m_ref[j], ceilf(col_top));     // a whole number: see the rounding of the weights below
                 const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_ref[j] - m_new);   // 2^-inf = 0
                 m_ref[j] = m_new;
 #pragma unroll

@@ -17,10 +17,12 @@ int leone_embed(const void* table, int dtype, const int* tokens, float* out, int
 
 // x += delta (delta may be null); y = rmsnorm(x) * gain.  With `rows` given,
 // y[r] is computed from row rows[r] and x is not written.  delta may be delta_planes (1..16) planes,
-// delta_plane elements apart, whose sum in order is what is added.
+// delta_plane elements apart, whose sum in order is what is added.  With squares_out (float32 [n_rows,
+// ceil(hidden / 16)]) the norm is only prepared for leone_gemm_fused_bf16's in_mode 2: y = x * gain, not yet
+// scaled, and the row's sum of squares in squares_out[r][0], zeros behind it.
 int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, int delta_planes, long delta_plane, const void* gain,
                       int gain_dtype, float eps, void* y, int y_dtype, const int* rows, int n_rows, int hidden,
-                      hipStream_t stream);
+                      float* squares_out, hipStream_t stream);
 
 // out[r, c] = silu(gate) * up, where gate_up[r] holds, in every block of 16 columns, 8 gate values
 // and then the 8 up values that belong to them; ffn is a multiple of 8.

@@ -39,7 +39,7 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
 template <typename TD, typename TY, int kThreads>
 __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int planes, long plane,
                                    AnyVec gain, float eps, TY* __restrict__ y,
-                                   const int* __restrict__ rows, int hidden) {
+                                   const int* __restrict__ rows, int hidden, float* __restrict__ squares_out) {
     __shared__ float scratch[kThreads / kWave];
     const int out_row = blockIdx.x;
     const long in_row = rows ? rows[out_row] : out_row;
@@ -56,7 +56,11 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__
         ss = fmaf(v, v, ss);
     }
     const float total = block_sum<kThreads>(ss, scratch);
-    const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+    const float inv = squares_out ? 1.0f : 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+    if (squares_out) {                                 // the row's sum first, zeros for the other parts
+        const int parts = (hidden + 15) / 16;
+        for (int i = threadIdx.x; i < parts; i += kThreads) squares_out[static_cast<long>(out_row) * parts + i] = i == 0 ? total : 0.f;
+    }
     for (int c = threadIdx.x; c < hidden; c += kThreads) {
         float v = xr[c];
         if (dr && rows)
@@ -91,7 +95,7 @@ template <typename TD, typename TG, typename TY, int kThreads, int kChunks>
 __global__ void __launch_bounds__(kThreads)
 add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, int planes, long plane,
                        const TG* __restrict__ gain, float eps, TY* __restrict__ y, const int* __restrict__ rows,
-                       int hidden) {
+                       int hidden, float* __restrict__ squares_out) {
     __shared__ float scratch[kThreads / kWave];
     const int out_row = blockIdx.x;
     const long in_row = rows ? rows[out_row] : out_row;
@@ -120,7 +124,11 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, int 
         }
     }
     const float total = block_sum<kThreads>(ss, scratch);
-    const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+    const float inv = squares_out ? 1.0f : 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
+    if (squares_out) {                                 // the row's sum first, zeros for the other parts
+        const int parts = (hidden + 15) / 16;
+        for (int i = threadIdx.x; i < parts; i += kThreads) squares_out[static_cast<long>(out_row) * parts + i] = i == 0 ? total : 0.f;
+    }
 #pragma unroll
     for (int i = 0; i < kChunks; ++i) {
         const int c = 4 * (threadIdx.x + i * kThreads);
@@ -239,6 +247,9 @@ __global__ void qk_norm_rope_write_kernel(
                 a[i] += to_float(src[s * plane + p]);
                 b[i] += to_float(src[s * plane + p + half]);
             }
+            // rounded as a product stored in the outputs' type would be: the same bits whichever way it came
+            a[i] = to_float(from_float<T>(a[i]));
+            b[i] = to_float(from_float<T>(b[i]));
             ss = fmaf(a[i], a[i], ss);
             ss = fmaf(b[i], b[i], ss);
         }
@@ -351,6 +362,9 @@ qk_norm_rope_write_runs_kernel(
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
+            // rounded as a product stored in the outputs' type would be: the same bits whichever way it came
+            a[i] = to_float(from_float<T>(a[i]));
+            b[i] = to_float(from_float<T>(b[i]));
             ss = fmaf(a[i], a[i], ss);
             ss = fmaf(b[i], b[i], ss);
         }
@@ -516,39 +530,39 @@ extern "C" int leone_embed(const void* table, int dtype, const int* tokens, floa
 
 template <typename TD, typename TG, typename TY>
 static void launch_add_rmsnorm_vec(float* x, const void* delta, int planes, long plane, const void* gain, float eps,
-                                   void* y, const int* rows, int n_rows, int hidden, hipStream_t stream) {
+                                   void* y, const int* rows, int n_rows, int hidden, float* squares, hipStream_t stream) {
     const TD* d = static_cast<const TD*>(delta);
     const TG* g = static_cast<const TG*>(gain);
     TY* out = static_cast<TY*>(y);
     if (hidden <= 4 * 64 * 2)
-        add_rmsnorm_vec_kernel<TD, TG, TY, 64, 2><<<n_rows, 64, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden);
+        add_rmsnorm_vec_kernel<TD, TG, TY, 64, 2><<<n_rows, 64, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden, squares);
     else if (hidden <= 4 * 256 * 2)
-        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 2><<<n_rows, 256, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden);
+        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 2><<<n_rows, 256, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden, squares);
     else if (hidden <= 4 * 256 * 4)
-        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 4><<<n_rows, 256, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden);
+        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 4><<<n_rows, 256, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden, squares);
     else
-        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 8><<<n_rows, 256, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden);
+        add_rmsnorm_vec_kernel<TD, TG, TY, 256, 8><<<n_rows, 256, 0, stream>>>(x, d, planes, plane, g, eps, out, rows, hidden, squares);
 }
 
 template <typename TD, typename TY>
 static void launch_add_rmsnorm(float* x, const void* delta, int planes, long plane, AnyVec gain, float eps, void* y,
-                               const int* rows, int n_rows, int hidden, hipStream_t stream) {
+                               const int* rows, int n_rows, int hidden, float* squares, hipStream_t stream) {
     if (hidden % 4 == 0 && hidden <= 4 * 256 * 8) {
         if (gain.dtype == kF32)
-            launch_add_rmsnorm_vec<TD, float, TY>(x, delta, planes, plane, gain.ptr, eps, y, rows, n_rows, hidden, stream);
+            launch_add_rmsnorm_vec<TD, float, TY>(x, delta, planes, plane, gain.ptr, eps, y, rows, n_rows, hidden, squares, stream);
         else
-            launch_add_rmsnorm_vec<TD, bf16_t, TY>(x, delta, planes, plane, gain.ptr, eps, y, rows, n_rows, hidden, stream);
+            launch_add_rmsnorm_vec<TD, bf16_t, TY>(x, delta, planes, plane, gain.ptr, eps, y, rows, n_rows, hidden, squares, stream);
         return;
     }
     if (hidden > 512)
-        add_rmsnorm_kernel<TD, TY, 256><<<n_rows, 256, 0, stream>>>(x, static_cast<const TD*>(delta), planes, plane, gain, eps, static_cast<TY*>(y), rows, hidden);
+        add_rmsnorm_kernel<TD, TY, 256><<<n_rows, 256, 0, stream>>>(x, static_cast<const TD*>(delta), planes, plane, gain, eps, static_cast<TY*>(y), rows, hidden, squares);
     else
-        add_rmsnorm_kernel<TD, TY, 64><<<n_rows, 64, 0, stream>>>(x, static_cast<const TD*>(delta), planes, plane, gain, eps, static_cast<TY*>(y), rows, hidden);
+        add_rmsnorm_kernel<TD, TY, 64><<<n_rows, 64, 0, stream>>>(x, static_cast<const TD*>(delta), planes, plane, gain, eps, static_cast<TY*>(y), rows, hidden, squares);
 }
 
 extern "C" int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, int delta_planes, long delta_plane,
                                  const void* gain, int gain_dtype, float eps, void* y, int y_dtype, const int* rows,
-                                 int n_rows, int hidden, hipStream_t stream) {
+                                 int n_rows, int hidden, float* squares_out, hipStream_t stream) {
     if (check_dtype(delta_dtype, "add_rmsnorm delta") || check_dtype(gain_dtype, "add_rmsnorm gain") ||
         check_dtype(y_dtype, "add_rmsnorm output"))
         return 1;
@@ -561,13 +575,13 @@ extern "C" int leone_add_rmsnorm(float* x, const void* delta, int delta_dtype, i
     const long plane = delta_plane;
     AnyVec g{gain, gain_dtype};
     if (delta_dtype == kF32 && y_dtype == kF32)
-        launch_add_rmsnorm<float, float>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, stream);
+        launch_add_rmsnorm<float, float>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, squares_out, stream);
     else if (delta_dtype == kBF16 && y_dtype == kBF16)
-        launch_add_rmsnorm<bf16_t, bf16_t>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, stream);
+        launch_add_rmsnorm<bf16_t, bf16_t>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, squares_out, stream);
     else if (delta_dtype == kF32 && y_dtype == kBF16)
-        launch_add_rmsnorm<float, bf16_t>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, stream);
+        launch_add_rmsnorm<float, bf16_t>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, squares_out, stream);
     else
-        launch_add_rmsnorm<bf16_t, float>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, stream);
+        launch_add_rmsnorm<bf16_t, float>(x, delta, planes, plane, g, eps, y, rows, n_rows, hidden, squares_out, stream);
     LEONE_LAUNCH_CHECK("add_rmsnorm");
     return 0;
 }

@@ -89,14 +89,17 @@ def embed(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor]
 
 def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
-                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out: Optional[torch.Tensor] = None, prepare: bool = False):
     """x += delta, then y = rmsnorm(x) * gain; with ``rows``, y[i] comes from row rows[i] and x is not written.
     ``delta`` is [n, hidden] or a stack of planes [p, n, hidden] whose sum, taken in order, is meant (the
-    parts of a product whose inner dimension was cut, see ``linear``)."""
+    parts of a product whose inner dimension was cut, see ``linear``).  With ``prepare`` the norm is left for
+    the product that consumes it to finish: ``PreparedRows`` comes back (the operand x * gain, and the rows'
+    sums of squares), which rounds where the product with the norm folded in rounds."""
     n, hidden = x.shape
     n_out = n if rows is None else rows.numel()
     if out is None:
         out = torch.empty((n_out, hidden), dtype=out_dtype, device=x.device)
+    squares = torch.empty((n_out, -(-hidden // 16)), dtype=torch.float32, device=x.device) if prepare else None
     delta_code = _code(delta, "add_rmsnorm delta") if delta is not None else _CODES[out_dtype]
     stacked = delta is not None and delta.dim() == 3
     planes = delta.shape[0] if stacked else 1
@@ -107,8 +110,8 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tens
          n * hidden,
          _dev(gain, "add_rmsnorm gain", None, (hidden,)), _code(gain, "add_rmsnorm gain"), float(eps),
          _dev(out, "add_rmsnorm out", out_dtype, (n_out, hidden)), _CODES[out_dtype],
-         _dev(rows, "add_rmsnorm rows", torch.int32), n_out, hidden, _stream())
-    return out
+         _dev(rows, "add_rmsnorm rows", torch.int32), n_out, hidden, _dev(squares, "add_rmsnorm sums"), _stream())
+    return PreparedRows(x, gain, eps, out_dtype, out, squares, rows) if prepare else out
 
 
 def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -348,16 +351,21 @@ class NormedRows:
     def materialize(self) -> torch.Tensor:
         return add_rmsnorm(self.x, None, self.gain, self.eps, self.dtype, self.rows)
 
+    def prepare(self) -> "PreparedRows":
+        """The norm kernel runs, but leaves the scaling to the product (see ``add_rmsnorm``)."""
+        return add_rmsnorm(self.x, None, self.gain, self.eps, self.dtype, self.rows, prepare=True)
+
 
 class PreparedRows(NormedRows):
-    """A norm of the whole stream ``x`` whose operand the product before has left behind: ``operand`` is
-    bf16(x * gain), ``squares`` float32 ``[rows, ceil(hidden / 16)]`` partial sums of x^2, so that the
-    product that consumes it needs no norm kernel and no second read of the stream.  The stream itself is
+    """A norm of the stream ``x`` (of its rows ``rows``) whose operand lies ready: ``operand`` is
+    bf16(x * gain), ``squares`` float32 ``[rows, ceil(hidden / 16)]`` partial sums of x^2.  The product before
+    leaves them behind (``linear(..., next_norm=)``), so that the product that consumes them needs no norm
+    kernel and no second read of the stream; or the norm kernel does (``add_rmsnorm(..., prepare=True)``).  The stream itself is
     up to date: any other consumer normalises it in the usual way (``materialize``)."""
 
     def __init__(self, x: torch.Tensor, gain: torch.Tensor, eps: float, dtype: torch.dtype,
-                 operand: torch.Tensor, squares: torch.Tensor):
-        super().__init__(x, gain, eps, dtype, None)
+                 operand: torch.Tensor, squares: torch.Tensor, rows: Optional[torch.Tensor] = None):
+        super().__init__(x, gain, eps, dtype, rows)
         self.operand, self.squares = operand, squares
 
 
@@ -553,7 +561,7 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         # Every workgroup (16 weight rows) would redo a folded norm for its own use: that pays only for
         # matrices with few rows; for the others the norm kernel runs once and the product reads its result.
         if isinstance(x, NormedRows) and not isinstance(x, PreparedRows) and weight.shape[0] > FUSED_NORM_WEIGHT_ROWS:
-            x = x.materialize()
+            x = x.prepare()                   # rounds where the folded norm rounds, whatever the weight's size
         if next_norm is not None and (residual is None or weight.shape[0] % 8 or next_norm[2] != torch.bfloat16):
             next_norm = None
         return gemm_fused(x, weight, out_dtype, residual, gated, next_norm)

@@ -185,3 +185,39 @@ def test_q_and_k_norm_come_before_the_rotation_and_skip_v(tiny):
     # shifting every position by the same amount changes nothing: only distances count
     shifted = plain.attention_block(x, weights, "model.layers.0.self_attn", config, list(range(100, 106)))
     assert torch.allclose(shifted, base, atol=1e-8)
+
+
+def test_gate_is_the_activated_projection_by_numbers():
+    """silu goes on gate_proj's result, up_proj's multiplies it (crates/leone/src/cpu.rs:892-907 with the
+    operands of crates/leone/src/runtime.rs:9283-9319).  One input, one unit each: gate 2, up 3 gives
+    2 / (1 + e^-2) * 3 = 5.2847...; the other way round it would be 3 / (1 + e^-3) * 2 = 5.7154..."""
+    weights = {"f.gate_proj.weight": torch.tensor([[2.0]]), "f.up_proj.weight": torch.tensor([[3.0]]),
+               "f.down_proj.weight": torch.tensor([[1.0]])}
+    out = plain.feed_forward(torch.tensor([[1.0]]), weights, "f")
+    assert abs(float(out) - 5.284782467867294) < 1e-12
+    assert abs(float(out) - 5.715445096562234) > 0.4
+
+
+def test_head_norms_use_the_layer_norms_eps_by_numbers():
+    """q and k are normalised with rms_norm_eps (crates/leone/src/runtime.rs:9227-9241 passes the model's one
+    epsilon).  Activations small enough for eps to matter: q = (3e-3, 4e-3), mean square 1.25e-5, eps 1e-5:
+    q / sqrt(2.25e-5) = (0.63246, 0.84327); with another eps (1e-6) it would be (0.81650, 1.08866).  One head
+    of size 2, one position, so rotation by angle 0 and attention over one key change nothing: the output is v."""
+    config = dict(num_attention_heads=1, num_key_value_heads=1, head_dim=2, rms_norm_eps=1e-5, rope_theta=1e4)
+    eye = torch.eye(2)
+    weights = {"a.q_proj.weight": eye, "a.k_proj.weight": eye, "a.v_proj.weight": eye, "a.o_proj.weight": eye,
+               "a.q_norm.weight": torch.ones(2), "a.k_norm.weight": torch.ones(2)}
+    y = torch.tensor([[3e-3, 4e-3]])
+    normed = plain.rms_norm(y.view(1, 1, 2), weights["a.q_norm.weight"], config["rms_norm_eps"])
+    assert torch.allclose(normed.view(2), torch.tensor([0.6324555320336759, 0.8432740427115678], dtype=torch.float64), atol=1e-12)
+    # and through the block, two positions: the second attends both keys with weights that depend on q . k,
+    # which depends on that factor: softmax over (q1.k0, q1.k1) / sqrt(2)
+    y2 = torch.tensor([[3e-3, 4e-3], [4e-3, -3e-3]])
+    out = plain.attention_block(y2, weights, "a", config, [0, 0])       # both at position 0: no rotation
+    n0, n1 = [v / math.sqrt((v * v).sum() / 2 + 1e-5) for v in (y2[0].double(), y2[1].double())]
+    scores = torch.stack([n1 @ n0, n1 @ n1]) / math.sqrt(2)
+    w = torch.softmax(scores, dim=0)
+    assert torch.allclose(out[1], w[0] * y2[0].double() + w[1] * y2[1].double(), atol=1e-12)
+    wrong = [v / math.sqrt((v * v).sum() / 2 + 1e-6) for v in (y2[0].double(), y2[1].double())]
+    wrong_w = torch.softmax(torch.stack([wrong[1] @ wrong[0], wrong[1] @ wrong[1]]) / math.sqrt(2), dim=0)
+    assert (wrong_w - w).abs().max() > 0.02
