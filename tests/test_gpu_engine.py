@@ -374,3 +374,95 @@ def test_bfloat16_engine_against_the_oracle_that_rounds_where_it_rounds(tmp_path
     # the first position of a request sees one key, whose weight is exactly 1: only the other roundings are left there
     first = max(float(np.abs(got[rid][0] - expected[rid][0]).max()) for rid in requests)
     assert first <= 2e-3, f"{name}/{schedule}: first positions differ by {first:.2e}"
+
+
+# ---- the layer sizes of the large models ----------------------------------------------------------------
+_REAL_BASE = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", rope_theta=1000000.0, rms_norm_eps=1e-6,
+                  tie_word_embeddings=False, max_position_embeddings=1024, vocab_size=8200)
+REAL = {
+    # one and two layers of the 8B widths, one of the 32B head shape (64 query heads of 128 over a width of 5,120)
+    "8b-1": dict(_REAL_BASE, num_hidden_layers=1, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                 head_dim=128, intermediate_size=12288),
+    "8b-2": dict(_REAL_BASE, num_hidden_layers=2, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                 head_dim=128, intermediate_size=12288),
+    "32b-1": dict(_REAL_BASE, num_hidden_layers=1, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
+                  head_dim=128, intermediate_size=25600),
+}
+REAL_LENGTHS = {"8b-1": [150, 600], "8b-2": [300, 160], "32b-1": [200, 330]}
+REAL_SCHEDULES = dict(SCHEDULES, portions=lambda requests: schedules.portions(
+    requests, sizes=(10, 11, 64, 65, 128, 129, 2, 40)))      # both sides of every change of kernel
+
+
+@pytest.fixture(scope="module")
+def real_cases(tmp_path_factory):
+    cache = {}
+
+    def get(name):
+        if name not in cache:
+            folder = make_model_dir(str(tmp_path_factory.mktemp(f"real_{name}")), REAL[name], seed=71, dtype=torch.bfloat16)
+            config, weights = read_config(folder), read_weights(folder)
+            requests = {f"r{i}": random_tokens(100 * i + 9, n, config["vocab_size"]) for i, n in enumerate(REAL_LENGTHS[name])}
+            expected = {rid: qwen3_plain.forward(weights, config, toks).numpy() for rid, toks in requests.items()}
+            cache[name] = (folder, requests, expected, config, weights)
+        return cache[name]
+
+    return get
+
+
+@pytest.mark.parametrize("schedule", list(REAL_SCHEDULES))
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+@pytest.mark.parametrize("name", list(REAL))
+def test_layers_of_the_large_models_match_plain(real_cases, name, dtype_name, schedule):
+    """The widths at which the products' plans, the cuts of K and the changes of kernel at 10/11, 64/65 and
+    128/129 rows were chosen (crates/leone-cuda/tests/gpu.rs:653-711 tests at the model's own shapes).
+    Logits reach 7.5 here, so the bounds are taken relative to the largest logit: float32 as everywhere
+    (measured 4e-5), bfloat16 1.5 % for a single logit and 0.25 % on average (measured 0.9 % and 0.16 %)."""
+    from leone_amd import ops
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+
+    folder, requests, expected, config, weights = real_cases(name)
+    steps = REAL_SCHEDULES[schedule](requests)
+    engine = Engine(load_model(folder, dtype_name), num_pages=schedules.max_live_tokens(steps, round_to=64) // 64,
+                    page_tokens=64, max_requests=4, poison_freed=True)
+    outputs = run_steps(engine, steps)
+    scale = max(float(np.abs(v).max()) for v in expected.values())
+    assert scale > 3.0
+    if dtype_name == "float32":
+        compare(steps, outputs, expected, tolerance("float32"), f"{name}/float32/{schedule}")
+        return
+    compare(steps, outputs, expected, 1.5e-2 * scale, f"{name}/bfloat16/{schedule}")
+    got = schedules.collect(steps, outputs)
+    mean = np.mean([np.abs(np.stack(got[rid]) - expected[rid]).mean() for rid in requests])
+    assert mean <= 2.5e-3 * scale, f"{name}/{schedule}: mean difference {mean:.2e} of logits up to {scale:.2f}"
+    if schedule == "mixed":
+        from tests.plain import qwen3_rounded
+        sizes = qwen3_rounded.step_sizes(steps, requests)
+        rounded = {rid: qwen3_rounded.forward(weights, config, toks, sizes[rid][0], sizes[rid][1], ops.FUSED_ROWS,
+                                              ops.ROWS_MAX).numpy() for rid, toks in requests.items()}
+        mean = np.mean([np.abs(np.stack(got[rid]) - rounded[rid]).mean() for rid in requests])
+        assert mean <= 1e-3 * scale, f"{name}: mean difference from the rounding oracle {mean:.2e}"
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+@pytest.mark.parametrize("name", ["B", "M"])
+def test_twenty_live_requests_decoding_side_by_side(tmp_path, name, dtype_name):
+    """Up to twenty live requests, most of them decoding: steps of 11 to 30 rows of single tokens beside short
+    portions, which is where the multi-row weight-streaming products and the split-KV kernel serve many
+    requests at once; few pages, so that finished requests' pages are used again."""
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+
+    folder = make_model_dir(str(tmp_path / "m"), TINY[name], seed=81, dtype=DTYPES[dtype_name],
+                            sharpen=2.0 if dtype_name == "float32" else 1.0)
+    config, weights = read_config(folder), read_weights(folder)
+    gen = np.random.default_rng(5)
+    requests = {f"d{i}": random_tokens(900 + i, int(gen.integers(18, 60)), config["vocab_size"]) for i in range(30)}
+    expected = {rid: qwen3_plain.forward(weights, config, toks).numpy() for rid, toks in requests.items()}
+    steps = schedules.mixed(requests, max_live=20, prompt_fraction=0.3, sizes=(5, 2, 9, 3))
+    decode_rows = [sum(1 for e in s["entries"] if len(e["tokens"]) == 1) for s in steps]
+    assert max(decode_rows) >= 16 and sum(1 for n in decode_rows if n >= 11) >= 20
+    engine = Engine(load_model(folder, dtype_name), num_pages=schedules.max_live_tokens(steps, round_to=16) // 16,
+                    page_tokens=16, max_requests=20, poison_freed=True)
+    outputs = run_steps(engine, steps)
+    compare(steps, outputs, expected, tolerance(dtype_name), f"{name}/{dtype_name}/twenty live")
