@@ -58,7 +58,8 @@ class Runtime:
 
     def __init__(self, model, *, num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  page_tokens: int = 64, max_requests: int = 64, max_context: Optional[int] = None,
-                 policy: Optional[SchedulerPolicy] = None, tokenizer=None, graphs: bool = True):
+                 policy: Optional[SchedulerPolicy] = None, tokenizer=None, graphs: bool = True,
+                 poison_freed: bool = False):
         self.model = model
         self.config = getattr(model, "config", None)
         context = min(max_context or model.spec.max_positions, model.spec.max_positions)
@@ -68,7 +69,8 @@ class Runtime:
                             if hasattr(need, "kv_heads"))
             num_pages = default_num_pages(model, page_tokens, max_requests, context, per_token)
         self.engine = Engine(model, num_pages=num_pages, max_tokens=max_tokens, page_tokens=page_tokens,
-                             max_requests=max_requests, max_context=context, graphs=graphs)
+                             max_requests=max_requests, max_context=context, graphs=graphs,
+                             poison_freed=poison_freed)
         self.policy = policy or SchedulerPolicy(max_live_requests=max_requests)
         self.tokenizer = tokenizer
         self.last_stats: Optional[GenerationStats] = None

@@ -201,6 +201,17 @@ class CacheManager:
     def shared_pages(self, group: int) -> int:
         return self._checked(self._lib.leone_cache_shared_pages(self.handle, group))
 
+    def log_freed(self, on: bool = True) -> None:
+        """Has the manager note every page whose last holder lets go, whoever frees it (``drain_freed``)."""
+        self._checked(self._lib.leone_cache_log_freed(self.handle, 1 if on else 0))
+
+    def drain_freed(self, group: int) -> List[int]:
+        """Pages of ``group`` that became free since the last call (the log must be on); some may have been
+        handed out again already, to a holder that has not written them yet."""
+        buffer = (c_int * self.groups[group].num_pages)()
+        n = self._checked(self._lib.leone_cache_drain_freed(self.handle, group, buffer, self.groups[group].num_pages))
+        return list(buffer[:n])
+
     @property
     def pages_high_water(self) -> List[int]:
         return [self._lib.leone_cache_high_water(self.handle, g) for g in range(len(self.groups))]

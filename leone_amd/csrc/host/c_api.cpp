@@ -149,6 +149,24 @@ int leone_cache_shared_pages(void* cache, int group) {
 int leone_cache_high_water(void* cache, int group) {
     return guarded([&]() -> long { return cache_of(cache).pages_high_water(group); });
 }
+int leone_cache_log_freed(void* cache, int on) {
+    return guarded([&]() -> long {
+        cache_of(cache).log_freed(on != 0);
+        return 0;
+    });
+}
+int leone_cache_drain_freed(void* cache, int group, int* out, int capacity) {
+    return guarded([&]() -> long {
+        // nothing is taken off the log unless it fits: a caller with too little room asks again
+        CacheManager& manager = cache_of(cache);
+        std::vector<int> pages = manager.drain_freed(group);
+        if (static_cast<long>(pages.size()) > capacity || (!out && !pages.empty()))
+            throw CacheError("the freed pages of group " + std::to_string(group) + " need room for " +
+                             std::to_string(pages.size()) + " entries");
+        for (size_t i = 0; i < pages.size(); ++i) out[i] = pages[i];
+        return static_cast<long>(pages.size());
+    });
+}
 int leone_cache_max_blocks(void* cache, int group) {
     return guarded([&]() -> long { return cache_of(cache).max_blocks(group); });
 }

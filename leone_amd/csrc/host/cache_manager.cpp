@@ -104,7 +104,24 @@ void CacheManager::drop(int g, int page) {
     if (refs_[g][page] <= 0)
         throw CacheError("group " + std::to_string(g) + ": page " + std::to_string(page) +
                          " is given back more often than it was taken");
-    if (--refs_[g][page] == 0) free_[g].push_back(page);
+    if (--refs_[g][page] == 0) {
+        free_[g].push_back(page);
+        if (log_freed_) freed_log_[g].push_back(page);
+    }
+}
+
+void CacheManager::log_freed(bool on) {
+    log_freed_ = on;
+    freed_log_.assign(groups_.size(), {});
+}
+
+std::vector<int> CacheManager::drain_freed(int g) {
+    if (g < 0 || g >= group_count()) throw CacheError("no cache group " + std::to_string(g));
+    std::vector<int> out;
+    if (log_freed_) out.swap(freed_log_[g]);
+    std::sort(out.begin(), out.end());
+    out.erase(std::unique(out.begin(), out.end()), out.end());      // a page freed twice since is one page
+    return out;
 }
 
 int CacheManager::fork(RequestKey parent, RequestKey child, int tokens) {

@@ -75,6 +75,11 @@ public:
     int holders(int g, int page) const { return refs_.at(g).at(page); }
     int shared_pages(int g) const;
     int pages_high_water(int g) const { return high_water_.at(g); }
+    // With the log switched on, every page whose last holder lets go is noted (whoever frees it: release,
+    // a window that has passed, a rollback, a truncation); drain_freed hands the notes out and clears them.
+    // For a caller that wants to overwrite what freed pages hold before anyone gets them again.
+    void log_freed(bool on);
+    std::vector<int> drain_freed(int g);
     // New pages each group must map to append `tokens` to `request` now.
     std::vector<int> pages_needed(RequestKey request, int tokens) const;
 
@@ -118,6 +123,8 @@ private:
     std::vector<int> free_slots_;
     std::vector<std::vector<int>> refs_;    // holders of every page
     std::vector<int> high_water_;
+    bool log_freed_ = false;
+    std::vector<std::vector<int>> freed_log_;
     std::unordered_map<RequestKey, Request> requests_;
 };
 

@@ -45,6 +45,8 @@ int leone_cache_free_slot_list(void* cache, int* out, int capacity);
 int leone_cache_holders(void* cache, int group, int page);
 int leone_cache_shared_pages(void* cache, int group);
 int leone_cache_high_water(void* cache, int group);
+int leone_cache_log_freed(void* cache, int on);                                       // note pages as they become free
+int leone_cache_drain_freed(void* cache, int group, int* out, int capacity);          // the notes so far; clears them
 int leone_cache_max_blocks(void* cache, int group);
 void leone_cache_shortage(int* group, int* needed, int* free);   // of the last LEONE_HOST_OUT_OF_PAGES
 

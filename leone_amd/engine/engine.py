@@ -164,7 +164,12 @@ class Engine:
             num_pages = (max_tokens + page_tokens - 1) // page_tokens
         self.pools = DevicePools(model.cache_needs(), self.dtype, self.device, num_pages, page_tokens, max_requests)
         self.cache = CacheManager(self.pools.group_specs, max_requests, self.max_context)
+        # With poison_freed every page is filled with NaN when its last holder lets go of it, whoever frees it
+        # (this engine, a scheduler on the same cache manager, a window that has passed): the manager notes
+        # such pages and they are overwritten before the next kernel runs.
         self.poison_freed = poison_freed
+        if poison_freed:
+            self.cache.log_freed(True)
         self.vocab_size = model.spec.vocab_size
         # Steps of single decoded tokens are recorded once per batch size and replayed.
         self.graphs = bool(graphs) and model.graph_safe
@@ -179,12 +184,15 @@ class Engine:
         return slot
 
     def release(self, request: Hashable) -> None:
-        if self.poison_freed:
-            tables = [list(self.cache.table(request, g)) for g in range(len(self.cache.groups))]
         self.cache.release(request)
+        self.poison_freed_pages()
+
+    def poison_freed_pages(self) -> None:
+        """Overwrites the pages that became free since the last call (nothing unless ``poison_freed``).  A page
+        that was handed out again meanwhile has not been written by its new holder: no kernel ran in between."""
         if self.poison_freed:
-            for g, table in enumerate(tables):
-                self.pools.poison_pages(g, [p for p in table if p >= 0 and self.cache.holders(g, p) == 0])
+            for g in range(len(self.cache.groups)):
+                self.pools.poison_pages(g, self.cache.drain_freed(g))
 
     def length(self, request: Hashable) -> int:
         return self.cache.length(request)
@@ -248,6 +256,7 @@ class Engine:
 
     def run_reserved(self, entries: Sequence[StepEntry]) -> StepOutput:
         """Runs a step whose pages the caller has reserved; commits on success, rolls back on failure."""
+        self.poison_freed_pages()              # what a scheduler on the same manager has freed since the last step
         try:
             for e in entries:
                 if self.cache.length(e.request) == 0:
@@ -264,19 +273,9 @@ class Engine:
                 if self.cache.has(e.request):
                     self.cache.rollback(e.request)
             raise
-        freed_before = None
-        if self.poison_freed:
-            freed_before = [[list(self.cache.table(e.request, g)) for g in range(len(self.cache.groups))]
-                            for e in entries]
         for e in entries:
             self.cache.commit(e.request, len(e.tokens))
-        if self.poison_freed:
-            for e, before in zip(entries, freed_before):
-                for g, old in enumerate(before):
-                    new = self.cache.table(e.request, g)
-                    gone = [p for b, p in enumerate(old)
-                            if p >= 0 and (b >= len(new) or new[b] != p) and self.cache.holders(g, p) == 0]
-                    self.pools.poison_pages(g, gone)
+        self.poison_freed_pages()              # pages a window has passed
         return StepOutput(logits, rows)
 
     def _run_decode_graph(self, entries: Sequence[StepEntry]):

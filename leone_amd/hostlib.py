@@ -47,6 +47,8 @@ _PROTOTYPES = {
     "leone_cache_holders": (c_int, [H, c_int, c_int]),
     "leone_cache_shared_pages": (c_int, [H, c_int]),
     "leone_cache_high_water": (c_int, [H, c_int]),
+    "leone_cache_log_freed": (c_int, [H, c_int]),
+    "leone_cache_drain_freed": (c_int, [H, c_int, PI, c_int]),
     "leone_cache_max_blocks": (c_int, [H, c_int]),
     "leone_cache_shortage": (None, [PI, PI, PI]),
     "leone_scheduler_create": (H, [H, PI64]),

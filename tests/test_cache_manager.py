@@ -234,3 +234,45 @@ def test_random_orders_with_forks(seed):
         m.release(rid)
     m.check()
     assert m.free_pages(0) == 30 and m.shared_pages(0) == 0
+
+
+def test_the_log_of_freed_pages_names_every_page_whoever_frees_it():
+    """With the log on, release, rollback, truncation and a window that has passed all leave their pages in
+    it, once each; a shared page only when its last holder lets go; nothing while the log is off."""
+    m = CacheManager([GroupSpec(12, 4), GroupSpec(12, 4, window=6)], max_requests=4, max_context=64)
+    m.admit("a")
+    m.reserve("a", 10)
+    m.commit("a")
+    m.release("a")
+    assert m.drain_freed(0) == [] and m.drain_freed(1) == []           # off
+    m.log_freed(True)
+    m.admit("b")
+    m.reserve("b", 9)
+    table0 = [p for p in m.table("b", 0) if p >= 0]
+    m.rollback("b")
+    assert sorted(m.drain_freed(0)) == sorted(table0) and len(m.drain_freed(1)) == len(table0)
+    m.reserve("b", 13)
+    before = list(m.table("b", 1))
+    m.commit("b")                                                       # the window of 6 has passed the first pages
+    after = m.table("b", 1)
+    passed = [p for b, p in enumerate(before) if p >= 0 and after[b] < 0]
+    assert passed and sorted(m.drain_freed(1)) == sorted(passed) and m.drain_freed(0) == []
+    m.release("b")
+    m.check()
+    assert m.free_pages(0) == 12 and m.free_pages(1) == 12
+    # a shared page is named only when its last holder lets go
+    m = CacheManager([GroupSpec(12, 4)], max_requests=4, max_context=64)
+    m.log_freed(True)
+    m.admit("b")
+    m.reserve("b", 13)
+    m.commit("b")
+    m.fork("b", "c", 8)
+    shared = [p for p in m.table("c", 0) if p >= 0]
+    held = [p for p in m.table("b", 0) if p >= 0]
+    assert len(shared) == 2
+    m.release("b")
+    assert sorted(m.drain_freed(0)) == sorted(set(held) - set(shared))     # the child still holds the shared ones
+    m.release("c")
+    assert sorted(m.drain_freed(0)) == sorted(shared)
+    assert m.drain_freed(0) == []                                          # drained
+    m.check()

@@ -466,3 +466,38 @@ def test_twenty_live_requests_decoding_side_by_side(tmp_path, name, dtype_name):
                     page_tokens=16, max_requests=20, poison_freed=True)
     outputs = run_steps(engine, steps)
     compare(steps, outputs, expected, tolerance(dtype_name), f"{name}/{dtype_name}/twenty live")
+
+
+@pytest.mark.parametrize("name", ["A", "B", "D"])
+def test_many_groups_of_prompt_tiles_at_few_heads(tmp_path, name):
+    """Four prompt portions of 40 tokens in one step (a group of tiles each), then a prompt of 420 tokens whole
+    (four groups of one request), at 4, 6 and 2 query heads: head counts at which the prompt kernel's numbering
+    of workgroups by die once left heads out.  bfloat16 with sharpened scores against the oracle that rounds
+    where the engine rounds (a width that is no multiple of 8 takes other kernels: against the plain one)."""
+    from leone_amd import ops
+    from leone_amd.engine.engine import Engine, StepEntry
+    from leone_amd.runtime import load_model
+    from tests.plain import qwen3_rounded
+
+    raw = dict(TINY[name], max_position_embeddings=512)
+    runs_of_8 = raw["hidden_size"] % 8 == 0  # the oracle knows the roundings of the 16-byte-run kernels only
+    folder = make_model_dir(str(tmp_path / "m"), raw, seed=91, dtype=torch.bfloat16, sharpen=2.0 if runs_of_8 else 1.0)
+    config, weights = read_config(folder), read_weights(folder)
+    requests = {f"g{i}": random_tokens(40 + i, 40, config["vocab_size"]) for i in range(4)}
+    requests["long"] = random_tokens(50, 420, config["vocab_size"])
+    steps = [{"step": 0, "entries": [{"id": f"g{i}", "tokens": requests[f"g{i}"], "want": list(range(40))} for i in range(4)],
+              "end": [f"g{i}" for i in range(4)]},
+             {"step": 1, "entries": [{"id": "long", "tokens": requests["long"], "want": list(range(420))}], "end": ["long"]}]
+    engine = Engine(load_model(folder, "bfloat16"), max_tokens=448, page_tokens=16, max_requests=4, poison_freed=True)
+    outputs = run_steps(engine, steps)
+    if not runs_of_8:
+        expected = {rid: qwen3_plain.forward(weights, config, toks).numpy() for rid, toks in requests.items()}
+        compare(steps, outputs, expected, tolerance("bfloat16"), f"{name}/groups of tiles")
+        return
+    sizes = qwen3_rounded.step_sizes(steps, requests)
+    rounded = {rid: qwen3_rounded.forward(weights, config, toks, sizes[rid][0], sizes[rid][1], ops.FUSED_ROWS,
+                                          ops.ROWS_MAX).numpy() for rid, toks in requests.items()}
+    compare(steps, outputs, rounded, ROUNDED_MAX[name], f"{name}/groups of tiles")
+    got = schedules.collect(steps, outputs)
+    mean = np.mean([np.abs(np.stack(got[rid]) - rounded[rid]).mean() for rid in requests])
+    assert mean <= ROUNDED_MEAN[name], f"{name}: mean difference from the rounding oracle {mean:.2e}"
