@@ -1,76 +1,87 @@
-"""Device storage behind the cache manager: key/value pages per group, state per slot."""
+"""Device storage behind the cache manager: pages per group, state per slot."""
 from __future__ import annotations
 
 from typing import Dict, List, Union
 
 import torch
 
-from ..parts.base import KvNeed, StateNeed
-from ..parts.context import CacheView, KvCacheView, StateCacheView
+from ..parts.context import CacheView
 from .manager import GroupSpec
 
 
 class DevicePools:
     """Allocates, once, the tensors that layer runs read and write.
 
-    Cache slots with the same key/value need (heads, head size, window) form one
-    group and share page ids and block tables; each slot has its own key and
-    value tensor, packed in runs of 8 (keys ``[pages, kv_heads, head_dim/8, page_tokens, 8]``,
-    values ``[pages, kv_heads, page_tokens/8, head_dim, 8]``).  A slot with a state
-    need gets ``[max_requests, *shape]``.
+    What a cache slot holds is its need's affair (``parts/base.py``: ``KvNeed``, ``StateNeed``, or any class
+    with the same methods): the pools only sort the slots.  Paged needs with the same ``group_key()`` form one
+    group and share page ids and block tables, each slot with storage of its own; a group's pages hold
+    the need's ``page_tokens`` tokens, or the engine's if it names none.  The other needs get storage per
+    request slot.
     """
 
     def __init__(self, needs: Dict[int, object], dtype: torch.dtype, device, num_pages: Union[int, Dict[int, int]],
                  page_tokens: int, max_requests: int):
         self.dtype, self.device = dtype, torch.device(device)
         self.page_tokens = page_tokens
-        self.group_needs: List[KvNeed] = []
+        self.needs = dict(needs)
+        self.group_needs: List[object] = []
         self.group_of_slot: Dict[int, int] = {}
-        self.kv: Dict[int, tuple] = {}
-        self.state: Dict[int, torch.Tensor] = {}
+        self.paged: Dict[int, object] = {}        # slot -> storage of a paged need
+        self.state: Dict[int, object] = {}        # slot -> storage of a per-request need
         for slot in sorted(needs):
             need = needs[slot]
-            if isinstance(need, KvNeed):
-                if need not in self.group_needs:
+            if not hasattr(need, "paged"):
+                raise TypeError(f"cache slot {slot}: {need!r} is no cache need (see parts/base.py)")
+            if need.paged:
+                key = need.group_key()
+                if key not in [n.group_key() for n in self.group_needs]:
                     self.group_needs.append(need)
-                self.group_of_slot[slot] = self.group_needs.index(need)
-            elif isinstance(need, StateNeed):
-                self.state[slot] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=self.device)
+                self.group_of_slot[slot] = [n.group_key() for n in self.group_needs].index(key)
             else:
-                raise TypeError(f"cache slot {slot}: unknown need {need!r}")
+                self.state[slot] = need.allocate_slots(max_requests, self.device)
         self.group_specs: List[GroupSpec] = []
         for gi, need in enumerate(self.group_needs):
             pages = num_pages[gi] if isinstance(num_pages, dict) else num_pages
-            self.group_specs.append(GroupSpec(pages, page_tokens, need.window))
+            self.group_specs.append(GroupSpec(pages, getattr(need, "page_tokens", None) or page_tokens,
+                                              getattr(need, "window", None)))
         for slot, gi in self.group_of_slot.items():
-            need, pages = self.group_needs[gi], self.group_specs[gi].num_pages
-            # keys [page][head][element / 8][token][8]; values [page][head][token / 8][element][8]
-            if need.head_dim % 8 or page_tokens % 8:
-                raise ValueError(f"the cache packs runs of 8: head_dim {need.head_dim} and page_tokens "
-                                 f"{page_tokens} must be multiples of 8")
-            self.kv[slot] = (torch.zeros((pages, need.kv_heads, need.head_dim // 8, page_tokens, 8), dtype=dtype,
-                                         device=self.device),
-                             torch.zeros((pages, need.kv_heads, page_tokens // 8, need.head_dim, 8), dtype=dtype,
-                                         device=self.device))
+            spec = self.group_specs[gi]
+            self.paged[slot] = needs[slot].allocate(spec.num_pages, spec.page_tokens, dtype, self.device)
+
+    @property
+    def kv(self) -> Dict[int, tuple]:
+        """slot -> (key pool, value pool) of the slots whose need is a ``KvNeed``."""
+        return {slot: storage for slot, storage in self.paged.items() if isinstance(storage, tuple) and len(storage) == 2}
 
     def bytes_per_token(self) -> int:
         size = torch.empty((), dtype=self.dtype).element_size()
-        return sum(2 * self.group_needs[g].kv_heads * self.group_needs[g].head_dim * size
-                   for g in self.group_of_slot.values())
+        return sum(self.needs[slot].bytes_per_token(size) for slot in self.group_of_slot)
 
     def views(self, block_tables: Dict[int, torch.Tensor]) -> Dict[int, CacheView]:
         out: Dict[int, CacheView] = {}
         for slot, gi in self.group_of_slot.items():
-            k, v = self.kv[slot]
-            out[slot] = KvCacheView(writes=True, k_pool=k, v_pool=v, block_table=block_tables[gi],
-                                    page_tokens=self.page_tokens)
-        for slot, tensor in self.state.items():
-            out[slot] = StateCacheView(writes=True, state=tensor)
+            out[slot] = self.needs[slot].view(self.paged[slot], block_tables[gi], self.group_specs[gi].page_tokens)
+        for slot, storage in self.state.items():
+            out[slot] = self.needs[slot].view(storage)
         return out
 
     def zero_state(self, slot_index: int) -> None:
-        for tensor in self.state.values():
-            tensor[slot_index].zero_()
+        for slot, storage in self.state.items():
+            self.needs[slot].zero(storage, slot_index)
+
+    def snapshot_state(self, slot_indices: List[int]):
+        """What the per-request storage of these request slots holds, to be put back by ``restore_state``."""
+        if not self.state:
+            return None
+        index = torch.tensor(sorted(set(slot_indices)), dtype=torch.long, device=self.device)
+        return index, {slot: self.needs[slot].snapshot(storage, index) for slot, storage in self.state.items()}
+
+    def restore_state(self, saved) -> None:
+        if saved is None:
+            return
+        index, kept = saved
+        for slot, value in kept.items():
+            self.needs[slot].restore(self.state[slot], index, value)
 
     def poison_pages(self, group: int, pages: List[int]) -> None:
         """Fills pages with NaN so that a read of a page that was given back shows up."""
@@ -79,5 +90,4 @@ class DevicePools:
         index = torch.tensor(pages, dtype=torch.long, device=self.device)
         for slot, gi in self.group_of_slot.items():
             if gi == group:
-                for pool in self.kv[slot]:
-                    pool.index_fill_(0, index, float("nan"))
+                self.needs[slot].poison(self.paged[slot], index)

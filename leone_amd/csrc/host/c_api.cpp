@@ -326,17 +326,23 @@ long leone_step_pack(void* cache, int n_entries, const int64_t* requests, const 
             token_at += std::max(counts[i], 0);
             want_at += std::max(want_counts[i], 0);
         }
-        const StepShape step_shape{shape[0], shape[1], shape[2], shape[3] != 0, shape[4]};
-        if (step_shape.tile_rows <= 0 || step_shape.group_tiles <= 0)
-            throw std::invalid_argument("step_pack: tile_rows and group_tiles must be positive");
+        // shape: vocabulary, all rows wanted, number of tilings, then (tile_rows, min_rows, group_tiles) of each
+        StepShape step_shape{shape[0], shape[1] != 0, {}};
+        if (shape[2] < 0 || shape[2] > 16) throw std::invalid_argument("step_pack: at most 16 tilings");
+        for (int i = 0; i < shape[2]; ++i) {
+            const RowTiling t{shape[3 + 3 * i], shape[4 + 3 * i], shape[5 + 3 * i]};
+            if (t.tile_rows <= 0 || t.group_tiles <= 0 || t.min_rows <= 0)
+                throw std::invalid_argument("step_pack: tile_rows, min_rows and group_tiles must be positive");
+            step_shape.tilings.push_back(t);
+        }
         const StepSections layout = step_sections(manager, entries, step_shape);
         std::copy(layout.offsets.begin(), layout.offsets.end(), sections);
         if (!out || capacity < layout.total()) return layout.total();
         std::vector<PlacedEntry> where;
         const StepSummary s = pack_step(manager, entries, step_shape, layout, out, where);
-        if (summary) {
-            summary[0] = s.rows, summary[1] = s.prefill_rows, summary[2] = s.max_position;
-            summary[3] = s.tiles, summary[4] = s.wanted, summary[5] = s.decode_only ? 1 : 0;
+        if (summary) {   // rows, largest position, wanted rows, decode only, then (rows, tiles) of each tiling
+            summary[0] = s.rows, summary[1] = s.max_position, summary[2] = s.wanted, summary[3] = s.decode_only ? 1 : 0;
+            for (size_t i = 0; i < s.tiled.size(); ++i) summary[4 + 2 * i] = s.tiled[i].rows, summary[5 + 2 * i] = s.tiled[i].tiles;
         }
         if (placed)
             for (int i = 0; i < n_entries; ++i) {

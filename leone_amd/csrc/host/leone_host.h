@@ -83,10 +83,11 @@ int leone_scheduler_events(void* scheduler, int first, int count, int* kinds, in
 void leone_scheduler_stats(void* scheduler, int64_t* out15);
 
 // ---- step layout.  Entries are given flat: request, token count and wanted count per entry, then
-// all tokens and all wanted places in entry order.  shape: vocab_size, tile_rows, min_tile_rows,
-// all_rows_wanted, group_tiles.  Returns the words the packed step takes; writes nothing but `sections`
-// (7 + groups offsets) if `capacity` is smaller.  summary: rows, prefill_rows, max_position, tiles,
-// wanted, decode_only.  placed: per entry in running order given_index, slot, first_row, count, start.
+// all tokens and all wanted places in entry order.  shape: vocab_size, all_rows_wanted, the number of
+// row tilings, then (tile_rows, min_rows, group_tiles) of each.  Returns the words the packed step takes;
+// writes nothing but `sections` (6 + tilings + groups offsets) if `capacity` is smaller.  summary: rows,
+// max_position, wanted, decode_only, then (tiled rows, tiles) of each tiling.  placed: per entry in running
+// order given_index, slot, first_row, count, start.
 long leone_step_pack(void* cache, int n_entries, const int64_t* requests, const int* counts, const int* want_counts,
                      const int32_t* tokens, const int32_t* wants, const int* shape, int32_t* out, long capacity,
                      long* sections, int* summary, int* placed);

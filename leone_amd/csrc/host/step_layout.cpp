@@ -8,12 +8,22 @@ namespace leone::host {
 
 namespace {
 
-bool tiled(const StepEntryView& e, const StepShape& shape) { return !shape.all_rows_wanted && e.count >= shape.min_tile_rows; }
+bool tiled(const StepEntryView& e, const StepShape& shape, const RowTiling& t) {
+    return !shape.all_rows_wanted && e.count >= t.min_rows;
+}
+
+// How many of the tilings cut this entry: thresholds nest, so the entries a tiling cuts are those that reach
+// a certain number.
+int tilings_met(const StepEntryView& e, const StepShape& shape) {
+    int met = 0;
+    for (const RowTiling& t : shape.tilings) met += tiled(e, shape, t) ? 1 : 0;
+    return met;
+}
 
 // Places the tiles of a portion of `count` rows take: whole groups.
-long tile_places(int count, const StepShape& shape) {
-    const long tiles = (count + shape.tile_rows - 1) / shape.tile_rows;
-    return (tiles + shape.group_tiles - 1) / shape.group_tiles * shape.group_tiles;
+long tile_places(int count, const RowTiling& t) {
+    const long tiles = (count + t.tile_rows - 1) / t.tile_rows;
+    return (tiles + t.group_tiles - 1) / t.group_tiles * t.group_tiles;
 }
 
 void check(const std::vector<StepEntryView>& entries, const StepShape& shape) {
@@ -37,16 +47,19 @@ void check(const std::vector<StepEntryView>& entries, const StepShape& shape) {
 }  // namespace
 
 StepSections step_sections(const CacheManager& cache, const std::vector<StepEntryView>& entries, const StepShape& shape) {
-    long rows = 0, wanted = 0, tiles = 0;
+    long rows = 0, wanted = 0;
+    std::vector<long> tiles(shape.tilings.size(), 0);
     for (const StepEntryView& e : entries) {
         rows += e.count;
         wanted += e.want_count;
-        if (tiled(e, shape)) tiles += tile_places(e.count, shape);
+        for (size_t i = 0; i < shape.tilings.size(); ++i)
+            if (tiled(e, shape, shape.tilings[i])) tiles[i] += tile_places(e.count, shape.tilings[i]);
     }
     if (shape.all_rows_wanted) wanted = rows;
     const long n = static_cast<long>(entries.size());
     StepSections s;
-    s.offsets = {0, rows, 2 * rows, 3 * rows, 3 * rows + n, 3 * rows + n + wanted, 3 * rows + n + wanted + 3 * tiles};
+    s.offsets = {0, rows, 2 * rows, 3 * rows, 3 * rows + n, 3 * rows + n + wanted};
+    for (long count : tiles) s.offsets.push_back(s.offsets.back() + 3 * count);
     for (int g = 0; g < cache.group_count(); ++g) s.offsets.push_back(s.offsets.back() + n * cache.max_blocks(g));
     return s;
 }
@@ -60,19 +73,21 @@ StepSummary pack_step(const CacheManager& cache, const std::vector<StepEntryView
     std::vector<int> order(n);
     for (int i = 0; i < n; ++i) order[i] = i;
     std::stable_sort(order.begin(), order.end(),
-                     [&](int a, int b) { return tiled(entries[a], shape) && !tiled(entries[b], shape); });
+                     [&](int a, int b) { return tilings_met(entries[a], shape) > tilings_met(entries[b], shape); });
 
     std::int32_t* tokens = out + sections.offsets[0];
     std::int32_t* positions = out + sections.offsets[1];
     std::int32_t* row_entry = out + sections.offsets[2];
     std::int32_t* slots = out + sections.offsets[3];
     std::int32_t* want_rows = out + sections.offsets[4];
-    std::int32_t* tiles = out + sections.offsets[5];
+    const int n_tilings = static_cast<int>(shape.tilings.size());
+    const int first_table = 5 + n_tilings;          // index of the first block table's offset
 
     StepSummary summary;
+    summary.tiled.assign(n_tilings, TiledRows{});
     placed.assign(n, PlacedEntry{});
     std::vector<int> first_row(n, 0);
-    int row = 0, tile = 0;
+    int row = 0;
     for (int ei = 0; ei < n; ++ei) {
         const StepEntryView& e = entries[order[ei]];
         const int start = cache.length(e.request);
@@ -86,23 +101,27 @@ StepSummary pack_step(const CacheManager& cache, const std::vector<StepEntryView
         for (int g = 0; g < cache.group_count(); ++g) {
             const std::vector<int>& table = cache.table(e.request, g);
             const int width = cache.max_blocks(g);
-            std::int32_t* dst = out + sections.offsets[6 + g] + static_cast<long>(ei) * width;
+            std::int32_t* dst = out + sections.offsets[first_table + g] + static_cast<long>(ei) * width;
             const int held = std::min<int>(width, static_cast<int>(table.size()));
             std::copy(table.begin(), table.begin() + held, dst);
             std::fill(dst + held, dst + width, -1);
         }
-        if (tiled(e, shape)) {
-            const int n_tiles = (e.count + shape.tile_rows - 1) / shape.tile_rows;
-            const long places = tile_places(e.count, shape);
+        for (int ti = 0; ti < n_tilings; ++ti) {
+            const RowTiling& t = shape.tilings[ti];
+            if (!tiled(e, shape, t)) continue;
+            std::int32_t* tiles = out + sections.offsets[5 + ti];
+            int& tile = summary.tiled[ti].tiles;
+            const int n_tiles = (e.count + t.tile_rows - 1) / t.tile_rows;
+            const long places = tile_places(e.count, t);
             for (long index = 0; index < places; ++index) {
                 const bool used = index < n_tiles;
-                const int at = static_cast<int>(index) * shape.tile_rows;
+                const int at = static_cast<int>(index) * t.tile_rows;
                 tiles[3 * tile] = ei;
                 tiles[3 * tile + 1] = used ? row + at : row;
-                tiles[3 * tile + 2] = used ? std::min(shape.tile_rows, e.count - at) : 0;
+                tiles[3 * tile + 2] = used ? std::min(t.tile_rows, e.count - at) : 0;
                 ++tile;
             }
-            summary.prefill_rows = row + e.count;
+            summary.tiled[ti].rows = row + e.count;
         }
         if (e.count != 1) summary.decode_only = false;
         summary.max_position = std::max(summary.max_position, start + e.count - 1);
@@ -117,7 +136,6 @@ StepSummary pack_step(const CacheManager& cache, const std::vector<StepEntryView
             for (int w = 0; w < entries[i].want_count; ++w) want_rows[wanted++] = first_row[i] + entries[i].want[w];
     }
     summary.rows = row;
-    summary.tiles = tile;
     summary.wanted = wanted;
     return summary;
 }

@@ -24,7 +24,7 @@ from .. import hostlib, ops
 from ..ops import profile
 from ..cache.manager import CacheManager
 from ..cache.pools import DevicePools
-from ..parts.context import EntryInfo, StepContext
+from ..parts.context import TiledRows, EntryInfo, StepContext
 from ..parts.model import DecoderModel
 
 
@@ -47,12 +47,14 @@ class StepError(ValueError):
 
 class PackedStep:
     """One step's metadata as the native layout routine wrote it into a host buffer (int32 words):
-    tokens, positions, row -> entry, state slots, wanted rows, query tiles, one block table per cache group."""
+    tokens, positions, row -> entry, state slots, wanted rows, one tile list per row tiling, one block table
+    per cache group."""
 
     def __init__(self, cache: CacheManager, vocab_size: int, entries: Sequence[StepEntry], all_rows_wanted: bool = False,
-                 host=None):
+                 host=None, tilings: Sequence = ()):
         """``host``: nothing (a buffer is made), a buffer to write into (it must be large enough), or a
-        callable that is given the number of words and returns one."""
+        callable that is given the number of words and returns one.  ``tilings``: the ``RowTiling`` of the
+        model's parts; each gets a tile list."""
         n = len(entries)
         lib = hostlib.library()
         requests = (c_int64 * max(1, n))()
@@ -77,10 +79,11 @@ class PackedStep:
         if wants.size and (wants.min() < limit.min or wants.max() > limit.max):
             raise StepError("a wanted place lies outside its entry")
         tokens, wants = tokens.astype(np.int32), wants.astype(np.int32)
-        shape = (c_int * 5)(vocab_size, ops.PREFILL_TILE_ROWS, ops.PREFILL_MIN_ROWS, int(all_rows_wanted),
-                            ops.PREFILL_GROUP_TILES)
-        sections = (c_long * (7 + len(cache.groups)))()
-        summary, placed = (c_int * 6)(), (c_int * (5 * max(1, n)))()
+        tilings = list(tilings)
+        flat = [v for t in tilings for v in (t.tile_rows, t.min_rows, t.group_tiles)]
+        shape = (c_int * (3 + len(flat)))(vocab_size, int(all_rows_wanted), len(tilings), *flat)
+        sections = (c_long * (6 + len(tilings) + len(cache.groups)))()
+        summary, placed = (c_int * (4 + 2 * len(tilings)))(), (c_int * (5 * max(1, n)))()
         as_i32 = lambda a: a.ctypes.data_as(hostlib.PI32)
         args = (cache.handle, n, requests, counts, want_counts, as_i32(tokens), as_i32(wants), shape)
         total = lib.leone_step_pack(*args, None, 0, sections, None, None)
@@ -98,8 +101,11 @@ class PackedStep:
         self.host = host
         self.total = int(total)
         self.offsets = list(sections)
-        self.rows, self.prefill_rows, self.max_position, self.tiles, self.wanted = list(summary)[:5]
-        self.decode_only = bool(summary[5])
+        self.rows, self.max_position, self.wanted = summary[0], summary[1], summary[2]
+        self.decode_only = bool(summary[3])
+        self.tilings = tilings
+        self.tiled = [(summary[4 + 2 * i], summary[5 + 2 * i]) for i in range(len(tilings))]   # (rows, tiles) of each
+        self.first_table = 5 + len(tilings)      # index of the first block table among the pieces
         # Entries in the order they run in: (index in the caller's list, slot, first row, rows, start).
         self.placed = [tuple(placed[5 * i:5 * i + 5]) for i in range(n)]
 
@@ -119,7 +125,8 @@ class _DecodeGraph:
     def __init__(self, engine: "Engine", rows: int):
         groups = len(engine.cache.groups)
         widths = [engine.cache.max_blocks(g) for g in range(groups)]
-        sizes = [rows] * 5 + [0] + [rows * w for w in widths]   # tokens, positions, row_entry, slots, want, tiles, tables
+        tilings = engine.tilings
+        sizes = [rows] * 5 + [0] * len(tilings) + [rows * w for w in widths]   # tokens, positions, row_entry, slots, want, tiles, tables
         self.offsets = [int(v) for v in np.cumsum([0] + sizes)]
         total = self.offsets[-1]
         self.host = torch.empty(total, dtype=torch.int32).pin_memory()
@@ -130,7 +137,7 @@ class _DecodeGraph:
         self.context = StepContext(
             rows=rows, dtype=engine.dtype, device=engine.device, positions=pieces[1], row_entry=pieces[2],
             entries=[], entry_slots=pieces[3], want_rows=pieces[4],
-            block_tables={g: pieces[6 + g].view(rows, widths[g]) for g in range(groups)},
+            block_tables={g: pieces[5 + len(tilings) + g].view(rows, widths[g]) for g in range(groups)},
             max_position=engine.max_context - 1, decode_only=True)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
@@ -138,7 +145,8 @@ class _DecodeGraph:
 
     def fill(self, engine: "Engine", entries: Sequence[StepEntry]) -> None:
         self.copied.synchronize()                     # the last upload has left the pinned buffer
-        packed = PackedStep(engine.cache, engine.vocab_size, entries, all_rows_wanted=True, host=self.host)
+        packed = PackedStep(engine.cache, engine.vocab_size, entries, all_rows_wanted=True, host=self.host,
+                            tilings=engine.tilings)
         if packed.offsets != self.offsets:
             raise StepError("the step does not fit the recorded layout")
         self.dev.copy_(self.host, non_blocking=True)
@@ -171,6 +179,7 @@ class Engine:
         if poison_freed:
             self.cache.log_freed(True)
         self.vocab_size = model.spec.vocab_size
+        self.tilings = model.row_tilings()      # what the parts want long portions cut into
         # Steps of single decoded tokens are recorded once per batch size and replayed.
         self.graphs = bool(graphs) and model.graph_safe
         self._decode_graphs: Dict[int, _DecodeGraph] = {}
@@ -257,6 +266,8 @@ class Engine:
     def run_reserved(self, entries: Sequence[StepEntry]) -> StepOutput:
         """Runs a step whose pages the caller has reserved; commits on success, rolls back on failure."""
         self.poison_freed_pages()              # what a scheduler on the same manager has freed since the last step
+        # A failed step gives its pages back (rollback) and leaves per-request state as it found it.
+        saved_state = self.pools.snapshot_state([self.cache.slot(e.request) for e in entries])
         try:
             for e in entries:
                 if self.cache.length(e.request) == 0:
@@ -272,6 +283,7 @@ class Engine:
             for e in entries:
                 if self.cache.has(e.request):
                     self.cache.rollback(e.request)
+            self.pools.restore_state(saved_state)
             raise
         for e in entries:
             self.cache.commit(e.request, len(e.tokens))
@@ -323,7 +335,7 @@ class Engine:
 
     def _build_context(self, entries: Sequence[StepEntry]):
         """The step's metadata, laid out by the native routine and uploaded in one copy."""
-        packed = PackedStep(self.cache, self.vocab_size, entries, host=self._staging_buffer)
+        packed = PackedStep(self.cache, self.vocab_size, entries, host=self._staging_buffer, tilings=self.tilings)
         device = torch.empty(max(1, packed.total), dtype=torch.int32, device=self.device)
         device.copy_(packed.host[:max(1, packed.total)], non_blocking=True)
         self._staging[self._staging_turn][1].record()
@@ -332,13 +344,16 @@ class Engine:
                  for given, slot, first_row, count, start in packed.placed]
         rows_map = [(e.request, int(w)) for e in entries for w in e.want]
         n_groups = len(self.cache.groups)
-        tiled = [(count, start) for _, _, first_row, count, start in packed.placed if first_row < packed.prefill_rows]
-        mean_keys = sum(count * (start + (count + 1) // 2) for count, start in tiled) // max(1, sum(c for c, _ in tiled))
+        tiled = {}
+        for i, (tiling, (tiled_rows, tiles)) in enumerate(zip(packed.tilings, packed.tiled)):
+            if not tiles:
+                continue
+            cut = [(count, start) for _, _, first_row, count, start in packed.placed if first_row < tiled_rows]
+            mean_keys = sum(count * (start + (count + 1) // 2) for count, start in cut) // max(1, sum(c for c, _ in cut))
+            tiled[tiling] = TiledRows(tiled_rows, pieces[5 + i].view(-1, 3), mean_keys)
         context = StepContext(
             rows=packed.rows, dtype=self.dtype, device=self.device, positions=pieces[1], row_entry=pieces[2],
             entries=infos, entry_slots=pieces[3], want_rows=pieces[4] if packed.wanted else None,
-            block_tables={g: pieces[6 + g].view(len(entries), -1) for g in range(n_groups)},
-            max_position=packed.max_position, decode_only=packed.decode_only,
-            prefill_rows=packed.prefill_rows, q_tiles=pieces[5].view(-1, 3) if packed.tiles else None,
-            prefill_mean_keys=mean_keys)
+            block_tables={g: pieces[packed.first_table + g].view(len(entries), -1) for g in range(n_groups)},
+            max_position=packed.max_position, decode_only=packed.decode_only, tiled=tiled)
         return pieces[0], context, rows_map

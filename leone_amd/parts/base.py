@@ -14,6 +14,7 @@ position      ``prepare(max_positions, device)``; what it exposes to a mixer is
               the position part's own affair (the rotary part exposes tables).
 mixer         ``tensor_specs()``, ``bind(tensors)``, ``cache_need()`` -> ``KvNeed`` /
               ``StateNeed`` / ``None``, ``forward(y, step, cache)`` -> delta ``[rows, hidden]``.
+              Optional: ``row_tiling()`` -> ``RowTiling`` if it has a kernel that works on tiles of rows.
 feed_forward  ``tensor_specs()``, ``bind(tensors)``, ``forward(y, step)`` -> delta.
               A mixer or feed-forward that sets ``fused_io = True`` is instead called with
               ``forward(y, step[, cache], residual=x)``: ``y`` may then be an ``ops.NormedRows`` (a norm
@@ -55,12 +56,51 @@ class PartSpec:
         return self.params.get(key, default)
 
 
+# ---- what a mixer keeps between steps --------------------------------------------------------------------
+# A need says what kind of storage a cache slot wants and how to make, view, clear and spoil it; the pools
+# (``cache/pools.py``) know needs only through these methods, so another kind of cache is another class here
+# or beside the mixer that uses it.  Two families:
+#   paged = True   one entry per token, in pages handed out by the cache manager.  Slots with equal
+#                  ``group_key()`` share page ids and block tables (a group); ``window`` and ``page_tokens``
+#                  (None: the engine's) are the group's.  ``allocate(pages, page_tokens, dtype, device)`` ->
+#                  storage, ``view(storage, block_table, page_tokens)`` -> what the mixer's forward receives,
+#                  ``poison(storage, page index tensor)``, ``bytes_per_token(element size)``.
+#   paged = False  storage of fixed size per request slot.  ``allocate_slots(max_requests, device)`` -> storage,
+#                  ``view(storage)``, ``zero(storage, slot)``, ``snapshot(storage, slots)`` -> saved,
+#                  ``restore(storage, slots, saved)`` (a failed step puts the state back).
+
 @dataclass(frozen=True)
 class KvNeed:
-    """A mixer that caches one key and one value vector per token and kv head."""
+    """A mixer that caches one key and one value vector per token and kv head, packed in runs of 8:
+    keys ``[pages, kv_heads, head_dim/8, page_tokens, 8]``, values ``[pages, kv_heads, page_tokens/8, head_dim, 8]``."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None   # only the last `window` positions are ever read
+    page_tokens: Optional[int] = None   # tokens a page of this group holds; None: the engine's choice
+
+    paged = True
+
+    def group_key(self):
+        return self
+
+    def allocate(self, pages: int, page_tokens: int, dtype: torch.dtype, device):
+        if self.head_dim % 8 or page_tokens % 8:
+            raise ValueError(f"the cache packs runs of 8: head_dim {self.head_dim} and page_tokens "
+                             f"{page_tokens} must be multiples of 8")
+        return (torch.zeros((pages, self.kv_heads, self.head_dim // 8, page_tokens, 8), dtype=dtype, device=device),
+                torch.zeros((pages, self.kv_heads, page_tokens // 8, self.head_dim, 8), dtype=dtype, device=device))
+
+    def view(self, storage, block_table, page_tokens: int):
+        from .context import KvCacheView
+        return KvCacheView(writes=True, k_pool=storage[0], v_pool=storage[1], block_table=block_table,
+                           page_tokens=page_tokens)
+
+    def poison(self, storage, index: torch.Tensor) -> None:
+        for pool in storage:
+            pool.index_fill_(0, index, float("nan"))
+
+    def bytes_per_token(self, element_size: int) -> int:
+        return 2 * self.kv_heads * self.head_dim * element_size
 
 
 @dataclass(frozen=True)
@@ -68,6 +108,35 @@ class StateNeed:
     """A mixer that keeps per-request state of fixed size (float32 unless said otherwise)."""
     shape: tuple
     dtype: torch.dtype = torch.float32
+
+    paged = False
+
+    def allocate_slots(self, max_requests: int, device):
+        return torch.zeros((max_requests, *self.shape), dtype=self.dtype, device=device)
+
+    def view(self, storage):
+        from .context import StateCacheView
+        return StateCacheView(writes=True, state=storage)
+
+    def zero(self, storage, slot: int) -> None:
+        storage[slot].zero_()
+
+    def snapshot(self, storage, slots: torch.Tensor):
+        return storage.index_select(0, slots)
+
+    def restore(self, storage, slots: torch.Tensor, saved) -> None:
+        storage.index_copy_(0, slots, saved)
+
+
+@dataclass(frozen=True)
+class RowTiling:
+    """How a part wants long portions cut for a kernel of its own: portions of at least ``min_rows`` rows in
+    tiles of ``tile_rows`` consecutive rows of one request, ``group_tiles`` tiles to a group (a portion's last
+    group is filled up with tiles of no rows).  A part that declares one (``row_tiling()``) finds the tile
+    list of every step in ``StepContext.tiled[tiling]``; the step's layout knows nothing else about it."""
+    tile_rows: int
+    group_tiles: int
+    min_rows: int
 
 
 class Registry:

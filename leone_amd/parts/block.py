@@ -43,6 +43,10 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def row_tilings(self):
+        """The tilings its parts declare (``RowTiling``)."""
+        return [part.row_tiling() for part in self.parts() if hasattr(part, "row_tiling")]
+
     prepares_next = True
 
     def entry_norm(self, out_dtype):

@@ -24,6 +24,15 @@ class EntryInfo:
 
 
 @dataclass
+class TiledRows:
+    """What a step holds for one ``RowTiling``: rows [0, rows) belong to the portions it cuts, ``tiles`` is
+    int32 [n, 3] (entry, first row, rows) in groups, places of no rows filling a group up."""
+    rows: int
+    tiles: torch.Tensor
+    mean_keys: int = 0                 # positions a row of these portions looks back on, on average (a hint for grids)
+
+
+@dataclass
 class StepContext:
     rows: int
     dtype: torch.dtype                 # activation type of the engine
@@ -36,12 +45,9 @@ class StepContext:
     block_tables: Dict[int, torch.Tensor] = field(default_factory=dict)  # group -> int32 [entries, max_blocks]
     max_position: int = 0              # largest position in the step (an upper bound when the step is replayed)
     decode_only: bool = False          # every entry brings exactly one row
-    # Long prompt portions come first in a step: rows [0, prefill_rows) belong to them, cut into
-    # q_tiles (int32 [n, 3]: entry, first row, rows; tiles of consecutive rows of one request, in the groups
-    # the prompt-attention kernel takes; places of no rows fill a group up).
-    prefill_rows: int = 0
-    q_tiles: Optional[torch.Tensor] = None
-    prefill_mean_keys: int = 0         # keys a row of these portions sees on average (steers the kernel's grid only)
+    # Long portions come first in a step.  For every tiling a part of the model declared (``RowTiling``) that
+    # cuts at least one portion of this step: the tile list and the rows it covers.
+    tiled: Dict[object, TiledRows] = field(default_factory=dict)
 
 
 @dataclass

@@ -8,7 +8,7 @@ import torch
 
 from .. import ops
 from ..weights.loader import MATRIX, VECTOR, TensorSpec
-from .base import MIXERS, KvNeed, Part, PartSpec
+from .base import MIXERS, KvNeed, Part, PartSpec, RowTiling
 from .context import KvCacheView, StepContext
 
 
@@ -52,6 +52,10 @@ class GqaAttention(Part):
 
     def cache_need(self) -> KvNeed:
         return KvNeed(self.kv_heads, self.head_dim, self.window)
+
+    def row_tiling(self) -> RowTiling:
+        """The tiles of the prompt-attention kernel."""
+        return RowTiling(ops.PREFILL_TILE_ROWS, ops.PREFILL_GROUP_TILES, ops.PREFILL_MIN_ROWS)
 
     def tensor_specs(self) -> List[TensorSpec]:
         qw, kvw = self.q_heads * self.head_dim, self.kv_heads * self.head_dim
@@ -104,13 +108,13 @@ class GqaAttention(Part):
                                       cache.block_table, self.q_heads, self.scale, window)
         first = 0
         out = torch.empty_like(q)
-        if (step.prefill_rows and step.q_tiles is not None
+        tiled = step.tiled.get(self.row_tiling())
+        if (tiled is not None and tiled.rows
                 and ops.prefill_attention_supported(q.dtype, self.head_dim, cache.page_tokens, max_blocks)):
-            ops.attention_prefill(q, out, cache.k_pool, cache.v_pool, step.positions, step.q_tiles,
+            ops.attention_prefill(q, out, cache.k_pool, cache.v_pool, step.positions, tiled.tiles,
                                   cache.block_table, self.q_heads, self.scale, window,
-                                  mean_keys=step.prefill_mean_keys or step.max_position + 1,
-                                  covered_rows=step.prefill_rows)
-            first = step.prefill_rows
+                                  mean_keys=tiled.mean_keys or step.max_position + 1, covered_rows=tiled.rows)
+            first = tiled.rows
         if first < step.rows:
             ops.attention_decode(q[first:], cache.k_pool, cache.v_pool, step.positions[first:],
                                  step.row_entry[first:], cache.block_table, self.q_heads, self.scale, window,

@@ -89,6 +89,15 @@ class DecoderModel:
         for position in self.positions.values():
             position.prepare(self.spec.max_positions, self.device)
 
+    def row_tilings(self) -> list:
+        """Every distinct tiling a part of the model declares, in a fixed order (``RowTiling``)."""
+        found = []
+        for layer in self.layers:
+            for tiling in (layer.row_tilings() if hasattr(layer, "row_tilings") else []):
+                if tiling is not None and tiling not in found:
+                    found.append(tiling)
+        return found
+
     # ---- bytes ---------------------------------------------------------------
     def weight_accounting(self, nbytes=None, rows: int = 1) -> Dict[str, object]:
         """Bytes of the model's tensors by class, as they lie in memory (``resident``) and as a decode step

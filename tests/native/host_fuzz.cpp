@@ -47,8 +47,8 @@ int main() {
                 if (sm[i]) wants.push_back(ct[i] - 1);
             }
             wants.push_back(0); toks.push_back(0);
-            int shape[5] = {1000, 32, 16, 0, 4};
-            long sections[16]; int summary[6]; std::vector<int> placed(5 * n + 5);
+            int shape[9] = {1000, 0, 2, 32, 16, 4, 8, 5, 2};   // two row tilings
+            long sections[16]; int summary[8]; std::vector<int> placed(5 * n + 5);
             long need = leone_step_pack(cache, n, req.data(), ct.data(), wc.data(), toks.data(), wants.data(), shape, nullptr, 0, sections, nullptr, nullptr);
             if (need <= 0) { std::printf("pack failed (%ld): %s n=%d\n", need, leone_host_last_error(), n); return 1; }
             std::vector<int32_t> out(need);

@@ -118,7 +118,8 @@ DECAY = 0.75
 def register_toy():
     from leone_amd.architectures import register_architecture
     from leone_amd.config.base import FieldReader
-    from leone_amd.parts import MIXERS, Part, PartSpec, StateNeed
+    from leone_amd.parts import MIXERS, Part, PartSpec, RowTiling, StateNeed
+    from leone_amd.parts.context import CacheView
     from leone_amd.parts.model import LayerRun, ModelSpec
     from leone_amd.weights.loader import MATRIX, TensorSpec
     from leone_amd import ops
@@ -149,8 +150,88 @@ def register_toy():
                     cache.state[entry.slot] = s
             return ops.linear(states.to(y.dtype), self.weight)
 
+    @dataclass(frozen=True)
+    class VectorNeed:
+        """A kind of cache the framework does not have: one float32 vector per token, in pages of its own size."""
+        width: int
+        page_tokens: int = 4
+        window = None
+        paged = True
+
+        def group_key(self):
+            return self
+
+        def allocate(self, pages, page_tokens, dtype, device):
+            return torch.zeros((pages, page_tokens, self.width), dtype=torch.float32, device=device)
+
+        def view(self, storage, block_table, page_tokens):
+            view = CacheView(writes=True)
+            view.vectors, view.block_table, view.page_tokens = storage, block_table, page_tokens
+            return view
+
+        def poison(self, storage, index):
+            storage.index_fill_(0, index, float("nan"))
+
+        def bytes_per_token(self, element_size):
+            return 4 * self.width
+
+    class PrefixMeanMixer(Part):
+        """out_t = W mean(y_0 .. y_t) per request: every y is kept in the cache (a ``VectorNeed``), so that a
+        later step finds the earlier ones.  It has a row kernel of its own, as it were: portions of 6 rows and
+        more it takes tile by tile (tiles of 8 rows, two to a group), the other rows one by one."""
+
+        TILING = RowTiling(tile_rows=8, group_tiles=2, min_rows=6)
+
+        def __init__(self, spec, **_):
+            self.hidden, self.name = spec["hidden"], spec["weight"]
+            self.tiles_seen = []
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name, (self.hidden, self.hidden), MATRIX)]
+
+        def bind(self, tensors):
+            self.weight = tensors.pop(self.name).contiguous()
+
+        def cache_need(self):
+            return VectorNeed(self.hidden)
+
+        def row_tiling(self):
+            return self.TILING
+
+        def forward(self, y, step, cache):
+            assert cache.page_tokens == 4
+            table = cache.block_table.cpu()
+            positions, row_entry = step.positions.cpu().tolist(), step.row_entry.cpu().tolist()
+            for r in range(step.rows):                                   # every row's vector into its page
+                page = int(table[row_entry[r], positions[r] // 4])
+                cache.vectors[page, positions[r] % 4] = y[r].float()
+            means = torch.empty((step.rows, self.hidden), dtype=torch.float32, device=y.device)
+
+            def mean_of(r):
+                pages = table[row_entry[r], :positions[r] // 4 + 1].to(y.device).long()
+                return cache.vectors[pages].reshape(-1, self.hidden)[:positions[r] + 1].mean(dim=0)
+
+            tiled = step.tiled.get(self.TILING)
+            covered = 0
+            if tiled is not None:
+                listed = tiled.tiles.cpu().tolist()
+                assert len(listed) % 2 == 0
+                self.tiles_seen.append(listed)
+                for entry, first_row, rows in listed:
+                    assert rows <= 8 and all(row_entry[r] == entry for r in range(first_row, first_row + rows))
+                    for r in range(first_row, first_row + rows):
+                        means[r] = mean_of(r)
+                covered = tiled.rows
+                assert sum(rows for _, _, rows in listed) == covered
+            for info in step.entries:                                    # the layout's promise about the rest
+                assert (info.first_row < covered) == (info.count >= 6)
+            for r in range(covered, step.rows):
+                means[r] = mean_of(r)
+            return ops.linear(means.to(y.dtype), self.weight)
+
     if "toy_decay" not in MIXERS.kinds():
         MIXERS.register("toy_decay", DecayMixer)
+        MIXERS.register("toy_prefix_mean", PrefixMeanMixer)
 
     @dataclass(frozen=True)
     class ToyConfig:
@@ -196,10 +277,14 @@ def register_toy():
                                  "norm2": norm("l1.n2"), "feed_forward": ffn("l1")}),
             PartSpec("prenorm", {"norm1": norm("l2.n1"), "mixer": attention("l2", c.window, False, False),
                                  "norm2": norm("l2.n2"), "feed_forward": ffn("l2")}),
+            PartSpec("prenorm", {"norm1": norm("l3.n1"),
+                                 "mixer": PartSpec("toy_prefix_mean", {"hidden": c.hidden, "weight": "l3.w"}),
+                                 "norm2": norm("l3.n2"), "feed_forward": ffn("l3")}),
         ]
         # layer 1 runs twice, each run with state of its own; the last run is layer 0 again, reading the
         # keys and values its first run wrote, writing none
-        order = [LayerRun(0, 0), LayerRun(1, 1), LayerRun(2, 2), LayerRun(1, 3), LayerRun(0, 0, writes=False)]
+        order = [LayerRun(0, 0), LayerRun(1, 1), LayerRun(2, 2), LayerRun(3, 4), LayerRun(1, 3),
+                 LayerRun(0, 0, writes=False)]
         return ModelSpec(hidden_size=c.hidden, vocab_size=c.vocab, max_positions=c.max_positions, embedding="emb",
                          layers=layers, schedule=order, final_norm=norm("final"), head="head",
                          positions={"rope": PartSpec("rope_half_split", {"rotary_dim": c.head_dim, "theta": 5000.0})})
@@ -245,8 +330,12 @@ def toy_plain(w, tokens):
     y = plain.rms_norm(x, w["l2.n1"], c["eps"])
     att = plain.causal_attention(heads(y, "l2.q", 3), heads(y, "l2.k", 1), heads(y, "l2.v", 1), window=c["window"])
     x = ffn(x + plain.linear(att.reshape(n, -1), w["l2.o"]), "l2")
-    x = decay_layer(x)                      # run 4: layer 1 again, state of its own, starting from zero
-    # run 5: layer 0 again: new queries over the keys and values of run 1
+    # run 4: layer 3, the mean of everything so far
+    y = plain.rms_norm(x, w["l3.n1"], c["eps"])
+    means = torch.cumsum(y, dim=0) / torch.arange(1, n + 1, dtype=torch.float64)[:, None]
+    x = ffn(x + plain.linear(means, w["l3.w"]), "l3")
+    x = decay_layer(x)                      # run 5: layer 1 again, state of its own, starting from zero
+    # run 6: layer 0 again: new queries over the keys and values of run 1
     y = plain.rms_norm(x, w["l0.n1"], c["eps"])
     q = plain.rope_half_split(plain.rms_norm(heads(y, "l0.q", 3), w["l0.qn"], c["eps"]), positions, 5000.0)
     x = ffn(x + plain.linear(plain.causal_attention(q, k0, v0).reshape(n, -1), w["l0.o"]), "l0")
@@ -279,9 +368,12 @@ def test_toy_architecture_with_state_window_repeat_and_shared_cache(tmp_path, dt
         write_file(os.path.join(folder, "model.safetensors"), tensors)
         model = load_model(folder, dtype_name)
         needs = model.cache_needs()
-        assert sorted(needs) == [0, 1, 2, 3]
-        engine = Engine(model, num_pages=20, page_tokens=8, max_requests=3, poison_freed=True)
-        assert len(engine.cache.groups) == 2 and sorted(g.window or 0 for g in engine.cache.groups) == [0, 11]
+        assert sorted(needs) == [0, 1, 2, 3, 4]
+        engine = Engine(model, num_pages=36, page_tokens=8, max_requests=3, poison_freed=True)
+        # three groups: all keys, a window of 11, and the toy's own kind of cache with pages of 4 tokens
+        assert [(g.window or 0, g.page_tokens) for g in engine.cache.groups] == [(0, 8), (11, 8), (0, 4)]
+        # two tilings: the attention mixer's and the toy's
+        assert len(engine.tilings) == 2 and {t.tile_rows for t in engine.tilings} == {8, 32}
         requests = {f"t{i}": random_tokens(900 + i, n, TOY["vocab"]) for i, n in enumerate([45, 30, 9, 38])}
         weights = {k: v.float() for k, v in tensors.items()}
         expected = {rid: toy_plain(weights, toks).numpy() for rid, toks in requests.items()}
@@ -300,10 +392,42 @@ def test_toy_architecture_with_state_window_repeat_and_shared_cache(tmp_path, dt
                 err = np.abs(np.stack(rows) - expected[rid]).max(axis=1)
                 assert np.isfinite(err).all() and err.max() <= tol, (mode, rid, int(err.argmax()), float(err.max()))
             # the windowed group never holds more than ceil((window - 1 + longest portion) / page) + 1 pages a request
-            assert engine.cache.free_pages(0) == 20 and engine.cache.free_pages(1) == 20
+            assert all(engine.cache.free_pages(g) == 36 for g in range(3))
+        assert any(len(listed) > 2 for listed in model.layers[3].mixer.tiles_seen)        # the toy's tiles were used
+        # A step that fails half way leaves pages and per-request state as they were: the first half of a
+        # request, then its second half fails after the state mixers have run; run again it gives the same
+        # logits as if nothing had happened.
+        tokens = requests["t0"]
+        engine.step([StepEntry("f", tokens[:20], [])])
+        state_before = {slot: tensor.clone() for slot, tensor in engine.pools.state.items()}
+        free_before = [engine.cache.free_pages(g) for g in range(3)]
+        last = model.layers[0].feed_forward
+        real = last.forward
+        calls = []
+
+        def failing(*args, **kwargs):
+            calls.append(1)
+            if len(calls) == 2:                     # layer 0 runs twice a step: its second run comes last
+                raise RuntimeError("injected")
+            return real(*args, **kwargs)
+        last.forward = failing
+        try:
+            with pytest.raises(RuntimeError, match="injected"):
+                engine.step([StepEntry("f", tokens[20:], list(range(len(tokens) - 20)))])
+        finally:
+            last.forward = real
+        assert engine.cache.length("f") == 20 and [engine.cache.free_pages(g) for g in range(3)] == free_before
+        for slot, tensor in engine.pools.state.items():
+            assert torch.equal(tensor, state_before[slot])
+        out = engine.step([StepEntry("f", tokens[20:], list(range(len(tokens) - 20)))])
+        err = np.abs(out.logits.cpu().numpy() - expected["t0"][20:]).max()
+        assert err <= tol, err
+        engine.release("f")
+        engine.cache.check()
     finally:
         unregister_architecture("ToyForCausalLM")
         MIXERS.unregister("toy_decay")
+        MIXERS.unregister("toy_prefix_mean")
 
 
 # ---- a second toy: a feed-forward that routes rows to experts, and another position encoding -------------

@@ -5,6 +5,9 @@ import pytest
 from leone_amd import ops
 from leone_amd.cache.manager import CacheManager, GroupSpec
 from leone_amd.engine.engine import PackedStep, StepEntry, StepError
+from leone_amd.parts.base import RowTiling
+
+PROMPT = RowTiling(ops.PREFILL_TILE_ROWS, ops.PREFILL_GROUP_TILES, ops.PREFILL_MIN_ROWS)   # the attention mixer's
 
 
 def reserved(cache, entries):
@@ -27,7 +30,7 @@ def test_rows_positions_tables_and_wanted_rows():
     entries = [StepEntry("old", [7], [0]), StepEntry("long", list(range(100, 150)), [49, 0]),
                StepEntry("short", [1, 2, 3], [])]
     reserved(cache, entries)
-    packed = PackedStep(cache, 1000, entries)
+    packed = PackedStep(cache, 1000, entries, tilings=[PROMPT])
     tokens, positions, row_entry, slots, want, tiles, table0, table1 = sections(packed)
     # the portion long enough for the tiled kernel runs first, the others keep their order
     assert [p[0] for p in packed.placed] == [1, 0, 2]
@@ -36,7 +39,7 @@ def test_rows_positions_tables_and_wanted_rows():
     assert row_entry.tolist() == [0] * 50 + [1] + [2] * 3
     assert slots.tolist() == [cache.slot("long"), cache.slot("old"), cache.slot("short")]
     assert want.tolist() == [50, 49, 0]                       # in the caller's order of entries and places
-    assert (packed.rows, packed.prefill_rows, packed.max_position, packed.decode_only) == (54, 50, 49, False)
+    assert (packed.rows, packed.tiled[0][0], packed.max_position, packed.decode_only) == (54, 50, 49, False)
     width0, width1 = cache.max_blocks(0), cache.max_blocks(1)
     for place, name in enumerate(["long", "old", "short"]):
         for table, width, group in ((table0, width0, 0), (table1, width1, 1)):
@@ -54,7 +57,7 @@ def test_every_tile_is_listed_once_in_groups_of_one_entry(rows):
     other = StepEntry("b", list(range(40)), [])
     entry = StepEntry("a", [5] * rows, [rows - 1])
     reserved(cache, [other, entry])
-    packed = PackedStep(cache, 100, [other, entry])
+    packed = PackedStep(cache, 100, [other, entry], tilings=[PROMPT])
     tiles = sections(packed)[5].reshape(-1, 3)
     group = ops.PREFILL_GROUP_TILES
     assert len(tiles) % group == 0
@@ -76,7 +79,7 @@ def test_decode_layout_wants_every_row():
     cache = CacheManager([GroupSpec(8, 16)], max_requests=3, max_context=64)
     entries = [StepEntry(i, [i + 1], [0] if i else []) for i in range(3)]
     reserved(cache, entries)
-    packed = PackedStep(cache, 10, entries, all_rows_wanted=True)
+    packed = PackedStep(cache, 10, entries, all_rows_wanted=True, tilings=[PROMPT])
     tokens, positions, row_entry, slots, want, tiles = sections(packed)[:6]
     assert tokens.tolist() == [1, 2, 3] and want.tolist() == [0, 1, 2] and tiles.size == 0 and packed.decode_only
 
@@ -91,3 +94,27 @@ def test_malformed_steps_are_refused(entries, message):
     cache.admit("a")
     with pytest.raises(StepError, match=message):
         PackedStep(cache, 10, entries)
+
+
+def test_two_tilings_each_find_their_portions_at_the_front():
+    """Parts with kernels of different shapes each declare a tiling; the entries that more tilings cut come
+    first, so the rows of a tiling's portions are the step's first rows whatever its threshold; a model
+    without any gets no tile list at all."""
+    cache = CacheManager([GroupSpec(100, 16)], max_requests=6, max_context=400)
+    entries = [StepEntry("one", [1], [0]), StepEntry("mid", [2] * 10, []), StepEntry("long", [3] * 70, [69]),
+               StepEntry("two", [4, 4], []), StepEntry("mid2", [5] * 24, [0])]
+    reserved(cache, entries)
+    coarse, fine = RowTiling(32, 4, 16), RowTiling(8, 2, 5)
+    packed = PackedStep(cache, 10, entries, tilings=[coarse, fine])
+    assert [p[0] for p in packed.placed] == [2, 4, 1, 0, 3]      # cut by both, by the fine one only, by none
+    tokens, positions, row_entry, slots, want, tiles_coarse, tiles_fine, table = sections(packed)
+    assert packed.tiled == [(94, 8), (104, 16)]                  # (rows, tile places) of each
+    assert tiles_coarse.reshape(-1, 3).tolist() == [[0, 0, 32], [0, 32, 32], [0, 64, 6], [0, 0, 0],
+                                                    [1, 70, 24], [1, 70, 0], [1, 70, 0], [1, 70, 0]]
+    listed = tiles_fine.reshape(-1, 3).tolist()
+    assert listed[:9] == [[0, 8 * i, 8] for i in range(8)] + [[0, 64, 6]] and listed[9] == [0, 0, 0]
+    assert listed[10:14] == [[1, 70, 8], [1, 78, 8], [1, 86, 8], [1, 70, 0]]
+    assert listed[14:] == [[2, 94, 8], [2, 102, 2]]
+    assert want.tolist() == [104, 69, 70]
+    none = PackedStep(cache, 10, entries)
+    assert none.tiled == [] and len(sections(none)) == 6 and [p[0] for p in none.placed] == [0, 1, 2, 3, 4]
