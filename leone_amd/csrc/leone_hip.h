@@ -11,9 +11,12 @@ extern "C" {
 const char* leone_last_error();
 int leone_library_version();
 
-// out[r, :] = table[tokens[r], :] widened to float.
+// out[r, :] = table[tokens[r], :] widened to float, times scale (1 for none).
 int leone_embed(const void* table, int dtype, const int* tokens, float* out, int rows, int hidden, int vocab,
-                hipStream_t stream);
+                float scale, hipStream_t stream);
+
+// x = cap * tanh(x / cap) in place, n floats.
+int leone_soft_cap(float* x, long n, float cap, hipStream_t stream);
 
 // x += delta (delta may be null); y = rmsnorm(x) * gain.  With `rows` given,
 // y[r] is computed from row rows[r] and x is not written.  delta may be delta_planes (1..16) planes,

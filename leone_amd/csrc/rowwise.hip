@@ -17,7 +17,7 @@ namespace leone {
 // ---- embedding -------------------------------------------------------------
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
-                             float* __restrict__ out, int hidden, int vocab) {
+                             float* __restrict__ out, int hidden, int vocab, float scale) {
     const int row = blockIdx.x;
     const int token = tokens[row];
     float* dst = out + static_cast<long>(row) * hidden;
@@ -27,7 +27,14 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
         return;
     }
     const T* src = table + static_cast<long>(token) * hidden;
-    for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = to_float(src[c]);
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = to_float(src[c]) * scale;
+}
+
+// ---- a soft cap on logits -----------------------------------------------------
+// x = cap * tanh(x / cap), in place: what some architectures put between the head and the sampler.
+__global__ void __launch_bounds__(256) soft_cap_kernel(float* __restrict__ x, long n, float cap) {
+    const long stride = static_cast<long>(gridDim.x) * blockDim.x;
+    for (long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) x[i] = cap * tanhf(x[i] / cap);
 }
 
 // ---- residual add + RMSNorm -------------------------------------------------
@@ -514,16 +521,24 @@ static int check_dtype(int dtype, const char* what) {
 
 using namespace leone;
 
+extern "C" int leone_soft_cap(float* x, long n, float cap, hipStream_t stream) {
+    LEONE_REQUIRE(x && n > 0 && cap > 0.f, "soft_cap: needs values and a positive cap");
+    const long blocks = (n + 255) / 256;
+    soft_cap_kernel<<<static_cast<int>(blocks < 4096 ? blocks : 4096), 256, 0, stream>>>(x, n, cap);
+    LEONE_LAUNCH_CHECK("soft_cap");
+    return 0;
+}
+
 extern "C" int leone_embed(const void* table, int dtype, const int* tokens, float* out, int rows,
-                           int hidden, int vocab, hipStream_t stream) {
+                           int hidden, int vocab, float scale, hipStream_t stream) {
     if (check_dtype(dtype, "embed")) return 1;
     LEONE_REQUIRE(table && tokens && out, "embed: null pointer");
     LEONE_REQUIRE(rows > 0 && hidden > 0 && vocab > 0, "embed: rows %d hidden %d vocab %d must be positive", rows, hidden, vocab);
     const int threads = hidden >= 1024 ? 256 : 64;
     if (dtype == kF32)
-        embed_kernel<float><<<rows, threads, 0, stream>>>(static_cast<const float*>(table), tokens, out, hidden, vocab);
+        embed_kernel<float><<<rows, threads, 0, stream>>>(static_cast<const float*>(table), tokens, out, hidden, vocab, scale);
     else
-        embed_kernel<bf16_t><<<rows, threads, 0, stream>>>(static_cast<const bf16_t*>(table), tokens, out, hidden, vocab);
+        embed_kernel<bf16_t><<<rows, threads, 0, stream>>>(static_cast<const bf16_t*>(table), tokens, out, hidden, vocab, scale);
     LEONE_LAUNCH_CHECK("embed");
     return 0;
 }

@@ -75,16 +75,23 @@ def pack_values(v: torch.Tensor) -> torch.Tensor:
     return v.reshape(*lead, tokens // 8, 8, dim).transpose(-2, -1).contiguous()
 
 
-def embed(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[r] = table[tokens[r]] as float32.  Token ids must have been checked against the table."""
+def embed(table: torch.Tensor, tokens: torch.Tensor, out: Optional[torch.Tensor] = None,
+          scale: float = 1.0) -> torch.Tensor:
+    """out[r] = table[tokens[r]] * scale as float32.  Token ids must have been checked against the table."""
     vocab, hidden = table.shape
     rows = tokens.numel()
     if out is None:
         out = torch.empty((rows, hidden), dtype=torch.float32, device=table.device)
     call("leone_embed", _dev(table, "embed table"), _code(table, "embed table"),
          _dev(tokens, "embed tokens", torch.int32, (rows,)), _dev(out, "embed out", torch.float32, (rows, hidden)),
-         rows, hidden, vocab, _stream())
+         rows, hidden, vocab, float(scale), _stream())
     return out
+
+
+def soft_cap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x = cap * tanh(x / cap), in place (float32)."""
+    call("leone_soft_cap", _dev(x, "soft_cap values", torch.float32), x.numel(), float(cap), _stream())
+    return x
 
 
 def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, eps: float,

@@ -22,7 +22,8 @@ _lib: ctypes.CDLL | None = None
 
 P = c_void_p
 _PROTOTYPES = {
-    "leone_embed": [P, c_int, P, P, c_int, c_int, c_int, P],
+    "leone_embed": [P, c_int, P, P, c_int, c_int, c_int, c_float, P],
+    "leone_soft_cap": [P, ctypes.c_long, c_float, P],
     "leone_add_rmsnorm": [P, P, c_int, c_int, ctypes.c_long, P, c_int, c_float, P, c_int, P, c_int, c_int, P, P],
     "leone_swiglu": [P, P, c_int, c_int, c_int, P],
     "leone_rope_table": [P, P, c_double, c_int, c_int, P],

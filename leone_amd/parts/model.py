@@ -38,6 +38,8 @@ class ModelSpec:
     head: Optional[str]                             # tensor name [vocab, hidden]; None = tied to the embedding
     positions: Dict[str, PartSpec] = field(default_factory=dict)
     ignore_tensors: Sequence[str] = ()              # names a file may hold that the model does not use
+    embedding_scale: Optional[float] = None         # the stream starts as table row * scale
+    logit_cap: Optional[float] = None               # logits = cap * tanh(logits / cap)
 
 
 def default_schedule(n_layers: int) -> List[LayerRun]:
@@ -161,7 +163,7 @@ class DecoderModel:
     # ---- forward ---------------------------------------------------------------
     def forward(self, tokens: torch.Tensor, step: StepContext, caches: Dict[int, CacheView]) -> Optional[torch.Tensor]:
         """Runs the step's rows through every scheduled layer; returns float32 logits of the wanted rows."""
-        x = ops.embed(self.embedding, tokens)
+        x = ops.embed(self.embedding, tokens, scale=self.spec.embedding_scale or 1.0)
         pending = None
         for at, run in enumerate(self.schedule):
             cache = caches.get(run.cache) if run.cache is not None else None
@@ -185,4 +187,5 @@ class DecoderModel:
             y = self.final_norm.lazy(x, pending, self.dtype, rows=step.want_rows)
         else:
             y = self.final_norm.add_norm(x, pending, self.dtype, rows=step.want_rows)
-        return ops.linear(y, self.head, out_dtype=torch.float32)
+        logits = ops.linear(y, self.head, out_dtype=torch.float32)
+        return ops.soft_cap(logits, self.spec.logit_cap) if self.spec.logit_cap else logits

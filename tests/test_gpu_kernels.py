@@ -34,6 +34,10 @@ def test_embed(dtype):
     out = ops.embed(table, tokens)
     assert out.dtype == torch.float32
     assert torch.equal(out, table.float()[tokens.long()])
+    assert torch.equal(ops.embed(table, tokens, scale=3.0), table.float()[tokens.long()] * 3.0)
+    values = torch.randn(7, 333, device=DEV) * 40
+    capped = ops.soft_cap(values.clone(), 30.0)
+    close(capped, 30.0 * torch.tanh(values.double() / 30.0), 1e-5, 1e-6, "soft cap")
 
 
 @pytest.mark.parametrize("hidden", [80, 1000, 4096, 5120])

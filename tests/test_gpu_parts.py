@@ -676,3 +676,31 @@ def test_block_part(dtype, rows):
     want = x1 + plain.feed_forward(plain.rms_norm(x1, wf["n2"], 1e-5), wf, "f")
     tol = 2e-5 if dtype == torch.float32 else 3e-2
     assert (got - want).abs().max() < tol
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_model_spec_with_embedding_scale_and_logit_cap(tmp_path, dtype_name):
+    """Two things a model description may ask for around the layers: the stream starts as table row * scale,
+    and logits pass through cap * tanh(logits / cap).  Checked on the Qwen3 parts with a spec changed here:
+    the plain side gets the scale through a scaled table (the head is not tied) and the cap applied after."""
+    import dataclasses
+    from leone_amd.architectures import config_from_dict, model_spec_for
+    from leone_amd.engine.engine import Engine, StepEntry
+    from leone_amd.parts.model import DecoderModel
+    from leone_amd.weights import loader
+    from tests.util import TINY, make_model_dir, read_weights
+    dtype = torch.float32 if dtype_name == "float32" else torch.bfloat16
+    folder = make_model_dir(str(tmp_path / "m"), TINY["B"], 5, dtype)
+    spec = dataclasses.replace(model_spec_for(config_from_dict(TINY["B"])), embedding_scale=4.0, logit_cap=0.5)
+    model = DecoderModel(spec, dtype, DEV)
+    model.bind(loader.load_from_dir(folder, model.tensor_specs(), dtype, torch.device(DEV)))
+    weights = {k: v.float() for k, v in read_weights(folder).items()}
+    tokens = random_tokens(3, 50, TINY["B"]["vocab_size"])
+    scaled = dict(weights)
+    scaled["model.embed_tokens.weight"] = weights["model.embed_tokens.weight"] * 4.0
+    want = 0.5 * torch.tanh(plain.forward(scaled, TINY["B"], tokens) / 0.5)
+    engine = Engine(model, max_tokens=64, page_tokens=16, max_requests=2)
+    out = engine.step([StepEntry("a", tokens[:37], list(range(37)))]).logits
+    out = torch.cat([out, engine.step([StepEntry("a", tokens[37:], list(range(13)))]).logits]).cpu().double()
+    assert float(want.abs().max()) > 0.3                                  # the cap bites
+    assert (out - want).abs().max() < (1e-4 if dtype_name == "float32" else 3e-2)
