@@ -23,6 +23,14 @@
 // finishes last do the merge was measured: the device-wide fences it needs
 // cost far more than the second launch, 8.8 against 6.0 ms a step.)
 //
+// A step in which every row is another request (single decoded tokens) can leave the work on the new token's
+// heads to this kernel (`FromProjection`): it takes the fused q/k/v projection as it comes, normalises and
+// rotates the query heads it needs in registers (per-head RMSNorm, half-split rotation:
+// crates/leone/src/backend.rs:2182-2208, crates/leone/src/cpu.rs:1721-1779), and the workgroup whose keys
+// end with the row's own position does the same for the new key, writes it and the new value into the cache
+// and only then walks its tiles.  One launch fewer a layer; the values are those of the separate kernel
+// (rowwise.hip).  Head sizes that are multiples of 64 only: there a lane holds both halves of its pairs.
+//
 // Operand layouts of the 16x16x32 instruction (lane l, c = l % 16, g = l / 16):
 //   A: row c,    k-slots 8g .. 8g+7        B: column c, k-slots 8g .. 8g+7
 //   C/D: column c, rows 4g .. 4g+3
@@ -53,16 +61,55 @@ __device__ inline bf16x8 zero8() {
     return __builtin_bit_cast(bf16x8, z);
 }
 
+// The fused q/k/v projection of the step's rows and what turns it into queries, keys and values.
+struct FromProjection {
+    const void* qkv;        // [rows, (q_heads + 2 kv_heads) * head_dim], bfloat16, or float32 in `planes` planes
+    int is_float;
+    int planes;
+    long plane;
+    AnyVec q_gain, k_gain;  // null pointers: no norm
+    float eps;
+    const float* cos_table; // [table_positions, head_dim / 2], or null: no rotation
+    const float* sin_table;
+    int table_positions;
+    bf16_t* k_out;          // the pools, for the new token; null: this run writes no cache
+    bf16_t* v_out;
+};
+
+// Eight elements of the projection from element offset `at` of row `row`: planes added in order, then rounded
+// to bfloat16 as a stored projection would be.
+__device__ inline void load_projection8(const FromProjection& f, long row_width, long row, long at, float out[8]) {
+    if (!f.is_float) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(f.qkv) + row * row_width + at);
+        const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            out[2 * i] = __uint_as_float(w[i] << 16);
+            out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+        return;
+    }
+    const float* src = static_cast<const float*>(f.qkv) + row * row_width + at;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = src[i];
+    for (int p = 1; p < f.planes; ++p)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] += src[p * f.plane + i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = to_float(from_float<bf16_t>(out[i]));
+}
+
 // kD16 = head_dim / 16.
 // Up to a head size of 128 the kernel fits three waves a SIMD without spilling if the compiler is asked to
 // (a little faster than two, measured); larger heads need their registers.
-template <int kD16>
+template <int kD16, bool kFused>
 __global__ void __launch_bounds__(kDecodeThreads, kD16 <= 8 ? 3 : 1)
 attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
                         const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
                         const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
                         float* __restrict__ part_acc, float* __restrict__ part_ml, bf16_t* __restrict__ out,
-                        int q_heads, int kv_heads, int page_shift, float to_log2, int window, int splits) {
+                        int q_heads, int kv_heads, int page_shift, float to_log2, int window, int splits,
+                        FromProjection from) {
     constexpr int kD = kD16 * 16;
     constexpr int kSteps = (kD16 + 1) / 2;           // 32-element steps of the q.k product
     extern __shared__ float smem[];                   // [waves][columns][kD] accumulators, then m and l
@@ -97,11 +144,142 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         const int n_pages = my_begin < my_end ? (last_key >> page_shift) - first_page + 1 : 0;
         for (int i = threadIdx.x; i < n_pages; i += kDecodeThreads) pages[i] = table[first_page + i];
     }
+    if constexpr (kFused) {
+        // The workgroup whose keys end with the row's own position makes that position's key and value and
+        // writes them into the cache; its waves read them from there after the barrier.  (With more than 16
+        // query heads a kv head several workgroups do, each for itself: the same bytes.)
+        if (from.k_out != nullptr && my_begin < my_end && my_end == t_end) {
+            const long width = static_cast<long>(q_heads + 2 * kv_heads) * kD;
+            const int pos = n - 1;
+            const int page = table[pos >> page_shift];
+            if (page >= 0) {                              // the host reserves the page before the launch
+                const long base = (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD;
+                const int token = pos & page_mask;
+                constexpr int kHalfRuns = kD16;           // runs of 8 elements in half a head
+                if (wave == 0) {
+                    // lane L < kHalfRuns: elements 8L .. 8L+7 and their partners in the other half
+                    const bool mine = lane < kHalfRuns;
+                    float a[8], b[8];
+                    float ss = 0.f;
+                    if (mine) {
+                        load_projection8(from, width, row, static_cast<long>(q_heads + kvh) * kD + 8 * lane, a);
+                        load_projection8(from, width, row, static_cast<long>(q_heads + kvh) * kD + kD / 2 + 8 * lane, b);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) {
+                            ss = fmaf(a[i], a[i], ss);
+                            ss = fmaf(b[i], b[i], ss);
+                        }
+                    }
+                    ss = wave_sum(ss);
+                    if (mine) {
+                        if (from.k_gain.ptr) {
+                            const float inv = 1.0f / sqrtf(ss / static_cast<float>(kD) + from.eps);
+                            float ga[8], gb[8];
+                            load_any8(from.k_gain, 8 * lane, ga);
+                            load_any8(from.k_gain, kD / 2 + 8 * lane, gb);
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) {
+                                a[i] = (a[i] * ga[i]) * inv;
+                                b[i] = (b[i] * gb[i]) * inv;
+                            }
+                        }
+                        if (from.cos_table != nullptr) {
+                            const int tpos = pos < from.table_positions ? pos : from.table_positions - 1;
+                            float cs[8], sn[8];
+                            load_any8(AnyVec{from.cos_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 8 * lane, cs);
+                            load_any8(AnyVec{from.sin_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 8 * lane, sn);
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) {
+                                const float ru = a[i] * cs[i] - b[i] * sn[i];
+                                const float rv = a[i] * sn[i] + b[i] * cs[i];
+                                a[i] = ru;
+                                b[i] = rv;
+                            }
+                        }
+                        uint4 lo, hi;
+                        unsigned* wl = reinterpret_cast<unsigned*>(&lo);
+                        unsigned* wh = reinterpret_cast<unsigned*>(&hi);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            wl[i] = bf16_bits_from_float(a[2 * i]) | (static_cast<unsigned>(bf16_bits_from_float(a[2 * i + 1])) << 16);
+                            wh[i] = bf16_bits_from_float(b[2 * i]) | (static_cast<unsigned>(bf16_bits_from_float(b[2 * i + 1])) << 16);
+                        }
+                        *reinterpret_cast<uint4*>(from.k_out + base + key_offset(token, 8 * lane, page_tokens)) = lo;
+                        *reinterpret_cast<uint4*>(from.k_out + base + key_offset(token, kD / 2 + 8 * lane, page_tokens)) = hi;
+                    }
+                } else if (wave == 1) {
+                    // values are copied as they are, one element of one token at a time
+                    const long value_at = static_cast<long>(q_heads + kv_heads + kvh) * kD;
+                    for (int e = 8 * lane; e < kD; e += 8 * kWave) {
+                        float v[8];
+                        load_projection8(from, width, row, value_at + e, v);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i)
+                            from.v_out[base + value_offset(token, e + i, kD)] = from_float<bf16_t>(v[i]);
+                    }
+                }
+            }
+            __threadfence_block();                         // the waves of this workgroup read what was written
+        }
+    }
     __syncthreads();
 
     // Q^T operand: column c is query head kvh*group + col0 + c.
     bf16x8 qreg[kSteps];
-    {
+    if constexpr (kFused) {
+        // Lane (c, g) holds elements 32s + 8g .. + 7 of head c for every step s; with a head size that is a
+        // multiple of 64 the partner of such a run in the other half of the head is the same lane's run of
+        // step s + kSteps / 2.
+        static_assert(!kFused || kD16 % 4 == 0, "the fused query path needs a head size that is a multiple of 64");
+        constexpr int kHalfSteps = kSteps / 2;
+        const bool head_ok = c < cols;
+        const long width = static_cast<long>(q_heads + 2 * kv_heads) * kD;
+        const long head_at = static_cast<long>(kvh * group + col0 + (head_ok ? c : 0)) * kD;
+        // everything is asked for first (heads, gains, angles), 16 or 32 bytes at a time, then worked on
+        float v[kSteps][8], gain[kSteps][8], cs[kHalfSteps][8], sn[kHalfSteps][8];
+        const int tpos = n - 1 < from.table_positions ? n - 1 : from.table_positions - 1;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            load_projection8(from, width, row, head_at + 32 * s + 8 * g, v[s]);
+            if (from.q_gain.ptr) load_any8(from.q_gain, 32 * s + 8 * g, gain[s]);
+        }
+        if (from.cos_table != nullptr) {
+#pragma unroll
+            for (int s = 0; s < kHalfSteps; ++s) {
+                load_any8(AnyVec{from.cos_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 32 * s + 8 * g, cs[s]);
+                load_any8(AnyVec{from.sin_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 32 * s + 8 * g, sn[s]);
+            }
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss = fmaf(v[s][i], v[s][i], ss);
+        ss += __shfl_xor(ss, 16, kWave);                  // the four lanes that share head c
+        ss += __shfl_xor(ss, 32, kWave);
+        if (from.q_gain.ptr) {
+            const float inv = 1.0f / sqrtf(ss / static_cast<float>(kD) + from.eps);
+#pragma unroll
+            for (int s = 0; s < kSteps; ++s)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[s][i] = (v[s][i] * gain[s][i]) * inv;
+        }
+        if (from.cos_table != nullptr) {
+#pragma unroll
+            for (int s = 0; s < kHalfSteps; ++s) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float a = v[s][i], b = v[s + kHalfSteps][i];
+                    v[s][i] = a * cs[s][i] - b * sn[s][i];
+                    v[s + kHalfSteps][i] = a * sn[s][i] + b * cs[s][i];
+                }
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) qreg[s][i] = head_ok ? static_cast<__bf16>(v[s][i]) : static_cast<__bf16>(0.0f);
+    } else {
         const bool head_ok = c < cols;
         const bf16_t* qrow = q + (static_cast<long>(row) * q_heads + kvh * group + col0 + (head_ok ? c : 0)) * kD;
 #pragma unroll
@@ -315,33 +493,39 @@ template <int kD16>
 static void launch_decode(const void* q, const void* k_pool, const void* v_pool, const int* positions,
                           const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
                           float* part_ml, void* out, int rows, int q_heads, int kv_heads, int page_shift, float scale,
-                          int window, int splits, hipStream_t stream) {
+                          int window, int splits, const FromProjection* from, hipStream_t stream) {
     const int group = q_heads / kv_heads;
     dim3 grid(rows, kv_heads * ((group + 15) / 16), splits);
     const size_t smem = decode_smem_bytes(kD16 * 16, group, max_blocks);
-    attention_decode_kernel<kD16><<<grid, kDecodeThreads, smem, stream>>>(
+    const float to_log2 = scale * 1.4426950408889634f;
+    if constexpr (kD16 % 4 == 0) {
+        if (from != nullptr) {
+            attention_decode_kernel<kD16, true><<<grid, kDecodeThreads, smem, stream>>>(
+                nullptr, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), positions, row_entry,
+                block_table, max_blocks, part_acc, part_ml, static_cast<bf16_t*>(out), q_heads, kv_heads, page_shift,
+                to_log2, window, splits, *from);
+            return;
+        }
+    }
+    attention_decode_kernel<kD16, false><<<grid, kDecodeThreads, smem, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
         positions, row_entry, block_table, max_blocks, part_acc, part_ml, static_cast<bf16_t*>(out), q_heads, kv_heads,
-        page_shift, scale * 1.4426950408889634f, window, splits);
+        page_shift, to_log2, window, splits, FromProjection{});
 }
 
-}  // namespace leone
-
-using namespace leone;
-
-// Workspace for splits > 1: part_acc holds rows*q_heads*splits*head_dim floats, part_ml rows*q_heads*splits*2.
-extern "C" int leone_attention_decode(const void* q, void* out, const void* k_pool, const void* v_pool,
-                                      const int* positions, const int* row_entry, const int* block_table,
-                                      int max_blocks, float* part_acc, float* part_ml, int rows, int q_heads,
-                                      int kv_heads, int head_dim, int page_tokens, float scale, int window,
-                                      int splits, hipStream_t stream) {
-    LEONE_REQUIRE(q && out && k_pool && v_pool && positions && row_entry && block_table,
+static int decode_checked(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
+                          const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
+                          float* part_ml, int rows, int q_heads, int kv_heads, int head_dim, int page_tokens,
+                          float scale, int window, int splits, const FromProjection* from, hipStream_t stream) {
+    LEONE_REQUIRE((q || from) && out && k_pool && v_pool && positions && row_entry && block_table,
                   "attention_decode: null pointer");
     LEONE_REQUIRE(splits == 1 || (part_acc && part_ml), "attention_decode: %d splits need the workspace", splits);
     LEONE_REQUIRE(rows > 0 && q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
                   "attention_decode: rows %d, %d query heads over %d kv heads", rows, q_heads, kv_heads);
     LEONE_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
                   "attention_decode: head_dim %d must be a multiple of 16 in 16..256", head_dim);
+    LEONE_REQUIRE(!from || head_dim % 64 == 0, "attention_decode: the projection is taken only at head sizes that are "
+                  "multiples of 64, not %d", head_dim);
     LEONE_REQUIRE(page_tokens >= 16 && (page_tokens & (page_tokens - 1)) == 0,
                   "attention_decode: page_tokens %d must be a power of two, at least 16", page_tokens);
     LEONE_REQUIRE(decode_smem_bytes(head_dim, q_heads / kv_heads, max_blocks) <= 64 * 1024,
@@ -355,7 +539,7 @@ extern "C" int leone_attention_decode(const void* q, void* out, const void* k_po
 #define LEONE_DECODE_CASE(N)                                                                                      \
     case N:                                                                                                       \
         launch_decode<N>(q, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml,     \
-                         out, rows, q_heads, kv_heads, page_shift, scale, window, splits, stream);                \
+                         out, rows, q_heads, kv_heads, page_shift, scale, window, splits, from, stream);          \
         break;
     switch (head_dim / 16) {
         LEONE_DECODE_CASE(1) LEONE_DECODE_CASE(2) LEONE_DECODE_CASE(3) LEONE_DECODE_CASE(4)
@@ -374,4 +558,51 @@ extern "C" int leone_attention_decode(const void* q, void* out, const void* k_po
         LEONE_LAUNCH_CHECK("attention_reduce");
     }
     return 0;
+}
+
+}  // namespace leone
+
+using namespace leone;
+
+// Workspace for splits > 1: part_acc holds rows*q_heads*splits*head_dim floats, part_ml rows*q_heads*splits*2.
+extern "C" int leone_attention_decode(const void* q, void* out, const void* k_pool, const void* v_pool,
+                                      const int* positions, const int* row_entry, const int* block_table,
+                                      int max_blocks, float* part_acc, float* part_ml, int rows, int q_heads,
+                                      int kv_heads, int head_dim, int page_tokens, float scale, int window,
+                                      int splits, hipStream_t stream) {
+    return decode_checked(q, out, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml, rows,
+                          q_heads, kv_heads, head_dim, page_tokens, scale, window, splits, nullptr, stream);
+}
+
+// The same for a step in which every row is another request, taking the fused q/k/v projection instead of
+// finished queries: per-head RMSNorm (gains may be null) and half-split rotation (tables may be null) of the
+// query heads, and with write_cache of the new key too, which goes into the cache with the new value before the
+// keys are read.  qkv is bfloat16 [rows, (q_heads + 2 kv_heads) * head_dim], or float32 in qkv_planes planes
+// (qkv_plane elements apart) that are added up in order.  head_dim a multiple of 64.
+extern "C" int leone_attention_decode_projected(const void* qkv, int qkv_dtype, int qkv_planes, long qkv_plane,
+                                                const void* q_gain, const void* k_gain, int gain_dtype, float eps,
+                                                const float* cos_table, const float* sin_table, int table_positions,
+                                                void* out, void* k_pool, void* v_pool, int write_cache,
+                                                const int* positions, const int* row_entry, const int* block_table,
+                                                int max_blocks, float* part_acc, float* part_ml, int rows, int q_heads,
+                                                int kv_heads, int head_dim, int page_tokens, float scale, int window,
+                                                int splits, hipStream_t stream) {
+    LEONE_REQUIRE(qkv && (qkv_dtype == kBF16 || qkv_dtype == kF32), "attention_decode: the projection is bfloat16 or float32");
+    LEONE_REQUIRE(qkv_planes >= 1 && qkv_planes <= 64 && (qkv_dtype == kF32 || qkv_planes == 1),
+                  "attention_decode: %d planes of the projection", qkv_planes);
+    LEONE_REQUIRE((q_gain == nullptr) == (k_gain == nullptr), "attention_decode: q and k gains come together");
+    LEONE_REQUIRE(!q_gain || ((gain_dtype == kF32 || gain_dtype == kBF16) && eps > 0.f),
+                  "attention_decode: the head norms need gains of a known type and a positive eps");
+    LEONE_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "attention_decode: cos and sin tables come together");
+    LEONE_REQUIRE(!cos_table || table_positions > 0, "attention_decode: empty rotary table");
+    LEONE_REQUIRE(reinterpret_cast<uintptr_t>(qkv) % 32 == 0 &&
+                      (!cos_table || (reinterpret_cast<uintptr_t>(cos_table) % 32 == 0 && reinterpret_cast<uintptr_t>(sin_table) % 32 == 0)) &&
+                      (!q_gain || (reinterpret_cast<uintptr_t>(q_gain) % 32 == 0 && reinterpret_cast<uintptr_t>(k_gain) % 32 == 0)),
+                  "attention_decode: the projection, the gains and the rotary tables must be aligned to 32 bytes");
+    FromProjection from{qkv, qkv_dtype == kF32 ? 1 : 0, qkv_planes, qkv_plane, AnyVec{q_gain, gain_dtype},
+                        AnyVec{k_gain, gain_dtype}, eps, cos_table, sin_table, table_positions,
+                        write_cache ? static_cast<bf16_t*>(k_pool) : nullptr,
+                        write_cache ? static_cast<bf16_t*>(v_pool) : nullptr};
+    return decode_checked(nullptr, out, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml,
+                          rows, q_heads, kv_heads, head_dim, page_tokens, scale, window, splits, &from, stream);
 }

@@ -65,6 +65,27 @@ __device__ inline float load_any(const AnyVec& v, long i) {
                            : to_float(static_cast<const bf16_t*>(v.ptr)[i]);
 }
 
+// Eight elements of such a vector from an offset that is a multiple of 8 (the vector aligned to 32 bytes).
+__device__ inline void load_any8(const AnyVec& v, long at, float out[8]) {
+    if (v.dtype == kF32) {
+        const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(v.ptr) + at);
+        const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(v.ptr) + at + 4);
+        out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+        out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+    } else {
+        const uint4 t = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(v.ptr) + at);
+        const unsigned w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            union { uint32_t u; float f; } lo, hi;
+            lo.u = w[i] << 16;
+            hi.u = w[i] & 0xffff0000u;
+            out[2 * i] = lo.f;
+            out[2 * i + 1] = hi.f;
+        }
+    }
+}
+
 __device__ inline float wave_sum(float v) {
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);

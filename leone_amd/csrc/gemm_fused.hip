@@ -95,15 +95,13 @@ gemm_fused_kernel(FusedArgs a) {
     float ss = 0.f;
     const int xr = c < m ? c : m - 1;
     const long xrow_index = (kIn == kInNorm && a.rows) ? a.rows[xr] : xr;
-    if (kIn == kInPrepared) {
-        // The partial sums of squares of row c, a contiguous share for every (wave, g), summed in index order.
-        const int parts = (k + 15) / 16;
-        const int share = (parts + 4 * kWaves - 1) / (4 * kWaves);
-        const int begin = (wave * 4 + g) * share;
-        const int end = begin + share < parts ? begin + share : parts;
-        const float* from = a.squares_in + static_cast<long>(xr) * parts;
-        for (int i = begin; i < end; ++i) ss += from[i];
-    }
+    // Prepared input: the rows' partial sums of squares ([m][k / 16] floats, k a multiple of 64) go to shared
+    // memory after the walk over K, all threads side by side in 16-byte loads, and wave 0 adds each row's up
+    // in index order.  (Asked for before the walk and kept in registers they cost the kernel a third of the
+    // waves a compute unit holds, and with them the loads in flight that it lives on.)
+    constexpr int kQuads = 8;                        // 16-byte loads a thread takes; the entry point checks that they suffice
+    extern __shared__ float4 sums_of_squares[];      // [m * k / 64]
+    const int quads = kIn == kInPrepared ? m * (k / 64) : 0;
     const bf16_t* xb = static_cast<const bf16_t*>(a.x) + xrow_index * k + 16 * g;   // plain
     const float* xf = static_cast<const float*>(a.x) + xrow_index * k + 16 * g;     // norm
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -159,7 +157,20 @@ gemm_fused_kernel(FusedArgs a) {
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) partial[wave][lane][r] = acc[r];
-    if (kIn != kInPlain) {
+    if (kIn == kInPrepared) {
+        float4 held[kQuads];
+#pragma unroll
+        for (int i = 0; i < kQuads; ++i) {
+            const int at = i * kWaves * kWave + static_cast<int>(threadIdx.x);
+            held[i] = at < quads ? reinterpret_cast<const float4*>(a.squares_in)[at] : float4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int i = 0; i < kQuads; ++i) {
+            const int at = i * kWaves * kWave + static_cast<int>(threadIdx.x);
+            if (at < quads) sums_of_squares[at] = held[i];
+        }
+    }
+    if (kIn == kInNorm) {
         ss += __shfl_xor(ss, 16, kWave);             // the four lanes that share X row c
         ss += __shfl_xor(ss, 32, kWave);
         if (g == 0) squares[wave][c] = ss;
@@ -175,8 +186,24 @@ gemm_fused_kernel(FusedArgs a) {
         for (int r = 0; r < 4; ++r) sum[r] += partial[v][lane][r];
     if (kIn != kInPlain) {
         float total = 0.f;
+        if (kIn == kInPrepared) {
+            // lane (c, g) adds the g-th quarter of row c's partial sums, then the four quarters meet
+            const int per = k / 64;                  // 16-byte runs of a quarter: k / 16 sums a row
+            const float4* from = sums_of_squares + static_cast<long>(xr) * per;
+            const int begin = g * (per / 4) + (g < per % 4 ? g : per % 4), end = begin + per / 4 + (g < per % 4 ? 1 : 0);
+            for (int i = begin; i < end; i += 8) {       // eight reads on their way at a time
+                float4 v[8];
 #pragma unroll
-        for (int v = 0; v < kWaves; ++v) total += squares[v][c];
+                for (int u = 0; u < 8; ++u) v[u] = i + u < end ? from[i + u] : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int u = 0; u < 8; ++u) total += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+            }
+            total += __shfl_xor(total, 16, kWave);
+            total += __shfl_xor(total, 32, kWave);
+        } else {
+#pragma unroll
+            for (int v = 0; v < kWaves; ++v) total += squares[v][c];
+        }
         const float inv = 1.0f / sqrtf(total / static_cast<float>(k) + a.eps);
 #pragma unroll
         for (int r = 0; r < 4; ++r) sum[r] *= inv;
@@ -238,8 +265,9 @@ static void launch_fused(const FusedArgs& a, hipStream_t stream) {
     const int steps = ceil_div(a.k, 64);
     const bool tail = a.k % 64 != 0;
     const bool many = tiles * 4 >= 4096 || steps < 16;    // workgroups enough to fill the chip, or too little of K to split further
+    const size_t shared = kIn == kInPrepared ? static_cast<size_t>(a.m) * (a.k / 16) * sizeof(float) : 0;
 #define LEONE_FUSED(TAIL, WAVES) \
-    gemm_fused_kernel<kIn, kOut, TAIL, WAVES, TOut><<<tiles, WAVES * kWave, 0, stream>>>(a)
+    gemm_fused_kernel<kIn, kOut, TAIL, WAVES, TOut><<<tiles, WAVES * kWave, shared, stream>>>(a)
     // Measured at the 8B shapes: about one workgroup a compute unit (output and down projections) wants
     // sixteen waves to keep enough loads in flight; matrices with many rows want four waves when X has many
     // rows and eight when it has few.
@@ -273,6 +301,10 @@ extern "C" int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows
                   "gemm_fused: the norm input needs a gain and a positive eps");
     LEONE_REQUIRE(in_mode != kInPrepared || (squares_in && eps > 0.f),
                   "gemm_fused: the prepared input needs the sums of squares and a positive eps");
+    // the sums travel as 16-byte runs, eight to a thread of the smallest workgroup (256 threads)
+    LEONE_REQUIRE(in_mode != kInPrepared || (k % 64 == 0 && static_cast<long>(m) * (k / 64) <= 8 * 256 &&
+                                             reinterpret_cast<uintptr_t>(squares_in) % 16 == 0),
+                  "gemm_fused: the prepared input takes K %d a multiple of 64 with rows x K / 64 up to 2048", k);
     LEONE_REQUIRE(out_mode >= kOutStore && out_mode <= kOutPrepare, "gemm_fused: unknown output mode %d", out_mode);
     LEONE_REQUIRE(out_mode != kOutGated || n % 16 == 0, "gemm_fused: gated output needs N %d to be a multiple of 16", n);
     LEONE_REQUIRE(out_mode != kOutStore || out_dtype == kF32 || out_dtype == kBF16, "gemm_fused: unknown output type");

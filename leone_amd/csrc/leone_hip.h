@@ -60,6 +60,19 @@ int leone_attention_decode(const void* q, void* out, const void* k_pool, const v
                            float* part_ml, int rows, int q_heads, int kv_heads, int head_dim, int page_tokens,
                            float scale, int window, int splits, hipStream_t stream);
 
+// The same for a step in which every row is another request, from the fused q/k/v projection instead of finished
+// queries: the kernel normalises and rotates the query heads itself and, with write_cache, makes the new key,
+// and writes it and the new value into the cache before the keys are read (what leone_qk_norm_rope_write does,
+// without its launch).  qkv: bfloat16, or float32 in qkv_planes planes added up in order.  head_dim a multiple
+// of 64.  A row's keys must not be another row's new key: one row a request.
+int leone_attention_decode_projected(const void* qkv, int qkv_dtype, int qkv_planes, long qkv_plane, const void* q_gain,
+                                     const void* k_gain, int gain_dtype, float eps, const float* cos_table,
+                                     const float* sin_table, int table_positions, void* out, void* k_pool, void* v_pool,
+                                     int write_cache, const int* positions, const int* row_entry, const int* block_table,
+                                     int max_blocks, float* part_acc, float* part_ml, int rows, int q_heads, int kv_heads,
+                                     int head_dim, int page_tokens, float scale, int window, int splits,
+                                     hipStream_t stream);
+
 // Causal attention of prompt portions on the matrix cores for bfloat16.  `tiles` lists (entry, first
 // row, rows) for runs of at most leone_attention_prefill_tile_rows() consecutive rows of one request;
 // the rows of a tile sit at consecutive positions; leone_attention_prefill_group_tiles() tiles of one

@@ -250,6 +250,47 @@ def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
     return out
 
 
+def attention_decode_projected(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int,
+                               q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
+                               cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], k_pool: torch.Tensor,
+                               v_pool: torch.Tensor, positions: torch.Tensor, row_entry: torch.Tensor,
+                               block_table: torch.Tensor, scale: float, window: int = 0, max_context: int = 1,
+                               splits: Optional[int] = None, write_cache: bool = True) -> torch.Tensor:
+    """``qk_norm_rope_write`` and ``attention_decode`` in one launch, for a step in which every row is another
+    request (single decoded tokens): the kernel takes the fused q/k/v projection (bfloat16 ``[rows, width]``, or
+    float32 planes ``[p, rows, width]``), makes queries and the new key itself and writes key and value into
+    the cache before it reads the keys.  Head sizes that are multiples of 64."""
+    planes = qkv.shape[0] if qkv.dim() == 3 else 1
+    rows, width = qkv.shape[-2:]
+    pages, pool_heads, page_tokens, pool_dim = cache_dims(k_pool, v_pool)
+    if (pool_heads, pool_dim) != (kv_heads, head_dim) or width != (q_heads + 2 * kv_heads) * head_dim:
+        raise KernelError(f"attention_decode_projected: width {width} and pool {tuple(k_pool.shape)} do not fit "
+                          f"{q_heads}+2*{kv_heads} heads of {head_dim}")
+    if head_dim % 64:
+        raise KernelError(f"attention_decode_projected: head size {head_dim} is no multiple of 64")
+    if cos is not None and (cos.shape[1] != head_dim // 2 or sin is None or sin.shape != cos.shape):
+        raise KernelError("attention_decode_projected: rotary table does not fit the head size")
+    if q_gain is not None and (k_gain is None or k_gain.dtype != q_gain.dtype):
+        raise KernelError("attention_decode_projected: q and k gains must come together in one type")
+    if splits is None:
+        splits = choose_splits(rows, kv_heads, q_heads // kv_heads, max_context)
+    out = torch.empty((rows, q_heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    part_acc = part_ml = None
+    if splits > 1:
+        part_acc = torch.empty((rows * q_heads * splits * head_dim,), dtype=torch.float32, device=qkv.device)
+        part_ml = torch.empty((rows * q_heads * splits * 2,), dtype=torch.float32, device=qkv.device)
+    call("leone_attention_decode_projected", _dev(qkv, "qkv"), _code(qkv, "qkv"), planes, rows * width,
+         _dev(q_gain, "q gain", None, (head_dim,)), _dev(k_gain, "k gain", None, (head_dim,)),
+         _code(q_gain, "q gain") if q_gain is not None else F32, float(eps),
+         _dev(cos, "rope cos", torch.float32), _dev(sin, "rope sin", torch.float32), 0 if cos is None else cos.shape[0],
+         _dev(out, "attention out"), _dev(k_pool, "k pool", torch.bfloat16), _dev(v_pool, "v pool", torch.bfloat16),
+         1 if write_cache else 0, _dev(positions, "positions", torch.int32, (rows,)),
+         _dev(row_entry, "row map", torch.int32, (rows,)), _dev(block_table, "block table", torch.int32),
+         block_table.shape[1], _dev(part_acc, "partials"), _dev(part_ml, "partial sums"), rows, q_heads, kv_heads,
+         head_dim, page_tokens, float(scale), int(window), int(splits), _stream())
+    return out
+
+
 PREFILL_TILE_ROWS = 32       # rows of one request a wave of the prompt kernel takes (checked against the library)
 PREFILL_GROUP_TILES = 4      # tiles of one request a workgroup of the prompt kernel takes (likewise)
 PREFILL_MIN_ROWS = 16        # shorter portions go through the split-KV kernel row by row
@@ -374,6 +415,12 @@ class PreparedRows(NormedRows):
                  operand: torch.Tensor, squares: torch.Tensor, rows: Optional[torch.Tensor] = None):
         super().__init__(x, gain, eps, dtype, rows)
         self.operand, self.squares = operand, squares
+
+
+def prepared_fits(rows: int, hidden: int) -> bool:
+    """Whether ``gemm_fused`` takes rows of this width as ``PreparedRows`` (its sums of squares travel in
+    16-byte runs, at most 2,048 of them)."""
+    return hidden % 64 == 0 and rows * (hidden // 64) <= 2048
 
 
 def materialize(x) -> torch.Tensor:
@@ -568,8 +615,10 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
         # Every workgroup (16 weight rows) would redo a folded norm for its own use: that pays only for
         # matrices with few rows; for the others the norm kernel runs once and the product reads its result.
         if isinstance(x, NormedRows) and not isinstance(x, PreparedRows) and weight.shape[0] > FUSED_NORM_WEIGHT_ROWS:
-            x = x.prepare()                   # rounds where the folded norm rounds, whatever the weight's size
-        if next_norm is not None and (residual is None or weight.shape[0] % 8 or next_norm[2] != torch.bfloat16):
+            # rounds where the folded norm rounds, whatever the weight's size
+            x = x.prepare() if prepared_fits(rows, k) else x.materialize()
+        if next_norm is not None and (residual is None or not prepared_fits(rows, weight.shape[0])
+                                      or next_norm[2] != torch.bfloat16):
             next_norm = None
         return gemm_fused(x, weight, out_dtype, residual, gated, next_norm)
     x = materialize(x)

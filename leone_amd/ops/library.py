@@ -31,6 +31,8 @@ _PROTOTYPES = {
                                  c_int, c_int, c_int, c_int, c_int, c_int, P],
     "leone_attention_rows": [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                              c_int, P],
+    "leone_attention_decode_projected": [P, c_int, c_int, ctypes.c_long, P, P, c_int, c_float, P, P, c_int, P, P, P, c_int,
+                                         P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, P],
     "leone_attention_decode": [P, P, P, P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                c_int, P],
     "leone_attention_prefill": [P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P, P,

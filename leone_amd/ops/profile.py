@@ -25,6 +25,7 @@ OPERATIONS = {
     "leone_add_rmsnorm": "norm",
     "leone_qk_norm_rope_write": "qknorm rope kv",
     "leone_attention_decode": "attention",
+    "leone_attention_decode_projected": "attention",
     "leone_attention_rows": "attention",
     "leone_attention_prefill": "attention",
     "leone_gemm_fused_bf16": "gemv fused",

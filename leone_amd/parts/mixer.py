@@ -90,6 +90,16 @@ class GqaAttention(Part):
         cos, sin = self.position.tables() if self.position is not None else (None, None)
         if cos is not None and step.max_position >= cos.shape[0]:
             raise ValueError(f"position {step.max_position} is beyond the rotary table of {cos.shape[0]} positions")
+        if (step.decode_only and step.dtype == torch.bfloat16 and self.head_dim % 64 == 0
+                and ops.decode_attention_supported(step.dtype, self.head_dim, cache.page_tokens,
+                                                   self.q_heads // self.kv_heads, cache.block_table.shape[1])):
+            # Single decoded tokens, every row another request: the attention kernel makes the heads itself.
+            attended = ops.attention_decode_projected(
+                qkv, self.q_heads, self.kv_heads, self.head_dim, self.q_gain, self.k_gain,
+                self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin, cache.k_pool, cache.v_pool,
+                step.positions, step.row_entry, cache.block_table, self.scale, int(self.window or 0),
+                max_context=step.max_position + 1, write_cache=cache.writes)
+            return ops.linear(attended, self.w_o, residual=residual, next_norm=next_norm)
         q = ops.qk_norm_rope_write(qkv, self.q_heads, self.kv_heads, self.head_dim, self.q_gain, self.k_gain,
                                    self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin,
                                    step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,

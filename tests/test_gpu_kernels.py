@@ -789,7 +789,7 @@ def test_gemm_rows_gated(mfk):
 
 
 @pytest.mark.parametrize("gain_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("mnk", [(1, 4096, 4096), (7, 80, 176), (10, 1000, 64), (16, 4096, 12288)])
+@pytest.mark.parametrize("mnk", [(1, 4096, 4096), (7, 128, 176), (10, 960, 64), (16, 4096, 12288), (4, 5120, 5120)])
 def test_gemm_fused_prepares_the_next_norm(mnk, gain_dtype):
     """The product that adds into the stream leaves bf16(stream * gain) and partial sums of squares behind;
     the next product takes them in place of a norm kernel (the reference's fused norm + residual store,
@@ -830,3 +830,52 @@ def test_gemm_fused_prepares_the_next_norm(mnk, gain_dtype):
     got = ops.linear(prepared, ops.interleave_gate_up(wg, wu).contiguous(), gated=True)
     operand = prepared.operand.double()
     close(got, plain.swiglu((operand @ wg.double().T) * inv, (operand @ wu.double().T) * inv), 1e-2, 1e-2, "gated")
+
+
+@pytest.mark.parametrize("planes", [1, 3])
+@pytest.mark.parametrize("window", [0, 37])
+@pytest.mark.parametrize("shape", [(32, 8, 128, 64), (6, 1, 64, 16), (40, 2, 128, 32), (4, 4, 192, 16)])
+def test_attention_decode_from_the_projection(shape, window, planes):
+    """One launch for head norms, rotation, cache write and attention of single decoded tokens gives what the
+    two kernels give one after the other: the same cache contents bit for bit, the same output to the rounding
+    of the queries (a product and a sum may be contracted differently in the two kernels)."""
+    from leone_amd import ops
+    q_heads, kv_heads, dim, page = shape
+    torch.manual_seed(41)
+    lengths = [1, 5, page, page + 1, 3 * page + 7, 700]               # keys each row sees, its own included
+    rows = len(lengths)
+    blocks = -(-max(lengths) // page)
+    n_pages = rows * blocks + 2
+    order = torch.randperm(n_pages)[:rows * blocks].int().view(rows, blocks)
+    k_pool = (torch.randn(n_pages, kv_heads, dim // 8, page, 8) * 0.5).bfloat16().to(DEV)
+    v_pool = (torch.randn(n_pages, kv_heads, page // 8, dim, 8) * 0.5).bfloat16().to(DEV)
+    table = order.to(DEV).contiguous()
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32, device=DEV)
+    entry = torch.arange(rows, dtype=torch.int32, device=DEV)
+    width = (q_heads + 2 * kv_heads) * dim
+    if planes == 1:
+        qkv = torch.randn(rows, width, device=DEV).bfloat16()
+    else:
+        qkv = torch.randn(planes, rows, width, device=DEV) * torch.tensor([1.0, 0.02, 3e-4], device=DEV).view(3, 1, 1)
+    q_gain = (1 + 0.1 * torch.randn(dim, device=DEV)).bfloat16()
+    k_gain = (1 + 0.1 * torch.randn(dim, device=DEV)).bfloat16()
+    cos, sin = ops.rope_table(1e6, dim, 1024, DEV)
+    scale = 1 / math.sqrt(dim)
+    k1, v1, k2, v2 = k_pool.clone(), v_pool.clone(), k_pool.clone(), v_pool.clone()
+    q = ops.qk_norm_rope_write(qkv, q_heads, kv_heads, dim, q_gain, k_gain, 1e-6, cos, sin, positions, entry, table,
+                               k1, v1, out_dtype=torch.bfloat16)
+    want = ops.attention_decode(q, k1, v1, positions, entry, table, q_heads, scale, window, max_context=700)
+    got = ops.attention_decode_projected(qkv, q_heads, kv_heads, dim, q_gain, k_gain, 1e-6, cos, sin, k2, v2, positions,
+                                         entry, table, scale, window, max_context=700)
+    assert torch.equal(k1, k2) and torch.equal(v1, v2) and not torch.equal(k1, k_pool)
+    close(got, want.double(), 2e-2, 2e-2, "attention from the projection")
+    assert (got.double() - want.double()).abs().mean() < 2e-4
+    # a run that reads another run's cache writes nothing; no norm, no rotation
+    k3, v3 = k1.clone(), v1.clone()
+    plain_q = ops.qk_norm_rope_write(qkv, q_heads, kv_heads, dim, None, None, 1.0, None, None, positions, entry, table,
+                                     k3, v3, write_cache=False, out_dtype=torch.bfloat16)
+    want3 = ops.attention_decode(plain_q, k3, v3, positions, entry, table, q_heads, scale, window, max_context=700)
+    got3 = ops.attention_decode_projected(qkv, q_heads, kv_heads, dim, None, None, 1.0, None, None, k3, v3, positions,
+                                          entry, table, scale, window, max_context=700, write_cache=False)
+    assert torch.equal(k3, k1) and torch.equal(v3, v1)
+    assert torch.equal(got3, want3)                                   # nothing to contract: the same bits
