@@ -56,6 +56,9 @@ constexpr int kTileKeys = 32;
 __device__ inline bf16x8 load8(const bf16_t* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
+__device__ inline bf16x8 load8_streamed(const bf16_t* p) {   // keys and values: read once a step
+    return __builtin_bit_cast(bf16x8, load_streamed16(p));
+}
 __device__ inline bf16x8 zero8() {
     uint4 z = {0u, 0u, 0u, 0u};
     return __builtin_bit_cast(bf16x8, z);
@@ -336,11 +339,11 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         for (int s = 0; s < kSteps; ++s) {
             const bool in_head = 32 * s + 8 * g < kD;
             const long run = static_cast<long>(4 * s + g) * page_tokens * 8;   // elements 32s+8g .. +7 of the key
-            xa[s] = (va && in_head) ? load8(pk + run) : zero8();
-            xb[s] = (vb && in_head) ? load8(pk + run + 32) : zero8();           // four keys further
+            xa[s] = (va && in_head) ? load8_streamed(pk + run) : zero8();
+            xb[s] = (vb && in_head) ? load8_streamed(pk + run + 32) : zero8();           // four keys further
         }
 #pragma unroll
-        for (int dt = 0; dt < kD16; ++dt) xv[dt] = any ? load8(pv + (16 * dt + c) * 8) : zero8();
+        for (int dt = 0; dt < kD16; ++dt) xv[dt] = any ? load8_streamed(pv + (16 * dt + c) * 8) : zero8();
 
         // ---- S^T = K . Q^T for the two 16-key halves --------------------------------------------
         floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};

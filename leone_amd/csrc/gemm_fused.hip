@@ -62,6 +62,9 @@ __device__ inline bf16x8 fz8() {
 __device__ inline bf16x8 fld8(const bf16_t* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
+__device__ inline bf16x8 wld8(const bf16_t* p) {       // weights: read once
+    return __builtin_bit_cast(bf16x8, load_streamed16(p));
+}
 __device__ inline void gain8(const void* gain, int dtype, int at, float out[8]) {
     if (dtype == kF32) {
         const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(gain) + at);

@@ -48,6 +48,7 @@ struct RowsArgs {
 
 
 __device__ inline uint4 rld(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ inline uint4 wld(const bf16_t* p) { return load_streamed16(p); }   // weights: read once
 
 // kMT: tiles of 16 rows of X; kWaves: waves of a workgroup, each with one tile of 16 rows of W; kSteps: steps
 // of 64 elements a chunk.
