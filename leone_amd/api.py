@@ -59,8 +59,9 @@ class Runtime:
     def __init__(self, model, *, num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  page_tokens: int = 64, max_requests: int = 64, max_context: Optional[int] = None,
                  policy: Optional[SchedulerPolicy] = None, tokenizer=None, graphs: bool = True,
-                 poison_freed: bool = False):
+                 poison_freed: bool = False, streamed_weights: Optional[bool] = None):
         self.model = model
+        model.keep_streamed_copies(streamed_weights)       # before the cache is sized by what is free
         self.config = getattr(model, "config", None)
         context = min(max_context or model.spec.max_positions, model.spec.max_positions)
         if num_pages is None and max_tokens is None:
@@ -70,7 +71,7 @@ class Runtime:
             num_pages = default_num_pages(model, page_tokens, max_requests, context, per_token)
         self.engine = Engine(model, num_pages=num_pages, max_tokens=max_tokens, page_tokens=page_tokens,
                              max_requests=max_requests, max_context=context, graphs=graphs,
-                             poison_freed=poison_freed)
+                             poison_freed=poison_freed, streamed_weights=streamed_weights)
         self.policy = policy or SchedulerPolicy(max_live_requests=max_requests)
         self.tokenizer = tokenizer
         self.last_stats: Optional[GenerationStats] = None

@@ -82,8 +82,11 @@ def measure_peaks(device: str = "cuda:0", megabytes: int = 1024, repeats: int = 
         return found
 
     stream = ops._stream()
-    read_ms = best_ms(lambda: call("leone_peak_read", src.data_ptr(), count, sink.data_ptr(), 8 * units, stream))
-    copy_ms = best_ms(lambda: call("leone_peak_copy", src.data_ptr(), dst.data_ptr(), count, 8 * units, stream))
+    # how many workgroups a compute unit read fastest differs between a read and a copy: the best of a few
+    read_ms = min(best_ms(lambda: call("leone_peak_read", src.data_ptr(), count, sink.data_ptr(), per * units, stream))
+                  for per in (1, 2, 4, 8))
+    copy_ms = min(best_ms(lambda: call("leone_peak_copy", src.data_ptr(), dst.data_ptr(), count, per * units, stream))
+                  for per in (1, 2, 4, 8))
     blocks, iterations = 8 * units, 4000
     mfma_ms = best_ms(lambda: call("leone_peak_mfma", blocks, iterations, sink.data_ptr(), stream))
     flops = library().leone_peak_mfma_flops(blocks, iterations)
@@ -264,6 +267,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument("--no-kernels", action="store_true", help="skip the per-operation table of the decode step")
     parser.add_argument("--no-peaks", action="store_true", help="skip the measurement of this GPU's own peaks")
+    parser.add_argument("--no-streamed-weights", action="store_true",
+                        help="keep no second copy of the matrices in the decode kernels' order")
     parser.add_argument("--peaks", action="store_true", help="only measure this GPU's own peaks and print them")
     parser.add_argument("--scenario", choices=sorted(SCENARIOS), help="run a serving scenario instead of the headline figure")
     args = parser.parse_args(argv)
@@ -296,7 +301,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     largest = max([args.batch] + points_batches)
     pages = largest * (args.context // page_tokens + 1) + PREFILL_TOKENS // page_tokens
     engine = Engine(model, num_pages=pages, page_tokens=page_tokens, max_requests=largest + 1,
-                    max_context=args.context)
+                    max_context=args.context, streamed_weights=False if args.no_streamed_weights else None)
 
     peaks = None if args.no_peaks else measure_peaks()
     profile_steps = 0 if args.no_kernels else 4
@@ -317,12 +322,14 @@ def main(argv: Optional[List[str]] = None) -> int:
                    "head_dim": config.head_dim, "intermediate": config.intermediate_size, "vocab": config.vocab_size,
                    "global_batch": args.batch, "seq_len": args.context, "decode_start_context": start,
                    "prefill_tokens": PREFILL_TOKENS, "page_tokens": page_tokens, "rope_theta": config.rope_theta,
-                   "tied_head": config.tie_word_embeddings, "parallelism": "single GPU"},
+                   "tied_head": config.tie_word_embeddings, "parallelism": "single GPU",
+                   "weight_copies": 2 if model.streamed_copy_bytes else 1},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
     }
     weights = model.weight_accounting(rows=args.batch)
     record["bytes"] = {"weights_resident": weights["tensor_bytes"], "weights_a_step": sum(weights["decode"].values()),
+                       "weights_second_copy": weights["streamed_copy_bytes"],
                        "cache_a_token": cache_bytes_per_token(model), "a_step": int(step_bytes)}
     if peaks is not None:
         record["peaks_measured"] = peaks

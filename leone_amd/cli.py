@@ -88,6 +88,8 @@ def build_parser() -> argparse.ArgumentParser:
     g.add_argument("--debug-tokens", help="File that receives the generated ids as a JSON list")
     g.add_argument("--debug-logits", help="File that receives, step by step, the five largest logits with their bits")
     g.add_argument("--ignore-eos", action="store_true", help="Do not stop at the end token")
+    g.add_argument("--single-weight-copy", action="store_true",
+                   help="Keep no second copy of the matrices in the decode kernels' order (half the weight memory, slower decoding)")
     _add_sampling(g)
 
     d = sub.add_parser("doctor", help="Check the platform, the kernel library and a model folder")
@@ -133,6 +135,7 @@ def cmd_generate(args) -> int:
         raise SystemExit("error: give exactly one of -p/--prompt and --prompt-tokens")
     runtime = Runtime.load(args.model, args.dtype, max_requests=1, max_context=args.max_context,
                            graphs=not args.eager_decode,
+                           streamed_weights=False if args.single_weight_copy else None,
                            policy=SchedulerPolicy(max_live_requests=1, prefill_chunk_tokens=args.prefill_chunk,
                                                   max_step_tokens=max(args.prefill_chunk, 1)))
     if args.prompt is not None:
@@ -239,9 +242,16 @@ def cmd_doctor(args) -> int:
         per_token = sum(2 * need.kv_heads * need.head_dim * size for need in model.cache_needs().values()
                         if hasattr(need, "kv_heads"))
         print(f"cache bytes per token ({args.dtype}): {per_token}")
+        # the second copy of the matrices that decode steps read (kept for bfloat16 when there is ample room)
+        second = sum(v for family, v in accounting["decode"].items() if family not in ("embed", "norm"))
+        second = second if args.dtype == "bfloat16" and model.spec.hidden_size % 64 == 0 else 0
+        print(f"second copy of the matrices in the decode kernels' order: {second / 2**20:.1f} MiB "
+              f"(kept if that is at most {model.STREAMED_SHARE_OF_DEVICE:.0%} of the device's memory)")
         if torch.cuda.is_available():
-            free, _ = torch.cuda.mem_get_info(0)
+            free, device_total = torch.cuda.mem_get_info(0)
             room = free - total * (2 if args.dtype == "float32" else 1)
+            if second <= model.STREAMED_SHARE_OF_DEVICE * device_total and second <= model.STREAMED_SHARE_OF_FREE * room:
+                room -= second
             print(f"tokens of context that fit beside the weights: {max(0, int(room * 0.9) // max(1, per_token))}")
         if args.probe:
             from .runtime import load_model

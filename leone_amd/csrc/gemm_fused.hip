@@ -62,9 +62,6 @@ __device__ inline bf16x8 fz8() {
 __device__ inline bf16x8 fld8(const bf16_t* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
-__device__ inline bf16x8 wld8(const bf16_t* p) {       // weights: read once
-    return __builtin_bit_cast(bf16x8, load_streamed16(p));
-}
 __device__ inline void gain8(const void* gain, int dtype, int at, float out[8]) {
     if (dtype == kF32) {
         const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(gain) + at);
@@ -82,7 +79,7 @@ __device__ inline void gain8(const void* gain, int dtype, int at, float out[8]) 
     }
 }
 
-template <int kIn, int kOut, bool kTail, int kWaves, typename TOut>
+template <int kIn, int kOut, bool kTail, int kWaves, typename TOut, bool kTiled>
 __global__ void __launch_bounds__(kWaves * kWave)
 gemm_fused_kernel(FusedArgs a) {
     __shared__ float partial[kWaves][kWave][4];
@@ -94,7 +91,15 @@ gemm_fused_kernel(FusedArgs a) {
     const long n0 = static_cast<long>(blockIdx.x) * 16;
     // Rows past the end are clamped: they only feed output rows and columns that are never stored.
     const long wr = n0 + c < n ? n0 + c : n - 1;
-    const bf16_t* wrow = a.w + wr * k + 16 * g;
+    // Row-major weights: this lane's 32 bytes of step s lie at 64 s + 16 g of its row.  Tiled weights: the 16
+    // bytes of lane L for half h of step s lie at ((s * 2 + h) * 64 + L) * 16 in the tile, so that every load of
+    // a wave is 1 KB in one piece; such loads may carry the non-temporal hint.
+    const bf16_t* wrow = kTiled ? a.w + static_cast<long>(blockIdx.x) * (k / 64) * 1024 + lane * 8 : a.w + wr * k + 16 * g;
+    constexpr int kStepStride = kTiled ? 1024 : 64, kHalfStride = kTiled ? 512 : 8;
+    auto wld = [&](int s, int h) {
+        const bf16_t* p = wrow + static_cast<long>(s) * kStepStride + h * kHalfStride;
+        return kTiled ? __builtin_bit_cast(bf16x8, load_streamed16(p)) : fld8(p);
+    };
     float ss = 0.f;
     const int xr = c < m ? c : m - 1;
     const long xrow_index = (kIn == kInNorm && a.rows) ? a.rows[xr] : xr;
@@ -147,16 +152,16 @@ gemm_fused_kernel(FusedArgs a) {
         bf16x8 wa[kUnroll][2];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            wa[u][0] = fld8(wrow + 64 * (s + u));
-            wa[u][1] = fld8(wrow + 64 * (s + u) + 8);
+            wa[u][0] = wld(s + u, 0);
+            wa[u][1] = wld(s + u, 1);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) step(s + u, wa[u][0], wa[u][1], false);
     }
-    for (; s < s_end; ++s) step(s, fld8(wrow + 64 * s), fld8(wrow + 64 * s + 8), false);
+    for (; s < s_end; ++s) step(s, wld(s, 0), wld(s, 1), false);
     if (kTail && wave == kWaves - 1) {                 // the last wave also takes the step that holds the end of K
         const int left = k - (64 * whole + 16 * g);
-        step(whole, left >= 8 ? fld8(wrow + 64 * whole) : fz8(), left >= 16 ? fld8(wrow + 64 * whole + 8) : fz8(), true);
+        step(whole, left >= 8 ? wld(whole, 0) : fz8(), left >= 16 ? wld(whole, 1) : fz8(), true);
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) partial[wave][lane][r] = acc[r];
@@ -263,14 +268,17 @@ gemm_fused_kernel(FusedArgs a) {
 }
 
 template <int kIn, int kOut, typename TOut>
-static void launch_fused(const FusedArgs& a, hipStream_t stream) {
+static void launch_fused(const FusedArgs& a, bool tiled, hipStream_t stream) {
     const int tiles = ceil_div(a.n, 16);
     const int steps = ceil_div(a.k, 64);
     const bool tail = a.k % 64 != 0;
     const bool many = tiles * 4 >= 4096 || steps < 16;    // workgroups enough to fill the chip, or too little of K to split further
     const size_t shared = kIn == kInPrepared ? static_cast<size_t>(a.m) * (a.k / 16) * sizeof(float) : 0;
-#define LEONE_FUSED(TAIL, WAVES) \
-    gemm_fused_kernel<kIn, kOut, TAIL, WAVES, TOut><<<tiles, WAVES * kWave, shared, stream>>>(a)
+#define LEONE_FUSED(TAIL, WAVES)                                                                                  \
+    do {                                                                                                          \
+        if (tiled) gemm_fused_kernel<kIn, kOut, false, WAVES, TOut, true><<<tiles, WAVES * kWave, shared, stream>>>(a); \
+        else gemm_fused_kernel<kIn, kOut, TAIL, WAVES, TOut, false><<<tiles, WAVES * kWave, shared, stream>>>(a);  \
+    } while (0)
     // Measured at the 8B shapes: about one workgroup a compute unit (output and down projections) wants
     // sixteen waves to keep enough loads in flight; matrices with many rows want four waves when X has many
     // rows and eight when it has few.
@@ -293,10 +301,12 @@ using namespace leone;
 // out_mode: 0 store (y of out_dtype [m,n]), 1 residual (y float32 [m,n] += product), 2 gated (y bfloat16 [m,n/2]),
 // 3 prepare (as 1, and operand_out bfloat16 [m,n] = bf16(y * next_gain), squares_out float32 [m, ceil(n / 16)]).
 extern "C" int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const void* gain, int gain_dtype,
-                                     float eps, const void* w, void* y, int out_mode, int out_dtype, int m, int n,
+                                     float eps, const void* w, int w_tiled, void* y, int out_mode, int out_dtype, int m, int n,
                                      int k, const float* squares_in, void* operand_out, float* squares_out,
                                      const void* next_gain, int next_gain_dtype, hipStream_t stream) {
     LEONE_REQUIRE(x && w && y, "gemm_fused: null pointer");
+    LEONE_REQUIRE(!w_tiled || (k % 64 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0),
+                  "gemm_fused: tiled weights need K %d to be a multiple of 64", k);
     LEONE_REQUIRE(m > 0 && m <= 16, "gemm_fused: rows %d must be in 1..16", m);
     LEONE_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_fused: sizes %d x %d: K must be a positive multiple of 8", n, k);
     LEONE_REQUIRE(in_mode >= kInPlain && in_mode <= kInPrepared, "gemm_fused: unknown input mode %d", in_mode);
@@ -319,12 +329,12 @@ extern "C" int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows
 #define LEONE_FUSED_OUT(IN)                                                                  \
     switch (out_mode) {                                                                      \
         case kOutStore:                                                                      \
-            if (out_dtype == kF32) launch_fused<IN, kOutStore, float>(a, stream);            \
-            else launch_fused<IN, kOutStore, bf16_t>(a, stream);                             \
+            if (out_dtype == kF32) launch_fused<IN, kOutStore, float>(a, w_tiled != 0, stream);            \
+            else launch_fused<IN, kOutStore, bf16_t>(a, w_tiled != 0, stream);                             \
             break;                                                                           \
-        case kOutResidual: launch_fused<IN, kOutResidual, float>(a, stream); break;          \
-        case kOutPrepare: launch_fused<IN, kOutPrepare, float>(a, stream); break;            \
-        default: launch_fused<IN, kOutGated, bf16_t>(a, stream); break;                      \
+        case kOutResidual: launch_fused<IN, kOutResidual, float>(a, w_tiled != 0, stream); break;          \
+        case kOutPrepare: launch_fused<IN, kOutPrepare, float>(a, w_tiled != 0, stream); break;            \
+        default: launch_fused<IN, kOutGated, bf16_t>(a, w_tiled != 0, stream); break;                      \
     }
     if (in_mode == kInPlain) {
         LEONE_FUSED_OUT(kInPlain)

@@ -39,7 +39,7 @@ enum RowsOut : int { kRowsStore = 0, kRowsResidual = 1, kRowsGated = 2, kRowsPla
 
 struct RowsArgs {
     const bf16_t* x;   // [M,K]
-    const bf16_t* w;   // [N,K]
+    const bf16_t* w;   // [N,K], or its tiled copy
     void* y;
     long plane;        // elements between two planes of y (kRowsPlanes)
     int m, n, k;
@@ -52,7 +52,7 @@ __device__ inline uint4 wld(const bf16_t* p) { return load_streamed16(p); }   //
 
 // kMT: tiles of 16 rows of X; kWaves: waves of a workgroup, each with one tile of 16 rows of W; kSteps: steps
 // of 64 elements a chunk.
-template <int kMT, int kWaves, int kSteps, int kDepth, int kOut, typename TOut>
+template <int kMT, int kWaves, int kSteps, int kDepth, int kOut, typename TOut, bool kTiled>
 __global__ void __launch_bounds__(kWaves * kWave)
 gemm_rows_kernel(RowsArgs a) {
     constexpr int kChunk = 64 * kSteps;              // elements of K a chunk
@@ -74,6 +74,11 @@ gemm_rows_kernel(RowsArgs a) {
     const long tile = static_cast<long>(blockIdx.x) * kWaves + wave;
     const long wr = 16 * tile + c;
     const bf16_t* wrow = a.w + (wr < n ? wr : n - 1) * k;
+    // Tiled weights: the 16 bytes of lane L for half h of step S of a tile lie at ((S * 2 + h) * 64 + L) * 16 in
+    // the tile, so that every load of a wave is 1 KB in one piece; K is a multiple of 64 there.
+    const int all_steps = k / 64;
+    const long tiles_n = (n + 15) / 16;
+    const bf16_t* wtile = a.w + (tile < tiles_n ? tile : tiles_n - 1) * all_steps * 1024 + lane * 8;
     // The runs of X this thread copies: copy i is run (i * threads + tid) % kRuns of row (i * threads + tid) / kRuns.
     const bf16_t* xsrc[kCopies];
     int xdst[kCopies], xcol[kCopies];
@@ -107,8 +112,13 @@ gemm_rows_kernel(RowsArgs a) {
         }
     };
     auto w_at = [&](int ch, int u) {
-        const int at = ch * kChunk + 16 * g + 64 * (u >> 1) + 8 * (u & 1);
-        return rld(wrow + (at + 8 <= k ? at : k - 8));
+        if constexpr (kTiled) {
+            const int step = ch * kSteps + (u >> 1);
+            return load_streamed16(wtile + static_cast<long>(step < all_steps ? step : all_steps - 1) * 1024 + 512 * (u & 1));
+        } else {
+            const int at = ch * kChunk + 16 * g + 64 * (u >> 1) + 8 * (u & 1);
+            return rld(wrow + (at + 8 <= k ? at : k - 8));
+        }
     };
     auto deposit = [&](uint4* to, const uint4 (&xn)[kCopies], int ch) {
         const int k0 = ch * kChunk;
@@ -227,13 +237,13 @@ gemm_rows_kernel(RowsArgs a) {
     }
 }
 
-template <int kMT, int kWaves, int kDepth, int kOut, typename TOut>
-static int launch_rows(const RowsArgs& a, int splits, hipStream_t stream) {
+template <int kMT, int kWaves, int kDepth, int kOut, typename TOut, bool kTiled>
+static int launch_rows_laid(const RowsArgs& a, int splits, hipStream_t stream) {
     constexpr int kSteps = kMT <= 4 ? 4 : 2;
     const size_t shared = 2 * static_cast<size_t>(16 * kMT) * (64 * kSteps / 8) * sizeof(uint4);
     static size_t allowed = 48 * 1024;                 // what a kernel may use without asking
     if (shared > allowed) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_rows_kernel<kMT, kWaves, kSteps, kDepth, kOut, TOut>),
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_rows_kernel<kMT, kWaves, kSteps, kDepth, kOut, TOut, kTiled>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shared));
         if (e != hipSuccess) {
             set_error("gemm_rows: %zu bytes of shared memory were refused: %s", shared, hipGetErrorString(e));
@@ -242,28 +252,35 @@ static int launch_rows(const RowsArgs& a, int splits, hipStream_t stream) {
         allowed = shared;
     }
     const int groups = ceil_div(a.n, 16 * kWaves);
-    gemm_rows_kernel<kMT, kWaves, kSteps, kDepth, kOut, TOut><<<dim3(groups, splits), kWaves * kWave, shared, stream>>>(a);
+    gemm_rows_kernel<kMT, kWaves, kSteps, kDepth, kOut, TOut, kTiled><<<dim3(groups, splits), kWaves * kWave, shared, stream>>>(a);
     return 0;
 }
 
+template <int kMT, int kWaves, int kDepth, int kOut, typename TOut>
+static int launch_rows(const RowsArgs& a, int splits, bool tiled, hipStream_t stream) {
+    return tiled ? launch_rows_laid<kMT, kWaves, kDepth, kOut, TOut, true>(a, splits, stream)
+                 : launch_rows_laid<kMT, kWaves, kDepth, kOut, TOut, false>(a, splits, stream);
+}
+
 template <int kMT, int kWaves, int kDepth>
-static int launch_rows_out(const RowsArgs& a, int out_mode, int out_dtype, int splits, hipStream_t stream) {
+static int launch_rows_out(const RowsArgs& a, int out_mode, int out_dtype, int splits, bool tiled, hipStream_t stream) {
     switch (out_mode) {
         case kRowsStore:
-            return out_dtype == kF32 ? launch_rows<kMT, kWaves, kDepth, kRowsStore, float>(a, splits, stream)
-                                     : launch_rows<kMT, kWaves, kDepth, kRowsStore, bf16_t>(a, splits, stream);
-        case kRowsResidual: return launch_rows<kMT, kWaves, kDepth, kRowsResidual, float>(a, splits, stream);
-        case kRowsGated: return launch_rows<kMT, kWaves, kDepth, kRowsGated, bf16_t>(a, splits, stream);
-        default: return launch_rows<kMT, kWaves, kDepth, kRowsPlanes, float>(a, splits, stream);
+            return out_dtype == kF32 ? launch_rows<kMT, kWaves, kDepth, kRowsStore, float>(a, splits, tiled, stream)
+                                     : launch_rows<kMT, kWaves, kDepth, kRowsStore, bf16_t>(a, splits, tiled, stream);
+        case kRowsResidual: return launch_rows<kMT, kWaves, kDepth, kRowsResidual, float>(a, splits, tiled, stream);
+        case kRowsGated: return launch_rows<kMT, kWaves, kDepth, kRowsGated, bf16_t>(a, splits, tiled, stream);
+        default: return launch_rows<kMT, kWaves, kDepth, kRowsPlanes, float>(a, splits, tiled, stream);
     }
 }
 
 template <int kMT>
-static int launch_rows_waves(const RowsArgs& a, int out_mode, int out_dtype, int splits, int waves, hipStream_t stream) {
+static int launch_rows_waves(const RowsArgs& a, int out_mode, int out_dtype, int splits, int waves, bool tiled,
+                             hipStream_t stream) {
     switch (waves) {
-        case 4: return launch_rows_out<kMT, 4, 1>(a, out_mode, out_dtype, splits, stream);
-        case 6: return launch_rows_out<kMT, 6, 1>(a, out_mode, out_dtype, splits, stream);
-        default: return launch_rows_out<kMT, 8, 1>(a, out_mode, out_dtype, splits, stream);
+        case 4: return launch_rows_out<kMT, 4, 1>(a, out_mode, out_dtype, splits, tiled, stream);
+        case 6: return launch_rows_out<kMT, 6, 1>(a, out_mode, out_dtype, splits, tiled, stream);
+        default: return launch_rows_out<kMT, 8, 1>(a, out_mode, out_dtype, splits, tiled, stream);
     }
 }
 
@@ -274,15 +291,18 @@ using namespace leone;
 extern "C" int leone_gemm_rows_max_rows() { return 128; }
 extern "C" int leone_gemm_rows_chunk(int m) { return m <= 64 ? 256 : 128; }
 
-// x bfloat16 [m,k], w bfloat16 [n,k], m in 1..128, k a multiple of 8.  out_mode 0: y[m,n] of out_dtype;
+// x bfloat16 [m,k], w bfloat16 [n,k] (or, with w_tiled, what leone_weight_tiles made of it; k a multiple of 64
+// then), m in 1..128, k a multiple of 8.  out_mode 0: y[m,n] of out_dtype;
 // 1: y float32 [m,n] += product; 2: w interleaves 8 gate rows with their 8 up rows (n a multiple of 16),
 // y bfloat16 [m,n/2] = silu(gate) * up; 3: y float32 [splits][m,n], `plane` elements apart, the product over
 // the s-th range of k in plane s (every plane is written whole).  splits must be 1 unless out_mode is 3; the
 // ranges are whole chunks of k and none may be empty.  waves (4, 6 or 8): 16 * waves rows of w a
 // workgroup, a tuning choice; the result does not depend on it beyond the order of the sum over k.
-extern "C" int leone_gemm_rows_bf16(const void* x, const void* w, void* y, int out_mode, int out_dtype, int m, int n,
-                                    int k, int splits, long plane, int waves, hipStream_t stream) {
+extern "C" int leone_gemm_rows_bf16(const void* x, const void* w, int w_tiled, void* y, int out_mode, int out_dtype,
+                                    int m, int n, int k, int splits, long plane, int waves, hipStream_t stream) {
     LEONE_REQUIRE(x && w && y, "gemm_rows: null pointer");
+    LEONE_REQUIRE(!w_tiled || (k % 64 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0),
+                  "gemm_rows: tiled weights need K %d to be a multiple of 64", k);
     LEONE_REQUIRE(m > 0 && m <= 128, "gemm_rows: rows %d must be in 1..128", m);
     LEONE_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_rows: sizes %d x %d: K must be a positive multiple of 8", n, k);
     LEONE_REQUIRE(out_mode >= kRowsStore && out_mode <= kRowsPlanes, "gemm_rows: unknown output mode %d", out_mode);
@@ -299,7 +319,7 @@ extern "C" int leone_gemm_rows_bf16(const void* x, const void* w, void* y, int o
     RowsArgs a{static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, plane, m, n, k, per};
     int status = 0;
 #define LEONE_ROWS_CASE(MT) \
-    case MT: status = launch_rows_waves<MT>(a, out_mode, out_dtype, splits, waves, stream); break;
+    case MT: status = launch_rows_waves<MT>(a, out_mode, out_dtype, splits, waves, w_tiled != 0, stream); break;
     const int tiles = ceil_div(m, 16);
     switch (tiles <= 4 ? tiles : tiles <= 6 ? 6 : 8) {
         LEONE_ROWS_CASE(1) LEONE_ROWS_CASE(2) LEONE_ROWS_CASE(3) LEONE_ROWS_CASE(4) LEONE_ROWS_CASE(6) LEONE_ROWS_CASE(8)

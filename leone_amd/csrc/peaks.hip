@@ -13,7 +13,10 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 constexpr int kPeakThreads = 256;
 constexpr int kPeakUnroll = 8;
 
-// Every thread reads runs of 16 bytes, kPeakUnroll of them in flight, a workgroup's reads side by side.
+// Every thread reads runs of 16 bytes, kPeakUnroll of them in flight, a workgroup's reads side by side: every
+// instruction covers whole lines, and the loads carry the non-temporal hint (a tenth faster than plain loads for
+// data that is read once; measured 7.0-7.1 TB/s with one or two workgroups a compute unit, 6.1-6.4 without the
+// hint, 5.1 with eight workgroups a unit).
 __global__ void __launch_bounds__(kPeakThreads)
 peak_read_kernel(const uint4* __restrict__ src, long runs, unsigned* __restrict__ sink) {
     const long stride = static_cast<long>(gridDim.x) * kPeakThreads;
@@ -22,7 +25,7 @@ peak_read_kernel(const uint4* __restrict__ src, long runs, unsigned* __restrict_
     for (; at + (kPeakUnroll - 1) * stride < runs; at += kPeakUnroll * stride) {
         uint4 v[kPeakUnroll];
 #pragma unroll
-        for (int u = 0; u < kPeakUnroll; ++u) v[u] = src[at + u * stride];
+        for (int u = 0; u < kPeakUnroll; ++u) v[u] = load_streamed16(src + at + u * stride);
 #pragma unroll
         for (int u = 0; u < kPeakUnroll; ++u) seen ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
     }
@@ -40,7 +43,7 @@ peak_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, long ru
     for (; at + (kPeakUnroll - 1) * stride < runs; at += kPeakUnroll * stride) {
         uint4 v[kPeakUnroll];
 #pragma unroll
-        for (int u = 0; u < kPeakUnroll; ++u) v[u] = src[at + u * stride];
+        for (int u = 0; u < kPeakUnroll; ++u) v[u] = load_streamed16(src + at + u * stride);
 #pragma unroll
         for (int u = 0; u < kPeakUnroll; ++u) dst[at + u * stride] = v[u];
     }

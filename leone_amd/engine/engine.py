@@ -156,11 +156,14 @@ class _DecodeGraph:
 class Engine:
     def __init__(self, model: DecoderModel, *, num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  page_tokens: int = 64, max_requests: int = 64, max_context: Optional[int] = None,
-                 poison_freed: bool = False, graphs: bool = True):
+                 poison_freed: bool = False, graphs: bool = True, streamed_weights: Optional[bool] = None):
         if model.embedding is None:
             raise ValueError("the model has no weights bound")
         if not torch.cuda.is_available() or model.device.type != "cuda":
             raise RuntimeError("the engine runs on a GPU only; there is no CPU path")
+        # A second copy of the matrices in the order the decode kernels read fastest: by default if there is
+        # ample room (``DecoderModel.keep_streamed_copies``); before the pools take their memory.
+        model.keep_streamed_copies(streamed_weights)
         self.model = model
         self.device = model.device
         self.dtype = model.dtype

@@ -8,6 +8,8 @@ from __future__ import annotations
 
 from typing import Optional
 
+import weakref
+
 import numpy as np
 import torch
 
@@ -436,6 +438,47 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return torch.stack([gate.view(ffn // 8, 8, hidden), up.view(ffn // 8, 8, hidden)], dim=1).reshape(2 * ffn, hidden)
 
 
+def tile_weight(weight: torch.Tensor) -> torch.Tensor:
+    """The copy of ``weight[N, K]`` (bfloat16, K a multiple of 64) that the weight-streaming products read
+    fastest: rows in tiles of 16 (the last filled up with zero rows), K in steps of 64, a step in two halves;
+    element e of lane 16 g + c in half h of step s of tile t is ``weight[16 t + c][64 s + 16 g + 8 h + e]``, so
+    ``[tiles, K / 64, 2, 4, 16, 8]``.  Each load of a wave is then 1 KB in one piece."""
+    n, k = weight.shape
+    if weight.dtype != torch.bfloat16 or k % 64:
+        raise KernelError(f"tile_weight: a bfloat16 matrix with K a multiple of 64 is needed, not {weight.dtype} with K {k}")
+    tiles = -(-n // 16)
+    if tiles * 16 != n:
+        weight = torch.cat([weight, weight.new_zeros((tiles * 16 - n, k))])
+    return weight.view(tiles, 16, k // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
+
+
+_streamed: dict = {}         # (address, shape) of a weight -> (weak reference to the weight, its tiled copy)
+
+
+def keep_streamed_copy(weight: torch.Tensor) -> int:
+    """Makes and keeps the tiled copy of a weight; the products take it from then on whenever they are given
+    this weight, and it is dropped when the weight is.  Returns the copy's bytes (0 if the weight's shape or
+    type has no tiled form)."""
+    if weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.shape[1] % 64 or not weight.is_cuda:
+        return 0
+    key = (weight.data_ptr(), tuple(weight.shape))
+    held = _streamed.get(key)
+    if held is None or held[0]() is not weight:
+        def forget(_, key=key):
+            _streamed.pop(key, None)
+        _streamed[key] = (weakref.ref(weight, forget), tile_weight(weight))
+    return _streamed[key][1].numel() * 2
+
+
+def streamed_copy(weight: torch.Tensor) -> Optional[torch.Tensor]:
+    held = _streamed.get((weight.data_ptr(), tuple(weight.shape)))
+    return None if held is None or held[0]() is not weight else held[1]
+
+
+def drop_streamed_copies() -> None:
+    _streamed.clear()
+
+
 def gemm_fused(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
                residual: Optional[torch.Tensor] = None, gated: bool = False, next_norm=None):
     """The product for at most 16 rows with its neighbours folded in: ``x`` may be ``NormedRows`` or
@@ -471,10 +514,12 @@ def gemm_fused(x, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
         source, in_mode = _dev(x.x, "stream", torch.float32), 1
     else:
         source, in_mode = _dev(x, "gemm x", torch.bfloat16, (m, k)), 0
+    tiles = streamed_copy(weight) if _streamed else None
     with profile.span("gemv fused", weight):
         call("leone_gemm_fused_bf16", source, in_mode, _dev(x.rows, "rows", torch.int32) if normed else 0,
              _dev(x.gain, "gain", None, (k,)) if normed else 0, _code(x.gain, "gain") if normed else 0,
-             x.eps if (normed or prepared) else 0.0, _dev(weight, "gemm weight", torch.bfloat16),
+             x.eps if (normed or prepared) else 0.0,
+             _dev(weight if tiles is None else tiles, "gemm weight", torch.bfloat16), 0 if tiles is None else 1,
              _dev(out, "gemm out", out_dtype, (m, n // 2 if gated else n)), mode, _CODES[out_dtype], m, n, k,
              x.squares.data_ptr() if prepared else 0, _dev(operand, "operand out"), _dev(squares, "sums out"),
              _dev(next_norm[0], "next gain", None, (n,)) if next_norm is not None else 0,
@@ -563,9 +608,11 @@ def gemm_rows(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = to
         out, mode, kind = torch.empty((m, n // 2), dtype=torch.bfloat16, device=weight.device), 2, torch.bfloat16
     else:
         out, mode, kind = torch.empty((m, n), dtype=out_dtype, device=weight.device), 0, out_dtype
+    tiles = streamed_copy(weight) if _streamed else None
     with profile.span("gemm rows", weight):
         call("leone_gemm_rows_bf16", _dev(x, "gemm x", torch.bfloat16, (m, k)),
-             _dev(weight, "gemm weight", torch.bfloat16), _dev(out, "gemm out", kind), mode, _CODES[kind], m, n, k,
+             _dev(weight if tiles is None else tiles, "gemm weight", torch.bfloat16), 0 if tiles is None else 1,
+             _dev(out, "gemm out", kind), mode, _CODES[kind], m, n, k,
              splits, plane, int(waves), _stream())
     return None if (residual is not None and splits == 1) else out
 

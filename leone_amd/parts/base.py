@@ -196,3 +196,9 @@ class Part:
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         pass
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        """The matrices this part hands to ``ops.linear`` as weights in decode steps, every one streamed
+        through once a step: the model may keep a second copy of them in the order the weight-streaming
+        kernels read fastest (``ops.keep_streamed_copy``).  Naming none is always right."""
+        return []

@@ -40,6 +40,9 @@ class PreNormBlock(Part):
         for part in self.parts():
             part.bind(tensors)
 
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [w for part in self.parts() if hasattr(part, "streamed_weights") for w in part.streamed_weights()]
+
     def cache_need(self):
         return self.mixer.cache_need()
 

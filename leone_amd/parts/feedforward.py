@@ -50,6 +50,9 @@ class SwiGluMlp(Part):
         self.w_gate_up = ops.interleave_gate_up(gate, up).contiguous()
         self.w_down = down.contiguous()
 
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.w_gate_up, self.w_down]
+
     def forward(self, y, step: StepContext, residual: Optional[torch.Tensor] = None, next_norm=None):
         """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned),
         and with ``next_norm`` the norm that follows may come back prepared (see ``ops.linear``)."""

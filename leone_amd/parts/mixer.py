@@ -79,6 +79,9 @@ class GqaAttention(Part):
             if self.q_gain.dtype != self.k_gain.dtype:
                 self.q_gain, self.k_gain = self.q_gain.float(), self.k_gain.float()
 
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.w_qkv, self.w_o]
+
     fused_io = True
     prepares_next = True
 

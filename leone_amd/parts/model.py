@@ -64,6 +64,7 @@ class DecoderModel:
                 raise ValueError(f"schedule names layer {run.layer}, the model has {len(self.layers)}")
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
+        self.streamed_copy_bytes: Optional[int] = None    # None: not decided yet (``keep_streamed_copies``)
 
     @property
     def graph_safe(self) -> bool:
@@ -90,6 +91,40 @@ class DecoderModel:
         self.final_norm.bind(tensors)
         for position in self.positions.values():
             position.prepare(self.spec.max_positions, self.device)
+
+    # Auto: keep the second copies if they take at most this share of the device's memory and of what is free.
+    STREAMED_SHARE_OF_DEVICE = 0.25
+    STREAMED_SHARE_OF_FREE = 0.5
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        """Every matrix a decode step streams through ``ops.linear``: the layers' and the head."""
+        found = [w for layer in self.layers if hasattr(layer, "streamed_weights") for w in layer.streamed_weights()]
+        if self.head is not None:
+            found.append(self.head)
+        return found
+
+    def keep_streamed_copies(self, wanted: Optional[bool] = None) -> int:
+        """Keeps, beside every matrix that decode steps stream through, a second copy in the order in which
+        the weight-streaming kernels read it fastest (``ops.tile_weight``; the row-major one stays for the
+        library's products of prompt portions and for the token table).  The results are the same bit for
+        bit; a decode step of few rows takes a sixth less time; the weights take twice the memory.
+        ``wanted`` None decides by room: yes if the copies take at most a quarter of the device's memory
+        and half of what is free.  Returns the bytes the copies take (0: none kept).  Asked again, it
+        answers what it did the first time."""
+        if self.streamed_copy_bytes is not None:
+            return self.streamed_copy_bytes
+        self.streamed_copy_bytes = 0
+        weights = self.streamed_weights() if (self.dtype == torch.bfloat16 and wanted is not False) else []
+        weights = [w for w in weights if w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] % 64 == 0]
+        if not weights:
+            return 0
+        if wanted is None:
+            needed = sum(-(-w.shape[0] // 16) * 16 * w.shape[1] * 2 for w in weights)
+            free, total = torch.cuda.mem_get_info(weights[0].device)
+            if needed > self.STREAMED_SHARE_OF_DEVICE * total or needed > self.STREAMED_SHARE_OF_FREE * free:
+                return 0
+        self.streamed_copy_bytes = sum(ops.keep_streamed_copy(w) for w in weights)
+        return self.streamed_copy_bytes
 
     def row_tilings(self) -> list:
         """Every distinct tiling a part of the model declares, in a fixed order (``RowTiling``)."""
@@ -128,7 +163,8 @@ class DecoderModel:
         decode["embed"] = resident["embed"] // self.spec.vocab_size * rows
         if self.spec.head is None:
             decode["head"] = resident["embed"]
-        return {"tensor_bytes": sum(resident.values()), "resident": resident, "decode": decode}
+        return {"tensor_bytes": sum(resident.values()), "resident": resident, "decode": decode,
+                "streamed_copy_bytes": self.streamed_copy_bytes or 0}
 
     def weight_bytes(self) -> int:
         """Bytes of all tensors of the model."""

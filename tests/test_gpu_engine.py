@@ -468,6 +468,36 @@ def test_twenty_live_requests_decoding_side_by_side(tmp_path, name, dtype_name):
     compare(steps, outputs, expected, tolerance(dtype_name), f"{name}/{dtype_name}/twenty live")
 
 
+@pytest.mark.parametrize("name", ["A", "M", "B"])
+def test_second_copies_of_the_weights_change_no_bit(tmp_path, name):
+    """With a second copy of every matrix in the decode kernels' order (kept by default where the widths allow
+    it and memory is ample) the engine gives the logits it gives without, bit for bit, over a mixed schedule;
+    the model's accounting names the copies' bytes; a matrix whose inner size is no multiple of 64 gets none."""
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+
+    folder = make_model_dir(str(tmp_path / "m"), TINY[name], seed=83, dtype=torch.bfloat16)
+    config = read_config(folder)
+    requests = {f"s{i}": random_tokens(300 + i, 50 + 17 * i, config["vocab_size"]) for i in range(6)}
+    steps = schedules.mixed(requests, max_live=4, prompt_fraction=0.4, sizes=(11, 2, 30, 5))
+    pages = schedules.max_live_tokens(steps, round_to=16) // 16
+    outputs = {}
+    for wanted in (False, None):
+        model = load_model(folder, "bfloat16")
+        engine = Engine(model, num_pages=pages, page_tokens=16, max_requests=4, streamed_weights=wanted)
+        copies = model.weight_accounting()["streamed_copy_bytes"]
+        if wanted is None:                            # every matrix whose inner size allows it, and no other
+            fitting = [w for w in model.streamed_weights() if w.shape[1] % 64 == 0]
+            assert copies == sum(-(-w.shape[0] // 16) * 16 * w.shape[1] * 2 for w in fitting) > 0
+            assert (len(fitting) == len(model.streamed_weights())) == (config["hidden_size"] % 64 == 0)
+        else:
+            assert copies == 0
+        outputs[wanted] = run_steps(engine, steps)
+    assert outputs[False].keys() == outputs[None].keys()
+    for step, logits in outputs[False].items():
+        assert np.array_equal(logits, outputs[None][step]), f"step {step} differs"
+
+
 @pytest.mark.parametrize("name", ["A", "B", "D"])
 def test_many_groups_of_prompt_tiles_at_few_heads(tmp_path, name):
     """Four prompt portions of 40 tokens in one step (a group of tiles each), then a prompt of 420 tokens whole

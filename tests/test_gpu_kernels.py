@@ -734,6 +734,65 @@ def test_gemm_rows_plain(mnk):
     assert torch.equal(ops.gemm_rows(other, w, torch.float32, splits=1, waves=waves)[m - 1], whole[m - 1])
 
 
+@pytest.mark.parametrize("nk", [(4096, 4096), (777, 192), (6144, 4096), (130, 1024), (40, 64), (24576, 4096), (4096, 12288)])
+def test_products_read_the_tiled_copy_of_a_weight_to_the_same_bits(nk):
+    """Both weight-streaming products, given a weight whose tiled copy is kept, read that copy (every load of
+    a wave one piece of 1 KB, with the non-temporal hint) and give what they give from the rows: the same
+    bits, in every output mode, for rows of the last tile and columns of the last chunk that do not exist.
+    The copy goes when the weight goes."""
+    from leone_amd import ops
+    n, k = nk
+    torch.manual_seed(29)
+    w = (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    gain = (1 + 0.1 * torch.randn(k, device=DEV)).bfloat16()
+    next_gain = (1 + 0.1 * torch.randn(n, device=DEV)).bfloat16()
+    ops.drop_streamed_copies()
+
+    def run_all():
+        found = []
+        for m in (1, 3, 8, 10, 16, 37, 64, 128):
+            x = torch.randn(m, k, generator=torch.Generator(device=DEV).manual_seed(m), device=DEV).bfloat16()
+            stream = torch.randn(m, k, generator=torch.Generator(device=DEV).manual_seed(100 + m), device=DEV)
+            if m <= ops.FUSED_ROWS:
+                found.append(ops.gemm_fused(x, w, torch.float32))
+                found.append(ops.gemm_fused(x, w, torch.bfloat16))
+                found.append(ops.gemm_fused(ops.NormedRows(stream, gain, 1e-6, torch.bfloat16), w, torch.float32))
+                res = torch.ones(m, n, device=DEV)
+                ops.gemm_fused(x, w, residual=res)
+                found.append(res)
+                if n % 64 == 0 and ops.prepared_fits(m, n):
+                    res = torch.ones(m, n, device=DEV)
+                    prepared = ops.gemm_fused(x, w, residual=res, next_norm=(next_gain, 1e-6, torch.bfloat16))
+                    found += [res, prepared.operand, prepared.squares]
+                if ops.prepared_fits(m, k):
+                    found.append(ops.gemm_fused(ops.NormedRows(stream, gain, 1e-6, torch.bfloat16).prepare(), w, torch.float32))
+                if n % 16 == 0:
+                    found.append(ops.gemm_fused(x, w, gated=True))
+            found.append(ops.gemm_rows(x, w, torch.float32, may_split=False))
+            found.append(ops.gemm_rows(x, w, torch.float32, splits=3, waves=4))
+            found.append(ops.gemm_rows(x, w, torch.bfloat16, may_split=False, waves=8))
+            res = torch.ones(m, n, device=DEV)
+            ops.gemm_rows(x, w, residual=res, splits=1)
+            found.append(res)
+            if n % 16 == 0:
+                found.append(ops.gemm_rows(x, w, gated=True))
+        return found
+
+    from_rows = run_all()
+    assert ops.streamed_copy(w) is None
+    assert ops.keep_streamed_copy(w) == -(-n // 16) * 16 * k * 2
+    tiles = ops.streamed_copy(w)
+    assert tiles is not None and tiles.shape == (-(-n // 16), k // 64, 2, 4, 16, 8)
+    from_tiles = run_all()
+    assert len(from_rows) == len(from_tiles) > 40
+    for index, (a, b) in enumerate(zip(from_rows, from_tiles)):
+        assert torch.equal(a, b), f"result {index} differs"
+    # the copy is the weight's: another tensor of the same values has none, and it goes with the weight
+    assert ops.streamed_copy(w.clone()) is None
+    del w, tiles
+    assert not ops._streamed
+
+
 def test_gemm_rows_plan_fills_the_compute_units():
     """The plan at the shapes it was measured on, and that it never names an empty range of K."""
     from leone_amd import ops

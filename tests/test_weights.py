@@ -120,3 +120,31 @@ def test_sharded_folder(tmp_path):
     json.dump(index, open(os.path.join(folder, "model.safetensors.index.json"), "w"))
     loaded = loader.load_from_dir(folder, specs_for(TINY_A), torch.float32, "cpu")
     assert all(torch.equal(loaded[n], tensors[n]) for n in names)
+
+
+def test_tiled_copy_of_a_weight_puts_every_element_where_the_kernels_look():
+    """``ops.tile_weight``: element e of lane 16 g + c in half h of step s of tile t is
+    weight[16 t + c][64 s + 16 g + 8 h + e]; rows that fill the last tile are zero; widths that are no multiple
+    of 64 and other types are refused."""
+    import pytest
+    from leone_amd import ops
+    from leone_amd.ops.library import KernelError
+
+    n, k = 40, 192
+    weight = (torch.arange(n * k, dtype=torch.float32).view(n, k) % 251 - 125).bfloat16()
+    tiles = ops.tile_weight(weight)
+    assert tiles.shape == (3, 3, 2, 4, 16, 8) and tiles.is_contiguous()
+    flat = tiles.view(-1)
+    for t in range(3):
+        for s in range(3):
+            for h in range(2):
+                for lane in (0, 5, 16, 31, 47, 63):
+                    g, c = lane // 16, lane % 16
+                    at = (((t * 3 + s) * 2 + h) * 64 + lane) * 8
+                    row, col = 16 * t + c, 64 * s + 16 * g + 8 * h
+                    want = weight[row, col:col + 8] if row < n else torch.zeros(8, dtype=torch.bfloat16)
+                    assert torch.equal(flat[at:at + 8], want), (t, s, h, lane)
+    with pytest.raises(KernelError):
+        ops.tile_weight(weight[:, :100].contiguous())
+    with pytest.raises(KernelError):
+        ops.tile_weight(weight.float())
