@@ -87,8 +87,10 @@ def measure_peaks(device: str = "cuda:0", megabytes: int = 1024, repeats: int = 
                   for per in (1, 2, 4, 8))
     copy_ms = min(best_ms(lambda: call("leone_peak_copy", src.data_ptr(), dst.data_ptr(), count, per * units, stream))
                   for per in (1, 2, 4, 8))
-    blocks, iterations = 8 * units, 4000
-    mfma_ms = best_ms(lambda: call("leone_peak_mfma", blocks, iterations, sink.data_ptr(), stream))
+    iterations = 4000
+    mfma_ms, blocks = min((best_ms(lambda: call("leone_peak_mfma", per * units, iterations, wide, sink.data_ptr(), stream)) / per,
+                           per * units) for per in (4, 8) for wide in (0, 1))
+    mfma_ms *= blocks // units
     flops = library().leone_peak_mfma_flops(blocks, iterations)
     return {"hbm_read_gbs": round(count / read_ms / 1e6, 1), "hbm_copy_gbs": round(2 * count / copy_ms / 1e6, 1),
             "mfma_bf16_tflops": round(flops / mfma_ms / 1e9, 1), "buffer_mb": megabytes}

@@ -126,12 +126,13 @@ int leone_gemm_rows_bf16(const void* x, const void* w, int w_tiled, void* y, int
                          int splits, long plane, int waves, hipStream_t stream);
 
 // What the memory and the matrix cores give with nothing else going on: one read of `bytes` (a multiple of
-// 16), one copy, and blocks x 4 waves x iterations x 8 v_mfma_f32_16x16x32_bf16 (leone_peak_mfma_flops in all).
+// 16), one copy, and blocks x 4 waves x iterations x 8 v_mfma_f32_16x16x32_bf16, or with `wide` x 4
+// v_mfma_f32_32x32x16_bf16, the same work (leone_peak_mfma_flops in all).
 // The caller times them.  sink: four bytes of device memory that are practically never written.
 int leone_peak_read(const void* src, long bytes, void* sink, int blocks, hipStream_t stream);
 int leone_peak_copy(const void* src, void* dst, long bytes, int blocks, hipStream_t stream);
 double leone_peak_mfma_flops(int blocks, int iterations);
-int leone_peak_mfma(int blocks, int iterations, void* sink, hipStream_t stream);
+int leone_peak_mfma(int blocks, int iterations, int wide, void* sink, hipStream_t stream);
 
 // Highest finite logit of each row, lowest index on ties, -1 if none.  Workspace: part_value and
 // part_index with rows * ceil(vocab / leone_argmax_chunk()) entries each.

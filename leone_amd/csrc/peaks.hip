@@ -50,24 +50,44 @@ peak_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, long ru
     for (; at < runs; at += stride) dst[at] = src[at];
 }
 
-// Eight independent accumulator tiles a wave, so that no instruction waits for the one before.
+// Independent accumulator tiles a wave, so that no instruction waits for the one before: eight of 16 x 16 or
+// four of 32 x 32 (the same registers).  Which instruction shape runs faster is the chip's affair; the bench
+// takes the better.
 constexpr int kPeakTiles = 8;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 
+template <bool kWide>
 __global__ void __launch_bounds__(kPeakThreads)
 peak_mfma_kernel(int iterations, float* __restrict__ sink) {
     const unsigned seed = 0x3f803f80u + (threadIdx.x & 7u);            // small bfloat16 values
     const bf16x8 a = __builtin_bit_cast(bf16x8, uint4{seed, seed, seed, seed});
     const bf16x8 b = __builtin_bit_cast(bf16x8, uint4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u});
-    floatx4 acc[kPeakTiles];
-#pragma unroll
-    for (int t = 0; t < kPeakTiles; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int i = 0; i < iterations; ++i) {
-#pragma unroll
-        for (int t = 0; t < kPeakTiles; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
-    }
     float total = 0.f;
+    if constexpr (kWide) {
+        floatx16 acc[kPeakTiles / 2];
 #pragma unroll
-    for (int t = 0; t < kPeakTiles; ++t) total += acc[t][0] + acc[t][1] + acc[t][2] + acc[t][3];
+        for (int t = 0; t < kPeakTiles / 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+        for (int i = 0; i < iterations; ++i) {
+#pragma unroll
+            for (int t = 0; t < kPeakTiles / 2; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
+        }
+#pragma unroll
+        for (int t = 0; t < kPeakTiles / 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) total += acc[t][r];
+    } else {
+        floatx4 acc[kPeakTiles];
+#pragma unroll
+        for (int t = 0; t < kPeakTiles; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < iterations; ++i) {
+#pragma unroll
+            for (int t = 0; t < kPeakTiles; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+        }
+#pragma unroll
+        for (int t = 0; t < kPeakTiles; ++t) total += acc[t][0] + acc[t][1] + acc[t][2] + acc[t][3];
+    }
     if (total == -1.0f) sink[0] = total;          // keeps the loop; never true for these operands
 }
 
@@ -94,15 +114,17 @@ extern "C" int leone_peak_copy(const void* src, void* dst, long bytes, int block
     return 0;
 }
 
-// blocks workgroups of four waves run `iterations` rounds of eight matrix instructions each:
-// leone_peak_mfma_flops(blocks, iterations) floating-point operations in all.
+// blocks workgroups of four waves run `iterations` rounds of eight 16 x 16 x 32 matrix instructions each, or
+// (wide) of four 32 x 32 x 16 ones, the same work: leone_peak_mfma_flops(blocks, iterations) floating-point
+// operations in all.
 extern "C" double leone_peak_mfma_flops(int blocks, int iterations) {
     return static_cast<double>(blocks) * (kPeakThreads / kWave) * iterations * kPeakTiles * (2.0 * 16 * 16 * 32);
 }
 
-extern "C" int leone_peak_mfma(int blocks, int iterations, void* sink, hipStream_t stream) {
+extern "C" int leone_peak_mfma(int blocks, int iterations, int wide, void* sink, hipStream_t stream) {
     LEONE_REQUIRE(sink && blocks > 0 && iterations > 0, "peak_mfma: bad arguments");
-    peak_mfma_kernel<<<blocks, kPeakThreads, 0, stream>>>(iterations, static_cast<float*>(sink));
+    if (wide) peak_mfma_kernel<true><<<blocks, kPeakThreads, 0, stream>>>(iterations, static_cast<float*>(sink));
+    else peak_mfma_kernel<false><<<blocks, kPeakThreads, 0, stream>>>(iterations, static_cast<float*>(sink));
     LEONE_LAUNCH_CHECK("peak_mfma");
     return 0;
 }

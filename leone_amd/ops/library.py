@@ -44,7 +44,7 @@ _PROTOTYPES = {
     "leone_argmax": [P, P, P, P, c_int, c_int, P],
     "leone_peak_read": [P, ctypes.c_long, P, c_int, P],
     "leone_peak_copy": [P, P, ctypes.c_long, c_int, P],
-    "leone_peak_mfma": [c_int, c_int, P, P],
+    "leone_peak_mfma": [c_int, c_int, c_int, P, P],
     "leone_sample_temperature": [P, P, P, P, P, P, P, P, c_int, c_int, P],
     "leone_top_candidates": [P, P, P, P, c_int, c_int, c_int, P],
 }
