@@ -1,7 +1,7 @@
 // Causal attention of prompt portions over the paged cache on the matrix cores, bfloat16.
 //
 // A portion's rows are cut into tiles of 32 consecutive rows; a wave takes one tile and one query
-// head, its rows as two 16-column operands.  A workgroup is four waves whose tiles belong to the
+// head, its rows as one 32-column operand.  A workgroup is four waves whose tiles belong to the
 // same request (the host lists them: entry, first row, row count, four to a workgroup).  The
 // workgroup walks the keys its tiles can see once, 64 at a time: the next 64 keys and values travel
 // from the cache to shared memory while the waves work on the present 64 (by loads that write to
@@ -10,10 +10,15 @@
 // running reference, sum and accumulator of the reference's recurrence
 // (crates/leone/src/cpu.rs:2359-2421) per query in registers; nothing of size rows x keys is ever
 // stored (the reference's prefill materialises the scores, crates/leone-cuda/cuda/ie_cuda.cu:5124-5220).
-// Products and operand layouts are those of the decode kernel: S^T = K . Q^T and O^T += V^T . P^T
-// with v_mfma_f32_16x16x32_bf16 on 16-byte runs of the packed cache layout.  Keys are stored in
-// shared memory in the order the first product's operand wants them, so that neighbouring lanes
-// read neighbouring runs.
+// The products are those of the decode kernel, S^T = K . Q^T and O^T += V^T . P^T, on 16-byte runs of the
+// packed cache layout, but with v_mfma_f32_32x32x16_bf16: 32 keys against 32 rows an instruction.  That
+// instruction does twice the work of the 16 x 16 x 32 one for the same operand registers, and operand
+// reads are what holds the small one back (measured in a register loop: 2.45 against 1.4-1.6 PFLOP/s).
+// Lane L gives row L % 32 of the first operand and column L % 32 of the second, elements 8 (L / 32) .. + 7 of
+// the 16 that are summed over, and gets column L % 32 of the result, rows 8 (v / 4) + 4 (L / 32) + v % 4
+// in register v.  Keys are stored in shared memory in the order in which the first product's rows want
+// them, chosen so that a lane's scores are those of 8 + 8 neighbouring keys: they go into the second
+// product as they are.
 //
 // The recurrence is kept in base-2 units: t = score * scale * log2(e), p = 2^(t - m).  m is a
 // reference, not always the maximum: it is raised (and sums and accumulators rescaled) only when
@@ -22,8 +27,8 @@
 // always a whole number (the maximum rounded up), so that the bfloat16 rounding of p gives the same
 // significant bits whatever m is: the weights do not depend on how the keys are cut into passes,
 // stages and ranges, and a raised reference rescales by an exact power of two.  The sum
-// of a query's p is one more row of the second product (a row of ones in V^T), so that numerator
-// and denominator are sums of the same rounded values.
+// of a query's p is taken over the rounded values, key by key, so that numerator and denominator are
+// sums of the same numbers.
 //
 // Few rows over many keys (a late portion of a long prompt) would leave most of the chip idle: then
 // the keys of a workgroup are cut into `splits` ranges of whole 64-key stages, one workgroup a range
@@ -39,16 +44,22 @@ namespace leone {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
 
 constexpr int kPrefillWaves = 4;
 constexpr int kPrefillThreads = kPrefillWaves * kWave;
-constexpr int kColsPerWave = 2;                                  // 16-query operands a wave carries
-constexpr int kRowsPerWave = 16 * kColsPerWave;                  // rows of a tile
+constexpr int kRowsPerWave = 32;                                 // rows of a tile: one operand of the matrix instruction
 constexpr int kStageKeys = 64;                                   // keys copied to shared memory at a time
 constexpr int kKeysPerPass = 32;                                 // keys of one pass of a wave
 constexpr float kRaise = 8.0f;                                   // a score this far above the reference raises it
 
 __device__ inline bf16x8 pf_bits(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+// Which key of a 32-key pass sits in row r of the first product's operand, and in which row key k sits: the
+// same swap of two bits either way.  Rows 8 b + 4 h + i (b 0..3, i 0..3) are what lane half h gets of the
+// result; with this order they are keys 8 h + 0..7 (b 0, 1) and 16 + 8 h + 0..7 (b 2, 3).
+__device__ inline int pass_key_or_row(int x) { return (x & 0x13) | ((x & 4) << 1) | ((x & 8) >> 1); }
 
 // Runs of 16 bytes one stage holds: keys [head_dim / 8][64], values [8][head_dim].
 __host__ __device__ constexpr int stage_runs(int head_dim) { return (head_dim / 8) * kStageKeys + 8 * head_dim; }
@@ -64,7 +75,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                          float* __restrict__ part_acc, float* __restrict__ part_ml, int splits) {
     constexpr int kD = kD16 * 16;
     constexpr int kRuns = kD / 8;                      // 16-byte runs of one key
-    constexpr int kSteps = (kD16 + 1) / 2;             // 32-element steps of the first product
+    constexpr int kDT = (kD + 31) / 32;                // 32-row tiles of the second product's result
     constexpr int kKeyRuns = kRuns * kStageKeys;       // runs of the keys of one stage; the values take as many
     constexpr int kStageRuns = stage_runs(kD);
     constexpr int kCopies = (kKeyRuns + kPrefillThreads - 1) / kPrefillThreads;   // runs a thread copies, keys and values each
@@ -72,7 +83,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int lane = threadIdx.x % kWave;
     const int tid = threadIdx.x;
-    const int c = lane & 15, g = lane >> 4;
+    const int j = lane & 31, h = lane >> 5;            // this lane's row of the tile, and which half of the summed-over elements
 
     // Which head and tile group this workgroup takes (an order that suits the dies' caches: prefill_order.h).
     const PrefillWork work = prefill_work(static_cast<int>(blockIdx.x), q_heads, n_groups);
@@ -120,15 +131,10 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         group_lo = mine_lo > group_lo ? mine_lo : group_lo;
         group_hi = mine_hi < group_hi ? mine_hi : group_hi;
         if (group_hi <= group_lo) {                              // more ranges than stages: this one is empty
-            if (g == 0) {
-#pragma unroll
-                for (int j = 0; j < kColsPerWave; ++j) {
-                    const int r = 16 * j + c;
-                    if (r >= wave_rows) continue;
-                    const long slot = (static_cast<long>(tile_row0 + r) * q_heads + head) * splits + blockIdx.y;
-                    part_ml[2 * slot] = -INFINITY;
-                    part_ml[2 * slot + 1] = 0.f;
-                }
+            if (h == 0 && j < wave_rows) {
+                const long slot = (static_cast<long>(tile_row0 + j) * q_heads + head) * splits + blockIdx.y;
+                part_ml[2 * slot] = -INFINITY;
+                part_ml[2 * slot + 1] = 0.f;
             }
             return;
         }
@@ -142,35 +148,26 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     for (int i = tid; i < n_pages; i += kPrefillThreads) pages[i] = table[first_page + i];
     __syncthreads();
 
-    // Q^T operands and each column's own position.
-    bf16x8 qreg[kColsPerWave][kSteps];
-    int col_pos[kColsPerWave];
+    // The Q^T operand and the row's own position.
+    const bool row_ok = j < wave_rows;
+    const int row_pos = row_ok ? p0 + j : -1;                                   // -1: the row sees no key
+    bf16x8 qreg[kD16];
+    {
+        const bf16_t* qrow = q + (static_cast<long>(tile_row0 + (row_ok ? j : 0)) * q_heads + head) * kD;
 #pragma unroll
-    for (int j = 0; j < kColsPerWave; ++j) {
-        const int r = 16 * j + c;
-        const bool ok = r < wave_rows;
-        col_pos[j] = ok ? p0 + r : -1;                                          // -1: the column sees no key
-        const bf16_t* qrow = q + (static_cast<long>(tile_row0 + (ok ? r : 0)) * q_heads + head) * kD;
-#pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-            const int d0 = 32 * s + 8 * g;
-            qreg[j][s] = (ok && d0 < kD) ? pf_bits(*reinterpret_cast<const uint4*>(qrow + d0)) : pf_bits(uint4{0u, 0u, 0u, 0u});
-        }
+        for (int s = 0; s < kD16; ++s)
+            qreg[s] = row_ok ? pf_bits(*reinterpret_cast<const uint4*>(qrow + 16 * s + 8 * h)) : pf_bits(uint4{0u, 0u, 0u, 0u});
     }
 
-    // Per column: the reference m (base-2 units), the accumulator, and the sum of p as one more
-    // accumulator tile (every row of it holds the sum).
-    float m_ref[kColsPerWave];
-    floatx4 acc[kColsPerWave][kD16], acc_sum[kColsPerWave];
+    // Per row: the reference m (base-2 units), the sum of p over this lane's half of the keys, and the
+    // accumulator (register v of tile dt: element 32 dt + 8 (v / 4) + 4 h + v % 4 of the row's result).
+    float m_ref = -INFINITY, l_run = 0.f;
+    floatx16 acc[kDT];
 #pragma unroll
-    for (int j = 0; j < kColsPerWave; ++j) {
-        m_ref[j] = -INFINITY;
-        acc_sum[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int dt = 0; dt < kDT; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < kD16; ++dt) acc[j][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-    }
+        for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
     const float to_log2 = scale * 1.44269504088896340736f;
-    const bf16x8 ones = pf_bits(uint4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
 
     // ---- copying a stage: keys [64 t, 64 t + 64) from the cache into registers, then into shared memory.
     // Copy i of a thread is run `idx / 64` of key `idx % 64` and, of the values, element `idx % kD`
@@ -190,9 +187,8 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         const int in_page = key_base & page_mask;
         const bf16_t* kp = k_pool + page * pool_stride + head_elems + static_cast<long>(in_page) * 8;
         const bf16_t* vp = v_pool + page * pool_stride + head_elems + static_cast<long>(in_page >> 3) * kD * 8;
-        // place -> key of the 32-key half: the inverse of `deposit`'s order
-        const int place = lane & 31;
-        const int kk = ((place >> 2) & 3) * 8 + (place >> 4) * 4 + (place & 3);
+        // place -> key of the 32-key half, as in `deposit`
+        const int kk = pass_key_or_row(lane & 31);
 #pragma unroll
         for (int i = 0; i < kDirect; ++i) {
             const int group = i * kPrefillWaves + wave;               // the same for the whole wave
@@ -270,11 +266,10 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         for (int i = 0; i < kCopies; ++i) {
             const int idx = i * kPrefillThreads + tid;
             if (kKeyRuns % kPrefillThreads != 0 && idx >= kKeyRuns) continue;
-            // Key kk of a 32-key half sits where the first product's operand row reads it: rows 0..15 are
-            // keys 8 (r / 4) + r % 4, rows 16..31 the keys four further on.
+            // Key kk of a 32-key half sits where the first product's operand row reads it.
             const int run = idx / kStageKeys, kl = idx % kStageKeys;
             const int half = kl >> 5, kk = kl & 31;
-            const int place = ((kk >> 2) & 1) * 16 + 4 * (kk >> 3) + (kk & 3);
+            const int place = pass_key_or_row(kk);
             to[(half * kRuns + run) * 32 + place] = held_k[i];
             to[kKeyRuns + idx] = held_v[i];
         }
@@ -282,80 +277,71 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 
     // ---- one pass of a wave: 32 keys against its 32 rows
     auto pass = [&](const uint4* from, int key0, int half, bool full) {
-        const int run0 = key0 + 8 * g;                         // the lane's eight keys in the second product
-        bf16x8 xa[kSteps], xb[kSteps];
+        // Two sums, over the even and the odd steps, so that no instruction waits for the one before.
+        floatx16 sc, sc_odd;
 #pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-            const bool in_head = 4 * s + g < kRuns;
-            const uint4* row = from + (half * kRuns + 4 * s + g) * 32;
-            xa[s] = in_head ? pf_bits(row[c]) : pf_bits(uint4{0u, 0u, 0u, 0u});
-            xb[s] = in_head ? pf_bits(row[16 + c]) : pf_bits(uint4{0u, 0u, 0u, 0u});
+        for (int v = 0; v < 16; ++v) sc[v] = sc_odd[v] = 0.f;
+#pragma unroll
+        for (int s = 0; s < kD16; ++s) {
+            // operand row j is key pass_key_or_row(j); this lane's elements 16 s + 8 h .. + 7 are run 2 s + h
+            const bf16x8 xk = pf_bits(from[(half * kRuns + 2 * s + h) * 32 + j]);
+            if (s % 2 == 0) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xk, qreg[s], sc, 0, 0, 0);
+            else sc_odd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xk, qreg[s], sc_odd, 0, 0, 0);
         }
-        float sc[kColsPerWave][8];
-        float top[kColsPerWave];
+        if (kD16 > 1) {
 #pragma unroll
-        for (int j = 0; j < kColsPerWave; ++j) {
-            floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < kSteps; ++s) {
-                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[s], qreg[j][s], sa, 0, 0, 0);
-                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb[s], qreg[j][s], sb, 0, 0, 0);
-            }
-            // lane (g, c): scores of keys run0 .. run0+7 for the query of column c
-#pragma unroll
-            for (int i = 0; i < 8; ++i) sc[j][i] = i < 4 ? sa[i & 3] : sb[i & 3];
+            for (int v = 0; v < 16; ++v) sc[v] += sc_odd[v];
         }
+        // lane (j, h): sc[v] is row j's score of key key0 + 8 h + v (v < 8) or key0 + 16 + 8 h + v - 8
         if (!full) {                                           // the same for the whole wave
+            const int p_lo = (window > 0) ? row_pos - window + 1 : 0;
 #pragma unroll
-            for (int j = 0; j < kColsPerWave; ++j) {
-                const int p = col_pos[j];
-                const int p_lo = (window > 0) ? p - window + 1 : 0;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int key = run0 + i;
-                    sc[j][i] = (key <= p && key >= p_lo) ? sc[j][i] : -INFINITY;
-                }
+            for (int v = 0; v < 16; ++v) {
+                const int key = key0 + 8 * h + (v & 7) + 16 * (v >> 3);
+                sc[v] = (key <= row_pos && key >= p_lo) ? sc[v] : -INFINITY;
             }
         }
-        bool raise = false;
+        float top = sc[0];
 #pragma unroll
-        for (int j = 0; j < kColsPerWave; ++j) {
-            top[j] = fmaxf(fmaxf(fmaxf(sc[j][0], sc[j][1]), fmaxf(sc[j][2], sc[j][3])),
-                           fmaxf(fmaxf(sc[j][4], sc[j][5]), fmaxf(sc[j][6], sc[j][7]))) * to_log2;
-            raise = raise || top[j] > m_ref[j] + kRaise;       // -inf + 8 is -inf: the first scores always raise
+        for (int v = 1; v < 16; ++v) top = fmaxf(top, sc[v]);
+        top *= to_log2;
+        if (__any(top > m_ref + kRaise)) {                     // -inf + 8 is -inf: the first scores always raise
+            // Some score outgrew its reference: every row takes its true maximum so far as the new one.
+            const float row_top = fmaxf(top, __shfl_xor(top, 32, kWave));
+            const float m_new = fmaxf(m_ref, ceilf(row_top));           // a whole number: see the rounding of the weights below
+            const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_ref - m_new);   // 2^-inf = 0
+            m_ref = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < kDT; ++dt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[dt][v] *= alpha;
         }
-        if (__any(raise)) {
-            // Some score outgrew its reference: every column takes its true maximum so far as the new one.
+        const float shift = m_ref == -INFINITY ? 0.f : -m_ref;         // a row that has seen no key yet
+        bf16x8 pt[2];
 #pragma unroll
-            for (int j = 0; j < kColsPerWave; ++j) {
-                float col_top = fmaxf(top[j], __shfl_xor(top[j], 16, kWave));
-                col_top = fmaxf(col_top, __shfl_xor(col_top, 32, kWave));
-                const float m_new = fmaxf(m_ref[j], ceilf(col_top));     // a whole number: see the rounding of the weights below
-                const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_ref[j] - m_new);   // 2^-inf = 0
-                m_ref[j] = m_new;
+        for (int v = 0; v < 16; ++v)
+            pt[v >> 3][v & 7] = static_cast<__bf16>(__builtin_amdgcn_exp2f(fmaf(sc[v], to_log2, shift)));
+        // the sum of what the second product sees: the rounded values, two to an instruction (p . 1 + p' . 1 + sum)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc_sum[j][r] *= alpha;
+        for (int ks = 0; ks < 2; ++ks) {
+            const uint4 packed = __builtin_bit_cast(uint4, pt[ks]);
+            const unsigned pairs[4] = {packed.x, packed.y, packed.z, packed.w};
 #pragma unroll
-                for (int dt = 0; dt < kD16; ++dt)
+            for (int i = 0; i < 4; ++i)
+                l_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pairs[i]), __builtin_bit_cast(bf16x2, 0x3f803f80u),
+                                                        l_run, false);
+        }
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[j][dt][r] *= alpha;
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int dt = 0; dt < kDT; ++dt) {
+                const int d = 32 * dt + j;                     // operand row j of tile dt is element d of the values
+                // this lane's keys 16 ks + 8 h .. + 7 of the pass are one run of the values' layout
+                const bf16x8 xv = (kD % 32 == 0 || d < kD) ? pf_bits(from[kKeyRuns + (4 * half + 2 * ks + h) * kD + d])
+                                                           : pf_bits(uint4{0u, 0u, 0u, 0u});
+                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xv, pt[ks], acc[dt], 0, 0, 0);
             }
-        }
-        bf16x8 pt[kColsPerWave];
-#pragma unroll
-        for (int j = 0; j < kColsPerWave; ++j) {
-            const float shift = m_ref[j] == -INFINITY ? 0.f : -m_ref[j];   // a column that has seen no key yet
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                pt[j][i] = static_cast<__bf16>(__builtin_amdgcn_exp2f(fmaf(sc[j][i], to_log2, shift)));
-            acc_sum[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pt[j], acc_sum[j], 0, 0, 0);
-        }
-#pragma unroll
-        for (int dt = 0; dt < kD16; ++dt) {
-            const bf16x8 xv = pf_bits(from[kKeyRuns + (4 * half + g) * kD + 16 * dt + c]);
-#pragma unroll
-            for (int j = 0; j < kColsPerWave; ++j)
-                acc[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv, pt[j], acc[j][dt], 0, 0, 0);
         }
     };
 
@@ -389,40 +375,42 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     }
 
     const bool poisoned = unmapped_seen != 0;                    // every write to it came before the last barrier
+    const float l_row = l_run + __shfl_xor(l_run, 32, kWave);    // both halves of the keys
     if (splits > 1) {
-#pragma unroll
-        for (int j = 0; j < kColsPerWave; ++j) {
-            const int r = 16 * j + c;
-            if (r >= wave_rows) continue;
-            const long slot = (static_cast<long>(tile_row0 + r) * q_heads + head) * splits + blockIdx.y;
-            if (g == 0) {
-                part_ml[2 * slot] = m_ref[j];
-                part_ml[2 * slot + 1] = poisoned ? __builtin_nanf("") : acc_sum[j][0];
-            }
-            if (m_ref[j] == -INFINITY) continue;                 // no key of this range for the row: nothing to merge
-#pragma unroll
-            for (int dt = 0; dt < kD16; ++dt)
-                *reinterpret_cast<floatx4*>(part_acc + slot * kD + 16 * dt + 4 * g) = acc[j][dt];
+        if (!row_ok) return;
+        const long slot = (static_cast<long>(tile_row0 + j) * q_heads + head) * splits + blockIdx.y;
+        if (h == 0) {
+            part_ml[2 * slot] = m_ref;
+            part_ml[2 * slot + 1] = poisoned ? __builtin_nanf("") : l_row;
         }
+        if (m_ref == -INFINITY) return;                          // no key of this range for the row: nothing to merge
+#pragma unroll
+        for (int dt = 0; dt < kDT; ++dt)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int d0 = 32 * dt + 8 * b + 4 * h;
+                if (kD % 32 == 0 || d0 < kD)
+                    *reinterpret_cast<floatx4*>(part_acc + slot * kD + d0) =
+                        floatx4{acc[dt][4 * b], acc[dt][4 * b + 1], acc[dt][4 * b + 2], acc[dt][4 * b + 3]};
+            }
         return;
     }
+    if (!row_ok) return;
+    const float inv = poisoned ? __builtin_nanf("") : 1.0f / l_row;
+    bf16_t* orow = out + (static_cast<long>(tile_row0 + j) * q_heads + head) * kD;
 #pragma unroll
-    for (int j = 0; j < kColsPerWave; ++j) {
-        const int r = 16 * j + c;
-        if (r >= wave_rows) continue;
-        const float inv = poisoned ? __builtin_nanf("") : 1.0f / acc_sum[j][0];
-        bf16_t* orow = out + (static_cast<long>(tile_row0 + r) * q_heads + head) * kD;
+    for (int dt = 0; dt < kDT; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < kD16; ++dt) {
-            // lane (g, c) holds elements 16dt + 4g .. +3 of query column c
+        for (int b = 0; b < 4; ++b) {
+            const int d0 = 32 * dt + 8 * b + 4 * h;              // registers 4 b .. 4 b + 3 are elements d0 .. d0 + 3
+            if (kD % 32 != 0 && d0 >= kD) continue;
             uint2 packed;
-            packed.x = bf16_bits_from_float(acc[j][dt][0] * inv) |
-                       (static_cast<uint32_t>(bf16_bits_from_float(acc[j][dt][1] * inv)) << 16);
-            packed.y = bf16_bits_from_float(acc[j][dt][2] * inv) |
-                       (static_cast<uint32_t>(bf16_bits_from_float(acc[j][dt][3] * inv)) << 16);
-            *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * g) = packed;
+            packed.x = bf16_bits_from_float(acc[dt][4 * b] * inv) |
+                       (static_cast<uint32_t>(bf16_bits_from_float(acc[dt][4 * b + 1] * inv)) << 16);
+            packed.y = bf16_bits_from_float(acc[dt][4 * b + 2] * inv) |
+                       (static_cast<uint32_t>(bf16_bits_from_float(acc[dt][4 * b + 3] * inv)) << 16);
+            *reinterpret_cast<uint2*>(orow + d0) = packed;
         }
-    }
 }
 
 // Merges the key ranges of one row and query head: out = sum_s acc_s 2^(m_s - M) / sum_s l_s 2^(m_s - M),
