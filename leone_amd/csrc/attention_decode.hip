@@ -103,10 +103,10 @@ __device__ inline void load_projection8(const FromProjection& f, long row_width,
 }
 
 // kD16 = head_dim / 16.
-// Up to a head size of 128 the kernel fits three waves a SIMD without spilling if the compiler is asked to
-// (a little faster than two, measured); larger heads need their registers.
+// Two tiles of keys and values are held at a time (one on its way, one being worked on): up to a head size of
+// 64 that fits three waves a SIMD, up to 128 two; larger heads need all registers.
 template <int kD16, bool kFused>
-__global__ void __launch_bounds__(kDecodeThreads, kD16 <= 8 ? 3 : 1)
+__global__ void __launch_bounds__(kDecodeThreads, kD16 <= 4 ? 3 : kD16 <= 8 ? 2 : 1)
 attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
                         const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
                         const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
@@ -227,6 +227,46 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     }
     __syncthreads();
 
+    // One 32-key tile in two steps: `issue` asks for its keys and values, `finish` does the arithmetic.  The
+    // next tile of the wave is asked for before the present one is finished, so that a wave always has loads
+    // in flight (with a row or two and a few thousand keys a wave has only a handful of tiles, and without
+    // this each of them waited out the memory's latency by itself).  Every call of `issue` gives the same
+    // number of load instructions whatever the tile: lanes with nothing to read (keys outside [lo, n), a key
+    // without a page, no further tile) read the pool's first bytes instead and the result is cleared in
+    // `finish`; the compiler counts loads in flight and would wait for all of them after a load that may or may
+    // not have been issued.  `full` tiles lie wholly inside [lo, n) and need no masks; at most the first and
+    // the last tile of a row are not.
+    struct Tile {
+        bf16x8 xa[kSteps], xb[kSteps], xv[kD16];
+    };
+    auto issue = [&](int t, bool exists, Tile& r) {
+        const int key0 = t * kTileKeys;
+        // A-operand row c of half a is key 8*(c/4) + c%4, of half b four keys further
+        const int ka = key0 + 8 * (c >> 2) + (c & 3);
+        const int run0 = key0 + 8 * g;                   // this lane's eight keys for the second product
+        const bool near = exists && ka + 4 >= lo && ka < n;   // ka or kb = ka + 4 in reach: they share a page (pages hold multiples of 8 keys)
+        const bool any = exists && run0 < n && run0 + 8 > lo;
+        const int page_k = near ? pages[(ka >> page_shift) - first_page] : -1;
+        const int page_v = any ? pages[(run0 >> page_shift) - first_page] : -1;
+        const bf16_t* pk = page_k < 0 ? k_pool
+                                      : k_pool + (static_cast<long>(page_k) * kv_heads + kvh) * page_tokens * kD + (ka & page_mask) * 8;
+        const bf16_t* pv = page_v < 0 ? v_pool
+                                      : v_pool + (static_cast<long>(page_v) * kv_heads + kvh) * page_tokens * kD +
+                                            static_cast<long>((run0 & page_mask) >> 3) * kD * 8;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            const bool in_head = 32 * s + 8 * g < kD;
+            const long run = in_head ? static_cast<long>(4 * s + g) * page_tokens * 8 : 0;   // elements 32s+8g .. +7 of the key
+            r.xa[s] = load8_streamed(pk + run);
+            r.xb[s] = load8_streamed(pk + run + 32);           // four keys further
+        }
+#pragma unroll
+        for (int dt = 0; dt < kD16; ++dt) r.xv[dt] = load8_streamed(pv + (16 * dt + c) * 8);
+    };
+    // The wave's first tile is asked for before the queries are made: neither waits for the other.
+    Tile one, two;
+    if (my_begin + wave < my_end) issue(my_begin + wave, true, one);
+
     // Q^T operand: column c is query head kvh*group + col0 + c.
     bf16x8 qreg[kSteps];
     if constexpr (kFused) {
@@ -298,59 +338,57 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
 #pragma unroll
     for (int dt = 0; dt < kD16; ++dt) acc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // One 32-key tile.  `full` tiles lie wholly inside [lo, n) and need no masks; at most the first
-    // and the last tile of a row are not.  All loads of a tile, keys and values, are issued before
-    // the first product, so that they are in flight together.
-    auto do_tile = [&](int t, auto full_tag) {
-        constexpr bool kFull = decltype(full_tag)::value;
+    auto finish = [&](int t, Tile& r) {
         const int key0 = t * kTileKeys;
-        // A-operand row c of half a is key 8*(c/4) + c%4, of half b four keys further
+        const bool full = key0 >= lo && key0 + kTileKeys <= n;      // the same for the whole wave
         const int ka = key0 + 8 * (c >> 2) + (c & 3);
         const int kb = ka + 4;
-        const int run0 = key0 + 8 * g;                   // this lane's eight keys for the second product
-        bool va = true, vb = true, any = true, whole = true;
-        if constexpr (!kFull) {
-            va = ka >= lo && ka < n;
-            vb = kb >= lo && kb < n;
-            any = run0 < n && run0 + 8 > lo;
-            whole = run0 >= lo && run0 + 8 <= n;
+        const int run0 = key0 + 8 * g;
+        bool va = ka >= lo && ka < n, vb = kb >= lo && kb < n, any = run0 < n && run0 + 8 > lo;
+        if ((va || vb) && pages[(ka >> page_shift) - first_page] < 0) {
+            unmapped = true;                              // never read outside the pool; the result is poisoned below
+            va = vb = false;
         }
-        const bf16_t* pk = k_pool;
-        const bf16_t* pv = v_pool;
-        if (va || vb) {                                   // ka and kb share a page: pages hold multiples of 8 keys
-            const int page = pages[(ka >> page_shift) - first_page];
-            if (page < 0) {
-                unmapped = true;                          // never read outside the pool; the result is poisoned below
-                va = vb = false;
-            }
-            pk = k_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD + (ka & page_mask) * 8;
+        if (any && pages[(run0 >> page_shift) - first_page] < 0) {
+            unmapped = true;
+            any = false;
         }
-        if (any) {
-            const int page = pages[(run0 >> page_shift) - first_page];
-            if (page < 0) {
-                unmapped = true;
-                any = false;
-            }
-            pv = v_pool + (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD +
-                 static_cast<long>((run0 & page_mask) >> 3) * kD * 8;
-        }
-        bf16x8 xa[kSteps], xb[kSteps], xv[kD16];
+        if (!full || kD16 % 2 != 0 || __any(unmapped)) {
+            // what was read in place of nothing counts as zero
 #pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-            const bool in_head = 32 * s + 8 * g < kD;
-            const long run = static_cast<long>(4 * s + g) * page_tokens * 8;   // elements 32s+8g .. +7 of the key
-            xa[s] = (va && in_head) ? load8_streamed(pk + run) : zero8();
-            xb[s] = (vb && in_head) ? load8_streamed(pk + run + 32) : zero8();           // four keys further
-        }
+            for (int s = 0; s < kSteps; ++s) {
+                const bool in_head = 32 * s + 8 * g < kD;
+                if (!(va && in_head)) r.xa[s] = zero8();
+                if (!(vb && in_head)) r.xb[s] = zero8();
+            }
+            const bool whole = run0 >= lo && run0 + 8 <= n;
 #pragma unroll
-        for (int dt = 0; dt < kD16; ++dt) xv[dt] = any ? load8_streamed(pv + (16 * dt + c) * 8) : zero8();
+            for (int dt = 0; dt < kD16; ++dt) {
+                if (!any) {
+                    r.xv[dt] = zero8();
+                } else if (!whole) {
+                    // slots outside [lo, n) may hold anything, even NaN: clear them, a zero weight is not enough
+                    uint4 raw = __builtin_bit_cast(uint4, r.xv[dt]);
+                    unsigned* w = reinterpret_cast<unsigned*>(&raw);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int e0 = run0 + 2 * i, e1 = e0 + 1;
+                        unsigned mask = 0u;
+                        if (e0 >= lo && e0 < n) mask |= 0x0000ffffu;
+                        if (e1 >= lo && e1 < n) mask |= 0xffff0000u;
+                        w[i] &= mask;
+                    }
+                    r.xv[dt] = __builtin_bit_cast(bf16x8, raw);
+                }
+            }
+        }
 
         // ---- S^T = K . Q^T for the two 16-key halves --------------------------------------------
         floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) {
-            sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[s], qreg[s], sa, 0, 0, 0);
-            sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb[s], qreg[s], sb, 0, 0, 0);
+            sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(r.xa[s], qreg[s], sa, 0, 0, 0);
+            sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(r.xb[s], qreg[s], sb, 0, 0, 0);
         }
         // lane (g, c) now holds, for query column c, the scores of keys key0 + 8g + j, j = 0..7
         float sc[8];
@@ -359,7 +397,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         for (int j = 0; j < 8; ++j) {
             const int key = run0 + j;
             const float raw = j < 4 ? sa[j & 3] : sb[j & 3];
-            sc[j] = (kFull || (key >= lo && key < n)) ? raw * to_log2 : -INFINITY;
+            sc[j] = (full || (key >= lo && key < n)) ? raw * to_log2 : -INFINITY;
             tile_max = fmaxf(tile_max, sc[j]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
@@ -380,34 +418,34 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         // ---- O^T += V^T . P^T ------------------------------------------------------------------
 #pragma unroll
         for (int dt = 0; dt < kD16; ++dt) {
-            if constexpr (!kFull) {
-                if (any && !whole) {
-                    // slots outside [lo, n) may hold anything, even NaN: clear them, a zero weight is not enough
-                    uint4 raw = __builtin_bit_cast(uint4, xv[dt]);
-                    unsigned* w = reinterpret_cast<unsigned*>(&raw);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int e0 = run0 + 2 * i, e1 = e0 + 1;
-                        unsigned mask = 0u;
-                        if (e0 >= lo && e0 < n) mask |= 0x0000ffffu;
-                        if (e1 >= lo && e1 < n) mask |= 0xffff0000u;
-                        w[i] &= mask;
-                    }
-                    xv[dt] = __builtin_bit_cast(bf16x8, raw);
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[dt][r] *= alpha;
-            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[dt], pt, acc[dt], 0, 0, 0);
+            for (int r4 = 0; r4 < 4; ++r4) acc[dt][r4] *= alpha;
+            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(r.xv[dt], pt, acc[dt], 0, 0, 0);
         }
     };
 
-    for (int t = my_begin + wave; t < my_end; t += kDecodeWaves) {
-        const int key0 = t * kTileKeys;
-        if (key0 >= lo && key0 + kTileKeys <= n)
-            do_tile(t, std::true_type{});
-        else
-            do_tile(t, std::false_type{});
+    // Two tiles in turn: while one is finished the other is on its way.  After its last tile the wave asks
+    // for a tile that does not exist (see `issue`).
+    if constexpr (kD16 > 8) {                           // two tiles of such heads do not fit the registers
+        for (int t = my_begin + wave; t < my_end; t += kDecodeWaves) {
+            if (t != my_begin + wave) issue(t, true, one);
+            finish(t, one);
+        }
+    } else {
+        int t = my_begin + wave;
+        if (t < my_end) {
+            while (true) {
+                const int t1 = t + kDecodeWaves;
+                issue(t1, t1 < my_end, two);
+                finish(t, one);
+                if (t1 >= my_end) break;
+                const int t2 = t1 + kDecodeWaves;
+                issue(t2, t2 < my_end, one);
+                finish(t1, two);
+                if (t2 >= my_end) break;
+                t = t2;
+            }
+        }
     }
 
     // ---- merge the four waves --------------------------------------------------------------------
