@@ -128,3 +128,46 @@ def forward(weights: Dict[str, torch.Tensor], config: dict, tokens) -> torch.Ten
     y = rms_norm(x, weights["model.norm.weight"], config["rms_norm_eps"])
     head = weights["model.embed_tokens.weight"] if config.get("tie_word_embeddings", False) else weights["lm_head.weight"]
     return linear(y, head)
+
+
+def rope_half_split_at_once(x: torch.Tensor, positions, theta: float) -> torch.Tensor:
+    """``rope_half_split`` for a hundred thousand positions: the same angles and pairs as array arithmetic
+    (``tests/test_plain.py`` holds the two against each other)."""
+    x = x.to(F64)
+    dim = x.shape[-1]
+    half = dim // 2
+    rates = torch.tensor([float(theta) ** (-2.0 * i / dim) for i in range(half)], dtype=F64)
+    angles = torch.as_tensor(positions, dtype=F64)[:, None] * rates[None, :]
+    c, s = torch.cos(angles)[:, None, :], torch.sin(angles)[:, None, :]
+    a, b = x[..., :half], x[..., half:]
+    return torch.cat([a * c - b * s, a * s + b * c], dim=-1)
+
+
+def forward_rows_of_one_layer(weights: Dict[str, torch.Tensor], config: dict, tokens, rows) -> torch.Tensor:
+    """Logits [len(rows), vocab] at the positions ``rows`` only, for a model of ONE layer: there the keys and
+    values of every position come straight from the embeddings, so a context of 100,000 tokens costs what its
+    length costs, not its square.  The same part functions in the same order as ``forward``."""
+    config = dict(config)
+    if config["num_hidden_layers"] != 1:
+        raise ValueError("only a model of one layer can be evaluated row by row")
+    config.setdefault("head_dim", config["hidden_size"] // config["num_attention_heads"])
+    config.setdefault("num_key_value_heads", config["num_attention_heads"])
+    heads, kv_heads, dim = config["num_attention_heads"], config["num_key_value_heads"], config["head_dim"]
+    eps, theta = config["rms_norm_eps"], config["rope_theta"]
+    count = len(tokens)
+    p, a = "model.layers.0", "model.layers.0.self_attn"
+    x = embedding(weights["model.embed_tokens.weight"], tokens)
+    y = rms_norm(x, weights[f"{p}.input_layernorm.weight"], eps)
+    k = rms_norm(linear(y, weights[f"{a}.k_proj.weight"]).view(count, kv_heads, dim), weights[f"{a}.k_norm.weight"], eps)
+    k = rope_half_split_at_once(k, list(range(count)), theta)
+    v = linear(y, weights[f"{a}.v_proj.weight"]).view(count, kv_heads, dim)
+    head = weights["model.embed_tokens.weight"] if config.get("tie_word_embeddings", False) else weights["lm_head.weight"]
+    out = []
+    for t in rows:
+        q = rms_norm(linear(y[t:t + 1], weights[f"{a}.q_proj.weight"]).view(1, heads, dim), weights[f"{a}.q_norm.weight"], eps)
+        q = rope_half_split(q, [t], theta)
+        attended = attend_one(q[0], k[:t + 1], v[:t + 1]).reshape(1, heads * dim)
+        xt = x[t:t + 1] + linear(attended, weights[f"{a}.o_proj.weight"])
+        xt = xt + feed_forward(rms_norm(xt, weights[f"{p}.post_attention_layernorm.weight"], eps), weights, f"{p}.mlp")
+        out.append(linear(rms_norm(xt, weights["model.norm.weight"], eps), head)[0])
+    return torch.stack(out)

@@ -188,6 +188,44 @@ def test_a_hundred_thousand_tokens_cut_three_ways(tmp_path):
         assert float((other - results[0]).abs().max()) <= tolerance("bfloat16")
 
 
+def test_a_hundred_thousand_tokens_against_the_plain_implementation(tmp_path):
+    """The same length against the plain implementation: a model of ONE layer, whose keys and values come
+    straight from the embeddings, can be evaluated at single positions for what the length costs.  Scores are
+    sharpened (q/k gains doubled in float32: the softmax of 100,000 keys then rests on the few hundred best,
+    which lie anywhere in the context; in the plain implementation a sixteenth of the keys left out moves these
+    logits by 0.4, a single page by 0.004 to 0.02; measured from the plain implementation: float32 6e-5,
+    bfloat16 1.3e-2).  The last prompt
+    position (the prompt kernel with key ranges, the last portion's rows over 98,000 earlier keys) and eight
+    decoded tokens (the split-KV kernel over 1,563 pages), in bfloat16 and float32."""
+    from leone_amd.engine.engine import Engine, StepEntry
+    from leone_amd.runtime import load_model
+
+    config = dict(TINY["M"], num_hidden_layers=1, max_position_embeddings=131072)
+    n = 100_000
+    tokens = random_tokens(6, n + 8, config["vocab_size"])
+    # bfloat16 with gains times 1.5: its own rounding of sharper scores comes close to its tolerance
+    for dtype_name, chunk, sharpen in (("bfloat16", 2048, 1.5), ("float32", 4096, 2.0)):
+        folder = make_model_dir(str(tmp_path / dtype_name), config, seed=10, dtype=DTYPES[dtype_name], sharpen=sharpen)
+        weights = read_weights(folder)
+        want = qwen3_plain.forward_rows_of_one_layer(weights, read_config(folder), tokens, list(range(n - 1, n + 8))).float()
+        engine = Engine(load_model(folder, dtype_name), max_tokens=n + 64, page_tokens=64, max_requests=1, max_context=n + 64)
+        at = 0
+        while at < n:
+            size = min(chunk, n - at)
+            out = engine.step([StepEntry("r", tokens[at:at + size], [size - 1] if at + size == n else [])])
+            at += size
+        rows = [out.logits[0].float().cpu()]
+        for i in range(8):
+            rows.append(engine.step([StepEntry("r", [tokens[n + i]], [0])]).logits[0].float().cpu())
+        got = torch.stack(rows)
+        engine.release("r")
+        engine.cache.check()
+        worst = float((got - want).abs().max())
+        assert float(want.abs().max()) > 0.5
+        print(f"100,000 tokens, {dtype_name}: {worst:.3e} from the plain implementation")
+        assert worst <= tolerance(dtype_name), f"{dtype_name}: {worst:.3e} from the plain implementation at 100,000 tokens"
+
+
 @pytest.mark.parametrize("schedule", ["whole", "portions", "mixed"])
 def test_a_wide_feed_forward_whose_down_projection_is_cut(tmp_path, schedule):
     """An intermediate size of 8,192 over a width of 64: for steps of more than 128 rows the down projection

@@ -221,3 +221,26 @@ def test_head_norms_use_the_layer_norms_eps_by_numbers():
     wrong = [v / math.sqrt((v * v).sum() / 2 + 1e-6) for v in (y2[0].double(), y2[1].double())]
     wrong_w = torch.softmax(torch.stack([wrong[1] @ wrong[0], wrong[1] @ wrong[1]]) / math.sqrt(2), dim=0)
     assert (wrong_w - w).abs().max() > 0.02
+
+
+def test_rows_of_one_layer_equal_the_whole_forward():
+    """The row-by-row evaluation of a one-layer model (used where the whole forward would cost the square of
+    100,000 tokens) gives what ``forward`` gives at those rows."""
+    torch.manual_seed(3)
+    config = dict(num_hidden_layers=1, hidden_size=48, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+                  intermediate_size=80, vocab_size=97, rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False)
+    names = {"model.embed_tokens.weight": (97, 48), "lm_head.weight": (97, 48), "model.norm.weight": (48,),
+             "model.layers.0.input_layernorm.weight": (48,), "model.layers.0.post_attention_layernorm.weight": (48,),
+             "model.layers.0.self_attn.q_proj.weight": (64, 48), "model.layers.0.self_attn.k_proj.weight": (32, 48),
+             "model.layers.0.self_attn.v_proj.weight": (32, 48), "model.layers.0.self_attn.o_proj.weight": (48, 64),
+             "model.layers.0.self_attn.q_norm.weight": (16,), "model.layers.0.self_attn.k_norm.weight": (16,),
+             "model.layers.0.mlp.gate_proj.weight": (80, 48), "model.layers.0.mlp.up_proj.weight": (80, 48),
+             "model.layers.0.mlp.down_proj.weight": (48, 80)}
+    weights = {name: torch.randn(shape) * (1.0 if len(shape) == 1 else 0.3) for name, shape in names.items()}
+    tokens = [int(t) for t in torch.randint(0, 97, (40,))]
+    whole = plain.forward(weights, config, tokens)
+    rows = [0, 7, 38, 39]
+    assert torch.allclose(plain.forward_rows_of_one_layer(weights, config, tokens, rows), whole[rows], rtol=0, atol=1e-12)
+    x = torch.randn(9, 3, 16, dtype=torch.float64)
+    positions = [0, 1, 2, 77, 1000, 31000, 99999, 5, 100007]
+    assert torch.allclose(plain.rope_half_split_at_once(x, positions, 1e6), plain.rope_half_split(x, positions, 1e6), rtol=0, atol=1e-12)
