@@ -264,6 +264,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=CONTEXT)
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    parser.add_argument("--shape", default="8b", choices=["8b", "14b", "32b"],
+                        help="layer sizes of which Qwen3 model (the headline figure is 8b)")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     parser.add_argument("--no-prefill", action="store_true")
@@ -290,7 +292,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     from .engine.engine import Engine
     from .runtime import random_model
 
-    raw = dict(QWEN3_8B)
+    raw = dict({"8b": QWEN3_8B, "14b": QWEN3_14B, "32b": QWEN3_32B}[args.shape])
     full_layers = raw["num_hidden_layers"]
     if args.layers is not None:
         raw["num_hidden_layers"] = args.layers
@@ -315,10 +317,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     step_bytes = decode_bytes(model, args.batch, mean_context)
     achieved = step_bytes / (elapsed / args.steps) / 1e9
     record = {
-        "metric": "decode tok/s (Qwen3-8B shape)", "value": round(value, 2), "unit": "tok/s", "n_gpus": 1,
+        "metric": f"decode tok/s (Qwen3-{args.shape.upper()} shape)", "value": round(value, 2), "unit": "tok/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dtype_name, "data": "synthetic",
-        "config": {"model": "Qwen3-8B shape, random weights", "layers": config.num_hidden_layers,
+        "config": {"model": f"Qwen3-{args.shape.upper()} shape, random weights", "layers": config.num_hidden_layers,
                    "layers_of_configuration": full_layers, "hidden": config.hidden_size,
                    "q_heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
                    "head_dim": config.head_dim, "intermediate": config.intermediate_size, "vocab": config.vocab_size,

@@ -272,19 +272,33 @@ static void launch_fused(const FusedArgs& a, bool tiled, hipStream_t stream) {
     const int tiles = ceil_div(a.n, 16);
     const int steps = ceil_div(a.k, 64);
     const bool tail = a.k % 64 != 0;
-    const bool many = tiles * 4 >= 4096 || steps < 16;    // workgroups enough to fill the chip, or too little of K to split further
     const size_t shared = kIn == kInPrepared ? static_cast<size_t>(a.m) * (a.k / 16) * sizeof(float) : 0;
 #define LEONE_FUSED(TAIL, WAVES)                                                                                  \
     do {                                                                                                          \
         if (tiled) gemm_fused_kernel<kIn, kOut, false, WAVES, TOut, true><<<tiles, WAVES * kWave, shared, stream>>>(a); \
         else gemm_fused_kernel<kIn, kOut, TAIL, WAVES, TOut, false><<<tiles, WAVES * kWave, shared, stream>>>(a);  \
     } while (0)
-    // Measured at the 8B shapes: about one workgroup a compute unit (output and down projections) wants
-    // sixteen waves to keep enough loads in flight; matrices with many rows want four waves when X has many
-    // rows and eight when it has few.
-    if (tiles <= 256 && steps >= 64) {
+    // How many waves share a workgroup's walk over K.  Measured in whole decode steps at the layer sizes of the
+    // 8B, 14B and 32B models (a product timed alone, without the norms and the residual folded in, says
+    // otherwise and misleads):
+    //   about one workgroup a compute unit and a long K (4,096 x 4,096 and x 12,288): 16 waves, or too few
+    //     loads are in flight;
+    //   somewhat more than one a unit, K at least as long as the matrix is high (5,120 x 5,120 .. x 25,600, the
+    //     output and down projections of the 14B and 32B sizes): 4 waves, fewer and longer streams (+2 % on a
+    //     step of 8 rows, +3 % on one row there);
+    //   many workgroups a unit: 4 waves when X has more than four rows and 8 when it has few.
+    static int units = 0;
+    if (units == 0) {
+        int device = 0, count = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0)
+            count = 256;
+        units = count;
+    }
+    const bool many = tiles >= 4 * units || steps < 16;   // workgroups enough to fill the chip, or too little of K to split further
+    if (tiles <= units && steps >= 64) {
         if (tail) LEONE_FUSED(true, 16); else LEONE_FUSED(false, 16);
-    } else if (many && a.m > 4) {
+    } else if ((tiles > units && tiles <= 2 * units && 4L * a.n <= 5L * a.k) || (many && a.m > 4)) {
         if (tail) LEONE_FUSED(true, 4); else LEONE_FUSED(false, 4);
     } else {
         if (tail) LEONE_FUSED(true, 8); else LEONE_FUSED(false, 8);
