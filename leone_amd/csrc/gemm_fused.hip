@@ -278,15 +278,16 @@ static void launch_fused(const FusedArgs& a, bool tiled, hipStream_t stream) {
         if (tiled) gemm_fused_kernel<kIn, kOut, false, WAVES, TOut, true><<<tiles, WAVES * kWave, shared, stream>>>(a); \
         else gemm_fused_kernel<kIn, kOut, TAIL, WAVES, TOut, false><<<tiles, WAVES * kWave, shared, stream>>>(a);  \
     } while (0)
-    // How many waves share a workgroup's walk over K.  Measured in whole decode steps at the layer sizes of the
-    // 8B, 14B and 32B models (a product timed alone, without the norms and the residual folded in, says
-    // otherwise and misleads):
-    //   about one workgroup a compute unit and a long K (4,096 x 4,096 and x 12,288): 16 waves, or too few
+    // How many waves share a workgroup's walk over K.  Measured in whole decode steps of 1 and 8 rows at the
+    // layer sizes of the 8B, 14B and 32B models, one engine, the choices in turn (a product timed alone, without
+    // the norms and the residual folded in, says otherwise and misleads: 16 waves for gate/up look 1 % better
+    // there and cost a step 8 %):
+    //   up to one workgroup a compute unit and a long K (4,096 x 4,096 and x 12,288): 16 waves, or too few
     //     loads are in flight;
-    //   somewhat more than one a unit, K at least as long as the matrix is high (5,120 x 5,120 .. x 25,600, the
-    //     output and down projections of the 14B and 32B sizes): 4 waves, fewer and longer streams (+2 % on a
-    //     step of 8 rows, +3 % on one row there);
-    //   many workgroups a unit: 4 waves when X has more than four rows and 8 when it has few.
+    //   up to four a unit (q/k/v everywhere, the output and down projections of the 14B and 32B sizes): 4 waves,
+    //     fewer and longer streams (against 8: 14B 7.90 : 8.08 ms a step of 8 rows, 32B 15.98 : 16.33, 8B 4.93 : 4.98);
+    //   more: 8 waves (4 or 16 for the head, 4 for gate/up: level; 16 for gate/up: 5.37 : 4.98).
+    // With little of K to share (under 16 steps of 64) four waves are plenty.
     static int units = 0;
     if (units == 0) {
         int device = 0, count = 0;
@@ -295,10 +296,9 @@ static void launch_fused(const FusedArgs& a, bool tiled, hipStream_t stream) {
             count = 256;
         units = count;
     }
-    const bool many = tiles >= 4 * units || steps < 16;   // workgroups enough to fill the chip, or too little of K to split further
     if (tiles <= units && steps >= 64) {
         if (tail) LEONE_FUSED(true, 16); else LEONE_FUSED(false, 16);
-    } else if ((tiles > units && tiles <= 2 * units && 4L * a.n <= 5L * a.k) || (many && a.m > 4)) {
+    } else if (steps < 16 || (tiles > units && tiles <= 4 * units)) {
         if (tail) LEONE_FUSED(true, 4); else LEONE_FUSED(false, 4);
     } else {
         if (tail) LEONE_FUSED(true, 8); else LEONE_FUSED(false, 8);
