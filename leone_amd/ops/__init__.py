@@ -218,12 +218,14 @@ def decode_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: i
             and page_tokens >= 16 and page_tokens & (page_tokens - 1) == 0)
 
 
-def choose_splits(rows: int, kv_heads: int, group: int, max_context: int) -> int:
-    """How many parts the keys of a row are cut into: about two workgroups for each of the 256 CUs,
-    at least four 32-key tiles a part so that each of a workgroup's four waves has one."""
+def choose_splits(rows: int, kv_heads: int, group: int, max_context: int, units: int = 256) -> int:
+    """How many parts the keys of a row are cut into: about one workgroup for each compute unit (measured in
+    whole decode steps at 8,192 keys: against two a unit 4.91 : 4.97 ms a step at 8 rows, 3.89 : 3.93 at 3,
+    level at 1 and from 16 rows on), at least four 32-key tiles a part so that each of a workgroup's four waves
+    has one, at most 32 parts."""
     blocks = rows * kv_heads * ((group + 15) // 16)
     tiles = (max_context + 31) // 32
-    return max(1, min(512 // max(1, blocks), (tiles + 3) // 4, 32))
+    return max(1, min(units // max(1, blocks), (tiles + 3) // 4, 32))
 
 
 def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
@@ -236,7 +238,7 @@ def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
     if q.shape[1] != q_heads * head_dim:
         raise KernelError(f"attention: query width {q.shape[1]} is not {q_heads}*{head_dim}")
     if splits is None:
-        splits = choose_splits(rows, kv_heads, q_heads // kv_heads, max_context)
+        splits = choose_splits(rows, kv_heads, q_heads // kv_heads, max_context, compute_units(q.device))
     if out is None:
         out = torch.empty_like(q)
     part_acc = part_ml = None
@@ -275,7 +277,7 @@ def attention_decode_projected(qkv: torch.Tensor, q_heads: int, kv_heads: int, h
     if q_gain is not None and (k_gain is None or k_gain.dtype != q_gain.dtype):
         raise KernelError("attention_decode_projected: q and k gains must come together in one type")
     if splits is None:
-        splits = choose_splits(rows, kv_heads, q_heads // kv_heads, max_context)
+        splits = choose_splits(rows, kv_heads, q_heads // kv_heads, max_context, compute_units(qkv.device))
     out = torch.empty((rows, q_heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
     part_acc = part_ml = None
     if splits > 1:
@@ -381,11 +383,12 @@ def gemm_f32(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = Non
     return out
 
 
-# Up to here norm, gate and residual are folded into the weight-streaming kernel (which takes up to 16 rows).
-# Beyond, its reads of X weigh as much as those of W and the library's product with separate row-wise kernels
-# is faster (measured at the 8B shape: 6.02 against 6.38 ms a step at 8 rows, 6.71 : 6.82 at 10, 7.57 : 7.36 at 12,
-# 8.68 : 8.19 at 16).
-FUSED_ROWS = 10
+# Up to here norm, gate and residual are folded into the weight-streaming kernel for few rows; beyond, the
+# multi-row kernel runs with the row-wise kernels between.  Measured in whole decode steps at the 8B layer sizes
+# with the second copies of the weights (ms a step, folded : multi-row): 5.98 : 6.40 at 11 rows, 6.17 : 6.47 at
+# 12, 6.51 : 6.66 at 14, level at 16, which is all the kernel takes.  (With row-major weights only, the folded
+# kernel's reads of X weighed more and the two crossed between 10 and 11 rows.)
+FUSED_ROWS = 16
 FUSED_NORM_WEIGHT_ROWS = 1024   # a norm is folded into the product only for weights of at most this many rows
 
 

@@ -229,7 +229,7 @@ def test_a_hundred_thousand_tokens_against_the_plain_implementation(tmp_path):
 @pytest.mark.parametrize("schedule", ["whole", "portions", "mixed"])
 def test_a_wide_feed_forward_whose_down_projection_is_cut(tmp_path, schedule):
     """An intermediate size of 8,192 over a width of 64: for steps of more than 128 rows the down projection
-    runs in parts on the library, for 11 to 128 on the multi-row weight-streaming kernel with K cut into
+    runs in parts on the library, for 17 to 128 on the multi-row weight-streaming kernel with K cut into
     ranges; either way the next norm adds up the planes, and the last block's planes go to the final norm."""
     from leone_amd import ops
     from leone_amd.engine.engine import Engine
@@ -409,9 +409,13 @@ def test_bfloat16_engine_against_the_oracle_that_rounds_where_it_rounds(tmp_path
     got = schedules.collect(steps, outputs)
     differences = np.concatenate([np.abs(np.stack(got[rid]) - expected[rid]).ravel() for rid in requests])
     assert differences.mean() <= ROUNDED_MEAN[name], f"{name}/{schedule}: mean difference {differences.mean():.2e}"
-    # the first position of a request sees one key, whose weight is exactly 1: only the other roundings are left there
-    first = max(float(np.abs(got[rid][0] - expected[rid][0]).max()) for rid in requests)
-    assert first <= 2e-3, f"{name}/{schedule}: first positions differ by {first:.2e}"
+    # The first position of a request sees one key, whose weight is exactly 1: only the other roundings are left
+    # there, and the oracle reproduces them: most first positions agree to the last bits of a float.  One in a
+    # few has a single bfloat16 value of the first layers fall the other way (which one depends on the order
+    # in which a kernel's waves add up K), and then nearly every logit of that position moves by up to 3e-3.
+    firsts = sorted(float(np.abs(got[rid][0] - expected[rid][0]).max()) for rid in requests)
+    assert firsts[(len(firsts) - 1) // 2] <= 1e-5, f"{name}/{schedule}: first positions differ by {firsts}"
+    assert firsts[-1] <= 5e-3, f"{name}/{schedule}: a first position differs by {firsts[-1]:.2e}"
 
 
 # ---- the layer sizes of the large models ----------------------------------------------------------------
@@ -428,7 +432,7 @@ REAL = {
 }
 REAL_LENGTHS = {"8b-1": [150, 600], "8b-2": [300, 160], "32b-1": [200, 330]}
 REAL_SCHEDULES = dict(SCHEDULES, portions=lambda requests: schedules.portions(
-    requests, sizes=(10, 11, 64, 65, 128, 129, 2, 40)))      # both sides of every change of kernel
+    requests, sizes=(16, 17, 64, 65, 128, 129, 2, 40)))      # both sides of every change of kernel
 
 
 @pytest.fixture(scope="module")
@@ -451,7 +455,7 @@ def real_cases(tmp_path_factory):
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 @pytest.mark.parametrize("name", list(REAL))
 def test_layers_of_the_large_models_match_plain(real_cases, name, dtype_name, schedule):
-    """The widths at which the products' plans, the cuts of K and the changes of kernel at 10/11, 64/65 and
+    """The widths at which the products' plans, the cuts of K and the changes of kernel at 16/17, 64/65 and
     128/129 rows were chosen (crates/leone-cuda/tests/gpu.rs:653-711 tests at the model's own shapes).
     Logits reach 7.5 here, so the bounds are taken relative to the largest logit: float32 as everywhere
     (measured 4e-5), bfloat16 1.5 % for a single logit and 0.25 % on average (measured 0.9 % and 0.16 %)."""
@@ -484,10 +488,11 @@ def test_layers_of_the_large_models_match_plain(real_cases, name, dtype_name, sc
 
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 @pytest.mark.parametrize("name", ["B", "M"])
-def test_twenty_live_requests_decoding_side_by_side(tmp_path, name, dtype_name):
-    """Up to twenty live requests, most of them decoding: steps of 11 to 30 rows of single tokens beside short
+def test_many_live_requests_decoding_side_by_side(tmp_path, name, dtype_name):
+    """Up to 28 live requests, most of them decoding: steps of 17 to 28 rows of single tokens beside short
     portions, which is where the multi-row weight-streaming products and the split-KV kernel serve many
     requests at once; few pages, so that finished requests' pages are used again."""
+    from leone_amd import ops
     from leone_amd.engine.engine import Engine
     from leone_amd.runtime import load_model
 
@@ -495,15 +500,15 @@ def test_twenty_live_requests_decoding_side_by_side(tmp_path, name, dtype_name):
                             sharpen=2.0 if dtype_name == "float32" else 1.0)
     config, weights = read_config(folder), read_weights(folder)
     gen = np.random.default_rng(5)
-    requests = {f"d{i}": random_tokens(900 + i, int(gen.integers(18, 60)), config["vocab_size"]) for i in range(30)}
+    requests = {f"d{i}": random_tokens(900 + i, int(gen.integers(18, 60)), config["vocab_size"]) for i in range(40)}
     expected = {rid: qwen3_plain.forward(weights, config, toks).numpy() for rid, toks in requests.items()}
-    steps = schedules.mixed(requests, max_live=20, prompt_fraction=0.3, sizes=(5, 2, 9, 3))
+    steps = schedules.mixed(requests, max_live=28, prompt_fraction=0.3, sizes=(5, 2, 9, 3))
     decode_rows = [sum(1 for e in s["entries"] if len(e["tokens"]) == 1) for s in steps]
-    assert max(decode_rows) >= 16 and sum(1 for n in decode_rows if n >= 11) >= 20
+    assert max(decode_rows) >= 20 and sum(1 for n in decode_rows if n > ops.FUSED_ROWS) >= 20
     engine = Engine(load_model(folder, dtype_name), num_pages=schedules.max_live_tokens(steps, round_to=16) // 16,
-                    page_tokens=16, max_requests=20, poison_freed=True)
+                    page_tokens=16, max_requests=28, poison_freed=True)
     outputs = run_steps(engine, steps)
-    compare(steps, outputs, expected, tolerance(dtype_name), f"{name}/{dtype_name}/twenty live")
+    compare(steps, outputs, expected, tolerance(dtype_name), f"{name}/{dtype_name}/many live")
 
 
 @pytest.mark.parametrize("name", ["A", "M", "B"])

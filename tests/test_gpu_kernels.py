@@ -831,7 +831,7 @@ def test_gemm_rows_residual(mnk):
     close(stream2, want, 2e-6 * k, 1e-5, "planes added by the norm")
 
 
-@pytest.mark.parametrize("mfk", [(16, 12288, 4096), (36, 88, 80), (128, 256, 96), (64, 17408, 5120)])
+@pytest.mark.parametrize("mfk", [(16, 12288, 4096), (17, 1024, 512), (36, 88, 80), (128, 256, 96), (64, 17408, 5120)])
 def test_gemm_rows_gated(mfk):
     from leone_amd import ops
     m, f, k = mfk
@@ -844,7 +844,8 @@ def test_gemm_rows_gated(mfk):
         assert out.shape == (m, f) and out.dtype == torch.bfloat16
         want = plain.swiglu(x.double() @ wg.double().T, x.double() @ wu.double().T)
         close(out, want, 1e-2, 1e-2, "gated product")
-    assert torch.equal(ops.linear(x, w, gated=True), ops.gemm_rows(x, w, gated=True))
+    if m > ops.FUSED_ROWS:                            # fewer rows go to the kernel for few rows
+        assert torch.equal(ops.linear(x, w, gated=True), ops.gemm_rows(x, w, gated=True))
 
 
 @pytest.mark.parametrize("gain_dtype", [torch.float32, torch.bfloat16])
