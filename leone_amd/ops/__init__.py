@@ -550,15 +550,15 @@ def rows_plan(m: int, n: int, k: int, may_split: bool, units: int = 256) -> tupl
     waiting for a second round (6,144 x 4,096 at 64 rows: 18 us with 256 workgroups, 22 with 480, 24 with
     288), so the plan minimises rounds x the longest workgroup's traffic, where a chunk of K costs a
     workgroup its waves' weight tiles plus half of X's tiles (those come from the cache) and starting up
-    costs as much as 1,536 elements of K (with 768 the plan cut a 12,288-long K of 96 and 128 rows into 8 ranges
-    for 8 waves: 29.2 and 34.1 us against 26.5 and 32.9 with 4 and 4); ties go to fewer ranges, then fewer waves.  Matrices with rows for many rounds (a vocabulary) take the workgroup size by
-    the rows of X alone."""
+    costs as much as 3,072 elements of K; ties go to fewer ranges, then fewer waves.  The constants were set
+    in whole decode steps of 17 to 128 rows at the layer sizes of the 8B, 14B and 32B models (a start of 768
+    or 1,536 elements cuts long K's into too many ranges: 8B 8.05 : 7.91 ms a step at 64 rows; a fixed choice
+    for matrices of many rows gave the 32B gate/up product 4 waves and four rounds where 8 waves need two:
+    21.7 : 20.3 ms at 64 rows)."""
     chunk = library().leone_gemm_rows_chunk(m)
     chunks = -(-k // chunk)
     tiles = -(-n // 16)
     x_tiles = -(-m // 16)
-    if tiles >= 8 * units:
-        return (4 if m <= 32 else 6 if m <= 80 else 8), 1
     best = None
     for waves in ROWS_WAVES:
         groups = -(-tiles // waves)
@@ -567,7 +567,7 @@ def rows_plan(m: int, n: int, k: int, may_split: bool, units: int = 256) -> tupl
             if per * (splits - 1) >= chunks:            # a range would be empty
                 continue
             rounds = -(-groups * splits // units)
-            cost = (rounds * (per + 1536 // chunk) * (waves + 0.5 * x_tiles), splits, waves)
+            cost = (rounds * (per + 3072 // chunk) * (waves + 0.5 * x_tiles), splits, waves)
             if best is None or cost < best:
                 best = cost
     return best[2], best[1]

@@ -796,7 +796,9 @@ def test_products_read_the_tiled_copy_of_a_weight_to_the_same_bits(nk):
 def test_gemm_rows_plan_fills_the_compute_units():
     """The plan at the shapes it was measured on, and that it never names an empty range of K."""
     from leone_amd import ops
-    assert ops.rows_plan(64, 6144, 4096, True) == (6, 4)
+    assert ops.rows_plan(64, 6144, 4096, True) == (4, 2)
+    assert ops.rows_plan(64, 51200, 5120, False) == (8, 1)        # 400 workgroups, two rounds; four waves would need four
+    assert ops.rows_plan(24, 34816, 5120, False) == (6, 1)
     assert ops.rows_plan(64, 4096, 4096, True) == (4, 4)
     assert ops.rows_plan(64, 24576, 4096, False) == (6, 1)
     assert ops.rows_plan(64, 4096, 12288, True) == (4, 4)
