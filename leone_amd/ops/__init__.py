@@ -218,14 +218,24 @@ def decode_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: i
             and page_tokens >= 16 and page_tokens & (page_tokens - 1) == 0)
 
 
+DECODE_SPLIT_START_TILES = 8   # what starting a workgroup of the split-KV kernel costs, in 32-key tiles
+
+
 def choose_splits(rows: int, kv_heads: int, group: int, max_context: int, units: int = 256) -> int:
-    """How many parts the keys of a row are cut into: about one workgroup for each compute unit (measured in
-    whole decode steps at 8,192 keys: against two a unit 4.91 : 4.97 ms a step at 8 rows, 3.89 : 3.93 at 3,
-    level at 1 and from 16 rows on), at least four 32-key tiles a part so that each of a workgroup's four waves
-    has one, at most 32 parts."""
+    """Into how many parts the keys of a row are cut: the number (up to 32, at least four 32-key tiles a part,
+    one for each of a workgroup's waves) for which the compute unit with the most workgroups has the least to
+    do: ceil(workgroups / units) x (tiles a part + a start worth 8 tiles).  Measured in whole decode steps at
+    8,192 keys, 1 to 48 rows, against a fixed aim of one or two workgroups a unit: level where those do well
+    (1, 8, 12, 17 rows) and up to 15 % of a step better where their workgroup counts leave units idle or a few
+    with one workgroup more than the rest (24 rows: 8.67 ms against 9.18, 40 rows: 11.8 against 13.9)."""
     blocks = rows * kv_heads * ((group + 15) // 16)
     tiles = (max_context + 31) // 32
-    return max(1, min(units // max(1, blocks), (tiles + 3) // 4, 32))
+    best = None
+    for splits in range(1, min(32, max(1, tiles // 4)) + 1):
+        cost = (-(-blocks * splits // units) * (-(-tiles // splits) + DECODE_SPLIT_START_TILES), splits)
+        if best is None or cost < best:
+            best = cost
+    return best[1]
 
 
 def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
