@@ -104,3 +104,24 @@ def test_rotary_base_from_rope_parameters_and_harmless_extras():
     raw.update(rope_parameters={"rope_type": "default", "rope_theta": 123456.0}, layer_types=["full_attention"] * 2,
                rope_scaling={"rope_type": "default"}, sliding_window=4096, use_sliding_window=False)
     assert config_from_dict(raw).rope_theta == 123456.0
+
+
+def test_decode_attention_cuts_keys_to_fill_the_compute_units():
+    """``ops.choose_splits`` (host arithmetic only): every part keeps at least four 32-key tiles, at most 32
+    parts; few rows over many keys are cut so that every unit has work, many rows are not cut at all; and
+    the choice never leaves a few units with one workgroup more than the rest where another choice would not
+    (17 rows of 8 kv heads: 136 workgroups; cut in two they would be 272 on 256 units, so it is three or five)."""
+    from leone_amd import ops
+
+    for rows in range(1, 200):
+        for context in (1, 31, 100, 128, 1000, 8192, 100_000):
+            splits = ops.choose_splits(rows, 8, 4, context)
+            tiles = -(-context // 32)
+            assert 1 <= splits <= 32 and (splits == 1 or tiles // splits >= 4 or tiles // 4 >= splits)
+    assert ops.choose_splits(1, 8, 4, 8192) == 32
+    assert ops.choose_splits(8, 8, 4, 8192) == 4
+    assert ops.choose_splits(64, 8, 4, 8192) == 1
+    assert ops.choose_splits(17, 8, 4, 8192) in (3, 5)
+    assert ops.choose_splits(40, 8, 4, 8192) in (2, 4)
+    assert ops.choose_splits(8, 8, 4, 100) == 1                     # four tiles in all: nothing to cut
+    assert ops.choose_splits(1, 64, 1, 8192, units=304) >= 4        # other head counts, another chip
