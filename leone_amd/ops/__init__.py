@@ -308,8 +308,10 @@ def attention_decode_projected(qkv: torch.Tensor, q_heads: int, kv_heads: int, h
 PREFILL_TILE_ROWS = 32       # rows of one request a wave of the prompt kernel takes (checked against the library)
 PREFILL_GROUP_TILES = 4      # tiles of one request a workgroup of the prompt kernel takes (likewise)
 PREFILL_MIN_ROWS = 16        # shorter portions go through the split-KV kernel row by row
-PREFILL_SPLIT_MIN_STAGES = 8 # a key range of the prompt kernel is worth a workgroup from this many 64-key stages
 PREFILL_MAX_SPLITS = 32      # most key ranges the prompt kernel takes (checked against the library)
+PREFILL_SPLIT_MIN_STAGES = 4 # a key range of the prompt kernel keeps at least this many 64-key stages
+PREFILL_SPLIT_START_STAGES = 8   # what a workgroup of the prompt kernel costs before its first stage, in stages
+PREFILL_SPLIT_MERGE_STAGES = 6   # what writing and merging a range's partial results adds, in stages
 
 
 def prefill_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: int, max_blocks: int = 0) -> bool:
@@ -318,14 +320,26 @@ def prefill_attention_supported(dtype: torch.dtype, head_dim: int, page_tokens: 
             and page_tokens >= 16 and page_tokens & (page_tokens - 1) == 0)
 
 
-def choose_prefill_splits(groups: int, q_heads: int, mean_keys: int, window: int = 0) -> int:
-    """How many ranges the keys of a prompt workgroup are cut into: enough for about two workgroups on each
-    of the 256 CUs, as long as a range keeps PREFILL_SPLIT_MIN_STAGES stages of 64 keys where a row sees
-    ``mean_keys`` keys.  (A prompt from position 0 gains nothing: its early rows see few keys.)"""
+def choose_prefill_splits(groups: int, q_heads: int, mean_keys: int, window: int = 0, units: int = 256) -> int:
+    """How many ranges the keys of a prompt workgroup are cut into, where a row sees ``mean_keys`` keys: the
+    number (a range keeps at least PREFILL_SPLIT_MIN_STAGES stages of 64 keys) for which the rounds of
+    workgroups over the chip (two fit a compute unit) x (stages a range + the start, + the merge where there
+    is more than one range) come out least.  Measured in whole
+    steps on portions of 128 to 1,536 rows after 30,720 positions against a fixed aim of two workgroups a unit:
+    level for 256, 512 and 1,024 rows, 28.9 against 30.2 ms for 768 rows, 51.3 against 54.4 for 1,536.  (A
+    prompt from position 0 gains nothing from ranges, its early rows see few keys: without the merge's term
+    the rule took two ranges for 1,024 and 3,072 rows and lost 3 and 4 % of the step by it.)"""
     reach = PREFILL_GROUP_TILES * PREFILL_TILE_ROWS
     keys = min(mean_keys, window + reach) if window > 0 else mean_keys
     stages = -(-keys // 64)
-    return max(1, min(512 // max(1, groups * q_heads), stages // PREFILL_SPLIT_MIN_STAGES, PREFILL_MAX_SPLITS))
+    blocks = max(1, groups * q_heads)
+    best = None
+    for splits in range(1, min(PREFILL_MAX_SPLITS, max(1, stages // PREFILL_SPLIT_MIN_STAGES)) + 1):
+        each = -(-stages // splits) + PREFILL_SPLIT_START_STAGES + (PREFILL_SPLIT_MERGE_STAGES if splits > 1 else 0)
+        cost = (-(-blocks * splits // (2 * units)) * each, splits)
+        if best is None or cost < best:
+            best = cost
+    return best[1]
 
 
 def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
@@ -351,7 +365,7 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, 
         raise KernelError(f"attention_prefill: tiles must be int32 [n, 3] with n a multiple of {PREFILL_GROUP_TILES}")
     groups = tiles.shape[0] // PREFILL_GROUP_TILES
     if splits is None:
-        splits = choose_prefill_splits(groups, q_heads, mean_keys, window)
+        splits = choose_prefill_splits(groups, q_heads, mean_keys, window, compute_units(q.device))
     part_acc = part_ml = None
     if splits > 1:
         covered = rows if covered_rows is None else covered_rows

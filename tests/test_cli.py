@@ -107,7 +107,11 @@ def test_key_ranges_of_the_prompt_kernel_are_chosen_by_rows_and_keys():
         for keys in (1, 63, 64, 1000, 5000, 200000):
             splits = ops.choose_prefill_splits(groups, heads, keys)
             assert 1 <= splits <= ops.PREFILL_MAX_SPLITS
-            assert splits == 1 or (splits * groups * heads <= 512 and -(-keys // 64) // splits >= ops.PREFILL_SPLIT_MIN_STAGES)
+            assert splits == 1 or -(-keys // 64) // splits >= ops.PREFILL_SPLIT_MIN_STAGES
+    assert ops.choose_prefill_splits(6, heads, 31000) == 5                       # 768 rows: 960 workgroups, two rounds of 512
+    assert ops.choose_prefill_splits(8, heads, 512) == 1                         # 1,024 rows from position 0: the merge costs more
+    assert ops.choose_prefill_splits(24, heads, 1536) == 1                       # and 3,072
+    assert ops.choose_prefill_splits(12, heads, 31000) == 4
 
 
 def test_version_and_build_info(capsys):

@@ -100,7 +100,7 @@ def test_engine_matches_plain(cases, name, dtype_name, schedule, page_tokens):
 @pytest.mark.parametrize("name", ["M", "C"])
 def test_prompt_key_ranges_agree_with_plain(cases, monkeypatch, name, schedule):
     """The prompt kernel cuts a workgroup's keys into ranges when rows are few and keys many; here every
-    64-key stage may be a range of its own, so that the tiny prompts go that way too."""
+    64-key stage may be a range of its own and ranges cost nothing, so that the tiny prompts go that way too."""
     from leone_amd import ops
     from leone_amd.engine.engine import Engine
     from leone_amd.runtime import load_model
@@ -113,6 +113,8 @@ def test_prompt_key_ranges_agree_with_plain(cases, monkeypatch, name, schedule):
         return chosen[-1]
 
     monkeypatch.setattr(ops, "PREFILL_SPLIT_MIN_STAGES", 1)
+    monkeypatch.setattr(ops, "PREFILL_SPLIT_START_STAGES", 0)
+    monkeypatch.setattr(ops, "PREFILL_SPLIT_MERGE_STAGES", 0)
     monkeypatch.setattr(ops, "choose_prefill_splits", recording)
     folder, requests, expected = cases(name, "bfloat16")
     steps = SCHEDULES[schedule](requests)
