@@ -59,7 +59,10 @@ class Runtime:
     def __init__(self, model, *, num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  page_tokens: int = 64, max_requests: int = 64, max_context: Optional[int] = None,
                  policy: Optional[SchedulerPolicy] = None, tokenizer=None, graphs: bool = True,
-                 poison_freed: bool = False, streamed_weights: Optional[bool] = None):
+                 poison_freed: bool = False, streamed_weights: Optional[bool] = None, tune_products: bool = False):
+        """``tune_products``: let the vendor library's products of a full prompt portion (the policy's
+        ``prefill_chunk_tokens``) run with the fastest of the library's algorithms, measured now (a few
+        seconds; ``Engine.tune_products``)."""
         self.model = model
         model.keep_streamed_copies(streamed_weights)       # before the cache is sized by what is free
         self.config = getattr(model, "config", None)
@@ -73,6 +76,11 @@ class Runtime:
                              max_requests=max_requests, max_context=context, graphs=graphs,
                              poison_freed=poison_freed, streamed_weights=streamed_weights)
         self.policy = policy or SchedulerPolicy(max_live_requests=max_requests)
+        self.tuned_products = []
+        if tune_products and model.dtype == torch.bfloat16:
+            portion = min(self.policy.prefill_chunk_tokens, self.policy.max_step_tokens, context)
+            if portion <= self.engine.cache.free_pages(0) * page_tokens:      # the trial step needs that room for a moment
+                self.tuned_products = self.engine.tune_products(portion)
         self.tokenizer = tokenizer
         self.last_stats: Optional[GenerationStats] = None
         self.last_decode_profile: Optional[StepProfile] = None

@@ -273,6 +273,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     parser.add_argument("--no-peaks", action="store_true", help="skip the measurement of this GPU's own peaks")
     parser.add_argument("--no-streamed-weights", action="store_true",
                         help="keep no second copy of the matrices in the decode kernels' order")
+    parser.add_argument("--no-tuned-products", action="store_true",
+                        help="leave the choice of the vendor library's algorithms for the prompt's products to its heuristic")
     parser.add_argument("--peaks", action="store_true", help="only measure this GPU's own peaks and print them")
     parser.add_argument("--scenario", choices=sorted(SCENARIOS), help="run a serving scenario instead of the headline figure")
     args = parser.parse_args(argv)
@@ -341,6 +343,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     if profile_steps:
         record["kernels"] = kernel_table(timed[2], model, args.batch, start + args.warmup + args.steps + 2)
     if not args.no_prefill:
+        # the vendor library's products of the prompt run with the fastest of the library's algorithms, found by
+        # timing them now on this model's matrices (Engine.tune_products)
+        tuned = [] if args.no_tuned_products or args.dtype != "bfloat16" else engine.tune_products(PREFILL_TOKENS, thorough=True)
+        record["config"]["library_products"] = "measured choice" if any(r["kept"] for r in tuned) else "heuristic"
         seconds = time_prefill(engine, PREFILL_TOKENS)
         flops = prefill_flops(config, PREFILL_TOKENS)
         record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,

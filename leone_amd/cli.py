@@ -90,6 +90,8 @@ def build_parser() -> argparse.ArgumentParser:
     g.add_argument("--ignore-eos", action="store_true", help="Do not stop at the end token")
     g.add_argument("--single-weight-copy", action="store_true",
                    help="Keep no second copy of the matrices in the decode kernels' order (half the weight memory, slower decoding)")
+    g.add_argument("--tune-products", action="store_true",
+                   help="Time the vendor library's algorithms for a full prompt portion first and use the fastest (a few seconds)")
     _add_sampling(g)
 
     d = sub.add_parser("doctor", help="Check the platform, the kernel library and a model folder")
@@ -136,6 +138,7 @@ def cmd_generate(args) -> int:
     runtime = Runtime.load(args.model, args.dtype, max_requests=1, max_context=args.max_context,
                            graphs=not args.eager_decode,
                            streamed_weights=False if args.single_weight_copy else None,
+                           tune_products=args.tune_products,
                            policy=SchedulerPolicy(max_live_requests=1, prefill_chunk_tokens=args.prefill_chunk,
                                                   max_step_tokens=max(args.prefill_chunk, 1)))
     if args.prompt is not None:

@@ -125,6 +125,25 @@ int leone_gemm_rows_chunk(int m);
 int leone_gemm_rows_bf16(const void* x, const void* w, int w_tiled, void* y, int out_mode, int out_dtype, int m, int n, int k,
                          int splits, long plane, int waves, hipStream_t stream);
 
+// The vendor library's product for more rows than the kernels above take, Y[M,N] = X[M,K] . W[N,K]^T (or Y +=
+// with `accumulate`, Y float32), X and W bfloat16, Y of out_dtype, float accumulation, with the library's
+// algorithm chosen by measurement.  leone_library_product_tune times up to max_candidates of the algorithms the
+// library's heuristic lists for the problem, with every_algorithm also all others the library has for it (some
+// thousands, a few seconds), on the caller's operands (x, the n_ws weights of that shape in turn, y as
+// scratch: it is overwritten) and keeps the fastest for this device and exactly this (m, n, k, out_dtype,
+// accumulate); it reports the time of the library's own first choice and of the winner in microseconds.
+// leone_library_product runs a problem that was tuned and refuses any other: the caller keeps its ordinary
+// call of the library for those.  _available: 1 if hipBLASLt could be found in the process or on the loader's
+// path (it is looked up at run time and only then); _tuned: 1 if the problem was tuned on the current device.
+int leone_library_product_available();
+int leone_library_product_tuned(int m, int n, int k, int out_dtype, int accumulate);
+int leone_library_product_forget(int m, int n, int k, int out_dtype, int accumulate);
+int leone_library_product(const void* x, const void* w, void* y, int m, int n, int k, int out_dtype, int accumulate,
+                          hipStream_t stream);
+int leone_library_product_tune(const void* x, const void* const* ws, int n_ws, void* y, int m, int n, int k,
+                               int out_dtype, int accumulate, int max_candidates, int every_algorithm, float* first_us,
+                               float* best_us, int* candidates_timed, hipStream_t stream);
+
 // What the memory and the matrix cores give with nothing else going on: one read of `bytes` (a multiple of
 // 16), one copy, and blocks x 4 waves x iterations x 8 v_mfma_f32_16x16x32_bf16, or with `wide` x 4
 // v_mfma_f32_32x32x16_bf16, the same work (leone_peak_mfma_flops in all).

@@ -223,6 +223,29 @@ class Engine:
             raise StepError("a model with per-request state cannot be cut back")
         self.cache.truncate(request, position)
 
+    # ---- the vendor library's products ---------------------------------------------------
+    def tune_products(self, rows: int, candidates: int = 256, thorough: bool = False) -> List[dict]:
+        """Lets the vendor library's products of a step of ``rows`` prompt tokens (the portion size a scheduler
+        cuts long prompts into) be run with the fastest of the library's algorithms instead of the one its
+        heuristic names: one such step runs on a request of its own to see which products it hands to the
+        library, and ``ops.tune_library_product`` times the candidates for each on the model's own matrices.
+        Takes a few seconds (``thorough``: every algorithm of the library, not only the heuristic's list; some
+        ten seconds); steps of other sizes are not affected.  Needs room for ``rows`` tokens in the
+        cache for the moment.  Returns a record for every product."""
+        if not ops.library_product_available():
+            return []
+        rows = min(int(rows), self.max_context)
+        request = ("tune products", id(self))
+        with ops.record_library_products() as recorded:
+            self.step([StepEntry(request, [0] * rows, [rows - 1])])
+        self.release(request)
+        torch.cuda.synchronize(self.device)
+        records = []
+        for (m, n, k, out_code, accumulate), weights in recorded.problems.items():
+            out_dtype = torch.float32 if out_code == ops.F32 else torch.bfloat16
+            records.append(ops.tune_library_product(m, weights, out_dtype, bool(accumulate), candidates, thorough))
+        return records
+
     # ---- the step --------------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]) -> None:
         """Refuses a malformed step before anything is reserved (the layout routine checks again)."""

@@ -659,6 +659,116 @@ def inner_parts(rows: int, n: int, k: int) -> int:
     return 1
 
 
+# ---- the vendor library's product with a measured choice of its algorithm -------------------------------------
+_tuned_products: set = set()     # (device index, m, n, k, output code, accumulate) of the problems tuned
+_recorded_products = None        # while ``record_library_products`` runs: problem -> weights it was asked with
+
+
+class record_library_products:
+    """Within this context ``linear`` notes every product that it hands to the vendor library: the problem
+    (rows, weight rows, inner size, output type, whether it adds into the stream) and the weights it came with.
+    ``problems`` maps each problem to its weights afterwards."""
+
+    def __enter__(self):
+        global _recorded_products
+        self.problems: dict = {}
+        self._before = _recorded_products
+        _recorded_products = self.problems
+        return self
+
+    def __exit__(self, *exc):
+        global _recorded_products
+        _recorded_products = self._before
+        return False
+
+
+def _library_problem(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype, accumulate: bool):
+    return (x.device.index or 0, x.shape[0], weight.shape[0], weight.shape[1], F32 if out_dtype == torch.float32 else BF16,
+            1 if accumulate else 0)
+
+
+def library_product_available() -> bool:
+    return bool(library().leone_library_product_available())
+
+
+def tune_library_product(rows: int, weights, out_dtype: torch.dtype, accumulate: bool, candidates: int = 256,
+                         thorough: bool = False) -> dict:
+    """Times the vendor library's algorithms for ``[rows, K] . W^T`` on ``weights`` (matrices of one shape, taken
+    in turn as a model's layers are; ``candidates`` from the library's heuristic, with ``thorough`` every
+    algorithm the library has) and keeps the fastest for ``linear`` to use on exactly this problem, after
+    checking its result against a float32 product: it must be no further from it than twice what the library's
+    ordinary call is.  Returns the problem, the microseconds of the library's own choice and of the winner, and
+    how many algorithms were timed; ``kept`` is False if the winner failed the check and was dropped."""
+    weights = list(weights)
+    weight = weights[0]
+    n, k = weight.shape
+    if any(w.shape != weight.shape or w.dtype != torch.bfloat16 or not w.is_contiguous() for w in weights):
+        raise KernelError("tune_library_product: the weights must be contiguous bfloat16 matrices of one shape")
+    if accumulate and out_dtype != torch.float32:
+        raise KernelError("tune_library_product: adding into the stream is a float32 product")
+    generator = torch.Generator(device=weight.device).manual_seed(rows * 31 + n)
+    x = torch.randn((rows, k), device=weight.device, generator=generator).to(torch.bfloat16)
+    y = torch.zeros((rows, n), dtype=out_dtype, device=weight.device)
+    import ctypes
+    pointers = (ctypes.c_void_p * len(weights))(*[w.data_ptr() for w in weights])
+    first, best, timed = ctypes.c_float(), ctypes.c_float(), ctypes.c_int()
+    out_code = F32 if out_dtype == torch.float32 else BF16
+    call("leone_library_product_tune", _dev(x, "x", torch.bfloat16), pointers, len(weights), _dev(y, "y"), rows, n, k,
+         out_code, 1 if accumulate else 0, int(candidates), 1 if thorough else 0, ctypes.byref(first), ctypes.byref(best),
+         ctypes.byref(timed), _stream())
+    problem = _library_problem(x, weight, out_dtype, accumulate)
+    # the check: the winner and the library's ordinary call against a float32 product, from a zero stream
+    exact = torch.mm(x.float(), weight.float().t())
+    y.zero_()
+    call("leone_library_product", _dev(x, "x"), _dev(weight, "w"), _dev(y, "y"), rows, n, k, out_code,
+         1 if accumulate else 0, _stream())
+    usual = torch.mm(x, weight.t(), out_dtype=torch.float32) if out_dtype == torch.float32 else torch.nn.functional.linear(x, weight)
+    off = (y.float() - exact).abs().max().item()
+    usual_off = (usual.float() - exact).abs().max().item()
+    kept = bool(off <= 2.0 * usual_off + 1e-6 * exact.abs().max().item())
+    if kept:
+        _tuned_products.add(problem)
+    else:
+        call("leone_library_product_forget", rows, n, k, out_code, 1 if accumulate else 0)
+    return {"rows": rows, "weight_rows": n, "inner": k, "float_out": out_dtype == torch.float32, "adds": bool(accumulate),
+            "library_us": round(first.value, 1), "tuned_us": round(best.value, 1), "timed": timed.value, "kept": kept,
+            "off": off, "library_off": usual_off}
+
+
+def forget_tuned_products() -> None:
+    for device, m, n, k, out_code, accumulate in list(_tuned_products):
+        with torch.cuda.device(device):
+            call("leone_library_product_forget", m, n, k, out_code, accumulate)
+    _tuned_products.clear()
+
+
+def _library_product(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,
+                     residual: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """The vendor library's product for many rows: bfloat16 or float32 out, or added into the float32 stream
+    (then nothing comes back).  A problem that was tuned runs with the algorithm that won; any other goes
+    through torch's call of the same library."""
+    problem = _library_problem(x, weight, out_dtype, residual is not None)
+    if _recorded_products is not None:
+        known = _recorded_products.setdefault(problem[1:], [])
+        if all(w is not weight for w in known):
+            known.append(weight)
+    if problem in _tuned_products and x.is_contiguous() and weight.is_contiguous():
+        y = residual if residual is not None else torch.empty((x.shape[0], weight.shape[0]), dtype=out_dtype, device=x.device)
+        call("leone_library_product", _dev(x, "x", torch.bfloat16), _dev(weight, "w", torch.bfloat16),
+             _dev(y, "y", out_dtype, (x.shape[0], weight.shape[0])), x.shape[0], weight.shape[0], weight.shape[1],
+             problem[4], problem[5], _stream())
+        return None if residual is not None else y
+    if residual is not None:
+        # the library adds into the stream itself (float product plus float stream, the same bits as adding the
+        # product afterwards), which saves the next norm's kernel the read of the product: 27.2 against 27.8 ms
+        # for a prompt of 2,048 tokens
+        torch.addmm(residual, x, weight.t(), out_dtype=torch.float32, out=residual)
+        return None
+    if out_dtype == torch.float32:
+        return torch.mm(x, weight.t(), out_dtype=torch.float32)
+    return torch.nn.functional.linear(x, weight)    # float accumulation
+
+
 def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
            residual: Optional[torch.Tensor] = None, gated: bool = False,
            planes_ok: bool = False, next_norm=None):
@@ -716,16 +826,12 @@ def linear(x, weight: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                 y = torch.bmm(x.view(rows, parts, k // parts).transpose(0, 1),
                               weight.view(weight.shape[0], parts, k // parts).permute(1, 2, 0), out_dtype=torch.float32)
             elif residual is not None:
-                # the library adds into the stream itself (float product plus float stream, the same bits as
-                # adding the product afterwards), which saves the next norm's kernel the read of the product:
-                # 27.2 against 27.8 ms for a prompt of 2,048 tokens
-                torch.addmm(residual, x, weight.t(), out_dtype=torch.float32, out=residual)
-                return None
+                return _library_product(x, weight, torch.float32, residual)
             else:
-                y = torch.mm(x, weight.t(), out_dtype=torch.float32)
+                y = _library_product(x, weight, torch.float32, None)
     else:
         with profile.span(profile.LIBRARY_PRODUCT, weight):
-            y = torch.nn.functional.linear(x, weight)  # library matrix product, float accumulation
+            y = _library_product(x, weight, torch.bfloat16, None)
         if out_dtype != y.dtype:
             y = y.to(out_dtype)
     return swiglu(y) if gated else y

@@ -45,6 +45,9 @@ _PROTOTYPES = {
     "leone_peak_read": [P, ctypes.c_long, P, c_int, P],
     "leone_peak_copy": [P, P, ctypes.c_long, c_int, P],
     "leone_peak_mfma": [c_int, c_int, c_int, P, P],
+    "leone_library_product": [P, P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "leone_library_product_tune": [P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, P],
+    "leone_library_product_forget": [c_int, c_int, c_int, c_int, c_int],
     "leone_sample_temperature": [P, P, P, P, P, P, P, P, c_int, c_int, P],
     "leone_top_candidates": [P, P, P, P, c_int, c_int, c_int, P],
 }
@@ -78,6 +81,10 @@ def library() -> ctypes.CDLL:
             lib.leone_gemm_rows_max_rows.argtypes = []
             lib.leone_gemm_rows_chunk.restype = c_int
             lib.leone_gemm_rows_chunk.argtypes = [c_int]
+            lib.leone_library_product_available.restype = c_int
+            lib.leone_library_product_available.argtypes = []
+            lib.leone_library_product_tuned.restype = c_int
+            lib.leone_library_product_tuned.argtypes = [c_int, c_int, c_int, c_int, c_int]
             for name, argtypes in _PROTOTYPES.items():
                 fn = getattr(lib, name)
                 fn.argtypes = argtypes

@@ -126,6 +126,38 @@ def test_prompt_key_ranges_agree_with_plain(cases, monkeypatch, name, schedule):
     compare(steps, outputs, expected, tolerance("bfloat16"), f"{name}/key ranges/{schedule}")
 
 
+def test_tuned_library_products_agree_with_plain(cases):
+    """After ``Engine.tune_products`` the prompt portions of that size run the vendor library's products with
+    the algorithms that were fastest when timed: the logits still agree with the plain implementation, for a
+    prompt of the tuned size and for one of another size, and every tuned product is used."""
+    from leone_amd import ops
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+
+    folder, requests, expected = cases("M", "bfloat16")
+    name, tokens = max(requests.items(), key=lambda item: len(item[1]))
+    rows = len(tokens) - 7
+    assert rows > ops.ROWS_MAX, "the prompt is too short to reach the vendor library"
+    model = load_model(folder, "bfloat16")
+    engine = Engine(model, max_tokens=2 * len(tokens) + 64, page_tokens=16, max_requests=2)
+    try:
+        records = engine.tune_products(rows)
+        assert len(records) >= 3 and all(r["kept"] and r["rows"] == rows for r in records), records
+        assert not engine.cache.live_requests()
+        with ops.record_library_products() as seen:
+            steps = [{"step": 0, "entries": [{"id": name, "tokens": tokens[:rows], "want": list(range(rows))}], "end": []},
+                     {"step": 1, "entries": [{"id": name, "tokens": tokens[rows:], "want": list(range(7))}], "end": [name]},
+                     {"step": 2, "entries": [{"id": "again", "tokens": tokens[:rows - 3], "want": list(range(rows - 3))}], "end": ["again"]}]
+            outputs = run_steps(engine, steps)
+        assert ops._tuned_products and ops._tuned_products <= {(0,) + problem for problem in seen.problems}   # all were used
+        assert any(problem[0] == rows for problem in seen.problems) and any(problem[0] == rows - 3 for problem in seen.problems)
+        compare(steps[:2], outputs, {name: expected[name]}, tolerance("bfloat16"), "tuned products")
+        again = {"again": expected[name][:rows - 3]}
+        compare(steps[2:], {2: outputs[2]}, again, tolerance("bfloat16"), "beside tuned products")
+    finally:
+        ops.forget_tuned_products()
+
+
 def test_late_portions_of_a_long_request(tmp_path):
     """One request of 2,200 tokens at the large models' head shape: a long first portion, then portions of
     changing size far into the context, where the prompt kernel cuts the keys into ranges by its own rule,

@@ -941,3 +941,45 @@ def test_attention_decode_from_the_projection(shape, window, planes):
                                           entry, table, scale, window, max_context=700, write_cache=False)
     assert torch.equal(k3, k1) and torch.equal(v3, v1)
     assert torch.equal(got3, want3)                                   # nothing to contract: the same bits
+
+
+def test_library_products_with_a_measured_choice_of_algorithm():
+    """The vendor library's product for many rows, once with the algorithm its heuristic names (through torch) and
+    once with the one that was fastest when timed: both against a float64 product, for the three forms ``linear``
+    asks for (bfloat16 out, float32 out, added into the float32 stream); a problem of another size stays with
+    the heuristic."""
+    from leone_amd import ops
+    assert ops.library_product_available(), "hipBLASLt was not found in the process"
+    generator = torch.Generator().manual_seed(31)
+    n, k, rows = 384, 512, 200
+    weights = [(torch.randn(n, k, generator=generator) * 0.05).bfloat16().cuda() for _ in range(3)]
+    x = torch.randn(rows, k, generator=generator).bfloat16().cuda()
+    stream = torch.randn(rows, n, generator=generator).cuda()
+    exact = x.double() @ weights[1].double().t()
+    try:
+        for out_dtype, adds in ((torch.bfloat16, False), (torch.float32, False), (torch.float32, True)):
+            record = ops.tune_library_product(rows, weights, out_dtype, adds, candidates=64)
+            assert record["kept"] and record["timed"] >= 1, record
+            assert 0 < record["tuned_us"] <= record["library_us"], record
+            problem = (0, rows, n, k, ops.F32 if out_dtype == torch.float32 else ops.BF16, int(adds))
+            assert problem in ops._tuned_products
+            for m in (rows, rows + 8):                          # tuned, and left to the heuristic
+                with ops.record_library_products() as seen:
+                    if adds:
+                        y = stream[:1].repeat(m, 1).contiguous()
+                        base = y.double().clone()
+                        assert ops.linear(x[:1].repeat(m, 1).contiguous() if m != rows else x, weights[1], residual=y) is None
+                    else:
+                        base = 0.0
+                        y = ops.linear(x[:1].repeat(m, 1).contiguous() if m != rows else x, weights[1], out_dtype=out_dtype)
+                assert list(seen.problems) == [(m, n, k, problem[4], problem[5])]
+                want = base + (exact if m == rows else exact[:1].expand(m, n))
+                err = (y.double() - want).abs().max().item()
+                bound = 2e-2 if out_dtype == torch.bfloat16 else 2e-5      # half a bfloat16 step at |y| < 4; float sums of 512 terms
+                assert err <= bound, (out_dtype, adds, m, err)
+    finally:
+        ops.forget_tuned_products()
+    assert not ops._tuned_products
+    with pytest.raises(ops.KernelError, match="not tuned"):
+        y = torch.empty(rows, n, dtype=torch.float32, device="cuda")
+        ops.call("leone_library_product", x.data_ptr(), weights[0].data_ptr(), y.data_ptr(), rows, n, k, ops.F32, 0, None)
