@@ -13,6 +13,7 @@ reserved first, written by the kernels, and committed only if the step succeeds
 from __future__ import annotations
 
 import ctypes
+import time
 from ctypes import c_int, c_int64, c_long
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence
@@ -224,26 +225,50 @@ class Engine:
         self.cache.truncate(request, position)
 
     # ---- the vendor library's products ---------------------------------------------------
-    def tune_products(self, rows: int, candidates: int = 256, thorough: bool = False) -> List[dict]:
+    def tune_products(self, rows: int, candidates: int = 256, thorough: bool = False,
+                      keep_only_faster_steps: bool = True) -> List[dict]:
         """Lets the vendor library's products of a step of ``rows`` prompt tokens (the portion size a scheduler
         cuts long prompts into) be run with the fastest of the library's algorithms instead of the one its
-        heuristic names: one such step runs on a request of its own to see which products it hands to the
-        library, and ``ops.tune_library_product`` times the candidates for each on the model's own matrices.
-        Takes a few seconds (``thorough``: every algorithm of the library, not only the heuristic's list; some
-        ten seconds); steps of other sizes are not affected.  Needs room for ``rows`` tokens in the
-        cache for the moment.  Returns a record for every product."""
+        heuristic names.  A trial step of that size on a request of its own shows which products reach the
+        library; ``ops.tune_library_product`` times the candidates for each on the model's own matrices; and a
+        winner is kept only if the whole trial step is faster with it than without (a product timed by itself
+        says too little: at 1,024 rows of the 8B shape the winners of the four products made the step 3 %
+        slower; ``keep_only_faster_steps=False`` skips this).  Takes a few seconds (``thorough``: every algorithm of the library, not only the heuristic's
+        list); steps of other sizes are not affected.  Needs room for ``rows`` tokens in the cache for the
+        moment.  Returns a record for every product; ``kept`` says whether its winner is in use."""
         if not ops.library_product_available():
             return []
         rows = min(int(rows), self.max_context)
         request = ("tune products", id(self))
+        tokens = [(i * 7919) % self.vocab_size for i in range(rows)]      # varied, as a prompt's are
+
+        def trial_step_ms(repeats: int = 3) -> float:
+            best = float("inf")
+            for _ in range(repeats):
+                torch.cuda.synchronize(self.device)
+                started = time.perf_counter()
+                self.step([StepEntry(request, tokens, [rows - 1])])
+                torch.cuda.synchronize(self.device)
+                best = min(best, (time.perf_counter() - started) * 1e3)
+                self.release(request)
+            return best
+
         with ops.record_library_products() as recorded:
-            self.step([StepEntry(request, [0] * rows, [rows - 1])])
-        self.release(request)
-        torch.cuda.synchronize(self.device)
+            trial_step_ms(1)
+        step_ms = trial_step_ms()
         records = []
         for (m, n, k, out_code, accumulate), weights in recorded.problems.items():
             out_dtype = torch.float32 if out_code == ops.F32 else torch.bfloat16
-            records.append(ops.tune_library_product(m, weights, out_dtype, bool(accumulate), candidates, thorough))
+            record = ops.tune_library_product(m, weights, out_dtype, bool(accumulate), candidates, thorough)
+            if record["kept"] and keep_only_faster_steps:
+                with_it = trial_step_ms()
+                record["step_ms"], record["step_ms_before"] = round(with_it, 3), round(step_ms, 3)
+                if with_it < step_ms * 0.998:
+                    step_ms = with_it
+                else:
+                    ops.forget_tuned_products([record["problem"]])
+                    record["kept"] = False
+            records.append(record)
         return records
 
     # ---- the step --------------------------------------------------------------------

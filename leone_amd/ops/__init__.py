@@ -730,16 +730,19 @@ def tune_library_product(rows: int, weights, out_dtype: torch.dtype, accumulate:
         _tuned_products.add(problem)
     else:
         call("leone_library_product_forget", rows, n, k, out_code, 1 if accumulate else 0)
-    return {"rows": rows, "weight_rows": n, "inner": k, "float_out": out_dtype == torch.float32, "adds": bool(accumulate),
+    return {"problem": problem, "rows": rows, "weight_rows": n, "inner": k, "float_out": out_dtype == torch.float32,
+            "adds": bool(accumulate),
             "library_us": round(first.value, 1), "tuned_us": round(best.value, 1), "timed": timed.value, "kept": kept,
             "off": off, "library_off": usual_off}
 
 
-def forget_tuned_products() -> None:
-    for device, m, n, k, out_code, accumulate in list(_tuned_products):
+def forget_tuned_products(problems=None) -> None:
+    """Gives the named problems (all, if none are named) back to the library's heuristic."""
+    for problem in list(_tuned_products if problems is None else problems):
+        device, m, n, k, out_code, accumulate = problem
         with torch.cuda.device(device):
             call("leone_library_product_forget", m, n, k, out_code, accumulate)
-    _tuned_products.clear()
+        _tuned_products.discard(problem)
 
 
 def _library_product(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype,

@@ -141,7 +141,7 @@ def test_tuned_library_products_agree_with_plain(cases):
     model = load_model(folder, "bfloat16")
     engine = Engine(model, max_tokens=2 * len(tokens) + 64, page_tokens=16, max_requests=2)
     try:
-        records = engine.tune_products(rows)
+        records = engine.tune_products(rows, keep_only_faster_steps=False)    # tiny products: no step would be faster
         assert len(records) >= 3 and all(r["kept"] and r["rows"] == rows for r in records), records
         assert not engine.cache.live_requests()
         with ops.record_library_products() as seen:
