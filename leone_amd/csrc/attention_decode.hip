@@ -130,28 +130,6 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
     const int page_tokens = 1 << page_shift;
     const int page_mask = page_tokens - 1;
 
-    // The new token's key (wave 0) and value (wave 1) with the key's gains are asked for before anything else:
-    // they depend on nothing that is read here, and the workgroup that writes them into the cache (below) would
-    // otherwise wait for the row's position, its page, the projection, the gains and the angles one after the other.
-    constexpr int kHalfRuns = kD16;                   // runs of 8 elements in half a head
-    static_assert(kD <= 8 * kWave, "a wave copies a value in one go");
-    const bool writes = kFused && from.k_out != nullptr;
-    const bool key_lane = writes && wave == 0 && lane < kHalfRuns;   // elements 8L .. 8L+7 and their partners in the other half
-    const bool value_lane = writes && wave == 1 && 8 * lane < kD;
-    float new_a[8], new_b[8], gain_a[8], gain_b[8], new_v[8];
-    if constexpr (kFused) {
-        const long width = static_cast<long>(q_heads + 2 * kv_heads) * kD;
-        if (key_lane) {
-            load_projection8(from, width, row, static_cast<long>(q_heads + kvh) * kD + 8 * lane, new_a);
-            load_projection8(from, width, row, static_cast<long>(q_heads + kvh) * kD + kD / 2 + 8 * lane, new_b);
-            if (from.k_gain.ptr) {
-                load_any8(from.k_gain, 8 * lane, gain_a);
-                load_any8(from.k_gain, kD / 2 + 8 * lane, gain_b);
-            }
-        }
-        if (value_lane) load_projection8(from, width, row, static_cast<long>(q_heads + kv_heads + kvh) * kD + 8 * lane, new_v);
-    }
-
     const int n = positions[row] + 1;                                    // keys 0 .. n-1 exist
     const int lo = (window > 0 && n - window > 0) ? n - window : 0;      // first key in reach
     const int* table = block_table + static_cast<long>(row_entry[row]) * max_blocks;
@@ -173,44 +151,52 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         // The workgroup whose keys end with the row's own position makes that position's key and value and
         // writes them into the cache; its waves read them from there after the barrier.  (With more than 16
         // query heads a kv head several workgroups do, each for itself: the same bytes.)
-        if (writes && my_begin < my_end && my_end == t_end) {
+        if (from.k_out != nullptr && my_begin < my_end && my_end == t_end) {
+            const long width = static_cast<long>(q_heads + 2 * kv_heads) * kD;
             const int pos = n - 1;
-            float cs[8], sn[8];                           // asked for together with the page
-            if (key_lane && from.cos_table != nullptr) {
-                const int tpos = pos < from.table_positions ? pos : from.table_positions - 1;
-                load_any8(AnyVec{from.cos_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 8 * lane, cs);
-                load_any8(AnyVec{from.sin_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 8 * lane, sn);
-            }
             const int page = table[pos >> page_shift];
             if (page >= 0) {                              // the host reserves the page before the launch
                 const long base = (static_cast<long>(page) * kv_heads + kvh) * page_tokens * kD;
                 const int token = pos & page_mask;
+                constexpr int kHalfRuns = kD16;           // runs of 8 elements in half a head
                 if (wave == 0) {
+                    // lane L < kHalfRuns: elements 8L .. 8L+7 and their partners in the other half
+                    const bool mine = lane < kHalfRuns;
+                    float a[8], b[8];
                     float ss = 0.f;
-                    if (key_lane) {
+                    if (mine) {
+                        load_projection8(from, width, row, static_cast<long>(q_heads + kvh) * kD + 8 * lane, a);
+                        load_projection8(from, width, row, static_cast<long>(q_heads + kvh) * kD + kD / 2 + 8 * lane, b);
 #pragma unroll
                         for (int i = 0; i < 8; ++i) {
-                            ss = fmaf(new_a[i], new_a[i], ss);
-                            ss = fmaf(new_b[i], new_b[i], ss);
+                            ss = fmaf(a[i], a[i], ss);
+                            ss = fmaf(b[i], b[i], ss);
                         }
                     }
                     ss = wave_sum(ss);
-                    if (key_lane) {
+                    if (mine) {
                         if (from.k_gain.ptr) {
                             const float inv = 1.0f / sqrtf(ss / static_cast<float>(kD) + from.eps);
+                            float ga[8], gb[8];
+                            load_any8(from.k_gain, 8 * lane, ga);
+                            load_any8(from.k_gain, kD / 2 + 8 * lane, gb);
 #pragma unroll
                             for (int i = 0; i < 8; ++i) {
-                                new_a[i] = (new_a[i] * gain_a[i]) * inv;
-                                new_b[i] = (new_b[i] * gain_b[i]) * inv;
+                                a[i] = (a[i] * ga[i]) * inv;
+                                b[i] = (b[i] * gb[i]) * inv;
                             }
                         }
                         if (from.cos_table != nullptr) {
+                            const int tpos = pos < from.table_positions ? pos : from.table_positions - 1;
+                            float cs[8], sn[8];
+                            load_any8(AnyVec{from.cos_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 8 * lane, cs);
+                            load_any8(AnyVec{from.sin_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 8 * lane, sn);
 #pragma unroll
                             for (int i = 0; i < 8; ++i) {
-                                const float ru = new_a[i] * cs[i] - new_b[i] * sn[i];
-                                const float rv = new_a[i] * sn[i] + new_b[i] * cs[i];
-                                new_a[i] = ru;
-                                new_b[i] = rv;
+                                const float ru = a[i] * cs[i] - b[i] * sn[i];
+                                const float rv = a[i] * sn[i] + b[i] * cs[i];
+                                a[i] = ru;
+                                b[i] = rv;
                             }
                         }
                         uint4 lo, hi;
@@ -218,17 +204,22 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                         unsigned* wh = reinterpret_cast<unsigned*>(&hi);
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
-                            wl[i] = bf16_bits_from_float(new_a[2 * i]) | (static_cast<unsigned>(bf16_bits_from_float(new_a[2 * i + 1])) << 16);
-                            wh[i] = bf16_bits_from_float(new_b[2 * i]) | (static_cast<unsigned>(bf16_bits_from_float(new_b[2 * i + 1])) << 16);
+                            wl[i] = bf16_bits_from_float(a[2 * i]) | (static_cast<unsigned>(bf16_bits_from_float(a[2 * i + 1])) << 16);
+                            wh[i] = bf16_bits_from_float(b[2 * i]) | (static_cast<unsigned>(bf16_bits_from_float(b[2 * i + 1])) << 16);
                         }
                         *reinterpret_cast<uint4*>(from.k_out + base + key_offset(token, 8 * lane, page_tokens)) = lo;
                         *reinterpret_cast<uint4*>(from.k_out + base + key_offset(token, kD / 2 + 8 * lane, page_tokens)) = hi;
                     }
-                } else if (value_lane) {
+                } else if (wave == 1) {
                     // values are copied as they are, one element of one token at a time
+                    const long value_at = static_cast<long>(q_heads + kv_heads + kvh) * kD;
+                    for (int e = 8 * lane; e < kD; e += 8 * kWave) {
+                        float v[8];
+                        load_projection8(from, width, row, value_at + e, v);
 #pragma unroll
-                    for (int i = 0; i < 8; ++i)
-                        from.v_out[base + value_offset(token, 8 * lane + i, kD)] = from_float<bf16_t>(new_v[i]);
+                        for (int i = 0; i < 8; ++i)
+                            from.v_out[base + value_offset(token, e + i, kD)] = from_float<bf16_t>(v[i]);
+                    }
                 }
             }
             __threadfence_block();                         // the waves of this workgroup read what was written

@@ -142,6 +142,21 @@ gemm_fused_kernel(FusedArgs a) {
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b[1], acc, 0, 0, 0);
     };
 
+    // Wave 0, which writes the result, asks for what the epilogue adds to (the stream's values, the next
+    // norm's gains) before the walk over K: after it they would cost one more trip to memory.
+    float stream_before[4] = {0.f, 0.f, 0.f, 0.f}, gain_after[4] = {0.f, 0.f, 0.f, 0.f};
+    if ((kOut == kOutPrepare || kOut == kOutResidual) && wave == 0) {
+        const long col = n0 + 4 * g;
+        const float* out = static_cast<const float*>(a.y) + static_cast<long>(c) * n + col;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            if (c < m && col + r < n) {
+                stream_before[r] = out[r];
+                if (kOut == kOutPrepare) gain_after[r] = load_any(AnyVec{a.next_gain, a.next_gain_dtype}, col + r);
+            }
+        }
+    }
+
     // Each wave takes a contiguous share of K, so that it reads long runs of every weight row.
     const int whole = k / 64;                        // steps of 64 elements without a tail
     const int share = (whole + kWaves - 1) / kWaves;
@@ -237,15 +252,14 @@ gemm_fused_kernel(FusedArgs a) {
     if (kOut == kOutPrepare) {
         // every lane takes part in the exchange; rows and columns past the end count as zero
         float* out = static_cast<float*>(a.y) + static_cast<long>(row) * n + col;
-        const AnyVec gain{a.next_gain, a.next_gain_dtype};
         float squares = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             if (row < m && col + r < n) {
-                const float v = out[r] + sum[r];
+                const float v = stream_before[r] + sum[r];
                 out[r] = v;
                 squares = fmaf(v, v, squares);
-                a.operand_out[static_cast<long>(row) * n + col + r] = from_float<bf16_t>(v * load_any(gain, col + r));
+                a.operand_out[static_cast<long>(row) * n + col + r] = from_float<bf16_t>(v * gain_after[r]);
             }
         }
         squares += __shfl_xor(squares, 16, kWave);
@@ -258,7 +272,7 @@ gemm_fused_kernel(FusedArgs a) {
         float* out = static_cast<float*>(a.y) + static_cast<long>(row) * n + col;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-            if (col + r < n) out[r] += sum[r];
+            if (col + r < n) out[r] = stream_before[r] + sum[r];
     } else {
         TOut* out = static_cast<TOut*>(a.y) + static_cast<long>(row) * n + col;
 #pragma unroll
