@@ -234,8 +234,9 @@ class Engine:
         winner is kept only if the whole trial step is faster with it than without (a product timed by itself
         says too little: at 1,024 rows of the 8B shape the winners of the four products made the step 3 %
         slower; ``keep_only_faster_steps=False`` skips this).  Takes a few seconds (``thorough``: every algorithm of the library, not only the heuristic's
-        list); steps of other sizes are not affected.  Needs room for ``rows`` tokens in the cache for the
-        moment.  Returns a record for every product; ``kept`` says whether its winner is in use."""
+        list); steps of other sizes are not affected.  Needs room for ``rows`` tokens and a free request slot in
+        the cache for the moment (without them nothing is tuned).  Returns a record for every product; ``kept``
+        says whether its winner is in use."""
         if not ops.library_product_available():
             return []
         rows = min(int(rows), self.max_context)
@@ -253,8 +254,12 @@ class Engine:
                 self.release(request)
             return best
 
-        with ops.record_library_products() as recorded:
-            trial_step_ms(1)
+        from ..cache.manager import OutOfPages, OutOfSlots
+        try:
+            with ops.record_library_products() as recorded:
+                trial_step_ms(1)
+        except (OutOfPages, OutOfSlots):
+            return []                                   # no room for the trial step now: nothing is tuned
         step_ms = trial_step_ms()
         records = []
         for (m, n, k, out_code, accumulate), weights in recorded.problems.items():

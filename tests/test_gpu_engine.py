@@ -154,6 +154,10 @@ def test_tuned_library_products_agree_with_plain(cases):
         compare(steps[:2], outputs, {name: expected[name]}, tolerance("bfloat16"), "tuned products")
         again = {"again": expected[name][:rows - 3]}
         compare(steps[2:], {2: outputs[2]}, again, tolerance("bfloat16"), "beside tuned products")
+        # without room for the trial step nothing is tuned and nothing is left behind
+        tight = Engine(model, max_tokens=64, page_tokens=16, max_requests=1)
+        assert tight.tune_products(rows) == [] and not tight.cache.live_requests()
+        assert tight.cache.free_pages(0) == tight.cache.groups[0].num_pages
     finally:
         ops.forget_tuned_products()
 
