@@ -184,6 +184,10 @@ def cmd_generate(args) -> int:
     print(f"prefill: {stats.prefill_rate:.2f} tok/s", file=sys.stderr)
     print(f"tokens emitted: {stats.emitted_tokens}", file=sys.stderr)
     print(f"finish: {results[0].finish_reason}", file=sys.stderr)
+    if args.tune_products:
+        tuned = runtime.tuned_products
+        print(f"library products of a portion of {tuned[0]['rows'] if tuned else 0} tokens: {len(tuned)} timed, "
+              f"{sum(1 for r in tuned if r['kept'])} run with another algorithm than the heuristic's", file=sys.stderr)
     if runtime.last_decode_profile is not None:
         print("\n".join(runtime.last_decode_profile.lines()), file=sys.stderr)
     return 0
