@@ -281,13 +281,34 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         floatx16 sc, sc_odd;
 #pragma unroll
         for (int v = 0; v < 16; ++v) sc[v] = sc_odd[v] = 0.f;
+        // All of the pass's keys are asked for from shared memory at once and the values right after the first
+        // product's instructions, so that the way out of shared memory is waited for once a pass and the
+        // values come while the weights are made.  (Left to the compiler the reads come in pairs right before
+        // the instruction that needs them, a wait each, which a wave that has its SIMD to itself sits out.)
+        bf16x8 xk[kD16];
 #pragma unroll
         for (int s = 0; s < kD16; ++s) {
             // operand row j is key pass_key_or_row(j); this lane's elements 16 s + 8 h .. + 7 are run 2 s + h
-            const bf16x8 xk = pf_bits(from[(half * kRuns + 2 * s + h) * 32 + j]);
-            if (s % 2 == 0) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xk, qreg[s], sc, 0, 0, 0);
-            else sc_odd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xk, qreg[s], sc_odd, 0, 0, 0);
+            xk[s] = pf_bits(from[(half * kRuns + 2 * s + h) * 32 + j]);
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < kD16; ++s) {
+            if (s % 2 == 0) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xk[s], qreg[s], sc, 0, 0, 0);
+            else sc_odd = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xk[s], qreg[s], sc_odd, 0, 0, 0);
+        }
+        bf16x8 xv[2][kDT];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int dt = 0; dt < kDT; ++dt) {
+                const int d = 32 * dt + j;                     // operand row j of tile dt is element d of the values
+                // this lane's keys 16 ks + 8 h .. + 7 of the pass are one run of the values' layout
+                xv[ks][dt] = (kD % 32 == 0 || d < kD) ? pf_bits(from[kKeyRuns + (4 * half + 2 * ks + h) * kD + d])
+                                                      : pf_bits(uint4{0u, 0u, 0u, 0u});
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
         if (kD16 > 1) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) sc[v] += sc_odd[v];
@@ -335,13 +356,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-            for (int dt = 0; dt < kDT; ++dt) {
-                const int d = 32 * dt + j;                     // operand row j of tile dt is element d of the values
-                // this lane's keys 16 ks + 8 h .. + 7 of the pass are one run of the values' layout
-                const bf16x8 xv = (kD % 32 == 0 || d < kD) ? pf_bits(from[kKeyRuns + (4 * half + 2 * ks + h) * kD + d])
-                                                           : pf_bits(uint4{0u, 0u, 0u, 0u});
-                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xv, pt[ks], acc[dt], 0, 0, 0);
-            }
+            for (int dt = 0; dt < kDT; ++dt) acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xv[ks][dt], pt[ks], acc[dt], 0, 0, 0);
         }
     };
 
