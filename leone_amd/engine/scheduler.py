@@ -54,6 +54,10 @@ class SchedulerError(RuntimeError):
 
 @dataclass(frozen=True)
 class SchedulerPolicy:
+    """``max_step_tokens`` is the number of rows a full step has: decoded tokens first, prompt portions cut to
+    what is left of it.  The vendor library's products, which a step of more than 128 rows uses, are built for
+    round row counts (at the 8B layer sizes a step of 2,049 rows takes 25 % longer than one of 2,048, one of
+    544 rows 17 % longer than one of 512): keep it a multiple of 256."""
     max_live_requests: int = 64
     max_queued_requests: int = 1024
     max_step_tokens: int = 2048          # token budget of one step (decode rows + prompt portions)
