@@ -325,6 +325,12 @@ __device__ inline void load_run(const AnyVec& v, int at, float out[8]) {
     }
 }
 
+template <typename T>
+__device__ inline void value_write_block(T* turned, int row_block, int kvh, const T* __restrict__ qkv, T* __restrict__ v_pool,
+                                         const int* __restrict__ positions, const int* __restrict__ row_entry,
+                                         const int* __restrict__ block_table, int max_blocks, int rows, int q_heads,
+                                         int kv_heads, int head_dim, int page_tokens);
+
 template <typename TIn, typename T, int kD16>
 __global__ void __launch_bounds__(256)
 qk_norm_rope_write_runs_kernel(
@@ -332,9 +338,20 @@ qk_norm_rope_write_runs_kernel(
     AnyVec q_gain, AnyVec k_gain, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int table_positions, const int* __restrict__ positions,
     const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
-    int rows, int q_heads, int kv_heads, int page_tokens, int write_cache, int write_values) {
+    int rows, int q_heads, int kv_heads, int page_tokens, int write_cache, int write_values, int value_blocks) {
     constexpr int kD = 16 * kD16;
     constexpr int kHalf = kD / 2;
+    // The last `value_blocks` workgroups write the values of many rows in whole runs (value_write_block: eight
+    // rows and one kv head each), in the same launch as the heads.
+    if (static_cast<int>(gridDim.x - blockIdx.x) <= value_blocks) {
+        if constexpr (std::is_same<TIn, T>::value) {
+            extern __shared__ __align__(32) unsigned char turned_raw[];
+            const int at = value_blocks - static_cast<int>(gridDim.x - blockIdx.x);
+            value_write_block<T>(reinterpret_cast<T*>(turned_raw), at / kv_heads, at % kv_heads, qkv, v_pool, positions, row_entry,
+                                 block_table, max_blocks, rows, q_heads, kv_heads, kD, page_tokens);
+        }
+        return;
+    }
     constexpr int kShare = kD16 <= 1 ? 1 : kD16 <= 2 ? 2 : kD16 <= 4 ? 4 : 8;   // lanes a head takes (a power of two)
     const int heads_total = q_heads + (write_cache ? (write_values ? 2 : 1) * kv_heads : 0);
     const long item = (static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x) / kShare;
@@ -445,15 +462,12 @@ qk_norm_rope_write_runs_kernel(
 // up like that (the first and last rows of a portion, single decoded tokens) are written one element
 // at a time.  One thread an element of the head.
 template <typename T>
-__global__ void __launch_bounds__(512)
-value_write_kernel(const T* __restrict__ qkv, T* __restrict__ v_pool, const int* __restrict__ positions,
-                   const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
-                   int rows, int q_heads, int kv_heads, int head_dim, int page_tokens) {
-    extern __shared__ __align__(32) unsigned char turned_raw[];
-    T* turned = reinterpret_cast<T*>(turned_raw);                       // [8][head_dim]
-    const int row0 = blockIdx.x * 8;
-    const int kvh = blockIdx.y;
-    const int d = threadIdx.x;                                          // blockDim.x == head_dim
+__device__ inline void value_write_block(T* turned, int row_block, int kvh, const T* __restrict__ qkv, T* __restrict__ v_pool,
+                                         const int* __restrict__ positions, const int* __restrict__ row_entry,
+                                         const int* __restrict__ block_table, int max_blocks, int rows, int q_heads,
+                                         int kv_heads, int head_dim, int page_tokens) {
+    const int row0 = row_block * 8;
+    const int d = threadIdx.x;                                          // blockDim.x >= head_dim; threads beyond it only copy
     const int qkv_width = (q_heads + 2 * kv_heads) * head_dim;
     const long head_at = static_cast<long>(q_heads + kv_heads + kvh) * head_dim;
     const int n = rows - row0 < 8 ? rows - row0 : 8;
@@ -467,6 +481,7 @@ value_write_kernel(const T* __restrict__ qkv, T* __restrict__ v_pool, const int*
             *reinterpret_cast<const HeadRun<T>*>(qkv + static_cast<long>(row0 + r) * qkv_width + head_at + 8 * chunk);
     }
     __syncthreads();
+    if (d >= head_dim) return;
     if (lined_up) {
         const int page = block_table[static_cast<long>(e0) * max_blocks + p0 / page_tokens];
         if (page < 0) return;  // host reserves pages before the launch
@@ -486,6 +501,16 @@ value_write_kernel(const T* __restrict__ qkv, T* __restrict__ v_pool, const int*
     }
 }
 
+template <typename T>
+__global__ void __launch_bounds__(512)
+value_write_kernel(const T* __restrict__ qkv, T* __restrict__ v_pool, const int* __restrict__ positions,
+                   const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
+                   int rows, int q_heads, int kv_heads, int head_dim, int page_tokens) {
+    extern __shared__ __align__(32) unsigned char turned_raw[];
+    value_write_block<T>(reinterpret_cast<T*>(turned_raw), blockIdx.x, blockIdx.y, qkv, v_pool, positions, row_entry, block_table,
+                         max_blocks, rows, q_heads, kv_heads, head_dim, page_tokens);
+}
+
 template <typename TIn, typename T, int kD16>
 static void launch_runs(const void* qkv, int planes, long plane, void* q_out, void* k_pool, void* v_pool, AnyVec qg, AnyVec kg, float eps,
                         const float* cos_table, const float* sin_table, int table_positions, const int* positions,
@@ -497,16 +522,22 @@ static void launch_runs(const void* qkv, int planes, long plane, void* q_out, vo
                               std::is_same<TIn, T>::value && planes == 1;
     const long items = static_cast<long>(rows) * (q_heads + (write_cache ? (values_apart ? 1 : 2) * kv_heads : 0));
     const int blocks = ceil_div(items * kShare, 256);
-    qk_norm_rope_write_runs_kernel<TIn, T, kD16><<<blocks, 256, 0, stream>>>(
-        static_cast<const TIn*>(qkv), planes, plane, static_cast<T*>(q_out), static_cast<T*>(k_pool), static_cast<T*>(v_pool), qg, kg, eps,
-        cos_table, sin_table, table_positions, positions, row_entry, block_table, max_blocks, rows, q_heads, kv_heads,
-        page_tokens, write_cache, values_apart ? 0 : 1);
-    if (values_apart) {
-        constexpr int kD = 16 * kD16;
+    constexpr int kD = 16 * kD16;
+    const long value_blocks = values_apart ? static_cast<long>(ceil_div(rows, 8)) * kv_heads : 0;
+    if (blocks + value_blocks > 0x7fffffffL) {          // too many for one launch: the values by themselves
+        qk_norm_rope_write_runs_kernel<TIn, T, kD16><<<blocks, 256, 0, stream>>>(
+            static_cast<const TIn*>(qkv), planes, plane, static_cast<T*>(q_out), static_cast<T*>(k_pool), static_cast<T*>(v_pool), qg, kg, eps,
+            cos_table, sin_table, table_positions, positions, row_entry, block_table, max_blocks, rows, q_heads, kv_heads,
+            page_tokens, write_cache, 0, 0);
         value_write_kernel<T><<<dim3(ceil_div(rows, 8), kv_heads), kD, 8 * kD * sizeof(T), stream>>>(
             reinterpret_cast<const T*>(qkv), static_cast<T*>(v_pool), positions, row_entry, block_table, max_blocks, rows,
             q_heads, kv_heads, kD, page_tokens);
+        return;
     }
+    qk_norm_rope_write_runs_kernel<TIn, T, kD16><<<static_cast<int>(blocks + value_blocks), 256, values_apart ? 8 * kD * sizeof(T) : 0, stream>>>(
+        static_cast<const TIn*>(qkv), planes, plane, static_cast<T*>(q_out), static_cast<T*>(k_pool), static_cast<T*>(v_pool), qg, kg, eps,
+        cos_table, sin_table, table_positions, positions, row_entry, block_table, max_blocks, rows, q_heads, kv_heads,
+        page_tokens, write_cache, values_apart ? 0 : 1, static_cast<int>(value_blocks));
 }
 
 static int check_dtype(int dtype, const char* what) {
