@@ -334,7 +334,8 @@ class Engine:
             else:
                 tokens, context, rows = self._build_context(entries)
                 caches = self.pools.views(context.block_tables)
-                logits = self.model.forward(tokens, context, caches)
+                with ops.one_stream():
+                    logits = self.model.forward(tokens, context, caches)
         except Exception:
             for e in entries:
                 if self.cache.has(e.request):
@@ -356,9 +357,10 @@ class Engine:
             # First step of this size: run it for real on the static buffers, then record the same
             # calls for later steps.  Recording executes nothing, so the cache is written once.
             caches = self.pools.views(state.context.block_tables)
-            logits = self.model.forward(state.tokens, state.context, caches)
+            with ops.one_stream():
+                logits = self.model.forward(state.tokens, state.context, caches)
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            with torch.cuda.graph(graph), ops.one_stream():
                 state.logits = self.model.forward(state.tokens, state.context, caches)
             state.graph = graph
         else:

@@ -8,6 +8,7 @@ from __future__ import annotations
 
 from typing import Optional
 
+import functools
 import weakref
 
 import numpy as np
@@ -45,12 +46,35 @@ def _dev(t: Optional[torch.Tensor], what: str, dtype=None, shape=None) -> int:
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
+_step_stream: Optional[int] = None     # inside ``one_stream``: the handle that was current when it began
+
+
 def _stream() -> int:
     """The current stream's handle.  Asked for before every launch, so the short way is taken where this
-    torch has it (a tenth of the time of building a Stream object)."""
+    torch has it (a tenth of the time of building a Stream object); within ``one_stream`` it was asked for once."""
+    if _step_stream is not None:
+        return _step_stream
     if _raw_stream is not None:
         return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
+
+
+class one_stream:
+    """Within this context every launch goes to the stream that is current at its beginning: the few hundred
+    launches of a step need not ask for it one by one (0.4 ms of the 4 ms the host takes to issue a step of the
+    8B shape).  Whoever changes the current stream inside (a graph capture does) opens a context of its own."""
+
+    def __enter__(self):
+        global _step_stream
+        self._before = _step_stream
+        _step_stream = None
+        _step_stream = _stream()
+        return self
+
+    def __exit__(self, *exc):
+        global _step_stream
+        _step_stream = self._before
+        return False
 
 
 def cache_dims(k_pool: torch.Tensor, v_pool: torch.Tensor):
@@ -579,12 +603,17 @@ def rows_plan(m: int, n: int, k: int, may_split: bool, units: int = 256) -> tupl
     or 1,536 elements cuts long K's into too many ranges: 8B 8.05 : 7.91 ms a step at 64 rows; a fixed choice
     for matrices of many rows gave the 32B gate/up product 4 waves and four rounds where 8 waves need two:
     21.7 : 20.3 ms at 64 rows)."""
-    chunk = library().leone_gemm_rows_chunk(m)
+    return _rows_plan(m, n, k, bool(may_split), units, library().leone_gemm_rows_chunk(m), tuple(ROWS_WAVES))
+
+
+@functools.lru_cache(maxsize=4096)
+def _rows_plan(m: int, n: int, k: int, may_split: bool, units: int, chunk: int, waves_offered: tuple) -> tuple[int, int]:
+    # the same few problems come back a few hundred times a step: 0.8 ms of a step's 4 on the host without this
     chunks = -(-k // chunk)
     tiles = -(-n // 16)
     x_tiles = -(-m // 16)
     best = None
-    for waves in ROWS_WAVES:
+    for waves in waves_offered:
         groups = -(-tiles // waves)
         for splits in range(1, (min(chunks, 16) if may_split else 1) + 1):
             per = -(-chunks // splits)
