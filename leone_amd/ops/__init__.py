@@ -62,7 +62,9 @@ def _stream() -> int:
 class one_stream:
     """Within this context every launch goes to the stream that is current at its beginning: the few hundred
     launches of a step need not ask for it one by one (0.4 ms of the 4 ms the host takes to issue a step of the
-    8B shape).  Whoever changes the current stream inside (a graph capture does) opens a context of its own."""
+    8B shape).  Whoever changes the current stream inside (a graph capture does) opens a context of its own.  The
+    handle is kept for the process, not for a thread: steps that run side by side in several threads on different
+    streams must not use it."""
 
     def __enter__(self):
         global _step_stream
