@@ -311,8 +311,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     points_batches = [] if args.no_points else [1, 64]
     largest = max([args.batch] + points_batches)
     pages = largest * (args.context // page_tokens + 1) + PREFILL_TOKENS // page_tokens
+    # the cache takes requests of the context asked for and, for the prompt's figure, one of PREFILL_TOKENS
     engine = Engine(model, num_pages=pages, page_tokens=page_tokens, max_requests=largest + 1,
-                    max_context=args.context, streamed_weights=False if args.no_streamed_weights else None)
+                    max_context=args.context if args.no_prefill else max(args.context, PREFILL_TOKENS),
+                    streamed_weights=False if args.no_streamed_weights else None)
 
     peaks = None if args.no_peaks else measure_peaks()
     profile_steps = 0 if args.no_kernels else 4

@@ -1,0 +1,34 @@
+"""The measurement program's record: what a reader of its one line relies on."""
+import json
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_the_record_of_a_short_run(capsys):
+    """Two layers of the headline shape, a few steps: one line of JSON with the decode figure, the prompt's, the
+    roofline's and the points', and a flat description of every size."""
+    from leone_amd import benchmark
+    assert benchmark.main(["--layers", "2", "--steps", "4", "--warmup", "1", "--batch", "8", "--context", "1024",
+                           "--no-peaks"]) == 0
+    lines = [line for line in capsys.readouterr().out.splitlines() if line.strip()]
+    assert len(lines) == 1
+    record = json.loads(lines[0])
+    for key, kind in (("metric", str), ("value", float), ("unit", str), ("n_gpus", int), ("steps", int), ("warmup", int),
+                      ("ms_per_step", float), ("higher_is_better", bool), ("scaling", str), ("dtype", str), ("data", str)):
+        assert isinstance(record[key], kind), key
+    assert record["n_gpus"] == 1 and record["steps"] == 4 and record["warmup"] == 1 and record["value"] > 0
+    assert abs(record["value"] - 8 / record["ms_per_step"] * 1e3) / record["value"] < 1e-3      # decoded tokens a second
+    config = record["config"]
+    assert len(config) <= 20 and all(isinstance(v, (str, int, float, bool)) for v in config.values()), config
+    assert config["layers"] == 2 and config["layers_of_configuration"] == 36 and config["global_batch"] == 8
+    assert config["library_products"] in ("measured choice", "heuristic")
+    prefill = record["prefill"]
+    assert prefill["tokens"] == 2048 and prefill["ms"] > 0 and 0 < prefill["frac"] < 1
+    assert abs(prefill["value"] - 2048 / prefill["ms"] * 1e3) / prefill["value"] < 1e-3
+    roofline = record["roofline"]
+    assert roofline["bound"] == "hbm" and roofline["unit"] == "GB/s" and roofline["peak"] == 8000.0
+    assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-3
+    assert abs(roofline["achieved"] - record["bytes"]["a_step"] / record["ms_per_step"] / 1e6) / roofline["achieved"] < 1e-2
+    assert {"decode_b1", "decode_b64"} <= set(record["points"]) and all(v > 0 for v in record["points"].values())
