@@ -32,3 +32,18 @@ def test_the_record_of_a_short_run(capsys):
     assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-3
     assert abs(roofline["achieved"] - record["bytes"]["a_step"] / record["ms_per_step"] / 1e6) / roofline["achieved"] < 1e-2
     assert {"decode_b1", "decode_b64"} <= set(record["points"]) and all(v > 0 for v in record["points"].values())
+
+
+@pytest.mark.parametrize("name", ["mixed14b", "pressure32b"])
+def test_a_serving_scenario_with_one_layer(name):
+    """The serving scenarios at their real widths and request mixes, one layer deep: every request finishes with
+    all its tokens, no page is lost (the scenario checks both itself), steps stay within the budget, and the
+    scenario with too few pages preempts."""
+    from leone_amd import benchmark
+    record = benchmark.run_scenario(name, layers=1)
+    scenario = benchmark.SCENARIOS[name]
+    assert record["value"] > 0 and record["config"]["layers"] == 1
+    assert record["max_step_rows"] <= scenario["chunk"] and record["max_live"] <= scenario["live"]
+    assert record["config"]["requests"] == scenario["requests"]
+    assert (record["preemptions"] > 0) == (scenario["pool_fraction"] < 1.0)
+    assert len(record["config"]) <= 20
