@@ -208,6 +208,12 @@ def cmd_doctor(args) -> int:
         from .csrc import build
         path = build.library_path() or build.build(verbose=True)
         print(f"kernel library: {path}")
+        if torch.cuda.is_available():
+            from .ops.library import library
+            found = library().leone_library_product_available()
+            print("vendor library for the products of prompt portions: "
+                  + ("hipBLASLt not found (torch's own calls of it remain; --tune-products has nothing to choose from)" if not found
+                     else "hipBLASLt, algorithms by its heuristic's list" + (" or all of them" if found == 2 else "")))
     except Exception as error:  # noqa: BLE001 - doctor reports, it does not raise
         print(f"kernel library: FAILED: {error}")
         ok = False

@@ -134,7 +134,7 @@ int leone_gemm_rows_bf16(const void* x, const void* w, int w_tiled, void* y, int
 // accumulate); it reports the time of the library's own first choice and of the winner in microseconds.
 // leone_library_product runs a problem that was tuned and refuses any other: the caller keeps its ordinary
 // call of the library for those.  _available: 1 if hipBLASLt could be found in the process or on the loader's
-// path (it is looked up at run time and only then); _tuned: 1 if the problem was tuned on the current device.
+// path (it is looked up at run time and only then), 2 if its list of all algorithms is there as well, else 0; _tuned: 1 if the problem was tuned on the current device.
 int leone_library_product_available();
 int leone_library_product_tuned(int m, int n, int k, int out_dtype, int accumulate);
 int leone_library_product_forget(int m, int n, int k, int out_dtype, int accumulate);

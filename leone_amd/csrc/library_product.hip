@@ -170,7 +170,7 @@ bool checked_shape(const char* who, int m, int n, int k, int out_dtype) {
 
 using namespace leone;
 
-extern "C" int leone_library_product_available() { return lt().ok ? 1 : 0; }
+extern "C" int leone_library_product_available() { return !lt().ok ? 0 : lt().all_algorithms ? 2 : 1; }
 
 extern "C" int leone_library_product_tuned(int m, int n, int k, int out_dtype, int accumulate) {
     int device = 0;
