@@ -6,6 +6,15 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def library_products_as_found():
+    """The measurement programs choose the vendor library's algorithms by measurement for the process: what they
+    chose goes back to the library's heuristic afterwards."""
+    yield
+    from leone_amd import ops
+    ops.forget_tuned_products()
+
+
 def test_the_record_of_a_short_run(capsys):
     """Two layers of the headline shape, a few steps: one line of JSON with the decode figure, the prompt's, the
     roofline's and the points', and a flat description of every size."""

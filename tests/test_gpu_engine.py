@@ -149,7 +149,8 @@ def test_tuned_library_products_agree_with_plain(cases):
                      {"step": 1, "entries": [{"id": name, "tokens": tokens[rows:], "want": list(range(7))}], "end": [name]},
                      {"step": 2, "entries": [{"id": "again", "tokens": tokens[:rows - 3], "want": list(range(rows - 3))}], "end": ["again"]}]
             outputs = run_steps(engine, steps)
-        assert ops._tuned_products and ops._tuned_products <= {(0,) + problem for problem in seen.problems}   # all were used
+        mine = {r["problem"] for r in records}
+        assert mine <= ops._tuned_products and mine <= {(0,) + problem for problem in seen.problems}    # all are in use
         assert any(problem[0] == rows for problem in seen.problems) and any(problem[0] == rows - 3 for problem in seen.problems)
         compare(steps[:2], outputs, {name: expected[name]}, tolerance("bfloat16"), "tuned products")
         again = {"again": expected[name][:rows - 3]}
