@@ -352,7 +352,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     if not args.no_prefill:
         # the vendor library's products of the prompt run with the fastest of the library's algorithms, found by
         # timing them now on this model's matrices (Engine.tune_products)
-        tuned = [] if args.no_tuned_products or args.dtype != "bfloat16" else engine.tune_products(PREFILL_TOKENS, thorough=True)
+        tuned = [] if args.no_tuned_products or args.dtype != "bfloat16" else engine.tune_products(PREFILL_TOKENS)
         record["config"]["library_products"] = "measured choice" if any(r["kept"] for r in tuned) else "heuristic"
         seconds = time_prefill(engine, PREFILL_TOKENS)
         flops = prefill_flops(config, PREFILL_TOKENS)
