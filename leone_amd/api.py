@@ -46,6 +46,13 @@ def sampling_params(temperature: Optional[float] = None, seed: int = 0, top_k: O
     return params
 
 
+def cache_bytes_per_token(model) -> int:
+    """Bytes one cached token takes over all cache slots of the model: every paged need says its own
+    (``bytes_per_token(element size)``), whatever kind of cache it is."""
+    size = torch.empty((), dtype=model.dtype).element_size()
+    return sum(need.bytes_per_token(size) for need in model.cache_needs().values() if getattr(need, "paged", False))
+
+
 def default_num_pages(model, page_tokens: int, max_requests: int, max_context: int, bytes_per_token: int) -> int:
     wanted = max_requests * ((max_context + page_tokens - 1) // page_tokens)
     free, _ = torch.cuda.mem_get_info(model.device)
@@ -68,10 +75,7 @@ class Runtime:
         self.config = getattr(model, "config", None)
         context = min(max_context or model.spec.max_positions, model.spec.max_positions)
         if num_pages is None and max_tokens is None:
-            size = torch.empty((), dtype=model.dtype).element_size()
-            per_token = sum(2 * need.kv_heads * need.head_dim * size for need in model.cache_needs().values()
-                            if hasattr(need, "kv_heads"))
-            num_pages = default_num_pages(model, page_tokens, max_requests, context, per_token)
+            num_pages = default_num_pages(model, page_tokens, max_requests, context, cache_bytes_per_token(model))
         self.engine = Engine(model, num_pages=num_pages, max_tokens=max_tokens, page_tokens=page_tokens,
                              max_requests=max_requests, max_context=context, graphs=graphs,
                              poison_freed=poison_freed, streamed_weights=streamed_weights)

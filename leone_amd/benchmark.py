@@ -40,9 +40,8 @@ def prefill_flops(c, tokens: int, start: int = 0) -> float:
 
 def cache_bytes_per_token(model) -> int:
     """Bytes of keys and values one cached token takes over all cache slots of the model."""
-    size = 2 if str(model.dtype).endswith("bfloat16") else 4
-    return sum(2 * need.kv_heads * need.head_dim * size for need in model.cache_needs().values()
-               if hasattr(need, "kv_heads"))
+    from .api import cache_bytes_per_token as per_token
+    return per_token(model)
 
 
 def decode_bytes(model, batch: int, context: float) -> float:
@@ -205,7 +204,19 @@ SCENARIOS = {
 }
 
 
-def run_scenario(name: str, dtype: str = "bfloat16", layers: Optional[int] = None) -> dict:
+def trial_portion(engine, rows: int) -> None:
+    """One prompt portion of ``rows`` tokens on a request of its own, released again: a process's first step of a
+    size costs a quarter of a second more than any later one (the libraries load their kernels), which is not
+    what a serving figure should hold."""
+    import torch
+    from .engine.engine import StepEntry
+    rows = min(rows, engine.max_context)
+    engine.step([StepEntry(("trial portion",), [(i * 7919) % engine.vocab_size for i in range(rows)], [rows - 1])])
+    engine.release(("trial portion",))
+    torch.cuda.synchronize()
+
+
+def run_scenario(name: str, dtype: str = "bfloat16", layers: Optional[int] = None, tuned_products: bool = False) -> dict:
     import torch
     from .architectures import config_from_dict
     from .engine.engine import Engine
@@ -235,7 +246,10 @@ def run_scenario(name: str, dtype: str = "bfloat16", layers: Optional[int] = Non
     # one of 512 rows 10.0).
     policy = SchedulerPolicy(max_live_requests=sc["live"], prefill_chunk_tokens=sc["chunk"],
                              max_step_tokens=sc["chunk"])
-    tuned = engine.tune_products(sc["chunk"]) if dtype == "bfloat16" else []     # before the clock starts
+    # before the clock starts: one trial portion, or (on request) the measured choice of the library's algorithms
+    tuned = engine.tune_products(sc["chunk"]) if dtype == "bfloat16" and tuned_products else []
+    if not tuned:
+        trial_portion(engine, sc["chunk"])
     generator = Generator(engine, policy)
     sampling = SamplingParams(temperature=sc["temperature"], seed=11)
     for i, prompt in enumerate(prompts):
@@ -278,8 +292,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     parser.add_argument("--no-peaks", action="store_true", help="skip the measurement of this GPU's own peaks")
     parser.add_argument("--no-streamed-weights", action="store_true",
                         help="keep no second copy of the matrices in the decode kernels' order")
-    parser.add_argument("--no-tuned-products", action="store_true",
-                        help="leave the choice of the vendor library's algorithms for the prompt's products to its heuristic")
+    parser.add_argument("--tuned-products", action="store_true",
+                        help="let the prompt's products run with the vendor library's algorithms that are fastest when "
+                             "timed now (Runtime(tune_products=True)); by default the library's heuristic chooses, as in "
+                             "Runtime and `leone generate`")
     parser.add_argument("--peaks", action="store_true", help="only measure this GPU's own peaks and print them")
     parser.add_argument("--scenario", choices=sorted(SCENARIOS), help="run a serving scenario instead of the headline figure")
     args = parser.parse_args(argv)
@@ -288,7 +304,7 @@ def main(argv: Optional[List[str]] = None) -> int:
         return 2
 
     if args.scenario:
-        print(json.dumps(run_scenario(args.scenario, args.dtype, args.layers)), flush=True)
+        print(json.dumps(run_scenario(args.scenario, args.dtype, args.layers, args.tuned_products)), flush=True)
         return 0
     if args.peaks:
         print(json.dumps({"metric": "measured peaks", **measure_peaks()}), flush=True)
@@ -350,9 +366,9 @@ def main(argv: Optional[List[str]] = None) -> int:
     if profile_steps:
         record["kernels"] = kernel_table(timed[2], model, args.batch, start + args.warmup + args.steps + 2)
     if not args.no_prefill:
-        # the vendor library's products of the prompt run with the fastest of the library's algorithms, found by
-        # timing them now on this model's matrices (Engine.tune_products)
-        tuned = [] if args.no_tuned_products or args.dtype != "bfloat16" else engine.tune_products(PREFILL_TOKENS)
+        # on request the vendor library's products of the prompt run with the fastest of the library's algorithms,
+        # found by timing them now on this model's matrices (Engine.tune_products)
+        tuned = engine.tune_products(PREFILL_TOKENS) if args.tuned_products and args.dtype == "bfloat16" else []
         record["config"]["library_products"] = "measured choice" if any(r["kept"] for r in tuned) else "heuristic"
         seconds = time_prefill(engine, PREFILL_TOKENS)
         flops = prefill_flops(config, PREFILL_TOKENS)

@@ -252,9 +252,21 @@ def cmd_doctor(args) -> int:
         print(f"weights a decode step reads: {sum(accounting['decode'].values()) / 2**20:.1f} MiB of "
               f"{accounting['tensor_bytes'] / 2**20:.1f} MiB")
         size = 2 if args.dtype == "bfloat16" else 4
-        per_token = sum(2 * need.kv_heads * need.head_dim * size for need in model.cache_needs().values()
-                        if hasattr(need, "kv_heads"))
+        per_token = sum(need.bytes_per_token(size) for need in model.cache_needs().values() if getattr(need, "paged", False))
         print(f"cache bytes per token ({args.dtype}): {per_token}")
+        # which attention kernels the layers' shapes get (pages of 64 tokens, the default)
+        kinds = {}
+        for layer in model.layers:
+            mixer = getattr(layer, "mixer", None)
+            if hasattr(mixer, "attention_kernels"):
+                chosen = mixer.attention_kernels(torch.bfloat16 if args.dtype == "bfloat16" else torch.float32, 64)
+                key = (mixer.q_heads, mixer.kv_heads, mixer.head_dim, chosen["decode"], chosen["prompt"])
+                kinds[key] = kinds.get(key, 0) + 1
+        names = {"projected": "split-KV matrix-core kernel that makes the heads itself", "split_kv": "split-KV matrix-core kernel",
+                 "flash": "matrix-core prompt kernel", "rows": "row kernel in float arithmetic"}
+        for (q_heads, kv_heads, head_dim, decode, prompt), count in kinds.items():
+            print(f"attention, {count} layer(s) of {q_heads}/{kv_heads} heads of {head_dim}: decoded tokens on the "
+                  f"{names[decode]}, prompt portions on the {names[prompt]}")
         # the second copy of the matrices that decode steps read (kept for bfloat16 when there is ample room)
         second = sum(v for family, v in accounting["decode"].items() if family not in ("embed", "norm"))
         second = second if args.dtype == "bfloat16" and model.spec.hidden_size % 64 == 0 else 0

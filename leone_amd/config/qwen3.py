@@ -62,6 +62,11 @@ class Qwen3Config:
             head_dim = hidden // heads
         if head_dim % 2 != 0:
             raise ConfigError("head_dim", f"rotary pairs need an even head_dim, found {head_dim}")
+        if head_dim % 8 != 0:
+            # the paged cache packs keys and values in runs of 8 elements; refused here, when the file is read
+            # (the reference validates shapes at load, crates/leone/src/backend.rs:1230), not when pools are made
+            raise ConfigError("head_dim", f"the key/value cache holds heads in runs of 8 elements: head_dim must "
+                                          f"be a multiple of 8, found {head_dim}")
         scaling = read.optional("rope_scaling")
         if scaling is not None and not (isinstance(scaling, dict) and
                                         scaling.get("rope_type", scaling.get("type")) == "default"):

@@ -623,7 +623,7 @@ extern "C" int leone_attention_decode(const void* q, void* out, const void* k_po
 extern "C" int leone_attention_decode_projected(const void* qkv, int qkv_dtype, int qkv_planes, long qkv_plane,
                                                 const void* q_gain, const void* k_gain, int gain_dtype, float eps,
                                                 const float* cos_table, const float* sin_table, int table_positions,
-                                                void* out, void* k_pool, void* v_pool, int write_cache,
+                                                int rotary_dim, int pairing, void* out, void* k_pool, void* v_pool, int write_cache,
                                                 const int* positions, const int* row_entry, const int* block_table,
                                                 int max_blocks, float* part_acc, float* part_ml, int rows, int q_heads,
                                                 int kv_heads, int head_dim, int page_tokens, float scale, int window,
@@ -636,6 +636,9 @@ extern "C" int leone_attention_decode_projected(const void* qkv, int qkv_dtype, 
                   "attention_decode: the head norms need gains of a known type and a positive eps");
     LEONE_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "attention_decode: cos and sin tables come together");
     LEONE_REQUIRE(!cos_table || table_positions > 0, "attention_decode: empty rotary table");
+    LEONE_REQUIRE(!cos_table || (rotary_dim == head_dim && pairing == 0),
+                  "attention_decode: the kernel that takes the projection rotates whole heads in half-split pairs, not "
+                  "%d of %d elements with pairing %d", rotary_dim, head_dim, pairing);
     LEONE_REQUIRE(reinterpret_cast<uintptr_t>(qkv) % 32 == 0 &&
                       (!cos_table || (reinterpret_cast<uintptr_t>(cos_table) % 32 == 0 && reinterpret_cast<uintptr_t>(sin_table) % 32 == 0)) &&
                       (!q_gain || (reinterpret_cast<uintptr_t>(q_gain) % 32 == 0 && reinterpret_cast<uintptr_t>(k_gain) % 32 == 0)),

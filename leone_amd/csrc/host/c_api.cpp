@@ -157,12 +157,14 @@ int leone_cache_log_freed(void* cache, int on) {
 }
 int leone_cache_drain_freed(void* cache, int group, int* out, int capacity) {
     return guarded([&]() -> long {
-        // nothing is taken off the log unless it fits: a caller with too little room asks again
+        // nothing is taken off the log unless it fits: the size is asked for first, so a caller with too
+        // little room loses no page and asks again
         CacheManager& manager = cache_of(cache);
-        std::vector<int> pages = manager.drain_freed(group);
-        if (static_cast<long>(pages.size()) > capacity || (!out && !pages.empty()))
+        const long waiting = manager.freed_count(group);
+        if (waiting > capacity || (!out && waiting > 0))
             throw CacheError("the freed pages of group " + std::to_string(group) + " need room for " +
-                             std::to_string(pages.size()) + " entries");
+                             std::to_string(waiting) + " entries");
+        std::vector<int> pages = manager.drain_freed(group);
         for (size_t i = 0; i < pages.size(); ++i) out[i] = pages[i];
         return static_cast<long>(pages.size());
     });

@@ -115,6 +115,14 @@ void CacheManager::log_freed(bool on) {
     freed_log_.assign(groups_.size(), {});
 }
 
+long CacheManager::freed_count(int g) const {
+    if (g < 0 || g >= group_count()) throw CacheError("no cache group " + std::to_string(g));
+    if (!log_freed_) return 0;
+    std::vector<int> pages = freed_log_[g];                               // a page freed twice since is one page
+    std::sort(pages.begin(), pages.end());
+    return static_cast<long>(std::unique(pages.begin(), pages.end()) - pages.begin());
+}
+
 std::vector<int> CacheManager::drain_freed(int g) {
     if (g < 0 || g >= group_count()) throw CacheError("no cache group " + std::to_string(g));
     std::vector<int> out;

@@ -80,6 +80,8 @@ public:
     // For a caller that wants to overwrite what freed pages hold before anyone gets them again.
     void log_freed(bool on);
     std::vector<int> drain_freed(int g);
+    long freed_count(int g) const;      // how many pages the next drain_freed will hand out
+
     // New pages each group must map to append `tokens` to `request` now.
     std::vector<int> pages_needed(RequestKey request, int tokens) const;
 

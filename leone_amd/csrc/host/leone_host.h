@@ -107,9 +107,9 @@ int leone_ref_add_rmsnorm(float* x, const float* delta, int planes, long plane, 
 int leone_ref_rope_table(float* cos_out, float* sin_out, double theta, int rotary_dim, int positions);
 int leone_ref_qk_norm_rope_write(const float* qkv, int planes, long plane, float* q_out, float* k_pool, float* v_pool,
                                  const float* q_gain, const float* k_gain, float eps, const float* cos_table,
-                                 const float* sin_table, int table_positions, const int* positions,
-                                 const int* row_entry, const int* block_table, int max_blocks, int rows, int q_heads,
-                                 int kv_heads, int head_dim, int page_tokens, int write_cache);
+                                 const float* sin_table, int table_positions, int rotary_dim, int pairing,
+                                 const int* positions, const int* row_entry, const int* block_table, int max_blocks,
+                                 int rows, int q_heads, int kv_heads, int head_dim, int page_tokens, int write_cache);
 int leone_ref_attention(const float* q, float* out, const float* k_pool, const float* v_pool, const int* positions,
                         const int* row_entry, const int* block_table, int max_blocks, int rows, int q_heads,
                         int kv_heads, int head_dim, int page_tokens, float scale, int window);

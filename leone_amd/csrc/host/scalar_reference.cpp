@@ -73,11 +73,14 @@ int leone_ref_rope_table(float* cos_out, float* sin_out, double theta, int rotar
     return 0;
 }
 
-// Per-head RMSNorm of q and k (gains may be null), half-split rotation (tables may be null), q to q_out, k and
-// v into the paged cache (crates/leone/src/backend.rs:2182-2208).  The input may come in planes to be added up.
+// Per-head RMSNorm of q and k (gains may be null), rotation of the head's first rotary_dim elements in half-split
+// (pairing 0) or adjacent (pairing 1) pairs (tables [positions, rotary_dim / 2], may be null), q to q_out, k and
+// v into the paged cache (crates/leone/src/backend.rs:2182-2208, crates/leone/src/cpu.rs:1765-1774).  The input
+// may come in planes to be added up.
 int leone_ref_qk_norm_rope_write(const float* qkv, int planes, long plane, float* q_out, float* k_pool, float* v_pool,
                                  const float* q_gain, const float* k_gain, float eps, const float* cos_table,
-                                 const float* sin_table, int table_positions, const int* positions,
+                                 const float* sin_table, int table_positions, int rotary_dim, int pairing,
+                                 const int* positions,
                                  const int* row_entry, const int* block_table, int max_blocks, int rows, int q_heads,
                                  int kv_heads, int head_dim, int page_tokens, int write_cache) {
     if (!qkv || !q_out || !positions || rows <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim % 2)
@@ -86,7 +89,9 @@ int leone_ref_qk_norm_rope_write(const float* qkv, int planes, long plane, float
                         head_dim % 8 || page_tokens % 8))
         return LEONE_HOST_INVALID;
     if ((q_gain == nullptr) != (k_gain == nullptr) || (cos_table == nullptr) != (sin_table == nullptr)) return LEONE_HOST_INVALID;
-    const int half = head_dim / 2;
+    if (cos_table && (rotary_dim <= 0 || rotary_dim % 2 || rotary_dim > head_dim || pairing < 0 || pairing > 1))
+        return LEONE_HOST_INVALID;
+    const int half = cos_table ? rotary_dim / 2 : 0;
     const long width = static_cast<long>(q_heads + 2 * kv_heads) * head_dim;
     std::vector<float> head(head_dim);
     for (int r = 0; r < rows; ++r) {
@@ -125,9 +130,10 @@ int leone_ref_qk_norm_rope_write(const float* qkv, int planes, long plane, float
                 const int tpos = pos < table_positions ? pos : table_positions - 1;
                 for (int i = 0; i < half; ++i) {
                     const float c = cos_table[static_cast<long>(tpos) * half + i], s = sin_table[static_cast<long>(tpos) * half + i];
-                    const float u = head[i], v = head[i + half];
-                    head[i] = u * c - v * s;
-                    head[i + half] = u * s + v * c;
+                    const int first = pairing == 0 ? i : 2 * i, second = pairing == 0 ? i + half : 2 * i + 1;
+                    const float u = head[first], v = head[second];
+                    head[first] = u * c - v * s;
+                    head[second] = u * s + v * c;
                 }
             }
             for (int d = 0; d < head_dim; ++d) dst[is_q ? d : key_offset(token, d, page_tokens)] = head[d];

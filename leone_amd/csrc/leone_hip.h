@@ -35,14 +35,16 @@ int leone_swiglu(const void* gate_up, void* out, int dtype, int rows, int ffn, h
 int leone_rope_table(float* cos_out, float* sin_out, double theta, int rotary_dim, int positions,
                      hipStream_t stream);
 
-// Per-head RMSNorm (gains may be null), half-split rotation (tables may be
-// null), q to q_out, k and v into the paged cache.  The input is of the outputs' type, or float32 in
-// qkv_planes planes (qkv_plane elements apart) that are added up in order: a product cut along K.
+// Per-head RMSNorm (gains may be null), rotation (tables may be null), q to q_out, k and v into the paged
+// cache.  The input is of the outputs' type, or float32 in qkv_planes planes (qkv_plane elements apart) that are
+// added up in order: a product cut along K.  The tables are [table_positions, rotary_dim / 2]; the first
+// rotary_dim elements of a head are rotated (rotary_dim even, at most head_dim), in pairs (i, i + rotary_dim / 2)
+// for pairing 0 (half split) or (2 i, 2 i + 1) for pairing 1 (adjacent); the rest is only normalised.
 int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_planes, long qkv_plane, void* q_out,
                              void* k_pool, void* v_pool, int dtype,
                              const void* q_gain, const void* k_gain, int gain_dtype, float eps,
                              const float* cos_table, const float* sin_table, int table_positions,
-                             const int* positions, const int* row_entry, const int* block_table, int max_blocks,
+                             int rotary_dim, int pairing, const int* positions, const int* row_entry, const int* block_table, int max_blocks,
                              int rows, int q_heads, int kv_heads, int head_dim, int page_tokens, int write_cache,
                              hipStream_t stream);
 
@@ -64,10 +66,11 @@ int leone_attention_decode(const void* q, void* out, const void* k_pool, const v
 // queries: the kernel normalises and rotates the query heads itself and, with write_cache, makes the new key,
 // and writes it and the new value into the cache before the keys are read (what leone_qk_norm_rope_write does,
 // without its launch).  qkv: bfloat16, or float32 in qkv_planes planes added up in order.  head_dim a multiple
-// of 64.  A row's keys must not be another row's new key: one row a request.
+// of 64.  A row's keys must not be another row's new key: one row a request.  The rotation it is built for is
+// the half-split one over the whole head (rotary_dim == head_dim, pairing 0); any other is refused.
 int leone_attention_decode_projected(const void* qkv, int qkv_dtype, int qkv_planes, long qkv_plane, const void* q_gain,
                                      const void* k_gain, int gain_dtype, float eps, const float* cos_table,
-                                     const float* sin_table, int table_positions, void* out, void* k_pool, void* v_pool,
+                                     const float* sin_table, int table_positions, int rotary_dim, int pairing, void* out, void* k_pool, void* v_pool,
                                      int write_cache, const int* positions, const int* row_entry, const int* block_table,
                                      int max_blocks, float* part_acc, float* part_ml, int rows, int q_heads, int kv_heads,
                                      int head_dim, int page_tokens, float scale, int window, int splits,

@@ -200,10 +200,15 @@ __global__ void rope_table_kernel(float* __restrict__ cos_out, float* __restrict
 //   k heads: the same, written into the request's page at `position`.
 //   v heads: copied into the page unchanged.
 // Keys and values go into the page in the packed layouts of key_offset() and value_offset().
-// A lane owns pairs p = lane, lane + 64, ... (p < D/2): elements p and p + D/2.
+// A lane owns pairs p = lane, lane + 64, ... (p < D/2).  Which two elements pair p is, and whether it is
+// rotated, is the position encoding's affair (crates/leone/src/cpu.rs:1765-1774 keeps the pairing a switch): of
+// the head's first `rotary_dim` = 2 * rotary_half elements, pair p < rotary_half is (p, p + rotary_half) for
+// the half-split pairing and (2p, 2p + 1) for the adjacent one and is rotated by the table's angle p; what
+// lies beyond rotary_dim is normalised but not rotated (pairs (2p, 2p + 1) either way).
 // When `write_cache` is 0 the k and v heads are skipped (a layer that reads
 // another layer's cache).
 constexpr int kMaxPairsPerLane = 4;  // head_dim up to 512
+enum RopePairing : int { kPairHalfSplit = 0, kPairAdjacent = 1 };
 
 template <typename TIn, typename T>
 __global__ void qk_norm_rope_write_kernel(
@@ -211,7 +216,7 @@ __global__ void qk_norm_rope_write_kernel(
     AnyVec q_gain, AnyVec k_gain, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int table_positions, const int* __restrict__ positions,
     const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
-    int q_heads, int kv_heads, int head_dim, int page_tokens, int write_cache) {
+    int q_heads, int kv_heads, int head_dim, int page_tokens, int write_cache, int rotary_half, int pairing) {
     const int row = blockIdx.x;
     const int head = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
     const int lane = threadIdx.x % kWave;
@@ -242,17 +247,20 @@ __global__ void qk_norm_rope_write_kernel(
         return kind == 0 ? d : kind == 1 ? key_offset(token, d, page_tokens) : value_offset(token, d, head_dim);
     };
 
+    // the two elements of pair p
+    auto first = [&](int p) { return pairing == kPairHalfSplit && p < rotary_half ? p : 2 * p; };
+    auto second = [&](int p) { return pairing == kPairHalfSplit && p < rotary_half ? p + rotary_half : 2 * p + 1; };
     float a[kMaxPairsPerLane], b[kMaxPairsPerLane];
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < kMaxPairsPerLane; ++i) {
         const int p = lane + i * kWave;
         if (p < half) {
-            a[i] = to_float(src[p]);
-            b[i] = to_float(src[p + half]);
+            a[i] = to_float(src[first(p)]);
+            b[i] = to_float(src[second(p)]);
             for (int s = 1; s < planes; ++s) {       // planes of a product cut along K: added in order
-                a[i] += to_float(src[s * plane + p]);
-                b[i] += to_float(src[s * plane + p + half]);
+                a[i] += to_float(src[s * plane + first(p)]);
+                b[i] += to_float(src[s * plane + second(p)]);
             }
             // rounded as a product stored in the outputs' type would be: the same bits whichever way it came
             a[i] = to_float(from_float<T>(a[i]));
@@ -266,8 +274,8 @@ __global__ void qk_norm_rope_write_kernel(
         for (int i = 0; i < kMaxPairsPerLane; ++i) {
             const int p = lane + i * kWave;
             if (p < half) {
-                dst[place(p)] = from_float<T>(a[i]);
-                dst[place(p + half)] = from_float<T>(b[i]);
+                dst[place(first(p))] = from_float<T>(a[i]);
+                dst[place(second(p))] = from_float<T>(b[i]);
             }
         }
         return;
@@ -286,19 +294,19 @@ __global__ void qk_norm_rope_write_kernel(
         if (p < half) {
             float u = a[i], v = b[i];
             if (gain.ptr) {
-                u = (u * load_any(gain, p)) * inv;
-                v = (v * load_any(gain, p + half)) * inv;
+                u = (u * load_any(gain, first(p))) * inv;
+                v = (v * load_any(gain, second(p))) * inv;
             }
-            if (rotate) {
-                const float c = cos_table[static_cast<long>(tpos) * half + p];
-                const float s = sin_table[static_cast<long>(tpos) * half + p];
+            if (rotate && p < rotary_half) {
+                const float c = cos_table[static_cast<long>(tpos) * rotary_half + p];
+                const float s = sin_table[static_cast<long>(tpos) * rotary_half + p];
                 const float ru = u * c - v * s;
                 const float rv = u * s + v * c;
                 u = ru;
                 v = rv;
             }
-            dst[place(p)] = from_float<T>(u);
-            dst[place(p + half)] = from_float<T>(v);
+            dst[place(first(p))] = from_float<T>(u);
+            dst[place(second(p))] = from_float<T>(v);
         }
     }
 }
@@ -667,6 +675,7 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_
                                         void* k_pool, void* v_pool, int dtype,
                                         const void* q_gain, const void* k_gain, int gain_dtype, float eps,
                                         const float* cos_table, const float* sin_table, int table_positions,
+                                        int rotary_dim, int pairing,
                                         const int* positions, const int* row_entry, const int* block_table,
                                         int max_blocks, int rows, int q_heads, int kv_heads, int head_dim,
                                         int page_tokens, int write_cache, hipStream_t stream) {
@@ -682,6 +691,11 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_
     LEONE_REQUIRE((q_gain == nullptr) == (k_gain == nullptr), "qk_norm_rope_write: q and k gains come together");
     LEONE_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "qk_norm_rope_write: cos and sin tables come together");
     LEONE_REQUIRE(!cos_table || table_positions > 0, "qk_norm_rope_write: empty rotary table");
+    LEONE_REQUIRE(!cos_table || (rotary_dim > 0 && rotary_dim % 2 == 0 && rotary_dim <= head_dim),
+                  "qk_norm_rope_write: rotary_dim %d must be even, positive and at most head_dim %d", rotary_dim, head_dim);
+    LEONE_REQUIRE(pairing == kPairHalfSplit || pairing == kPairAdjacent, "qk_norm_rope_write: unknown pairing %d", pairing);
+    // the kernel in runs of 8 is built for the half-split rotation of the whole head (or none)
+    const bool whole_head = !cos_table || (rotary_dim == head_dim && pairing == kPairHalfSplit);
     LEONE_REQUIRE(rows > 0 && q_heads > 0 && kv_heads > 0, "qk_norm_rope_write: rows %d heads %d/%d must be positive", rows, q_heads, kv_heads);
     LEONE_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && head_dim <= 2 * kWave * kMaxPairsPerLane,
                   "qk_norm_rope_write: head_dim %d must be even and at most %d", head_dim, 2 * kWave * kMaxPairsPerLane);
@@ -694,7 +708,7 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_
                          (!write_cache || (reinterpret_cast<uintptr_t>(k_pool) % run_bytes == 0 && page_tokens % 8 == 0));
     const bool tables_aligned = (!q_gain || (reinterpret_cast<uintptr_t>(q_gain) % 32 == 0 && reinterpret_cast<uintptr_t>(k_gain) % 32 == 0)) &&
                                 (!cos_table || (reinterpret_cast<uintptr_t>(cos_table) % 32 == 0 && reinterpret_cast<uintptr_t>(sin_table) % 32 == 0));
-    if (head_dim % 16 == 0 && head_dim <= 128 && aligned && tables_aligned && static_cast<long>(rows) * (q_heads + 2 * kv_heads) * 8 < 0x7fffffffL * 256) {
+    if (whole_head && head_dim % 16 == 0 && head_dim <= 128 && aligned && tables_aligned && static_cast<long>(rows) * (q_heads + 2 * kv_heads) * 8 < 0x7fffffffL * 256) {
 #define LEONE_RUNS_ARGS                                                                                             \
     qkv, qkv_planes, qkv_plane, q_out, k_pool, v_pool, qg, kg, eps, cos_table, sin_table, table_positions, positions, \
         row_entry, block_table, max_blocks, rows, q_heads, kv_heads, page_tokens, write_cache, stream
@@ -720,7 +734,7 @@ extern "C" int leone_qk_norm_rope_write(const void* qkv, int qkv_dtype, int qkv_
     qk_norm_rope_write_kernel<TIN, T><<<grid, waves_per_block * kWave, 0, stream>>>(                                \
         static_cast<const TIN*>(qkv), qkv_planes, qkv_plane, static_cast<T*>(q_out), static_cast<T*>(k_pool),       \
         static_cast<T*>(v_pool), qg, kg, eps, cos_table, sin_table, table_positions, positions, row_entry,          \
-        block_table, max_blocks, q_heads, kv_heads, head_dim, page_tokens, write_cache)
+        block_table, max_blocks, q_heads, kv_heads, head_dim, page_tokens, write_cache, cos_table ? rotary_dim / 2 : 0, pairing)
     if (dtype == kF32) LEONE_QK_ANY(float, float);
     else if (qkv_dtype == kF32) LEONE_QK_ANY(float, bf16_t);
     else LEONE_QK_ANY(bf16_t, bf16_t);

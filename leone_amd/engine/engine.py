@@ -255,25 +255,33 @@ class Engine:
             return best
 
         from ..cache.manager import OutOfPages, OutOfSlots
-        try:
-            with ops.record_library_products() as recorded:
-                trial_step_ms(1)
-        except (OutOfPages, OutOfSlots):
-            return []                                   # no room for the trial step now: nothing is tuned
-        step_ms = trial_step_ms()
         records = []
-        for (m, n, k, out_code, accumulate), weights in recorded.problems.items():
-            out_dtype = torch.float32 if out_code == ops.F32 else torch.bfloat16
-            record = ops.tune_library_product(m, weights, out_dtype, bool(accumulate), candidates, thorough)
-            if record["kept"] and keep_only_faster_steps:
-                with_it = trial_step_ms()
-                record["step_ms"], record["step_ms_before"] = round(with_it, 3), round(step_ms, 3)
-                if with_it < step_ms * 0.998:
-                    step_ms = with_it
-                else:
-                    ops.forget_tuned_products([record["problem"]])
-                    record["kept"] = False
-            records.append(record)
+        try:
+            try:
+                with ops.record_library_products() as recorded:
+                    trial_step_ms(1)
+            except (OutOfPages, OutOfSlots):
+                return []                                   # no room for the trial step now: nothing is tuned
+            step_ms = trial_step_ms()
+            for (m, n, k, out_code, accumulate), weights in recorded.problems.items():
+                out_dtype = torch.float32 if out_code == ops.F32 else torch.bfloat16
+                record = ops.tune_library_product(m, weights, out_dtype, bool(accumulate), candidates, thorough)
+                records.append(record)
+                if record["kept"] and keep_only_faster_steps:
+                    with_it = trial_step_ms()
+                    record["step_ms"], record["step_ms_before"] = round(with_it, 3), round(step_ms, 3)
+                    if with_it < step_ms * 0.998:
+                        step_ms = with_it
+                    else:
+                        ops.forget_tuned_products([record["problem"]])
+                        record["kept"] = False
+        except BaseException:
+            # whatever failed, the engine is left as it was found: no winner of this call stays in use
+            ops.forget_tuned_products([r["problem"] for r in records if r["kept"]])
+            raise
+        finally:
+            if self.cache.has(request):                     # a trial step that failed half way still holds its request
+                self.release(request)
         return records
 
     # ---- the step --------------------------------------------------------------------

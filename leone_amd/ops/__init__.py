@@ -169,15 +169,43 @@ def rope_table(theta: float, rotary_dim: int, positions: int, device) -> tuple[t
     return cos, sin
 
 
+PAIRINGS = {"half_split": 0, "adjacent": 1}   # which two elements of a head a rotation turns together
+
+
+def _rotation_shape(what: str, head_dim: int, cos, sin, pairing: str):
+    """(table positions, rotary_dim, pairing code) of a rotation given as cos/sin tables ``[positions,
+    rotary_dim / 2]``: the head's first ``rotary_dim`` elements are rotated, in pairs (i, i + rotary_dim / 2)
+    ("half_split") or (2 i, 2 i + 1) ("adjacent") (crates/leone/src/cpu.rs:1765-1774); the rest is left as it is."""
+    if pairing not in PAIRINGS:
+        raise KernelError(f"{what}: unknown pairing {pairing!r}; known: {', '.join(PAIRINGS)}")
+    if cos is None:
+        return 0, 0, PAIRINGS[pairing]
+    if sin is None or sin.shape != cos.shape or cos.dim() != 2:
+        raise KernelError(f"{what}: cos and sin tables must both be [positions, rotary_dim / 2]")
+    rotary_dim = 2 * cos.shape[1]
+    if not 0 < rotary_dim <= head_dim:
+        raise KernelError(f"{what}: the rotary tables cover {rotary_dim} elements, a head has {head_dim}")
+    return cos.shape[0], rotary_dim, PAIRINGS[pairing]
+
+
+def decode_projected_supported(head_dim: int, rotary_dim: int = 0, pairing: str = "half_split") -> bool:
+    """Whether ``attention_decode_projected`` takes this head and rotation: head sizes that are multiples of
+    64, no rotation (``rotary_dim`` 0) or the half-split one over the whole head."""
+    return head_dim % 64 == 0 and (rotary_dim == 0 or (rotary_dim == head_dim and pairing == "half_split"))
+
+
 def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim: int,
                        q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
                        cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
                        row_entry: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                        k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor], write_cache: bool = True,
-                       out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+                       out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
+                       pairing: str = "half_split") -> torch.Tensor:
     """Splits the fused projection, normalises and rotates q and k heads, writes k and v into the cache.
     ``qkv`` is ``[rows, width]`` of the cache's type, or float32 (also as planes ``[p, rows, width]`` whose
-    sum, in order, is meant: a product cut along K) with ``out_dtype`` naming the type of q and the cache."""
+    sum, in order, is meant: a product cut along K) with ``out_dtype`` naming the type of q and the cache.
+    The rotation's shape comes with its tables (``_rotation_shape``): their width says how much of a head is
+    rotated, ``pairing`` which elements go together."""
     planes = qkv.shape[0] if qkv.dim() == 3 else 1
     rows, width = qkv.shape[-2:]
     kind = out_dtype or qkv.dtype
@@ -196,11 +224,7 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim:
             raise KernelError(f"qk_norm_rope_write: pool shape {tuple(k_pool.shape)} does not fit "
                               f"{kv_heads} heads of {head_dim}")
         max_blocks = block_table.shape[1]
-    table_positions = 0
-    if cos is not None:
-        table_positions = cos.shape[0]
-        if cos.shape[1] != head_dim // 2 or sin is None or sin.shape != cos.shape:
-            raise KernelError("qk_norm_rope_write: rotary table does not fit the head size")
+    table_positions, rotary_dim, pairing_code = _rotation_shape("qk_norm_rope_write", head_dim, cos, sin, pairing)
     gain_code = _code(q_gain, "q gain") if q_gain is not None else F32
     if q_gain is not None and (k_gain is None or k_gain.dtype != q_gain.dtype):
         raise KernelError("qk_norm_rope_write: q and k gains must come together in one type")
@@ -210,7 +234,7 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_heads: int, kv_heads: int, head_dim:
          _dev(v_pool if write_cache else None, "v pool", kind), _CODES[kind],
          _dev(q_gain, "q gain", None, (head_dim,)), _dev(k_gain, "k gain", None, (head_dim,)), gain_code,
          float(eps), _dev(cos, "rope cos", torch.float32), _dev(sin, "rope sin", torch.float32), table_positions,
-         _dev(positions, "positions", torch.int32, (rows,)),
+         rotary_dim, pairing_code, _dev(positions, "positions", torch.int32, (rows,)),
          _dev(row_entry if write_cache else None, "row map", torch.int32, (rows,)),
          _dev(block_table if write_cache else None, "block table", torch.int32), max_blocks, rows, q_heads,
          kv_heads, head_dim, page_tokens, 1 if write_cache else 0, _stream())
@@ -295,7 +319,8 @@ def attention_decode_projected(qkv: torch.Tensor, q_heads: int, kv_heads: int, h
                                cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], k_pool: torch.Tensor,
                                v_pool: torch.Tensor, positions: torch.Tensor, row_entry: torch.Tensor,
                                block_table: torch.Tensor, scale: float, window: int = 0, max_context: int = 1,
-                               splits: Optional[int] = None, write_cache: bool = True) -> torch.Tensor:
+                               splits: Optional[int] = None, write_cache: bool = True,
+                               pairing: str = "half_split") -> torch.Tensor:
     """``qk_norm_rope_write`` and ``attention_decode`` in one launch, for a step in which every row is another
     request (single decoded tokens): the kernel takes the fused q/k/v projection (bfloat16 ``[rows, width]``, or
     float32 planes ``[p, rows, width]``), makes queries and the new key itself and writes key and value into
@@ -308,8 +333,11 @@ def attention_decode_projected(qkv: torch.Tensor, q_heads: int, kv_heads: int, h
                           f"{q_heads}+2*{kv_heads} heads of {head_dim}")
     if head_dim % 64:
         raise KernelError(f"attention_decode_projected: head size {head_dim} is no multiple of 64")
-    if cos is not None and (cos.shape[1] != head_dim // 2 or sin is None or sin.shape != cos.shape):
-        raise KernelError("attention_decode_projected: rotary table does not fit the head size")
+    table_positions, rotary_dim, pairing_code = _rotation_shape("attention_decode_projected", head_dim, cos, sin, pairing)
+    if not decode_projected_supported(head_dim, rotary_dim, pairing):
+        raise KernelError(f"attention_decode_projected: the kernel rotates whole heads in half-split pairs, not "
+                          f"{rotary_dim} of {head_dim} elements in {pairing} pairs (qk_norm_rope_write and "
+                          f"attention_decode take those)")
     if q_gain is not None and (k_gain is None or k_gain.dtype != q_gain.dtype):
         raise KernelError("attention_decode_projected: q and k gains must come together in one type")
     if splits is None:
@@ -322,8 +350,8 @@ def attention_decode_projected(qkv: torch.Tensor, q_heads: int, kv_heads: int, h
     call("leone_attention_decode_projected", _dev(qkv, "qkv"), _code(qkv, "qkv"), planes, rows * width,
          _dev(q_gain, "q gain", None, (head_dim,)), _dev(k_gain, "k gain", None, (head_dim,)),
          _code(q_gain, "q gain") if q_gain is not None else F32, float(eps),
-         _dev(cos, "rope cos", torch.float32), _dev(sin, "rope sin", torch.float32), 0 if cos is None else cos.shape[0],
-         _dev(out, "attention out"), _dev(k_pool, "k pool", torch.bfloat16), _dev(v_pool, "v pool", torch.bfloat16),
+         _dev(cos, "rope cos", torch.float32), _dev(sin, "rope sin", torch.float32), table_positions, rotary_dim,
+         pairing_code, _dev(out, "attention out"), _dev(k_pool, "k pool", torch.bfloat16), _dev(v_pool, "v pool", torch.bfloat16),
          1 if write_cache else 0, _dev(positions, "positions", torch.int32, (rows,)),
          _dev(row_entry, "row map", torch.int32, (rows,)), _dev(block_table, "block table", torch.int32),
          block_table.shape[1], _dev(part_acc, "partials"), _dev(part_ml, "partial sums"), rows, q_heads, kv_heads,
@@ -758,13 +786,24 @@ def tune_library_product(rows: int, weights, out_dtype: torch.dtype, accumulate:
     usual_off = (usual.float() - exact).abs().max().item()
     kept = bool(off <= 2.0 * usual_off + 1e-6 * exact.abs().max().item())
     if kept:
+        # An algorithm that reduces over K with atomics (split-K, stream-K) need not repeat bit for bit, and
+        # then neither would the logits of a replayed trace: the winner runs again from the same zero stream,
+        # and once more with the rows of x in reverse order (a row's bits must not depend on the other rows).
+        again = torch.zeros_like(y)
+        call("leone_library_product", _dev(x, "x"), _dev(weight, "w"), _dev(again, "y"), rows, n, k, out_code,
+             1 if accumulate else 0, _stream())
+        turned, x_turned = torch.zeros_like(y), x.flip(0).contiguous()
+        call("leone_library_product", _dev(x_turned, "x"), _dev(weight, "w"), _dev(turned, "y"), rows, n, k, out_code,
+             1 if accumulate else 0, _stream())
+        kept = bool(torch.equal(again, y) and torch.equal(turned.flip(0), y))
+    if kept:
         _tuned_products.add(problem)
     else:
         call("leone_library_product_forget", rows, n, k, out_code, 1 if accumulate else 0)
     return {"problem": problem, "rows": rows, "weight_rows": n, "inner": k, "float_out": out_dtype == torch.float32,
             "adds": bool(accumulate),
             "library_us": round(first.value, 1), "tuned_us": round(best.value, 1), "timed": timed.value, "kept": kept,
-            "off": off, "library_off": usual_off}
+            "off": off, "library_off": usual_off}      # ``kept`` False: too far off, or not the same bits twice
 
 
 def forget_tuned_products(problems=None) -> None:

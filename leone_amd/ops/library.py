@@ -27,11 +27,11 @@ _PROTOTYPES = {
     "leone_add_rmsnorm": [P, P, c_int, c_int, ctypes.c_long, P, c_int, c_float, P, c_int, P, c_int, c_int, P, P],
     "leone_swiglu": [P, P, c_int, c_int, c_int, P],
     "leone_rope_table": [P, P, c_double, c_int, c_int, P],
-    "leone_qk_norm_rope_write": [P, c_int, c_int, ctypes.c_long, P, P, P, c_int, P, P, c_int, c_float, P, P, c_int, P, P, P, c_int,
-                                 c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "leone_qk_norm_rope_write": [P, c_int, c_int, ctypes.c_long, P, P, P, c_int, P, P, c_int, c_float, P, P, c_int, c_int, c_int,
+                                 P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "leone_attention_rows": [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
                              c_int, P],
-    "leone_attention_decode_projected": [P, c_int, c_int, ctypes.c_long, P, P, c_int, c_float, P, P, c_int, P, P, P, c_int,
+    "leone_attention_decode_projected": [P, c_int, c_int, ctypes.c_long, P, P, c_int, c_float, P, P, c_int, c_int, c_int, P, P, P, c_int,
                                          P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, P],
     "leone_attention_decode": [P, P, P, P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                c_int, P],

@@ -10,6 +10,7 @@ from .. import ops
 from ..weights.loader import MATRIX, VECTOR, TensorSpec
 from .base import MIXERS, KvNeed, Part, PartSpec, RowTiling
 from .context import KvCacheView, StepContext
+from .position import rotation_of
 
 
 @MIXERS.register("gqa_attention")
@@ -90,25 +91,40 @@ class GqaAttention(Part):
         """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned),
         and with ``next_norm`` the norm that follows may come back prepared (see ``ops.linear``)."""
         qkv = ops.linear(y, self.w_qkv, planes_ok=True)
-        cos, sin = self.position.tables() if self.position is not None else (None, None)
+        # How much of a head is rotated and in which pairs is the position part's affair; the kernels are told.
+        rotation = rotation_of(self.position)
+        cos, sin = rotation.cos, rotation.sin
         if cos is not None and step.max_position >= cos.shape[0]:
             raise ValueError(f"position {step.max_position} is beyond the rotary table of {cos.shape[0]} positions")
-        if (step.decode_only and step.dtype == torch.bfloat16 and self.head_dim % 64 == 0
-                and ops.decode_attention_supported(step.dtype, self.head_dim, cache.page_tokens,
-                                                   self.q_heads // self.kv_heads, cache.block_table.shape[1])):
+        kernels = self.attention_kernels(step.dtype, cache.page_tokens, cache.block_table.shape[1])
+        if step.decode_only and kernels["decode"] == "projected":
             # Single decoded tokens, every row another request: the attention kernel makes the heads itself.
             attended = ops.attention_decode_projected(
                 qkv, self.q_heads, self.kv_heads, self.head_dim, self.q_gain, self.k_gain,
                 self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin, cache.k_pool, cache.v_pool,
                 step.positions, step.row_entry, cache.block_table, self.scale, int(self.window or 0),
-                max_context=step.max_position + 1, write_cache=cache.writes)
+                max_context=step.max_position + 1, write_cache=cache.writes, pairing=rotation.pairing)
             return ops.linear(attended, self.w_o, residual=residual, next_norm=next_norm)
         q = ops.qk_norm_rope_write(qkv, self.q_heads, self.kv_heads, self.head_dim, self.q_gain, self.k_gain,
                                    self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, cos, sin,
                                    step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
-                                   write_cache=cache.writes, out_dtype=step.dtype)
+                                   write_cache=cache.writes, out_dtype=step.dtype, pairing=rotation.pairing)
         attended = self._attend(q, step, cache)
         return ops.linear(attended, self.w_o, residual=residual, next_norm=next_norm)
+
+    def attention_kernels(self, dtype: torch.dtype, page_tokens: int, max_blocks: int = 0) -> Dict[str, str]:
+        """Which kernels this shape gets, by kind of work: ``decode`` (steps of single tokens): "projected" (the
+        split-KV matrix-core kernel that also makes the heads and writes the cache), "split_kv" (the same
+        kernel behind the norm/rotation/write kernel) or "rows" (the float kernel for any shape and type);
+        ``prompt`` (portions of at least ``ops.PREFILL_MIN_ROWS`` rows): "flash" (the matrix-core prompt
+        kernel), else what single tokens get."""
+        group = self.q_heads // self.kv_heads
+        if not ops.decode_attention_supported(dtype, self.head_dim, page_tokens, group, max_blocks):
+            return {"decode": "rows", "prompt": "rows"}
+        rotation = rotation_of(self.position)
+        projected = ops.decode_projected_supported(self.head_dim, rotation.rotary_dim, rotation.pairing)
+        return {"decode": "projected" if projected else "split_kv",
+                "prompt": "flash" if ops.prefill_attention_supported(dtype, self.head_dim, page_tokens, max_blocks) else "split_kv"}
 
     def _attend(self, q: torch.Tensor, step: StepContext, cache: KvCacheView) -> torch.Tensor:
         """Long prompt portions through the prompt kernel, the other rows through the split-KV kernel; the

@@ -53,6 +53,26 @@ def rope_half_split(x: torch.Tensor, positions, theta: float) -> torch.Tensor:
     return out
 
 
+def rope_pairs(x: torch.Tensor, positions, theta: float, rotary_dim: int, pairing: str) -> torch.Tensor:
+    """The rotation with its shape as parameters: of a head's first ``rotary_dim`` = R elements, pair i is
+    (x[i], x[i + R/2]) ("half_split") or (x[2i], x[2i + 1]) ("adjacent"), angle = pos * theta^(-2i/R); the
+    elements from R on are left as they are (the pairing switch of crates/leone/src/cpu.rs:1765-1774, the
+    frequencies of :1721-1743 with the rotated width in the exponent)."""
+    x = x.to(F64)
+    out = x.clone()
+    half = rotary_dim // 2
+    for t in range(x.shape[0]):
+        pos = float(int(positions[t]))
+        for i in range(half):
+            angle = pos * (float(theta) ** (-2.0 * i / rotary_dim))
+            c, s = math.cos(angle), math.sin(angle)
+            first, second = (i, i + half) if pairing == "half_split" else (2 * i, 2 * i + 1)
+            a, b = x[t, :, first], x[t, :, second]
+            out[t, :, first] = a * c - b * s
+            out[t, :, second] = a * s + b * c
+    return out
+
+
 def attend_one(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: Optional[int] = None) -> torch.Tensor:
     """One query [Hq, D] at position t = len(k) - 1 over the keys and values [t + 1, Hkv, D] of its
     sequence.  Query head h uses kv head h // (Hq/Hkv); score = (q . k) / sqrt(D), scale after the
@@ -95,8 +115,12 @@ def attention_block(y: torch.Tensor, weights: Dict[str, torch.Tensor], prefix: s
     v = linear(y, weights[f"{prefix}.v_proj.weight"]).view(tokens, kv_heads, dim)
     q = rms_norm(q, weights[f"{prefix}.q_norm.weight"], config["rms_norm_eps"])
     k = rms_norm(k, weights[f"{prefix}.k_norm.weight"], config["rms_norm_eps"])
-    q = rope_half_split(q, positions, config["rope_theta"])
-    k = rope_half_split(k, positions, config["rope_theta"])
+    if "rotary_dim" in config or "rope_pairing" in config:      # another shape of rotation than this architecture's
+        shape = (config.get("rotary_dim", dim), config.get("rope_pairing", "half_split"))
+        q, k = (rope_pairs(t, positions, config["rope_theta"], *shape) for t in (q, k))
+    else:
+        q = rope_half_split(q, positions, config["rope_theta"])
+        k = rope_half_split(k, positions, config["rope_theta"])
     attended = causal_attention(q, k, v).reshape(tokens, heads * dim)
     return linear(attended, weights[f"{prefix}.o_proj.weight"])
 

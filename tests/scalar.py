@@ -15,7 +15,7 @@ _PROTOTYPES = {
     "leone_ref_embed": [PF, PI, PF, c_int, c_int, c_int],
     "leone_ref_add_rmsnorm": [PF, PF, c_int, c_long, PF, c_float, PF, PI, c_int, c_int],
     "leone_ref_rope_table": [PF, PF, c_double, c_int, c_int],
-    "leone_ref_qk_norm_rope_write": [PF, c_int, c_long, PF, PF, PF, PF, PF, c_float, PF, PF, c_int, PI, PI, PI, c_int,
+    "leone_ref_qk_norm_rope_write": [PF, c_int, c_long, PF, PF, PF, PF, PF, c_float, PF, PF, c_int, c_int, c_int, PI, PI, PI, c_int,
                                      c_int, c_int, c_int, c_int, c_int, c_int],
     "leone_ref_attention": [PF, PF, PF, PF, PI, PI, PI, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int],
     "leone_ref_gemm": [PF, PF, PF, c_int, c_int, c_int],
@@ -88,7 +88,8 @@ def rope_table(theta, rotary_dim, positions):
 
 
 def qk_norm_rope_write(qkv, q_heads, kv_heads, head_dim, q_gain, k_gain, eps, cos, sin, positions, row_entry,
-                       block_table, k_pool, v_pool, write_cache=True):
+                       block_table, k_pool, v_pool, write_cache=True, pairing=0):
+    """The rotation covers the first 2 * (the tables' width) elements of a head; ``pairing`` 0 half split, 1 adjacent."""
     qkv = f32(qkv)
     planes = 1 if qkv.ndim == 2 else qkv.shape[0]
     rows, width = qkv.shape[-2:]
@@ -98,7 +99,7 @@ def qk_norm_rope_write(qkv, q_heads, kv_heads, head_dim, q_gain, k_gain, eps, co
     page_tokens = k_pool.shape[3] if k_pool is not None else 0
     _check(_lib().leone_ref_qk_norm_rope_write(
         _f(qkv), planes, rows * width, _f(q_out), _f(k_pool), _f(v_pool), _f(q_gain), _f(k_gain), eps, _f(cos), _f(sin),
-        0 if cos is None else cos.shape[0], _i(positions), _i(row_entry), _i(block_table), block_table.shape[1], rows,
+        0 if cos is None else cos.shape[0], 0 if cos is None else 2 * cos.shape[1], pairing, _i(positions), _i(row_entry), _i(block_table), block_table.shape[1], rows,
         q_heads, kv_heads, head_dim, page_tokens, 1 if write_cache else 0), "qk_norm_rope_write")
     return q_out
 

@@ -276,3 +276,12 @@ def test_the_log_of_freed_pages_names_every_page_whoever_frees_it():
     assert sorted(m.drain_freed(0)) == sorted(shared)
     assert m.drain_freed(0) == []                                          # drained
     m.check()
+    # a caller with too little room is refused and loses nothing: the pages come out when it asks again
+    from ctypes import c_int
+    m.admit("d")
+    m.reserve("d", 13)
+    held = sorted(p for p in m.table("d", 0) if p >= 0)
+    m.release("d")
+    small = (c_int * 2)()
+    assert m._lib.leone_cache_drain_freed(m.handle, 0, small, 2) < 0
+    assert sorted(m.drain_freed(0)) == held

@@ -134,3 +134,39 @@ def test_version_and_build_info(capsys):
         assert build.source_digest() != info["kernels"]["source_digest"]
     finally:
         build.FLAGS[:] = flags
+
+
+def test_cache_bytes_per_token_ask_every_kind_of_cache():
+    """The default size of the page pool and the roofline's cache bytes come from what each paged need says of
+    itself, so a mixer with another kind of cache than keys and values is not counted as caching nothing."""
+    from dataclasses import dataclass
+
+    import torch
+
+    from leone_amd.api import cache_bytes_per_token
+    from leone_amd.parts.base import KvNeed, StateNeed
+
+    @dataclass(frozen=True)
+    class VectorNeed:                      # one vector of `width` elements a token; no kv_heads, no head_dim
+        width: int
+        paged = True
+
+        def group_key(self):
+            return self
+
+        def bytes_per_token(self, element_size):
+            return self.width * element_size
+
+    class Model:
+        dtype = torch.bfloat16
+
+        def __init__(self, needs):
+            self.needs = needs
+
+        def cache_needs(self):
+            return self.needs
+
+    assert cache_bytes_per_token(Model({0: VectorNeed(24)})) == 48
+    assert cache_bytes_per_token(Model({0: VectorNeed(24), 1: KvNeed(2, 16), 2: StateNeed((5,))})) == 48 + 2 * 2 * 16 * 2
+    from leone_amd import benchmark
+    assert benchmark.cache_bytes_per_token(Model({0: VectorNeed(10), 3: KvNeed(8, 128)})) == 20 + 2 * 8 * 128 * 2

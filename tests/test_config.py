@@ -43,6 +43,7 @@ def test_defaults_and_head_dim_not_tied_to_hidden():
     ({"rope_theta": float("inf")}, "rope_theta"),
     ({"rms_norm_eps": 0.0}, "rms_norm_eps"),
     ({"head_dim": 15}, "head_dim"),
+    ({"head_dim": 20}, "head_dim"),          # even, but the cache packs heads in runs of 8
     ({"rope_scaling": {"type": "yarn", "factor": 4.0}}, "rope_scaling"),
     ({"attention_bias": True}, "attention_bias"),
     ({"use_sliding_window": True}, "use_sliding_window"),

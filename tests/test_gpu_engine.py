@@ -5,7 +5,7 @@ import torch
 
 from tests import schedules
 from tests.plain import qwen3_plain
-from tests.util import TINY, make_model_dir, random_tokens, read_config, read_weights, tolerance
+from tests.util import REAL_8B_ONE_LAYER, TINY, make_model_dir, random_tokens, read_config, read_weights, tolerance
 
 pytestmark = pytest.mark.gpu
 
@@ -462,8 +462,7 @@ _REAL_BASE = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", rope_t
                   tie_word_embeddings=False, max_position_embeddings=1024, vocab_size=8200)
 REAL = {
     # one and two layers of the 8B widths, one of the 32B head shape (64 query heads of 128 over a width of 5,120)
-    "8b-1": dict(_REAL_BASE, num_hidden_layers=1, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
-                 head_dim=128, intermediate_size=12288),
+    "8b-1": REAL_8B_ONE_LAYER,
     "8b-2": dict(_REAL_BASE, num_hidden_layers=2, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
                  head_dim=128, intermediate_size=12288),
     "32b-1": dict(_REAL_BASE, num_hidden_layers=1, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,

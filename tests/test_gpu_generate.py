@@ -84,6 +84,38 @@ def test_long_decoding_and_preemption_keep_the_tokens(folders, tmp_path, dtype_n
             assert margins[i][len(prompts[i]) + at - 1] < 3e-2, (i, at, margins[i][len(prompts[i]) + at - 1])
 
 
+def test_greedy_generation_at_the_widths_of_the_large_models(tmp_path):
+    """Scheduler, step and device sampler together at one layer of the 8B widths in bfloat16 (where the
+    products' plans, the cuts of K and the changes of kernel were chosen): four requests, prompts in portions
+    of 64 beside decoded tokens, so few pages that a request is preempted and recomputed.  Every token the
+    engine picks must be, for the plain implementation on the same (bfloat16) weights fed the same tokens,
+    the best one or within the type's noise of it: 1.5 % of the largest logit, the bound the step itself is
+    held to at these widths."""
+    from leone_amd.api import Runtime
+    from leone_amd.engine.scheduler import SchedulerPolicy
+    from tests.util import REAL_8B_ONE_LAYER
+
+    folder = make_model_dir(str(tmp_path / "m"), REAL_8B_ONE_LAYER, seed=73, dtype=torch.bfloat16)
+    weights, config = read_weights(folder), read_config(folder)
+    prompts = [random_tokens(50 + i, n, config["vocab_size"]) for i, n in enumerate([100, 37, 150, 70])]
+    new = 20
+    runtime = Runtime.load(folder, "bfloat16", num_pages=7, page_tokens=64, max_requests=4, poison_freed=True,
+                           policy=SchedulerPolicy(max_live_requests=4, prefill_chunk_tokens=64, max_step_tokens=96))
+    results = runtime.generate_tokens(prompts, new, eos_token_id=None)
+    runtime.engine.cache.check()
+    assert runtime.last_stats.emitted_tokens == new * len(prompts)
+    assert runtime.last_stats.preemptions >= 1
+    assert not runtime.engine.cache.live_requests()
+    for prompt, result in zip(prompts, results):
+        assert len(result.tokens) == new and result.finish_reason == "length"
+        logits = qwen3_plain.forward(weights, config, list(prompt) + result.tokens).numpy()
+        scale = float(np.abs(logits).max())
+        assert scale > 3.0
+        for i, token in enumerate(result.tokens):
+            row = logits[len(prompt) + i - 1]
+            assert row[token] >= row.max() - 1.5e-2 * scale, (i, token, float(row[token]), float(row.max()))
+
+
 def test_temperature_sampling_matches_oracle_and_ignores_batching(folders):
     """Config B's workload: prompts 5/40/130, portions of 32, 24 tokens at temperature 0.8, seeded."""
     from leone_amd.api import Runtime, sampling_params

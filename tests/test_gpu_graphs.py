@@ -58,36 +58,80 @@ def test_replayed_decode_steps_equal_eager_ones(tmp_path, dtype_name):
 
 
 def test_a_part_that_is_not_graph_safe_keeps_the_model_eager(tmp_path):
+    """A model one of whose parts does not declare itself safe to record is never replayed: the engine stays
+    eager, records nothing, and its decode steps still agree with the plain implementation."""
+    import dataclasses
+
+    from leone_amd.architectures import config_from_dir, model_spec_for
+    from leone_amd.engine.engine import Engine, StepEntry
     from leone_amd.parts import MIXERS, Part
+    from leone_amd.parts.base import PartSpec
     from leone_amd.parts.mixer import GqaAttention
+    from leone_amd.parts.model import DecoderModel
+    from leone_amd.weights import loader
+    from tests.plain import qwen3_plain
+    from tests.util import read_config, read_weights, tolerance
 
     class HostDependent(GqaAttention):
         graph_safe = False
 
     assert not Part.graph_safe and GqaAttention.graph_safe and not HostDependent.graph_safe
+    folder = make_model_dir(str(tmp_path / "m"), TINY["B"], 9, torch.float32)
+    spec = model_spec_for(config_from_dir(folder))
+    MIXERS.register("host_dependent_attention", HostDependent)
+    try:
+        spec = dataclasses.replace(spec, layers=[
+            PartSpec(layer.kind, {**layer.params, "mixer": PartSpec("host_dependent_attention", layer["mixer"].params)})
+            if i == 1 else layer for i, layer in enumerate(spec.layers)])
+        model = DecoderModel(spec, torch.float32, "cuda:0")
+        model.bind(loader.load_from_dir(folder, model.tensor_specs(), model.dtype, model.device))
+        assert not model.graph_safe
+        engine = Engine(model, num_pages=16, page_tokens=16, max_requests=2, graphs=True)
+        assert engine.graphs is False
+        tokens = random_tokens(31, 40, TINY["B"]["vocab_size"])
+        expected = qwen3_plain.forward(read_weights(folder), read_config(folder), tokens).numpy()
+        engine.step([StepEntry("a", tokens[:30], [])])
+        for at in range(30, 40):
+            logits = engine.step([StepEntry("a", [tokens[at]], [0])]).logits.cpu().numpy()
+            assert np.abs(logits[0] - expected[at]).max() <= tolerance("float32"), at
+        assert not engine._decode_graphs
+    finally:
+        MIXERS.unregister("host_dependent_attention")
 
 
-def test_replay_with_many_rows_uses_the_library_product_inside_the_graph(tmp_path):
-    """More than 16 decode rows take the library's matrix product; a recording that holds it is
-    replayed several times, with eager steps between, and every replay is compared with the eager engine."""
+@pytest.mark.parametrize("n", [20, 150])
+def test_replayed_decode_steps_of_many_rows_agree_with_plain(tmp_path, n):
+    """Decode steps of many requests, recorded and replayed, against the plain implementation: 20 rows take
+    the multi-row weight-streaming product, 150 rows (more than it takes) the vendor library's products and
+    the separate activation kernel inside the recording.  The recording is replayed several times, with eager
+    steps between, and every replay is compared."""
+    from leone_amd import ops
     from leone_amd.engine.engine import Engine, StepEntry
     from leone_amd.runtime import load_model
+    from tests.plain import qwen3_plain
+    from tests.util import read_config, read_weights, tolerance
 
     folder = make_model_dir(str(tmp_path / "m"), TINY["M"], 6, torch.bfloat16)
     model = load_model(folder, "bfloat16")
-    engines = [Engine(model, num_pages=64, page_tokens=16, max_requests=24, graphs=flag) for flag in (True, False)]
+    engines = [Engine(model, num_pages=n * 2 + 8, page_tokens=16, max_requests=n + 1, graphs=flag) for flag in (True, False)]
     vocab = TINY["M"]["vocab_size"]
-    n = 20
-    prompts = [random_tokens(700 + i, 3 + (i * 7) % 19, vocab) for i in range(n)]
+    steps = 5
+    sequences = [random_tokens(700 + i, 3 + (i * 7) % 19 + steps, vocab) for i in range(n)]
+    weights, config = read_weights(folder), read_config(folder)
+    expected = [qwen3_plain.forward(weights, config, s).numpy()[-steps:] for s in sequences]
     for e in engines:
-        e.step([StepEntry(i, prompts[i], []) for i in range(n)])
-    for step in range(6):
-        tokens = random_tokens(800 + step, n, vocab)
-        outs = [e.step([StepEntry(i, [tokens[i]], [0]) for i in range(n)]).logits.cpu().numpy() for e in engines]
-        assert np.isfinite(outs[0]).all()
-        assert np.abs(outs[0] - outs[1]).max() < 3e-2, f"replay {step}"
+        e.step([StepEntry(i, sequences[i][:-steps], []) for i in range(n)])
+    for step in range(steps):
+        entries = [StepEntry(i, [sequences[i][step - steps]], [0]) for i in range(n)]
+        with ops.record_library_products() as recorded:
+            outs = [e.step(entries).logits.cpu().numpy() for e in engines]
+        assert bool(recorded.problems) == (n > ops.ROWS_MAX)        # (a replay hands nothing to ``linear``)
+        want = np.stack([expected[i][step] for i in range(n)])
+        for which, out in zip(("replayed", "eager"), outs):
+            assert np.isfinite(out).all()
+            assert np.abs(out - want).max() <= tolerance("bfloat16"), f"{which} step {step}"
         if step % 2 == 0:                                      # eager work between the replays
             for e in engines:
                 e.step([StepEntry("other", random_tokens(900 + step, 21, vocab), [20])])
                 e.release("other")
-    assert engines[0]._decode_graphs[n].graph is not None
+    assert engines[0]._decode_graphs[n].graph is not None and not engines[1]._decode_graphs

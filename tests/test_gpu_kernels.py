@@ -371,6 +371,86 @@ def test_qk_norm_rope_write_many_rows(dtype, shape):
     assert (k_plain[untouched] == 7.0).all() and (v_plain[untouched] == 7.0).all()
 
 
+@pytest.mark.parametrize("pairing", ["half_split", "adjacent"])
+@pytest.mark.parametrize("shape", [(4, 2, 32, 16, 16), (3, 1, 64, 32, 16), (5, 5, 48, 24, 16), (8, 2, 128, 64, 64),
+                                   (2, 2, 128, 128, 64), (3, 3, 24, 8, 16)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_qk_norm_rope_write_with_the_rotation_shape_as_parameters(dtype, shape, pairing):
+    """The position encoding owns the rotation's shape: ``rotary_dim`` of the head's elements (here half, a
+    third or all of them) in half-split or adjacent pairs; the rest is normalised and left unrotated.  Against
+    the plain implementation and, in float32, the scalar reference of the entry point."""
+    from leone_amd import ops
+    from tests import scalar
+    q_heads, kv_heads, head_dim, rotary_dim, page_tokens = shape
+    torch.manual_seed(8)
+    rows_meta = [(0, 0), (0, 1), (1, 15), (1, 16), (2, 700)]
+    n = len(rows_meta)
+    qkv = torch.randn(n, (q_heads + 2 * kv_heads) * head_dim).to(dtype)
+    q_gain, k_gain = 1 + 0.1 * torch.randn(head_dim), 1 + 0.1 * torch.randn(head_dim)
+    eps, theta = 1e-5, 1e4
+    max_blocks = 700 // page_tokens + 1
+    table = torch.full((3, max_blocks), -1, dtype=torch.int32)
+    table[0, 0], table[1, 0], table[1, 16 // page_tokens], table[2, 700 // page_tokens] = 4, 2, 2 if page_tokens > 16 else 5, 1
+    n_pages = 6
+    kp = torch.zeros((n_pages, kv_heads, head_dim // 8, page_tokens, 8), dtype=dtype, device=DEV)
+    vp = torch.zeros((n_pages, kv_heads, page_tokens // 8, head_dim, 8), dtype=dtype, device=DEV)
+    cos, sin = ops.rope_table(theta, rotary_dim, 1024, DEV)
+    assert cos.shape == (1024, rotary_dim // 2)
+    positions = torch.tensor([p for _, p in rows_meta], dtype=torch.int32)
+    row_entry = torch.tensor([e for e, _ in rows_meta], dtype=torch.int32)
+    q_out = ops.qk_norm_rope_write(qkv.to(DEV), q_heads, kv_heads, head_dim, q_gain.to(DEV), k_gain.to(DEV), eps,
+                                   cos, sin, positions.to(DEV), row_entry.to(DEV), table.to(DEV), kp, vp, pairing=pairing)
+    x = qkv.float()
+    q = x[:, :q_heads * head_dim].view(n, q_heads, head_dim)
+    k = x[:, q_heads * head_dim:(q_heads + kv_heads) * head_dim].view(n, kv_heads, head_dim)
+    want_q = plain.rope_pairs(plain.rms_norm(q, q_gain, eps), positions, theta, rotary_dim, pairing)
+    want_k = plain.rope_pairs(plain.rms_norm(k, k_gain, eps), positions, theta, rotary_dim, pairing)
+    atol, rtol = (5e-6, 2e-5) if dtype == torch.float32 else (2e-2, 1e-2)
+    close(q_out.view(n, q_heads, head_dim), want_q, atol, rtol, "q")
+    k_plain = kp.cpu().transpose(2, 3).reshape(n_pages, kv_heads, page_tokens, head_dim)
+    for i, (e, p) in enumerate(rows_meta):
+        close(k_plain[int(table[e, p // page_tokens]), :, p % page_tokens], want_k[i], atol, rtol, f"k row {i}")
+    if rotary_dim < head_dim or pairing == "adjacent":
+        # the other shape would be far off: the test can tell them apart
+        other = plain.rope_pairs(plain.rms_norm(q, q_gain, eps), positions, theta, head_dim, "half_split")
+        assert (other - want_q).abs().max() > 0.1
+    if dtype == torch.float32:
+        k_ref = np.zeros(tuple(kp.shape), dtype=np.float32)
+        v_ref = np.zeros(tuple(vp.shape), dtype=np.float32)
+        q_ref = scalar.qk_norm_rope_write(qkv.numpy(), q_heads, kv_heads, head_dim, q_gain.numpy(), k_gain.numpy(), eps,
+                                          cos.cpu().numpy(), sin.cpu().numpy(), positions.numpy(), row_entry.numpy(),
+                                          table.numpy(), k_ref, v_ref, pairing=ops.PAIRINGS[pairing])
+        assert np.abs(q_ref - q_out.cpu().numpy()).max() < 2e-5
+        assert np.abs(k_ref - kp.cpu().numpy()).max() < 2e-5 and np.array_equal(v_ref, vp.cpu().numpy())
+
+
+def test_kernels_refuse_rotations_they_are_not_built_for():
+    """The decode kernel that takes the projection itself rotates whole heads in half-split pairs; given another
+    shape it says so instead of rotating wrongly, and tables wider than the head are refused everywhere."""
+    from leone_amd import ops
+    from leone_amd.ops import KernelError
+    q_heads, kv_heads, head_dim, page = 4, 1, 64, 16
+    qkv = torch.randn(2, (q_heads + 2 * kv_heads) * head_dim, device=DEV).bfloat16()
+    kp = torch.zeros((2, kv_heads, head_dim // 8, page, 8), dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros((2, kv_heads, page // 8, head_dim, 8), dtype=torch.bfloat16, device=DEV)
+    positions = torch.tensor([3, 5], dtype=torch.int32, device=DEV)
+    rows = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
+    table = torch.tensor([[0], [1]], dtype=torch.int32, device=DEV)
+    half_cos, half_sin = ops.rope_table(1e4, head_dim // 2, 32, DEV)
+    full_cos, full_sin = ops.rope_table(1e4, head_dim, 32, DEV)
+    wide_cos, wide_sin = ops.rope_table(1e4, 2 * head_dim, 32, DEV)
+    assert ops.decode_projected_supported(head_dim, head_dim) and not ops.decode_projected_supported(head_dim, head_dim // 2)
+    assert not ops.decode_projected_supported(head_dim, head_dim, "adjacent") and ops.decode_projected_supported(head_dim, 0)
+    for cos, sin, pairing, word in ((half_cos, half_sin, "half_split", "whole heads"), (full_cos, full_sin, "adjacent", "whole heads"),
+                                    (wide_cos, wide_sin, "half_split", "a head has"), (full_cos, full_sin, "spiral", "unknown pairing")):
+        with pytest.raises(KernelError, match=word):
+            ops.attention_decode_projected(qkv, q_heads, kv_heads, head_dim, None, None, 1e-6, cos, sin, kp, vp, positions,
+                                           rows, table, 0.125, pairing=pairing)
+    with pytest.raises(KernelError, match="a head has"):
+        ops.qk_norm_rope_write(qkv, q_heads, kv_heads, head_dim, None, None, 1e-6, wide_cos, wide_sin, positions, rows, table, kp, vp)
+    assert float(kp.abs().max()) == 0.0 and float(vp.abs().max()) == 0.0          # a refused call wrote nothing
+
+
 @pytest.mark.parametrize("mnk", [(1, 777, 80), (5, 64, 64), (130, 192, 96), (67, 1000, 333), (300, 130, 1029)])
 def test_gemm_f32(mnk):
     from leone_amd import ops

@@ -110,6 +110,60 @@ def test_attention_part_with_portions_and_two_requests(dtype):
         assert float(err.max()) < tol * (1 + float(want[r].abs().max())), (r, int(err.argmax()), float(err.max()))
 
 
+@pytest.mark.parametrize("position_kind, rotary_dim", [("rope_half_split", 32), ("rope_adjacent", 64), ("rope_half_split", 64)])
+def test_attention_part_takes_the_rotation_shape_from_its_position_part(position_kind, rotary_dim):
+    """The mixer assumes no shape of rotation: a position part that rotates half a head, or adjacent pairs,
+    is handed to the kernels as it is.  At head size 64 in bfloat16 the decode kernel that makes the heads
+    itself only knows the whole head in half-split pairs; for the other shapes the mixer must take the two
+    kernels instead, and says which it takes.  A prompt portion, then single tokens of two requests."""
+    from leone_amd.parts import MIXERS, POSITIONS, PartSpec
+    from leone_amd.parts.context import KvCacheView
+    dtype = torch.bfloat16
+    hidden, q_heads, kv_heads, dim, page = 64, 4, 2, 64, 16
+    rope = POSITIONS.build(PartSpec(position_kind, {"rotary_dim": rotary_dim, "theta": 1e4}))
+    rope.prepare(128, DEV)
+    pairing = "adjacent" if position_kind == "rope_adjacent" else "half_split"
+    assert rope.rotation().pairing == pairing and rope.rotation().rotary_dim == rotary_dim
+    names = {k: k for k in ("q", "k", "v", "o", "q_norm", "k_norm")}
+    mixer = MIXERS.build(PartSpec("gqa_attention", dict(hidden=hidden, q_heads=q_heads, kv_heads=kv_heads, head_dim=dim,
+                                                        qk_norm_eps=1e-5, window=None, position="rope", **names)),
+                         positions={"rope": rope})
+    whole = rotary_dim == dim and pairing == "half_split"
+    assert mixer.attention_kernels(dtype, page) == {"decode": "projected" if whole else "split_kv", "prompt": "flash"}
+    torch.manual_seed(4)
+    w = {"q": torch.randn(q_heads * dim, hidden) * 0.1, "k": torch.randn(kv_heads * dim, hidden) * 0.1,
+         "v": torch.randn(kv_heads * dim, hidden) * 0.1, "o": torch.randn(hidden, q_heads * dim) * 0.1,
+         "q_norm": torch.full((dim,), 3.0), "k_norm": torch.full((dim,), 3.0)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    mixer.bind({k: v.to(DEV) for k, v in w.items()})
+    lengths = [37, 22]
+    ys = [torch.randn(n, hidden).to(dtype) for n in lengths]
+    pw = {f"a.{k}_proj.weight": w[k].float() for k in ("q", "k", "v", "o")}
+    pw.update({"a.q_norm.weight": w["q_norm"].float(), "a.k_norm.weight": w["k_norm"].float()})
+    cfg = dict(num_attention_heads=q_heads, num_key_value_heads=kv_heads, head_dim=dim, rms_norm_eps=1e-5, rope_theta=1e4,
+               rotary_dim=rotary_dim, rope_pairing=pairing)
+    want = [plain.attention_block(y.float(), pw, "a", cfg, list(range(len(y)))) for y in ys]
+    other = plain.attention_block(ys[0].float(), pw, "a", dict(cfg, rotary_dim=dim, rope_pairing="half_split"), list(range(lengths[0])))
+    assert whole or (other - want[0]).abs().max() > 0.2 * want[0].abs().max()       # the shapes can be told apart
+    k_pool = torch.full((8, kv_heads, dim // 8, page, 8), float("nan"), dtype=dtype, device=DEV)
+    v_pool = torch.full((8, kv_heads, page // 8, dim, 8), float("nan"), dtype=dtype, device=DEV)
+    table = torch.tensor([[5, 0, 3, -1], [7, 2, -1, -1]], dtype=torch.int32, device=DEV)
+    cache = KvCacheView(writes=True, k_pool=k_pool, v_pool=v_pool, block_table=table, page_tokens=page)
+    meta = [(0, p) for p in range(33)] + [(1, p) for p in range(18)]
+    out = mixer.forward(torch.cat([ys[0][:33], ys[1][:18]]).to(DEV), step_context(meta, dtype, {0: table}), cache)
+    have = [[out[:33]], [out[33:]]]
+    for i in range(4):                                  # single tokens of both requests: a decode-only step
+        context = step_context([(0, 33 + i), (1, 18 + i)], dtype, {0: table})
+        context.decode_only = True
+        step = mixer.forward(torch.stack([ys[0][33 + i], ys[1][18 + i]]).to(DEV), context, cache)
+        have[0].append(step[0:1])
+        have[1].append(step[1:2])
+    for r in range(2):
+        got = torch.cat(have[r]).cpu().double()
+        err = (got - want[r]).abs().max(dim=1).values
+        assert float(err.max()) < 4e-2 * (1 + float(want[r].abs().max())), (r, int(err.argmax()), float(err.max()))
+
+
 # ---- a toy architecture assembled from the framework's parts and one part defined here --------------
 
 DECAY = 0.75

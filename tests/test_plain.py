@@ -65,6 +65,37 @@ def test_rope_scores_depend_only_on_distance():
     assert abs(score(10, 3) - score(10, 4)) > 1e-6
 
 
+def test_rotation_with_its_shape_as_parameters():
+    """``rope_pairs`` pinned by what fixes it: over the whole head in half-split pairs it is ``rope_half_split``;
+    the adjacent pairing is the same rotation on a permuted head (element 2i <-> i, 2i + 1 <-> i + R/2); elements
+    beyond rotary_dim come through untouched and the rotated ones do not depend on them; scores depend on
+    distances only, whatever the shape."""
+    dim, theta = 24, 5000.0
+    x = torch.randn(5, 2, dim, dtype=F64)
+    positions = [0, 3, 9, 100, 4000]
+    assert torch.equal(plain.rope_pairs(x, positions, theta, dim, "half_split"), plain.rope_half_split(x, positions, theta))
+    for rotary in (8, 16, 24):
+        half = rotary // 2
+        split = plain.rope_pairs(x, positions, theta, rotary, "half_split")
+        assert torch.equal(split[..., rotary:], x[..., rotary:])
+        assert torch.equal(split[..., :rotary], plain.rope_half_split(x[..., :rotary], positions, theta))
+        order = [2 * i for i in range(half)] + [2 * i + 1 for i in range(half)]     # adjacent slot of each half-split slot
+        permuted = x.clone()
+        permuted[..., order] = x[..., :rotary]
+        adjacent = plain.rope_pairs(permuted, positions, theta, rotary, "adjacent")
+        assert torch.allclose(adjacent[..., order], split[..., :rotary], atol=1e-14)
+        assert torch.equal(adjacent[..., rotary:], x[..., rotary:])
+        # a unit vector at slot 2 of an adjacent pairing moves into slots 2 and 3 by angle pos * theta^(-2/R)
+        e = torch.zeros(1, 1, dim, dtype=F64); e[0, 0, 2] = 1.0
+        r = plain.rope_pairs(e, [7], theta, rotary, "adjacent")[0, 0]
+        angle = 7 * theta ** (-2.0 / rotary)
+        assert abs(float(r[2]) - math.cos(angle)) < 1e-15 and abs(float(r[3]) - math.sin(angle)) < 1e-15
+        q, k = torch.randn(1, 1, dim, dtype=F64), torch.randn(1, 1, dim, dtype=F64)
+        for pairing in ("half_split", "adjacent"):
+            score = lambda m, n: float((plain.rope_pairs(q, [m], theta, rotary, pairing) * plain.rope_pairs(k, [n], theta, rotary, pairing)).sum())
+            assert abs(score(10, 3) - score(510, 503)) < 1e-9
+
+
 def test_attention_reference_vector():
     # 2 heads, 1 kv head, D=2; K rows [1,0],[0,1]; V rows [2,4],[6,8]; q [1,0] for head 0, [0,1] for head 1
     # (crates/leone/src/cpu.rs:2850-2898)

@@ -39,6 +39,13 @@ def test_argmax_without_allocation_equals_argmax_with_a_workspace():
         assert status == 0, lib.leone_last_error().decode()
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == before
+        # torch's figure covers torch's allocator only: the driver's count of free bytes would show a hipMalloc or
+        # hipFree inside the entry point (the first call has resolved the array's address, so this one is plain)
+        free_before, _ = torch.cuda.mem_get_info(device)
+        out.fill_(-7)
+        assert lib.leone_argmax_static(logits.data_ptr(), out.data_ptr(), rows, vocab, stream) == 0
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info(device)[0] == free_before
         want = ops.argmax(logits)
         assert torch.equal(out, want)
         assert int(out[rows - 1]) == vocab - 1
@@ -57,3 +64,27 @@ def test_argmax_without_allocation_refuses_what_its_array_cannot_hold():
                                      torch.cuda.current_stream().cuda_stream)
     assert status != 0
     assert "scratch array holds" in lib.leone_last_error().decode()
+
+
+def test_argmax_without_allocation_can_be_recorded_into_a_graph():
+    """Under stream capture an allocation is an error: the entry point records, and every replay (with eager
+    work between) gives the argmax of what the input buffer then holds."""
+    from leone_amd import ops
+    lib = _library()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    rows, vocab = 6, 40_000
+    logits = torch.randn(rows, vocab, device=device)
+    out = torch.full((rows,), -7, dtype=torch.int32, device=device)
+    assert lib.leone_argmax_static(logits.data_ptr(), out.data_ptr(), rows, vocab, torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        status = lib.leone_argmax_static(logits.data_ptr(), out.data_ptr(), rows, vocab, torch.cuda.current_stream().cuda_stream)
+    assert status == 0, lib.leone_last_error().decode()
+    for replay in range(3):
+        logits.copy_(torch.randn(rows, vocab, device=device))
+        out.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ops.argmax(logits)), replay

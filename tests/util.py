@@ -27,6 +27,11 @@ TINY_M = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden
 TINY_D = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, hidden_size=100,
               num_attention_heads=2, num_key_value_heads=1, head_dim=16, intermediate_size=75, vocab_size=333,
               max_position_embeddings=128, rope_theta=20000.0, rms_norm_eps=2e-6, tie_word_embeddings=True)
+# One layer of the 8B widths at a small vocabulary: where the products' plans and the changes of kernel were chosen.
+REAL_8B_ONE_LAYER = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", rope_theta=1000000.0, rms_norm_eps=1e-6,
+                         tie_word_embeddings=False, max_position_embeddings=1024, vocab_size=8200, num_hidden_layers=1,
+                         hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                         intermediate_size=12288)
 TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "M": TINY_M, "D": TINY_D}
 
 
