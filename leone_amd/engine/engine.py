@@ -114,13 +114,29 @@ class PackedStep:
         return [packed[self.offsets[i]:self.offsets[i + 1]] for i in range(len(self.offsets) - 1)]
 
 
+DECODE_BUCKET_MIN = 256      # the smallest context range a decode step is recorded for
+
+
+def context_bucket(positions: int, max_context: int) -> int:
+    """The context range a decode step whose longest request holds ``positions`` tokens is recorded for: the
+    next power of two from DECODE_BUCKET_MIN on, at most the engine's ``max_context``."""
+    bucket = DECODE_BUCKET_MIN
+    while bucket < positions:
+        bucket *= 2
+    return min(bucket, max_context)
+
+
 class _DecodeGraph:
-    """A recorded decode step for one batch size: static metadata buffers, the graph, its logits.
+    """Recorded decode steps for one batch size: static metadata buffers and, for every context range
+    (``context_bucket``) that came up, a graph and its logits.
 
     The step's metadata (tokens, positions, state slots, block tables) lives in one device buffer
     that is refilled before each replay; the recorded kernels read everything through it, so one
-    recording serves every step of that batch size (the reference replays one decode graph per
-    context bucket with a device-resident position, crates/leone/src/runtime.rs:4991-5013).
+    recording serves every step of that batch size whose contexts lie in its range.  What a recording fixes
+    beside the batch size is what the parts derive from ``StepContext.max_position`` on the host (into how
+    many parts the attention kernel cuts a row's keys), hence one recording a range: a chat of 300 tokens on
+    an engine built for 40,960 is cut as for 512, not as for 40,960 (the reference replays one decode graph per
+    context bucket with a device-resident position, crates/leone/src/runtime.rs:3555-3615, 4991-5013).
     """
 
     def __init__(self, engine: "Engine", rows: int):
@@ -135,16 +151,20 @@ class _DecodeGraph:
         pieces = [self.dev[self.offsets[i]:self.offsets[i + 1]] for i in range(len(sizes))]
         self.tokens = pieces[0]
         self.rows = rows
-        self.context = StepContext(
-            rows=rows, dtype=engine.dtype, device=engine.device, positions=pieces[1], row_entry=pieces[2],
-            entries=[], entry_slots=pieces[3], want_rows=pieces[4],
-            block_tables={g: pieces[5 + len(tilings) + g].view(rows, widths[g]) for g in range(groups)},
-            max_position=engine.max_context - 1, decode_only=True)
-        self.graph: Optional[torch.cuda.CUDAGraph] = None
-        self.logits: Optional[torch.Tensor] = None
+        self._pieces, self._tables = pieces, {g: pieces[5 + len(tilings) + g].view(rows, widths[g]) for g in range(groups)}
+        self._engine_type = (engine.dtype, engine.device)
+        self.recordings: Dict[int, tuple] = {}        # context range -> (graph, its logits)
         self.copied = torch.cuda.Event()
 
-    def fill(self, engine: "Engine", entries: Sequence[StepEntry]) -> None:
+    def context(self, bucket: int) -> StepContext:
+        """The step as the parts see it when it is recorded for contexts of up to ``bucket`` positions."""
+        pieces = self._pieces
+        return StepContext(
+            rows=self.rows, dtype=self._engine_type[0], device=self._engine_type[1], positions=pieces[1],
+            row_entry=pieces[2], entries=[], entry_slots=pieces[3], want_rows=pieces[4],
+            block_tables=self._tables, max_position=bucket - 1, decode_only=True)
+
+    def fill(self, engine: "Engine", entries: Sequence[StepEntry]) -> PackedStep:
         self.copied.synchronize()                     # the last upload has left the pinned buffer
         packed = PackedStep(engine.cache, engine.vocab_size, entries, all_rows_wanted=True, host=self.host,
                             tilings=engine.tilings)
@@ -152,6 +172,7 @@ class _DecodeGraph:
             raise StepError("the step does not fit the recorded layout")
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
+        return packed
 
 
 class Engine:
@@ -187,6 +208,7 @@ class Engine:
         # Steps of single decoded tokens are recorded once per batch size and replayed.
         self.graphs = bool(graphs) and model.graph_safe
         self._decode_graphs: Dict[int, _DecodeGraph] = {}
+        self._graph_pool = torch.cuda.graph_pool_handle() if self.graphs else None
         self._staging: List[Optional[tuple]] = [None, None]
         self._staging_turn = 0
 
@@ -360,20 +382,25 @@ class Engine:
         state = self._decode_graphs.get(len(entries))
         if state is None:
             state = self._decode_graphs[len(entries)] = _DecodeGraph(self, len(entries))
-        state.fill(self, entries)
-        if state.graph is None:
-            # First step of this size: run it for real on the static buffers, then record the same
-            # calls for later steps.  Recording executes nothing, so the cache is written once.
-            caches = self.pools.views(state.context.block_tables)
+        packed = state.fill(self, entries)
+        bucket = context_bucket(packed.max_position + 1, self.max_context)
+        recording = state.recordings.get(bucket)
+        if recording is None:
+            # First step of this size and context range: run it for real on the static buffers, then record
+            # the same calls for later steps.  Recording executes nothing, so the cache is written once.
+            context = state.context(bucket)
+            caches = self.pools.views(context.block_tables)
             with ops.one_stream():
-                logits = self.model.forward(state.tokens, state.context, caches)
+                logits = self.model.forward(state.tokens, context, caches)
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph), ops.one_stream():
-                state.logits = self.model.forward(state.tokens, state.context, caches)
-            state.graph = graph
+            # one pool of memory for all recordings: they run one after the other on one stream, and what a
+            # replay leaves in its logits is copied out before the next replay begins
+            with torch.cuda.graph(graph, pool=self._graph_pool), ops.one_stream():
+                recorded_logits = self.model.forward(state.tokens, context, caches)
+            state.recordings[bucket] = (graph, recorded_logits)
         else:
-            state.graph.replay()
-            logits = state.logits
+            recording[0].replay()
+            logits = recording[1]
         wanted, rows_map = [], []
         for i, e in enumerate(entries):
             for w in e.want:

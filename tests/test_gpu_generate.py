@@ -97,9 +97,9 @@ def test_greedy_generation_at_the_widths_of_the_large_models(tmp_path):
 
     folder = make_model_dir(str(tmp_path / "m"), REAL_8B_ONE_LAYER, seed=73, dtype=torch.bfloat16)
     weights, config = read_weights(folder), read_config(folder)
-    prompts = [random_tokens(50 + i, n, config["vocab_size"]) for i, n in enumerate([100, 37, 150, 70])]
-    new = 20
-    runtime = Runtime.load(folder, "bfloat16", num_pages=7, page_tokens=64, max_requests=4, poison_freed=True,
+    prompts = [random_tokens(50 + i, n, config["vocab_size"]) for i, n in enumerate([120, 60, 180, 50])]
+    new = 20        # every request grows over a page's edge while it decodes: 7 pages at first, 11 at the end, 8 there are
+    runtime = Runtime.load(folder, "bfloat16", num_pages=8, page_tokens=64, max_requests=4, poison_freed=True,
                            policy=SchedulerPolicy(max_live_requests=4, prefill_chunk_tokens=64, max_step_tokens=96))
     results = runtime.generate_tokens(prompts, new, eos_token_id=None)
     runtime.engine.cache.check()

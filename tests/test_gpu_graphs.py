@@ -52,7 +52,7 @@ def test_replayed_decode_steps_equal_eager_ones(tmp_path, dtype_name):
                 e.release("b")
             both([("b", prompts["b"], [])])               # its pages and slot are handed out again
             feed["b"] = feed["b"][:26] + random_tokens(77, 14, vocab)
-    assert len(engines[0]._decode_graphs) == 2 and all(g.graph is not None for g in engines[0]._decode_graphs.values())
+    assert len(engines[0]._decode_graphs) == 2 and all(g.recordings for g in engines[0]._decode_graphs.values())
     for e in engines:
         e.cache.check()
 
@@ -134,4 +134,72 @@ def test_replayed_decode_steps_of_many_rows_agree_with_plain(tmp_path, n):
             for e in engines:
                 e.step([StepEntry("other", random_tokens(900 + step, 21, vocab), [20])])
                 e.release("other")
-    assert engines[0]._decode_graphs[n].graph is not None and not engines[1]._decode_graphs
+    assert engines[0]._decode_graphs[n].recordings and not engines[1]._decode_graphs
+
+
+def test_decode_steps_are_recorded_for_the_context_range_they_run_in(tmp_path):
+    """An engine built for 40,960 positions records a decode step at context 300 for the range up to 512, not
+    for its largest context: the attention kernel then cuts the keys as an engine built for 512 positions
+    does, and the step takes the same time (within 5 %); as requests grow into the next range a further
+    recording is made; every replay equals the eager engine and the plain implementation."""
+    from leone_amd import ops
+    from leone_amd.engine.engine import Engine, StepEntry, context_bucket
+    from leone_amd.runtime import load_model
+    from tests.plain import qwen3_plain
+    from tests.util import read_config, read_weights, tolerance
+
+    assert [context_bucket(n, 40960) for n in (1, 256, 257, 512, 513, 40000, 40960)] == [256, 256, 512, 512, 1024, 40960, 40960]
+    assert context_bucket(300, 384) == 384
+    config = dict(TINY["M"], max_position_embeddings=40960)
+    folder = make_model_dir(str(tmp_path / "m"), config, 8, torch.bfloat16)
+    model = load_model(folder, "bfloat16")
+    wide = Engine(model, num_pages=40, page_tokens=16, max_requests=2, graphs=True)
+    narrow = Engine(model, num_pages=40, page_tokens=16, max_requests=2, graphs=True, max_context=512)
+    eager = Engine(model, num_pages=40, page_tokens=16, max_requests=2, graphs=False)
+    assert wide.max_context == 40960 and narrow.max_context == 512
+    chosen = []
+    choose = ops.choose_splits
+    ops.choose_splits = lambda rows, kv_heads, group, max_context, units=256: chosen.append(max_context) or choose(rows, kv_heads, group, max_context, units)
+    try:
+        vocab = config["vocab_size"]
+        tokens = {"a": random_tokens(1, 300, vocab), "b": random_tokens(2, 236, vocab)}
+        expected = {r: qwen3_plain.forward(read_weights(folder), read_config(folder), t).numpy() for r, t in tokens.items()}
+        engines = (wide, narrow, eager)
+        for e in engines:
+            e.step([StepEntry("a", tokens["a"][:270], []), StepEntry("b", tokens["b"][:206], [])])
+        chosen.clear()
+        for i in range(30):
+            entries = [StepEntry("a", [tokens["a"][270 + i]], [0]), StepEntry("b", [tokens["b"][206 + i]], [0])]
+            outs = [e.step(entries).logits.cpu().numpy() for e in engines]
+            want = np.stack([expected["a"][270 + i], expected["b"][206 + i]])
+            for which, out in zip(("wide", "narrow", "eager"), outs):
+                assert np.abs(out - want).max() <= tolerance("bfloat16"), f"{which} step {i}"
+            assert np.array_equal(outs[0], outs[1]), f"step {i}: the two recordings cut the keys differently"
+        # contexts 271..300 and 207..236: one range (up to 512) for both engines, cut as for 512 positions
+        assert set(wide._decode_graphs[2].recordings) == {512} and set(narrow._decode_graphs[2].recordings) == {512}
+        assert 40960 not in chosen and 512 in chosen
+        # the same steps again, timed: replays of the wide engine's recording against the narrow one's
+        def replay_ms(engine):
+            entries = [StepEntry("a", [5], [0]), StepEntry("b", [7], [0])]
+            best = float("inf")
+            first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            for _ in range(5):
+                first.record()
+                for _ in range(20):
+                    engine._decode_graphs[2].recordings[512][0].replay()
+                last.record()
+                torch.cuda.synchronize()
+                best = min(best, first.elapsed_time(last) / 20)
+            return best
+        assert replay_ms(wide) <= 1.05 * replay_ms(narrow)
+        # growing past 512 positions makes a second recording, which still agrees with the eager engine
+        long_tokens = random_tokens(3, 520, vocab)
+        for e in (wide, eager):
+            e.release("a"), e.release("b")
+            e.step([StepEntry("c", long_tokens[:505], [])])
+        for i in range(505, 520):
+            outs = [e.step([StepEntry("c", [long_tokens[i]], [0])]).logits.cpu().numpy() for e in (wide, eager)]
+            assert np.abs(outs[0] - outs[1]).max() < 2e-2, i
+        assert set(wide._decode_graphs[1].recordings) == {512, 1024}
+    finally:
+        ops.choose_splits = choose
