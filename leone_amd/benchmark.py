@@ -151,6 +151,44 @@ def time_decode(engine, batch: int, start_context: int, steps: int, warmup: int,
     return (elapsed, mean_context, profiled) if profile_steps else (elapsed, mean_context)
 
 
+def time_generate(engine, batch: int, prompt_tokens: int, new_tokens: int, seed: int = 3) -> dict:
+    """The stated workload through the generation loop itself, as the reference's bench runs it (prefill the
+    prompt, sample, then time decoding: crates/leone/src/runtime.rs:2006-2050): ``batch`` prompts of
+    ``prompt_tokens`` random tokens are submitted to a ``Generator`` (scheduler, real prefill a whole prompt a
+    step, pages taken as tokens arrive, greedy choice on the device, tokens reported back), ``new_tokens``
+    tokens each.  Timed, on the wall clock around ``Generator.step`` (planning, the step, sampling, the copy of
+    the tokens, completion), are the steps that hold one decoded token of every request and nothing else: the
+    same work as the bare step loop of ``time_decode`` plus everything the loop leaves out."""
+    import torch
+    from .engine.generate import Generator
+    from .engine.scheduler import SchedulerPolicy
+    from .sampling.sampler import SamplingParams
+    gen = torch.Generator().manual_seed(seed)
+    prompts = [torch.randint(0, engine.vocab_size, (prompt_tokens,), generator=gen).tolist() for _ in range(batch)]
+    # a whole prompt beside the tokens the earlier requests decode meanwhile; a multiple of 256 (see SchedulerPolicy)
+    policy = SchedulerPolicy(max_live_requests=batch, prefill_chunk_tokens=prompt_tokens,
+                             max_step_tokens=prompt_tokens + 256 * -(-batch // 256))
+    generator = Generator(engine, policy)
+    for i, prompt in enumerate(prompts):
+        generator.submit(("generate", i), prompt, new_tokens, SamplingParams(), None)
+    seconds, tokens, steps, total_started = 0.0, 0, 0, time.perf_counter()
+    while generator.scheduler.has_work():
+        before = (generator.stats.decode_tokens, generator.stats.prefill_tokens)
+        started = time.perf_counter()
+        generator.step()
+        elapsed = time.perf_counter() - started
+        if generator.stats.decode_tokens - before[0] == batch and generator.stats.prefill_tokens == before[1]:
+            steps += 1
+            if steps > 4:                         # the first steps of a size record their graph
+                seconds += elapsed
+                tokens += batch
+    torch.cuda.synchronize()
+    engine.cache.check()
+    assert not engine.cache.live_requests() and generator.stats.emitted_tokens == batch * new_tokens
+    return {"tok_s": tokens / seconds if seconds else 0.0, "timed_steps": steps - 4,
+            "prefill_tok_s": generator.stats.prefill_rate, "wall_s": time.perf_counter() - total_started}
+
+
 def kernel_table(profiled, model, batch: int, context: float) -> dict:
     """Per operation of a decode step: microseconds a step and, where the operation streams something, the
     GB/s it reached (products: their weight bytes; attention: the cache of the live requests)."""
@@ -168,7 +206,9 @@ def kernel_table(profiled, model, batch: int, context: float) -> dict:
     return table
 
 
-def time_prefill(engine, tokens: int, repeats: int = 3, seed: int = 2):
+def time_prefill(engine, tokens: int, repeats: int = 3, seed: int = 2, portion: Optional[int] = None):
+    """Seconds of the best of ``repeats`` runs of a prompt of ``tokens`` tokens from position 0, in one step or
+    (``portion``) in portions of that many tokens."""
     import torch
     from .engine.engine import StepEntry
     gen = torch.Generator().manual_seed(seed)
@@ -177,7 +217,9 @@ def time_prefill(engine, tokens: int, repeats: int = 3, seed: int = 2):
     for i in range(repeats + 1):
         torch.cuda.synchronize()
         started = time.perf_counter()
-        out = engine.step([StepEntry("prefill", prompt, [tokens - 1])])
+        for at in range(0, tokens, portion or tokens):
+            part = prompt[at:at + (portion or tokens)]
+            out = engine.step([StepEntry("prefill", part, [len(part) - 1] if at + len(part) == tokens else [])])
         out.logits.sum().item()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - started
@@ -287,6 +329,11 @@ def main(argv: Optional[List[str]] = None) -> int:
                         help="layer sizes of which Qwen3 model (the headline figure is 8b)")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    parser.add_argument("--no-generate", action="store_true",
+                        help="skip the stated workload through the generation loop (points generate_b*)")
+    parser.add_argument("--no-long", action="store_true",
+                        help="skip the points of a second engine built for the model's whole context (context 32,768, "
+                             "context 512 of 40,960, a prompt of 8,192 tokens)")
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument("--no-kernels", action="store_true", help="skip the per-operation table of the decode step")
     parser.add_argument("--no-peaks", action="store_true", help="skip the measurement of this GPU's own peaks")
@@ -388,6 +435,28 @@ def main(argv: Optional[List[str]] = None) -> int:
             break
         e, _ = time_decode(engine, batch, STATED_PROMPT, STATED_NEW - 8, 8)
         points[f"decode_b{batch}_prompt{STATED_PROMPT}_new{STATED_NEW}"] = round(batch * (STATED_NEW - 8) / e, 2)
+    # The same workload through the generation loop: scheduler, real prefill, page allocation, sampler.
+    if not (args.no_points or args.no_generate) and STATED_PROMPT + STATED_NEW + 1 <= args.context:
+        for batch in sorted({1, args.batch, 64}):
+            run = time_generate(engine, batch, STATED_PROMPT, STATED_NEW)
+            points[f"generate_b{batch}"] = round(run["tok_s"], 2)
+    # A second engine, built for the model's whole context: decoding at context 32,768, decoding a short
+    # context on an engine that could hold 40,960 positions (recordings are per context range), a long prompt.
+    if not (args.no_points or args.no_long) and config.max_position_embeddings >= 32768 + 64:
+        del engine
+        torch.cuda.empty_cache()
+        long_context, long_batch = 32768, 8
+        engine = Engine(model, num_pages=long_batch * (long_context // page_tokens + 1), page_tokens=page_tokens,
+                        max_requests=long_batch, streamed_weights=False if args.no_streamed_weights else None)
+        assert engine.max_context == config.max_position_embeddings
+        for batch in (1, long_batch):
+            e, _ = time_decode(engine, batch, long_context - 40, 24, 8)
+            points[f"decode_b{batch}_context{long_context}"] = round(batch * 24 / e, 2)
+            e, _ = time_decode(engine, batch, 512 - 72, 64, 8)
+            points[f"decode_b{batch}_context512_of_{engine.max_context}"] = round(batch * 64 / e, 2)
+        if not args.no_prefill:
+            seconds = time_prefill(engine, 8192, repeats=2)
+            points["prefill_8192"] = round(8192 / seconds, 1)
     if points:
         record["points"] = points
     print(json.dumps(record), flush=True)

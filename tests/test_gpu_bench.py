@@ -19,7 +19,7 @@ def test_the_record_of_a_short_run(capsys):
     """Two layers of the headline shape, a few steps: one line of JSON with the decode figure, the prompt's, the
     roofline's and the points', and a flat description of every size."""
     from leone_amd import benchmark
-    assert benchmark.main(["--layers", "2", "--steps", "4", "--warmup", "1", "--batch", "8", "--context", "1024",
+    assert benchmark.main(["--layers", "2", "--steps", "4", "--warmup", "1", "--batch", "8", "--context", "2560",
                            "--no-peaks"]) == 0
     lines = [line for line in capsys.readouterr().out.splitlines() if line.strip()]
     assert len(lines) == 1
@@ -41,6 +41,11 @@ def test_the_record_of_a_short_run(capsys):
     assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-3
     assert abs(roofline["achieved"] - record["bytes"]["a_step"] / record["ms_per_step"] / 1e6) / roofline["achieved"] < 1e-2
     assert {"decode_b1", "decode_b64"} <= set(record["points"]) and all(v > 0 for v in record["points"].values())
+    # the stated workload as a bare step loop and through the generation loop, and the second engine's points
+    for batch in (1, 8, 64):
+        assert {f"decode_b{batch}_prompt2048_new256", f"generate_b{batch}"} <= set(record["points"])
+    assert {"decode_b1_context32768", "decode_b8_context32768", "decode_b1_context512_of_40960",
+            "decode_b8_context512_of_40960", "prefill_8192"} <= set(record["points"])
 
 
 @pytest.mark.parametrize("name", ["mixed14b", "pressure32b"])
