@@ -69,6 +69,14 @@ class DevicePools:
         for slot, storage in self.state.items():
             self.needs[slot].zero(storage, slot_index)
 
+    def copy_state(self, from_slot: int, to_slot: int) -> None:
+        """Gives request slot ``to_slot`` a copy of what ``from_slot`` holds (a request that takes over another's
+        prefix at the other's latest position), through the needs' own ``snapshot`` and ``restore``."""
+        source = torch.tensor([from_slot], dtype=torch.long, device=self.device)
+        target = torch.tensor([to_slot], dtype=torch.long, device=self.device)
+        for slot, storage in self.state.items():
+            self.needs[slot].restore(storage, target, self.needs[slot].snapshot(storage, source))
+
     def snapshot_state(self, slot_indices: List[int]):
         """What the per-request storage of these request slots holds, to be put back by ``restore_state``."""
         if not self.state:

@@ -92,12 +92,27 @@ __device__ inline void load_projection8(const FromProjection& f, long row_width,
         }
         return;
     }
+    // The planes are asked for four at a time before any is added (a plane beyond the last is the last one again
+    // and is not added): one trip to memory for up to five planes instead of one a plane.  Added in their order.
     const float* src = static_cast<const float*>(f.qkv) + row * row_width + at;
+    const float4 a0 = *reinterpret_cast<const float4*>(src), b0 = *reinterpret_cast<const float4*>(src + 4);
+    out[0] = a0.x; out[1] = a0.y; out[2] = a0.z; out[3] = a0.w;
+    out[4] = b0.x; out[5] = b0.y; out[6] = b0.z; out[7] = b0.w;
+    for (int p0 = 1; p0 < f.planes; p0 += 4) {
+        float4 lo[4], hi[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) out[i] = src[i];
-    for (int p = 1; p < f.planes; ++p)
+        for (int q = 0; q < 4; ++q) {
+            const float* from = src + (p0 + q < f.planes ? p0 + q : f.planes - 1) * f.plane;
+            lo[q] = *reinterpret_cast<const float4*>(from);
+            hi[q] = *reinterpret_cast<const float4*>(from + 4);
+        }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) out[i] += src[p * f.plane + i];
+        for (int q = 0; q < 4; ++q)
+            if (p0 + q < f.planes) {
+                out[0] += lo[q].x; out[1] += lo[q].y; out[2] += lo[q].z; out[3] += lo[q].w;
+                out[4] += hi[q].x; out[5] += hi[q].y; out[6] += hi[q].z; out[7] += hi[q].w;
+            }
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i) out[i] = to_float(from_float<bf16_t>(out[i]));
 }
@@ -164,7 +179,18 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                     const bool mine = lane < kHalfRuns;
                     float a[8], b[8];
                     float ss = 0.f;
+                    // gains and angles are asked for together with the projection, not after the sum of squares
+                    float ga[8], gb[8], cs[8], sn[8];
                     if (mine) {
+                        if (from.k_gain.ptr) {
+                            load_any8(from.k_gain, 8 * lane, ga);
+                            load_any8(from.k_gain, kD / 2 + 8 * lane, gb);
+                        }
+                        if (from.cos_table != nullptr) {
+                            const int tpos = pos < from.table_positions ? pos : from.table_positions - 1;
+                            load_any8(AnyVec{from.cos_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 8 * lane, cs);
+                            load_any8(AnyVec{from.sin_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 8 * lane, sn);
+                        }
                         load_projection8(from, width, row, static_cast<long>(q_heads + kvh) * kD + 8 * lane, a);
                         load_projection8(from, width, row, static_cast<long>(q_heads + kvh) * kD + kD / 2 + 8 * lane, b);
 #pragma unroll
@@ -177,9 +203,6 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                     if (mine) {
                         if (from.k_gain.ptr) {
                             const float inv = 1.0f / sqrtf(ss / static_cast<float>(kD) + from.eps);
-                            float ga[8], gb[8];
-                            load_any8(from.k_gain, 8 * lane, ga);
-                            load_any8(from.k_gain, kD / 2 + 8 * lane, gb);
 #pragma unroll
                             for (int i = 0; i < 8; ++i) {
                                 a[i] = (a[i] * ga[i]) * inv;
@@ -187,10 +210,6 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                             }
                         }
                         if (from.cos_table != nullptr) {
-                            const int tpos = pos < from.table_positions ? pos : from.table_positions - 1;
-                            float cs[8], sn[8];
-                            load_any8(AnyVec{from.cos_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 8 * lane, cs);
-                            load_any8(AnyVec{from.sin_table, kF32}, static_cast<long>(tpos) * (kD / 2) + 8 * lane, sn);
 #pragma unroll
                             for (int i = 0; i < 8; ++i) {
                                 const float ru = a[i] * cs[i] - b[i] * sn[i];

@@ -3,9 +3,13 @@
 // own multi-row matrix-vector kernels with folded epilogues (crates/leone/src/runtime.rs:7865-7906,
 // crates/leone-cuda/cuda/ie_cuda.cu:1932, 2011, 6208): W is read from memory exactly once, X is small.
 //
-// A workgroup of 4, 6 or 8 waves owns 16 rows of W a wave and a range of K; the ranges of K (blockIdx.y,
+// A workgroup owns 4, 6 or 8 tiles of 16 rows of W and a range of K; the ranges of K (blockIdx.y,
 // `splits` of them) exist so that matrices with few rows still give every compute unit a workgroup (the
 // kernel is fastest with exactly one workgroup a compute unit: the caller picks waves and splits for that).
+// A tile of W belongs to one wave, or (more than 64 rows of X) to two waves that share out the 32-element
+// units of every chunk between them and add their sums up through shared memory at the end, in a fixed order:
+// the workgroup then has two waves a SIMD instead of one, so that one wave's wait for shared memory, for a
+// barrier or for its weights is the other's time on the matrix cores, and twice the weights are on their way.
 // What W costs in memory traffic X must not cost again in cache traffic: every wave needs all of X, so X
 // goes through shared memory, one chunk of K at a time (256 elements, 128 for more than 64 rows), copied
 // there once per workgroup with 16-byte loads that run along the rows, while the waves work on the chunk
@@ -50,28 +54,33 @@ struct RowsArgs {
 __device__ inline uint4 rld(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ inline uint4 wld(const bf16_t* p) { return load_streamed16(p); }   // weights: read once
 
-// kMT: tiles of 16 rows of X; kWaves: waves of a workgroup, each with one tile of 16 rows of W; kSteps: steps
-// of 64 elements a chunk.
-template <int kMT, int kWaves, int kSteps, int kDepth, int kOut, typename TOut, bool kTiled>
-__global__ void __launch_bounds__(kWaves * kWave)
+// kMT: tiles of 16 rows of X; kWaves: tiles of 16 rows of W a workgroup; kWays: waves that share a tile of W
+// (each takes kUnits / kWays units of every chunk); kSteps: steps of 64 elements a chunk; kDepth: chunks the
+// weights are asked for ahead.
+template <int kMT, int kWaves, int kWays, int kSteps, int kDepth, int kOut, typename TOut, bool kTiled>
+__global__ void __launch_bounds__(kWaves * kWays * kWave)
 gemm_rows_kernel(RowsArgs a) {
     constexpr int kChunk = 64 * kSteps;              // elements of K a chunk
     constexpr int kRuns = kChunk / 8;                // 16-byte runs of a row of the chunk
     constexpr int kXRows = 16 * kMT;
-    constexpr int kThreads = kWaves * kWave;
+    constexpr int kThreads = kWaves * kWays * kWave;
     constexpr int kCopies = (kXRows * kRuns + kThreads - 1) / kThreads;   // runs of X a thread copies per chunk
     constexpr bool kEven = kXRows * kRuns % kThreads == 0;
-    constexpr int kUnits = 2 * kSteps;               // matrix instructions per tile of X and chunk: 32 elements each
-    extern __shared__ uint4 lds[];                   // two chunks of X: [2][kXRows][kRuns]
+    constexpr int kChunkUnits = 2 * kSteps;          // 32-element units of a chunk
+    static_assert(kChunkUnits % kWays == 0, "the units of a chunk must share out evenly");
+    constexpr int kUnits = kChunkUnits / kWays;      // units of a chunk this wave takes: matrix instructions per tile of X
+    extern __shared__ uint4 lds[];                   // two chunks of X: [2][kXRows][kRuns]; at the end the waves' sums
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int lane = threadIdx.x % kWave;
     const int tid = threadIdx.x;
     const int c = lane & 15, g = lane >> 4;
     const int m = a.m, n = a.n, k = a.k;
+    const int way = wave / kWaves;                   // which share of every chunk's units
+    const int unit0 = way * kUnits;                  // its first unit in a chunk
 
     // This wave's weight rows; rows past the end are clamped and their results never stored.
-    const long tile = static_cast<long>(blockIdx.x) * kWaves + wave;
+    const long tile = static_cast<long>(blockIdx.x) * kWaves + wave % kWaves;
     const long wr = 16 * tile + c;
     const bf16_t* wrow = a.w + (wr < n ? wr : n - 1) * k;
     // Tiled weights: the 16 bytes of lane L for half h of step S of a tile lie at ((S * 2 + h) * 64 + L) * 16 in
@@ -111,7 +120,8 @@ gemm_rows_kernel(RowsArgs a) {
             xn[i] = rld(xsrc[i] + (at + 8 <= k ? at : k - 8));
         }
     };
-    auto w_at = [&](int ch, int u) {
+    auto w_at = [&](int ch, int mine) {
+        const int u = unit0 + mine;
         if constexpr (kTiled) {
             const int step = ch * kSteps + (u >> 1);
             return load_streamed16(wtile + static_cast<long>(step < all_steps ? step : all_steps - 1) * 1024 + 512 * (u & 1));
@@ -119,6 +129,14 @@ gemm_rows_kernel(RowsArgs a) {
             const int at = ch * kChunk + 16 * g + 64 * (u >> 1) + 8 * (u & 1);
             return rld(wrow + (at + 8 <= k ? at : k - 8));
         }
+    };
+    // Weights beyond the end of K count as zero themselves (not only through the zeros of X: a weight that is
+    // not finite would turn 0 into NaN).  The load is made all the same, from the row's end, and cleared when
+    // it is used: a select right behind the load would wait for it.
+    auto w_inside = [&](int ch, int mine) {
+        const int u = unit0 + mine;
+        if constexpr (kTiled) return ch * kSteps + (u >> 1) < all_steps;
+        else return ch * kChunk + 16 * g + 64 * (u >> 1) + 8 * (u & 1) + 8 <= k;
     };
     auto deposit = [&](uint4* to, const uint4 (&xn)[kCopies], int ch) {
         const int k0 = ch * kChunk;
@@ -134,9 +152,10 @@ gemm_rows_kernel(RowsArgs a) {
     // instructions ahead, so that their way out of shared memory is covered by the group before; a weight
     // register that has been used is filled again at once, from the next chunk.
     uint4 wreg[kDepth][kUnits];
-    auto compute = [&](const uint4* from, uint4 (&wreg)[kUnits], int next) {
+    auto compute = [&](const uint4* from, uint4 (&wreg)[kUnits], int present, int next) {
         bf16x8 xb[2][kMT];
-        auto read_x = [&](int u, bf16x8 (&to)[kMT]) {
+        auto read_x = [&](int mine, bf16x8 (&to)[kMT]) {
+            const int u = unit0 + mine;
             const int run = (4 * u + 2 * g - 3 * (u & 1)) ^ c;          // 8 (u / 2) + 2 g + u % 2
 #pragma unroll
             for (int t = 0; t < kMT; ++t) to[t] = __builtin_bit_cast(bf16x8, from[(16 * t + c) * kRuns + run]);
@@ -146,7 +165,10 @@ gemm_rows_kernel(RowsArgs a) {
         for (int u = 0; u < kUnits; ++u) {
             if (u + 1 < kUnits) read_x(u + 1, xb[(u + 1) & 1]);
             __builtin_amdgcn_sched_barrier(0);       // the reads stay ahead of the instructions they are not for
-            const bf16x8 wa = __builtin_bit_cast(bf16x8, wreg[u]);
+            const bool inside = w_inside(present, u);
+            const uint4 held = wreg[u];
+            const bf16x8 wa = __builtin_bit_cast(bf16x8, uint4{inside ? held.x : 0u, inside ? held.y : 0u,
+                                                               inside ? held.z : 0u, inside ? held.w : 0u});
 #pragma unroll
             for (int t = 0; t < kMT; ++t)
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xb[u & 1][t], acc[t], 0, 0, 0);
@@ -183,12 +205,32 @@ gemm_rows_kernel(RowsArgs a) {
             if (d > 0 && i + d >= count) break;
             const int next = chunk_or_last(i + d + 1);
             fetch_x(next, xn);
-            compute(lds + cur * kHalf, wreg[d], chunk_or_last(i + d + kDepth));
+            compute(lds + cur * kHalf, wreg[d], chunk_at(i + d), chunk_or_last(i + d + kDepth));
             cur ^= 1;
             __builtin_amdgcn_sched_barrier(0);
             deposit(lds + cur * kHalf, xn, next);
             __syncthreads();
         }
+    }
+
+    // The waves that shared a tile of W add up: every wave but the tile's first leaves its sums in shared
+    // memory (the chunks of X are done with), the first adds them in the order of the shares.
+    if constexpr (kWays > 1) {
+        floatx4* sums = reinterpret_cast<floatx4*>(lds);   // [kWays - 1][kWaves][kMT][64]
+        if (way > 0) {
+#pragma unroll
+            for (int t = 0; t < kMT; ++t) sums[(((way - 1) * kWaves + wave % kWaves) * kMT + t) * kWave + lane] = acc[t];
+        }
+        __syncthreads();
+        if (way > 0) return;
+#pragma unroll
+        for (int other = 1; other < kWays; ++other)
+#pragma unroll
+            for (int t = 0; t < kMT; ++t) {
+                const floatx4 part = sums[(((other - 1) * kWaves + wave) * kMT + t) * kWave + lane];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[t][r] += part[r];
+            }
     }
 
     // Lane (c, g) holds, for tile t, Y[16t + c][16 tile + 4g .. + 3].
@@ -237,13 +279,16 @@ gemm_rows_kernel(RowsArgs a) {
     }
 }
 
-template <int kMT, int kWaves, int kDepth, int kOut, typename TOut, bool kTiled>
+template <int kMT, int kWaves, int kWays, int kOut, typename TOut, bool kTiled>
 static int launch_rows_laid(const RowsArgs& a, int splits, hipStream_t stream) {
     constexpr int kSteps = kMT <= 4 ? 4 : 2;
-    const size_t shared = 2 * static_cast<size_t>(16 * kMT) * (64 * kSteps / 8) * sizeof(uint4);
+    constexpr int kDepth = kWays;                      // a wave keeps a whole chunk's worth of its weights on the way
+    const size_t chunks_of_x = 2 * static_cast<size_t>(16 * kMT) * (64 * kSteps / 8) * sizeof(uint4);
+    const size_t sums = static_cast<size_t>(kWays - 1) * kWaves * kMT * kWave * sizeof(floatx4);
+    const size_t shared = chunks_of_x > sums ? chunks_of_x : sums;
     static size_t allowed = 48 * 1024;                 // what a kernel may use without asking
     if (shared > allowed) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_rows_kernel<kMT, kWaves, kSteps, kDepth, kOut, TOut, kTiled>),
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_rows_kernel<kMT, kWaves, kWays, kSteps, kDepth, kOut, TOut, kTiled>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(shared));
         if (e != hipSuccess) {
             set_error("gemm_rows: %zu bytes of shared memory were refused: %s", shared, hipGetErrorString(e));
@@ -252,36 +297,56 @@ static int launch_rows_laid(const RowsArgs& a, int splits, hipStream_t stream) {
         allowed = shared;
     }
     const int groups = ceil_div(a.n, 16 * kWaves);
-    gemm_rows_kernel<kMT, kWaves, kSteps, kDepth, kOut, TOut, kTiled><<<dim3(groups, splits), kWaves * kWave, shared, stream>>>(a);
+    gemm_rows_kernel<kMT, kWaves, kWays, kSteps, kDepth, kOut, TOut, kTiled><<<dim3(groups, splits), kWaves * kWays * kWave, shared, stream>>>(a);
     return 0;
 }
 
-template <int kMT, int kWaves, int kDepth, int kOut, typename TOut>
+template <int kMT, int kWaves, int kWays, int kOut, typename TOut>
 static int launch_rows(const RowsArgs& a, int splits, bool tiled, hipStream_t stream) {
-    return tiled ? launch_rows_laid<kMT, kWaves, kDepth, kOut, TOut, true>(a, splits, stream)
-                 : launch_rows_laid<kMT, kWaves, kDepth, kOut, TOut, false>(a, splits, stream);
+    return tiled ? launch_rows_laid<kMT, kWaves, kWays, kOut, TOut, true>(a, splits, stream)
+                 : launch_rows_laid<kMT, kWaves, kWays, kOut, TOut, false>(a, splits, stream);
 }
 
-template <int kMT, int kWaves, int kDepth>
+template <int kMT, int kWaves, int kWays>
 static int launch_rows_out(const RowsArgs& a, int out_mode, int out_dtype, int splits, bool tiled, hipStream_t stream) {
     switch (out_mode) {
         case kRowsStore:
-            return out_dtype == kF32 ? launch_rows<kMT, kWaves, kDepth, kRowsStore, float>(a, splits, tiled, stream)
-                                     : launch_rows<kMT, kWaves, kDepth, kRowsStore, bf16_t>(a, splits, tiled, stream);
-        case kRowsResidual: return launch_rows<kMT, kWaves, kDepth, kRowsResidual, float>(a, splits, tiled, stream);
-        case kRowsGated: return launch_rows<kMT, kWaves, kDepth, kRowsGated, bf16_t>(a, splits, tiled, stream);
-        default: return launch_rows<kMT, kWaves, kDepth, kRowsPlanes, float>(a, splits, tiled, stream);
+            return out_dtype == kF32 ? launch_rows<kMT, kWaves, kWays, kRowsStore, float>(a, splits, tiled, stream)
+                                     : launch_rows<kMT, kWaves, kWays, kRowsStore, bf16_t>(a, splits, tiled, stream);
+        case kRowsResidual: return launch_rows<kMT, kWaves, kWays, kRowsResidual, float>(a, splits, tiled, stream);
+        case kRowsGated: return launch_rows<kMT, kWaves, kWays, kRowsGated, bf16_t>(a, splits, tiled, stream);
+        default: return launch_rows<kMT, kWaves, kWays, kRowsPlanes, float>(a, splits, tiled, stream);
+    }
+}
+
+// Which (tiles, shares) a workgroup may have.  Two waves a tile are built where they were measured to gain:
+// more than 64 rows of X (a wave then has twice the matrix instructions and reads of shared memory a unit of
+// K, and a second wave on its SIMD fills its waits: 6,144 x 4,096 at 128 rows 21.3 against 23.9 us, 4,096 x
+// 12,288 31.9 against 33.1); up to 64 rows they were level or 1 us slower, and four waves a tile no better.
+constexpr bool rows_shape_built(int mt, int waves, int ways) {
+    return ways == 1 || (ways == 2 && mt >= 6 && waves <= 6);
+}
+
+template <int kMT, int kWaves, int kWays>
+static int launch_rows_if_built(const RowsArgs& a, int out_mode, int out_dtype, int splits, bool tiled, hipStream_t stream) {
+    if constexpr (rows_shape_built(kMT, kWaves, kWays)) {
+        return launch_rows_out<kMT, kWaves, kWays>(a, out_mode, out_dtype, splits, tiled, stream);
+    } else {
+        set_error("gemm_rows: %d tiles of W shared by %d waves each are not built for %d rows", kWaves, kWays, a.m);
+        return 1;
     }
 }
 
 template <int kMT>
-static int launch_rows_waves(const RowsArgs& a, int out_mode, int out_dtype, int splits, int waves, bool tiled,
+static int launch_rows_waves(const RowsArgs& a, int out_mode, int out_dtype, int splits, int waves, int ways, bool tiled,
                              hipStream_t stream) {
-    switch (waves) {
-        case 4: return launch_rows_out<kMT, 4, 1>(a, out_mode, out_dtype, splits, tiled, stream);
-        case 6: return launch_rows_out<kMT, 6, 1>(a, out_mode, out_dtype, splits, tiled, stream);
-        default: return launch_rows_out<kMT, 8, 1>(a, out_mode, out_dtype, splits, tiled, stream);
-    }
+#define LEONE_ROWS_SHAPE(W, S) \
+    if (waves == W && ways == S) return launch_rows_if_built<kMT, W, S>(a, out_mode, out_dtype, splits, tiled, stream);
+    LEONE_ROWS_SHAPE(4, 1) LEONE_ROWS_SHAPE(6, 1) LEONE_ROWS_SHAPE(8, 1)
+    LEONE_ROWS_SHAPE(4, 2) LEONE_ROWS_SHAPE(6, 2)
+#undef LEONE_ROWS_SHAPE
+    set_error("gemm_rows: %d tiles of W a workgroup, %d waves a tile", waves, ways);
+    return 1;
 }
 
 }  // namespace leone
@@ -297,9 +362,16 @@ extern "C" int leone_gemm_rows_chunk(int m) { return m <= 64 ? 256 : 128; }
 // y bfloat16 [m,n/2] = silu(gate) * up; 3: y float32 [splits][m,n], `plane` elements apart, the product over
 // the s-th range of k in plane s (every plane is written whole).  splits must be 1 unless out_mode is 3; the
 // ranges are whole chunks of k and none may be empty.  waves (4, 6 or 8): 16 * waves rows of w a
-// workgroup, a tuning choice; the result does not depend on it beyond the order of the sum over k.
+// workgroup; ways (1 or 2, what leone_gemm_rows_shape_built allows): waves that share each of those tiles;
+// tuning choices both: the result does not depend on them beyond the order of the sum over k.
+extern "C" int leone_gemm_rows_shape_built(int m, int waves, int ways) {
+    const int tiles = ceil_div(m, 16);
+    const int mt = tiles <= 4 ? tiles : tiles <= 6 ? 6 : 8;
+    return (waves == 4 || waves == 6 || waves == 8) && (ways == 1 || ways == 2) && rows_shape_built(mt, waves, ways);
+}
+
 extern "C" int leone_gemm_rows_bf16(const void* x, const void* w, int w_tiled, void* y, int out_mode, int out_dtype,
-                                    int m, int n, int k, int splits, long plane, int waves, hipStream_t stream) {
+                                    int m, int n, int k, int splits, long plane, int waves, int ways, hipStream_t stream) {
     LEONE_REQUIRE(x && w && y, "gemm_rows: null pointer");
     LEONE_REQUIRE(!w_tiled || (k % 64 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0),
                   "gemm_rows: tiled weights need K %d to be a multiple of 64", k);
@@ -308,7 +380,9 @@ extern "C" int leone_gemm_rows_bf16(const void* x, const void* w, int w_tiled, v
     LEONE_REQUIRE(out_mode >= kRowsStore && out_mode <= kRowsPlanes, "gemm_rows: unknown output mode %d", out_mode);
     LEONE_REQUIRE(out_mode != kRowsGated || n % 16 == 0, "gemm_rows: gated output needs N %d to be a multiple of 16", n);
     LEONE_REQUIRE(out_mode != kRowsStore || out_dtype == kF32 || out_dtype == kBF16, "gemm_rows: unknown output type");
-    LEONE_REQUIRE(waves == 4 || waves == 6 || waves == 8, "gemm_rows: %d waves a workgroup", waves);
+    LEONE_REQUIRE(waves == 4 || waves == 6 || waves == 8, "gemm_rows: %d tiles of W a workgroup", waves);
+    LEONE_REQUIRE(leone_gemm_rows_shape_built(m, waves, ways), "gemm_rows: %d waves a tile of W are not built for %d tiles and %d rows",
+                  ways, waves, m);
     const int chunk = leone_gemm_rows_chunk(m);
     const int chunks = ceil_div(k, chunk);
     LEONE_REQUIRE(splits >= 1 && splits <= chunks && splits <= 65535, "gemm_rows: %d ranges of K for %d chunks", splits, chunks);
@@ -319,7 +393,7 @@ extern "C" int leone_gemm_rows_bf16(const void* x, const void* w, int w_tiled, v
     RowsArgs a{static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), y, plane, m, n, k, per};
     int status = 0;
 #define LEONE_ROWS_CASE(MT) \
-    case MT: status = launch_rows_waves<MT>(a, out_mode, out_dtype, splits, waves, w_tiled != 0, stream); break;
+    case MT: status = launch_rows_waves<MT>(a, out_mode, out_dtype, splits, waves, ways, w_tiled != 0, stream); break;
     const int tiles = ceil_div(m, 16);
     switch (tiles <= 4 ? tiles : tiles <= 6 ? 6 : 8) {
         LEONE_ROWS_CASE(1) LEONE_ROWS_CASE(2) LEONE_ROWS_CASE(3) LEONE_ROWS_CASE(4) LEONE_ROWS_CASE(6) LEONE_ROWS_CASE(8)

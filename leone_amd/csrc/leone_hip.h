@@ -121,12 +121,14 @@ int leone_gemm_fused_bf16(const void* x, int in_mode, const int* rows, const voi
 // 2: W interleaves 8 gate rows with their 8 up rows, y bfloat16 [M,N/2] = silu(gate) * up; 3: y float32
 // [splits][M,N], planes `plane` elements apart, plane s holding the product over the s-th range of K (whole
 // chunks of leone_gemm_rows_chunk(M) elements, ceil(chunks / splits) a range, no range empty).  splits > 1 only
-// with out_mode 3.  waves (4, 6 or 8; 16 rows of W each) is a tuning choice: it changes the result only through
-// the order of the sum over K.
+// with out_mode 3.  waves (4, 6 or 8 tiles of 16 rows of W a workgroup) and ways (1 or 2 waves that share a
+// tile's units of K; leone_gemm_rows_shape_built says which combinations exist for M rows) are tuning choices:
+// they change the result only through the order of the sum over K.
 int leone_gemm_rows_max_rows();
 int leone_gemm_rows_chunk(int m);
+int leone_gemm_rows_shape_built(int m, int waves, int ways);
 int leone_gemm_rows_bf16(const void* x, const void* w, int w_tiled, void* y, int out_mode, int out_dtype, int m, int n, int k,
-                         int splits, long plane, int waves, hipStream_t stream);
+                         int splits, long plane, int waves, int ways, hipStream_t stream);
 
 // The vendor library's product for more rows than the kernels above take, Y[M,N] = X[M,K] . W[N,K]^T (or Y +=
 // with `accumulate`, Y float32), X and W bfloat16, Y of out_dtype, float accumulation, with the library's

@@ -111,21 +111,47 @@ add_rmsnorm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, int 
     TY* yr = y + static_cast<long>(out_row) * hidden;
     float v[kChunks][4], gv[kChunks][4];
     float ss = 0.f;
+    // Everything a thread needs is asked for before anything is added: the row, the gains, and the planes four
+    // at a time (a plane beyond the last is the last one again and is not added), so that the trips to memory
+    // overlap instead of following one another plane by plane.  The planes are added in their order.
 #pragma unroll
     for (int i = 0; i < kChunks; ++i) {
         const int c = 4 * (threadIdx.x + i * kThreads);
         if (c < hidden) {
             load4(xr + c, v[i]);
             load4(gain + c, gv[i]);
-            if (dr) {
-                for (int p = 0; p < planes; ++p) {
-                    float d[4];
-                    load4(dr + p * plane + c, d);
+        }
+    }
+    if (dr) {
+        for (int p0 = 0; p0 < planes; p0 += 4) {
+            float d[kChunks][4][4];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) v[i][j] += d[j];
+            for (int i = 0; i < kChunks; ++i) {
+                const int c = 4 * (threadIdx.x + i * kThreads);
+                if (c < hidden) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) load4(dr + (p0 + q < planes ? p0 + q : planes - 1) * plane + c, d[i][q]);
                 }
-                if (!rows) store4(xr + c, v[i]);
             }
+#pragma unroll
+            for (int i = 0; i < kChunks; ++i) {
+                const int c = 4 * (threadIdx.x + i * kThreads);
+                if (c < hidden) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        if (p0 + q < planes) {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) v[i][j] += d[i][q][j];
+                        }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+        const int c = 4 * (threadIdx.x + i * kThreads);
+        if (c < hidden) {
+            if (dr && !rows) store4(xr + c, v[i]);
 #pragma unroll
             for (int j = 0; j < 4; ++j) ss = fmaf(v[i][j], v[i][j], ss);
         }

@@ -235,16 +235,31 @@ class Engine:
     def fork(self, parent: Hashable, child: Hashable, tokens: Optional[int] = None) -> int:
         """A new request that shares the full cache pages of ``parent``'s first ``tokens`` tokens.  Returns the
         number of tokens the child holds (a page boundary); the caller feeds it whatever comes after."""
-        if self.pools.state:
-            raise StepError("a model with per-request state cannot share a prefix: its state exists only "
-                            "for the parent's latest position")
-        return self.cache.fork(parent, child, tokens)
+        if not self.pools.state:
+            return self.cache.fork(parent, child, tokens)
+        # Per-request state exists only for the parent's latest position: the share point has to be there, and
+        # the child gets a copy of the state as it is now (pages are shared by reference, state by value).
+        length = self.cache.length(parent)
+        if tokens is not None and tokens < length:
+            raise StepError(f"a model with per-request state shares a prefix only at the parent's latest position "
+                            f"({length} tokens), where its state is; asked for {tokens}")
+        held = self.cache.fork(parent, child, tokens)
+        if held != length:
+            self.cache.release(child)
+            raise StepError(f"a model with per-request state shares a prefix only at the parent's latest position "
+                            f"({length} tokens), and pages are shared whole: {held} tokens could be shared")
+        self.pools.copy_state(self.cache.slot(parent), self.cache.slot(child))
+        return held
 
     def truncate(self, request: Hashable, position: int) -> None:
-        """Cuts a request back to its first ``position`` tokens."""
-        if self.pools.state:
-            raise StepError("a model with per-request state cannot be cut back")
+        """Cuts a request back to its first ``position`` tokens.  Per-request state cannot be wound back: a model
+        that has some can only be cut back to nothing (the state starts from zero again) or not at all."""
+        if self.pools.state and position not in (0, self.cache.length(request)):
+            raise StepError("a model with per-request state cannot be cut back to a position in between: its state "
+                            "exists only for the latest position")
         self.cache.truncate(request, position)
+        if self.pools.state and position == 0:
+            self.pools.zero_state(self.cache.slot(request))
 
     # ---- the vendor library's products ---------------------------------------------------
     def tune_products(self, rows: int, candidates: int = 256, thorough: bool = False,
@@ -395,7 +410,8 @@ class Engine:
             graph = torch.cuda.CUDAGraph()
             # one pool of memory for all recordings: they run one after the other on one stream, and what a
             # replay leaves in its logits is copied out before the next replay begins
-            with torch.cuda.graph(graph, pool=self._graph_pool), ops.one_stream():
+            # (errors of the capture are this thread's: an engine in another thread goes on with its own work)
+            with torch.cuda.graph(graph, pool=self._graph_pool, capture_error_mode="thread_local"), ops.one_stream():
                 recorded_logits = self.model.forward(state.tokens, context, caches)
             state.recordings[bucket] = (graph, recorded_logits)
         else:

@@ -9,6 +9,7 @@ from __future__ import annotations
 from typing import Optional
 
 import functools
+import threading
 import weakref
 
 import numpy as np
@@ -46,36 +47,35 @@ def _dev(t: Optional[torch.Tensor], what: str, dtype=None, shape=None) -> int:
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
-_step_stream: Optional[int] = None     # inside ``one_stream``: the handle that was current when it began
+_held = threading.local()                # .stream inside ``one_stream``: the handle that was current when it began
 
 
 def _stream() -> int:
     """The current stream's handle.  Asked for before every launch, so the short way is taken where this
     torch has it (a tenth of the time of building a Stream object); within ``one_stream`` it was asked for once."""
-    if _step_stream is not None:
-        return _step_stream
+    held = getattr(_held, "stream", None)
+    if held is not None:
+        return held
     if _raw_stream is not None:
         return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
 class one_stream:
-    """Within this context every launch goes to the stream that is current at its beginning: the few hundred
-    launches of a step need not ask for it one by one (0.4 ms of the 4 ms the host takes to issue a step of the
-    8B shape).  Whoever changes the current stream inside (a graph capture does) opens a context of its own.  The
-    handle is kept for the process, not for a thread: steps that run side by side in several threads on different
-    streams must not use it."""
+    """Within this context every launch of this thread goes to the stream that is current at its beginning: the
+    few hundred launches of a step need not ask for it one by one (0.4 ms of the 4 ms the host takes to issue a
+    step of the 8B shape).  Whoever changes the current stream inside (a graph capture does) opens a context of
+    its own.  The handle is kept per thread, as torch keeps the current stream: engines that step side by side
+    in threads of their own, each on its stream, do not see each other's."""
 
     def __enter__(self):
-        global _step_stream
-        self._before = _step_stream
-        _step_stream = None
-        _step_stream = _stream()
+        self._before = getattr(_held, "stream", None)
+        _held.stream = None
+        _held.stream = _stream()
         return self
 
     def __exit__(self, *exc):
-        global _step_stream
-        _step_stream = self._before
+        _held.stream = self._before
         return False
 
 
@@ -656,9 +656,22 @@ def _rows_plan(m: int, n: int, k: int, may_split: bool, units: int, chunk: int, 
     return best[2], best[1]
 
 
+ROWS_WAYS = 2                # most waves that share a tile of the weight in ``gemm_rows``
+
+
+def rows_ways(m: int, waves: int) -> int:
+    """How many waves share each tile of the weight in ``gemm_rows`` (each takes its share of a chunk's units of
+    K; their sums are added up in a fixed order at the end): the most the kernel is built with for this many
+    rows and tiles, up to ROWS_WAYS."""
+    ways = ROWS_WAYS
+    while ways > 1 and not library().leone_gemm_rows_shape_built(m, waves, ways):
+        ways //= 2
+    return ways
+
+
 def gemm_rows(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
               residual: Optional[torch.Tensor] = None, gated: bool = False, splits: Optional[int] = None,
-              waves: Optional[int] = None, may_split: bool = True) -> Optional[torch.Tensor]:
+              waves: Optional[int] = None, may_split: bool = True, ways: Optional[int] = None) -> Optional[torch.Tensor]:
     """The weight-streaming product for up to ROWS_MAX rows of bfloat16 ``x``.  With ``residual`` and one
     range of K the product is added into that float32 tensor (None returned); with ``gated`` the weight is
     an interleaved gate/up weight and silu(gate) * up comes out.  With more than one range of K (``splits``;
@@ -679,6 +692,8 @@ def gemm_rows(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = to
         plan = rows_plan(m, n, k, may_split and not gated, compute_units(weight.device))
         waves = plan[0] if waves is None else waves
         splits = plan[1] if splits is None else splits
+    if ways is None:
+        ways = rows_ways(m, int(waves))
     chunks = -(-k // library().leone_gemm_rows_chunk(m))
     splits = max(1, min(int(splits), chunks))
     splits = -(-chunks // -(-chunks // splits))        # no range of K may be empty
@@ -700,7 +715,7 @@ def gemm_rows(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = to
         call("leone_gemm_rows_bf16", _dev(x, "gemm x", torch.bfloat16, (m, k)),
              _dev(weight if tiles is None else tiles, "gemm weight", torch.bfloat16), 0 if tiles is None else 1,
              _dev(out, "gemm out", kind), mode, _CODES[kind], m, n, k,
-             splits, plane, int(waves), _stream())
+             splits, plane, int(waves), int(ways), _stream())
     return None if (residual is not None and splits == 1) else out
 
 

@@ -40,7 +40,8 @@ _PROTOTYPES = {
     "leone_gemm_f32": [P, P, P, c_int, c_int, c_int, P],
     "leone_gemm_fused_bf16": [P, c_int, P, P, c_int, c_float, P, c_int, P, c_int, c_int, c_int, c_int, c_int, P, P, P, P,
                               c_int, P],
-    "leone_gemm_rows_bf16": [P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_int, ctypes.c_long, c_int, P],
+    "leone_gemm_rows_bf16": [P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_int, ctypes.c_long, c_int, c_int, P],
+    "leone_gemm_rows_shape_built": [c_int, c_int, c_int],
     "leone_argmax": [P, P, P, P, c_int, c_int, P],
     "leone_peak_read": [P, ctypes.c_long, P, c_int, P],
     "leone_peak_copy": [P, P, ctypes.c_long, c_int, P],

@@ -612,3 +612,41 @@ def test_many_groups_of_prompt_tiles_at_few_heads(tmp_path, name):
     got = schedules.collect(steps, outputs)
     mean = np.mean([np.abs(np.stack(got[rid]) - rounded[rid]).mean() for rid in requests])
     assert mean <= ROUNDED_MEAN[name], f"{name}: mean difference from the rounding oracle {mean:.2e}"
+
+
+def test_two_engines_step_side_by_side_in_threads_on_streams_of_their_own(cases):
+    """Nothing a step relies on is kept for the process: two engines on one model, each in a thread with a
+    stream of its own, give bit for bit what they give one after the other."""
+    import threading
+
+    from leone_amd.engine.engine import Engine
+    from leone_amd.runtime import load_model
+
+    folder, requests, expected = cases("B", "float32")
+    model = load_model(folder, "float32")
+    halves = [dict(list(requests.items())[:3]), dict(list(requests.items())[2:])]
+    plans = [schedules.mixed(half, max_live=2) for half in halves]
+
+    def run(which, results, stream=None):
+        engine = Engine(model, num_pages=schedules.max_live_tokens(plans[which], 16) // 16 + 1, page_tokens=16, max_requests=2)
+        if stream is None:
+            results[which] = run_steps(engine, plans[which])
+            return
+        with torch.cuda.stream(stream):
+            for _ in range(3):                        # several times over, so that the two really overlap
+                results[which] = run_steps(engine, plans[which])
+            stream.synchronize()
+
+    alone, together = {}, {}
+    for which in range(2):
+        run(which, alone)
+    threads = [threading.Thread(target=run, args=(which, together, torch.cuda.Stream())) for which in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for which in range(2):
+        assert set(alone[which]) == set(together[which])
+        for step in alone[which]:
+            assert np.array_equal(alone[which][step], together[which][step]), (which, step)
+        compare(plans[which], together[which], {r: expected[r] for r in halves[which]}, tolerance("float32"), "side by side")

@@ -793,13 +793,20 @@ def test_gemm_rows_plain(mnk):
     x, w = torch.randn(m, k, device=DEV).bfloat16(), (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
     want = x.double() @ w.double().T
     big = n * k > 1 << 27
+    from leone_amd.ops.library import library
+    shared = 0
     for waves in ((6,) if big else ops.ROWS_WAVES):
-        for splits in ((1,) if big else (1, 2, 5)):
-            out = ops.gemm_rows(x, w, torch.float32, splits=splits, waves=waves)
-            if out.dim() == 3:
-                assert out.shape[1:] == (m, n)
-                out = out.double().sum(0)
-            close(out, want, 2e-6 * k, 1e-5, f"gemm_rows waves {waves} splits {splits}")
+        for ways in (1, 2):                       # waves that share a tile of the weight: built for more than 64 rows
+            if not library().leone_gemm_rows_shape_built(m, waves, ways):
+                continue
+            shared += ways > 1
+            for splits in ((1,) if big else (1, 2, 5)):
+                out = ops.gemm_rows(x, w, torch.float32, splits=splits, waves=waves, ways=ways)
+                if out.dim() == 3:
+                    assert out.shape[1:] == (m, n)
+                    out = out.double().sum(0)
+                close(out, want, 2e-6 * k, 1e-5, f"gemm_rows waves {waves} ways {ways} splits {splits}")
+    assert (shared > 0) == (m > 64)
     planned = ops.gemm_rows(x, w, torch.float32)
     assert torch.equal(planned, ops.gemm_rows(x, w, torch.float32))            # a launch repeats bit for bit
     close(planned.double().sum(0) if planned.dim() == 3 else planned, want, 2e-6 * k, 1e-5, "gemm_rows as planned")
@@ -871,6 +878,37 @@ def test_products_read_the_tiled_copy_of_a_weight_to_the_same_bits(nk):
     assert ops.streamed_copy(w.clone()) is None
     del w, tiles
     assert not ops._streamed
+
+
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("m", [5, 40, 100])
+def test_weight_streaming_products_do_not_read_weights_beyond_k_as_numbers(m, tiled):
+    """K that is no multiple of a chunk: the kernels load the row's end again for the runs beyond K and must count
+    those as zero themselves, not only through the zeros that stand for X there: with an infinite weight in a
+    row's last columns the sum of that row of W is infinite, as the plain sum is, and not NaN (infinity times
+    the zero beyond K)."""
+    from leone_amd import ops
+    n, k = 96, 320 if tiled else 328              # 256 + 64 (whole steps of the tiled copy), 256 + 72
+    torch.manual_seed(31)
+    x = torch.randn(m, k, device=DEV).bfloat16()
+    x[:, k - 1] = x[:, k - 1].abs() + 0.5
+    w = (torch.randn(n, k, device=DEV) * 0.05).bfloat16()
+    w[3, k - 1] = float("inf")
+    ops.drop_streamed_copies()
+    if tiled:
+        ops.keep_streamed_copy(w)
+    finite = w.clone()
+    finite[3, k - 1] = 0
+    want = x.double() @ finite.double().T
+    outs = {"rows": ops.gemm_rows(x, w, torch.float32, may_split=False)}
+    if m <= ops.FUSED_ROWS:
+        outs["fused"] = ops.gemm_fused(x, w, torch.float32)
+    keep = torch.ones(n, dtype=torch.bool, device=DEV)
+    keep[3] = False
+    for name, out in outs.items():
+        close(out[:, keep], want[:, keep], 2e-6 * k, 1e-5, name)
+        assert (out[:, 3] == float("inf")).all(), (name, out[:, 3])
+    ops.drop_streamed_copies()
 
 
 def test_gemm_rows_plan_fills_the_compute_units():

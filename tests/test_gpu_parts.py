@@ -478,6 +478,32 @@ def test_toy_architecture_with_state_window_repeat_and_shared_cache(tmp_path, dt
         assert err <= tol, err
         engine.release("f")
         engine.cache.check()
+        # A prefix is shared at the parent's latest position, where its state is: the child gets the pages by
+        # reference and a copy of the state, and both go on with tokens of their own.  Anywhere else it is refused
+        # and nothing is left behind; a request with state is cut back to nothing or not at all.
+        from leone_amd.engine.engine import StepError
+        first, second = requests["t0"], requests["t3"]
+        other = first[:24] + second[:14]
+        want_other = toy_plain(weights, other).numpy()
+        engine.step([StepEntry("p", first[:20], [])])
+        with pytest.raises(StepError, match="latest position"):
+            engine.fork("p", "c")                          # 20 tokens: pages are shared whole, 16 could be
+        with pytest.raises(StepError, match="latest position"):
+            engine.fork("p", "c", 16)
+        assert not engine.cache.has("c")
+        engine.step([StepEntry("p", first[20:24], [])])
+        assert engine.fork("p", "c") == 24 and engine.cache.shared_pages(0) > 0
+        out_child = engine.step([StepEntry("c", other[24:], list(range(14)))]).logits.cpu().numpy()
+        out_parent = engine.step([StepEntry("p", first[24:], list(range(len(first) - 24)))]).logits.cpu().numpy()
+        assert np.abs(out_child - want_other[24:]).max() <= tol and np.abs(out_parent - expected["t0"][24:]).max() <= tol
+        with pytest.raises(StepError, match="in between"):
+            engine.truncate("c", 8)
+        engine.truncate("c", 0)                            # its state starts from zero again
+        again = engine.step([StepEntry("c", second, list(range(len(second))))]).logits.cpu().numpy()
+        assert np.abs(again - expected["t3"]).max() <= tol
+        engine.release("p"), engine.release("c")
+        engine.cache.check()
+        assert all(engine.cache.free_pages(g) == 36 for g in range(3))
     finally:
         unregister_architecture("ToyForCausalLM")
         MIXERS.unregister("toy_decay")
