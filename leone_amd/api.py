@@ -114,15 +114,17 @@ class Runtime:
                         on_token: Optional[Callable[[Hashable, int], None]] = None,
                         logit_observer: Optional[Callable] = None,
                         profile_decode_steps: int = 0,
-                        cancelled: Optional[Callable[[], bool]] = None) -> List[GenerationResult]:
+                        cancelled: Optional[Callable[[], bool]] = None, look_ahead: bool = True) -> List[GenerationResult]:
         """Token ids in, token ids out, one result per prompt in order.  ``profile_decode_steps``: time
         that many decode steps operation by operation (they run without graph replay); the result is
         left in ``last_decode_profile``.  ``cancelled``: asked before every step; a yes ends every request
-        with the tokens it has (the reference's cancellation flag, crates/leone-cli/src/main.rs:1600-1602)."""
+        with the tokens it has (the reference's cancellation flag, crates/leone-cli/src/main.rs:1600-1602).
+        ``look_ahead`` False: every step waits for the tokens of the one before (``engine.generate.Generator``);
+        the tokens are the same."""
         eos = self.eos_token_id if eos_token_id == "config" else eos_token_id
         recorder = Recorder(profile_decode_steps) if profile_decode_steps > 0 else None
         results, stats = generate_tokens(self.engine, prompts, max_new_tokens, sampling, eos, self.policy, on_token,
-                                         logit_observer, recorder, cancelled)
+                                         logit_observer, recorder, cancelled, look_ahead)
         self.last_stats = stats
         self.last_decode_profile = recorder.profile if recorder is not None else None
         return results

@@ -115,7 +115,7 @@ def fill_cache(engine, batch: int, tokens: int, seed: int = 0):
 
 
 def time_decode(engine, batch: int, start_context: int, steps: int, warmup: int, seed: int = 1,
-                profile_steps: int = 0):
+                profile_steps: int = 0, pipelined: bool = True):
     """(seconds of ``steps`` decode steps, mean context over them[, per-operation profile of further steps])."""
     import torch
     from .engine.engine import StepEntry
@@ -124,9 +124,32 @@ def time_decode(engine, batch: int, start_context: int, steps: int, warmup: int,
     gen = torch.Generator().manual_seed(seed)
     tokens = torch.randint(0, engine.vocab_size, (batch,), generator=gen).tolist()
 
+    # A step is issued with the tokens the step before it is choosing still on the device; then that step's tokens
+    # are copied to the host (every step's are, one step late), as the generation loop does (``Generator``,
+    # ``look_ahead``): what the host does for a step overlaps the step before it.  ``pipelined`` False: the step,
+    # the choice and the copy one after the other, as the reference's loop.
+    waiting, waiting_turn = [], []
+    pinned = [torch.empty(batch, dtype=torch.int32).pin_memory() for _ in range(2)]
+
     def one_step(tokens):
-        out = engine.step([StepEntry(("bench", b), [tokens[b]], [0]) for b in range(batch)])
-        return ops.argmax(out.logits).cpu().tolist()       # the per-step copy of the chosen tokens
+        if not pipelined:
+            out = engine.step([StepEntry(("bench", b), [tokens[b]], [0]) for b in range(batch)])
+            return ops.argmax(out.logits).cpu().tolist()       # the per-step copy of the chosen tokens
+        chosen, on_host, arrived = waiting.pop() if waiting else (None, None, None)
+        out = engine.step([StepEntry(("bench", b), [tokens[b]], [0]) for b in range(batch)], device_tokens=chosen)
+        picked = ops.argmax(out.logits)
+        # the copy to the host is asked for at once and waited for by its event, one step later: asked for then, it
+        # would queue behind the step issued meanwhile
+        buffer = pinned[len(waiting_turn) % 2]
+        waiting_turn.append(0)
+        buffer.copy_(picked, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        waiting.append((picked, buffer, event))
+        if chosen is None:
+            return tokens
+        arrived.synchronize()
+        return on_host.tolist()
 
     for _ in range(warmup):
         tokens = one_step(tokens)
@@ -134,9 +157,12 @@ def time_decode(engine, batch: int, start_context: int, steps: int, warmup: int,
     started = time.perf_counter()
     for _ in range(steps):
         tokens = one_step(tokens)
+    if waiting:
+        waiting.pop()[2].synchronize()                       # the last step's tokens
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
     profiled = None
+    pipelined = False
     if profile_steps:
         from .ops.profile import Recorder
         recorder = Recorder(profile_steps)
@@ -399,7 +425,8 @@ def main(argv: Optional[List[str]] = None) -> int:
                    "global_batch": args.batch, "seq_len": args.context, "decode_start_context": start,
                    "prefill_tokens": PREFILL_TOKENS, "page_tokens": page_tokens, "rope_theta": config.rope_theta,
                    "tied_head": config.tie_word_embeddings, "parallelism": "single GPU",
-                   "weight_copies": 2 if model.streamed_copy_bytes else 1},
+                   "weight_copies": 2 if model.streamed_copy_bytes else 1,
+                   "decode_loop": "a step is issued before the last step's tokens reach the host"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
     }
@@ -424,6 +451,11 @@ def main(argv: Optional[List[str]] = None) -> int:
         if peaks is not None and dtype_name == "bf16":
             record["prefill"]["frac_of_measured"] = round(flops / seconds / (peaks["mfma_bf16_tflops"] * 1e12), 4)
     points = {}
+    if not args.no_points:
+        # the same steps one by one, as the reference's loop: step, choice, copy of the tokens, next step
+        e, _ = time_decode(engine, args.batch, args.context - args.steps - args.warmup - 1, args.steps, args.warmup,
+                           pipelined=False)
+        points[f"decode_b{args.batch}_one_by_one"] = round(args.batch * args.steps / e, 2)
     for batch in points_batches:
         steps = max(8, args.steps // 2)
         warm = max(2, args.warmup // 2)

@@ -227,6 +227,22 @@ int leone_scheduler_planned(void* scheduler, int64_t* requests, int* starts, int
         return n;
     });
 }
+int leone_scheduler_plan_ahead(void* scheduler) {
+    return guarded([&]() -> long { return static_cast<long>(scheduler_of(scheduler).plan_ahead().size()); });
+}
+int leone_scheduler_ahead(void* scheduler, int64_t* requests, int* starts, int* counts, int* samples, int capacity) {
+    return guarded([&]() -> long {
+        const std::vector<PlannedEntry>& entries = scheduler_of(scheduler).ahead();
+        const int n = static_cast<int>(entries.size());
+        for (int i = 0; i < std::min(n, capacity); ++i) {
+            requests[i] = entries[i].request;
+            starts[i] = entries[i].start;
+            counts[i] = entries[i].count;
+            samples[i] = entries[i].sample ? 1 : 0;
+        }
+        return n;
+    });
+}
 int leone_scheduler_complete(void* scheduler, const int64_t* requests, const int32_t* tokens, int n) {
     return guarded([&]() -> long {
         std::unordered_map<RequestKey, std::int32_t> sampled;

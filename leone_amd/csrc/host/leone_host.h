@@ -63,6 +63,10 @@ int leone_scheduler_has_work(void* scheduler);
 int leone_scheduler_plan(void* scheduler);     // number of entries
 // The planned entries: request, start, count, sample for each.
 int leone_scheduler_planned(void* scheduler, int64_t* requests, int* starts, int* counts, int* samples, int capacity);
+// One step beyond the planned one, before its tokens are known (Scheduler::plan_ahead): number of entries, 0 if
+// the next step cannot be known yet; leone_scheduler_ahead lists them as leone_scheduler_planned does.
+int leone_scheduler_plan_ahead(void* scheduler);
+int leone_scheduler_ahead(void* scheduler, int64_t* requests, int* starts, int* counts, int* samples, int capacity);
 int leone_scheduler_complete(void* scheduler, const int64_t* requests, const int32_t* tokens, int n);   // finished now
 int leone_scheduler_abort(void* scheduler);
 int leone_scheduler_history(void* scheduler, int64_t request, int32_t* out, int capacity);    // tokens known

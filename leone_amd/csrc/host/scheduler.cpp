@@ -88,7 +88,7 @@ bool Scheduler::cancel(RequestKey request) {
 
 const std::vector<PlannedEntry>& Scheduler::plan() {
     if (planned_valid_) throw SchedulerError("the previous step was neither completed nor aborted");
-    std::vector<LivePtr> gone;
+    std::vector<LivePtr> gone;   // (a step planned ahead became the planned step when the one before it was completed)
     for (const auto& kv : live_)
         if (kv.second->cancelled) gone.push_back(kv.second);
     std::sort(gone.begin(), gone.end(), [](const LivePtr& a, const LivePtr& b) { return a->order < b->order; });
@@ -116,6 +116,45 @@ const std::vector<PlannedEntry>& Scheduler::plan() {
             events_.push_back({EventKind::StepEntry, e.request, e.start, e.count, e.sample ? 1 : 0});
     }
     return planned_;
+}
+
+const std::vector<PlannedEntry>& Scheduler::plan_ahead() {
+    if (!planned_valid_) throw SchedulerError("no step is planned to look beyond");
+    if (ahead_valid_) throw SchedulerError("a step ahead is planned already");
+    ahead_.clear();
+    if (planned_.empty() || planned_.size() != live_.size() ||
+        static_cast<std::int64_t>(planned_.size()) > policy_.max_step_tokens)
+        return ahead_;
+    // somebody could be admitted into the next step: then it is not this step's rows once more
+    if (!queue_.empty() && static_cast<std::int64_t>(live_.size()) < policy_.max_live_requests && cache_.free_slots() > 0)
+        return ahead_;
+    for (const PlannedEntry& entry : planned_) {
+        const Live& state = *live_.at(entry.request);
+        if (!entry.sample || state.cancelled) return ahead_;
+        const std::int64_t generated = static_cast<std::int64_t>(state.tokens.size()) - state.prompt_len + 1;
+        if (generated >= state.max_new_tokens) return ahead_;           // this step's token is its last
+        if (cache_.length(entry.request) != entry.start + entry.count)
+            throw SchedulerError("request " + std::to_string(entry.request) +
+                                 ": the planned step has not run; there is nothing to look beyond yet");
+    }
+    std::vector<PlannedEntry> entries;
+    for (const PlannedEntry& entry : planned_) {
+        try {
+            cache_.reserve(entry.request, 1);
+        } catch (const std::runtime_error&) {    // no page (a preemption is the planned way's affair), or the context's end
+            for (const PlannedEntry& held : entries) cache_.rollback(held.request);
+            return ahead_;
+        }
+        entries.push_back({entry.request, entry.start + entry.count, 1, true});
+    }
+    ahead_ = std::move(entries);
+    ahead_valid_ = true;
+    ++stats_.steps;
+    stats_.decode_rows += static_cast<std::int64_t>(ahead_.size());
+    stats_.max_step_rows = std::max<std::int64_t>(stats_.max_step_rows, ahead_.size());
+    events_.push_back({EventKind::StepAhead, 0, static_cast<int>(ahead_.size()), 0, 0});
+    for (const PlannedEntry& e : ahead_) events_.push_back({EventKind::StepEntry, e.request, e.start, e.count, 1});
+    return ahead_;
 }
 
 Scheduler::LivePtr Scheduler::newest() const {
@@ -260,7 +299,8 @@ int Scheduler::complete(const std::unordered_map<RequestKey, std::int32_t>& samp
     if (!planned_valid_) throw SchedulerError("no step is planned");
     // Check everything before anything changes, so that a refused call leaves the step planned.
     for (const PlannedEntry& entry : planned_) {
-        if (cache_.length(entry.request) != entry.start + entry.count)
+        const int held = cache_.length(entry.request);           // a step ahead that ran has added its one token
+        if (held != entry.start + entry.count && !(ahead_valid_ && held == entry.start + entry.count + 1))
             throw SchedulerError("request " + std::to_string(entry.request) + ": the step was not committed to the cache");
         if (entry.sample && !sampled.count(entry.request))
             throw SchedulerError("request " + std::to_string(entry.request) + ": the step returned no token");
@@ -285,6 +325,15 @@ int Scheduler::complete(const std::unordered_map<RequestKey, std::int32_t>& samp
             ++done;
         }
     }
+    if (ahead_valid_) {
+        // The step ahead is the planned step now; a request that has just ended is no longer in it (what its
+        // row there wrote went back with everything else it held).
+        for (const PlannedEntry& entry : ahead_)
+            if (live_.count(entry.request)) planned_.push_back(entry);
+        ahead_.clear();
+        ahead_valid_ = false;
+        planned_valid_ = !planned_.empty();
+    }
     return done;
 }
 
@@ -293,6 +342,8 @@ int Scheduler::abort() {
     std::vector<PlannedEntry> planned = std::move(planned_);
     planned_.clear();
     planned_valid_ = false;
+    ahead_.clear();                     // its requests are the planned step's: they go with them
+    ahead_valid_ = false;
     for (const PlannedEntry& entry : planned) {
         LivePtr state = live_.at(entry.request);
         cache_.rollback(entry.request);

@@ -84,7 +84,8 @@ struct SchedulerStats {
 // that many StepEntry records (a = start, b = count, c = sample).  Submit: a = prompt tokens, b = most new
 // tokens; Reject: a = reason; Preempt: a = tokens known; Token: a = position of the row that gave it,
 // b = token; Finish: a = reason.
-enum class EventKind : int { Reject = 0, Submit, StepBegin, StepEntry, Admit, Preempt, Token, Finish };
+// A StepAhead record is a StepBegin for a step planned beyond one whose tokens are not known yet.
+enum class EventKind : int { Reject = 0, Submit, StepBegin, StepEntry, Admit, Preempt, Token, Finish, StepAhead };
 struct Event {
     EventKind kind;
     RequestKey request;
@@ -103,14 +104,29 @@ public:
     bool has_work() const { return !queue_.empty() || !live_.empty(); }
     // Decides the next step and reserves its pages.  Empty only if there is nothing to do.
     const std::vector<PlannedEntry>& plan();
+    // One step beyond the planned one, before that one's tokens are known: every request of the planned step
+    // once more, one row each at its next position, in the planned step's order, pages reserved.  The caller
+    // feeds the rows the tokens the planned step is still choosing (they never leave the device) and so has
+    // the next step running while it reads and reports the planned step's tokens.  Possible only where the
+    // next step is known without those tokens: the planned step ran and is committed, every live request is
+    // in it and gets a token from it, none of them uses up its output budget with that token, none is
+    // cancelled, nobody waits in the queue for a place that is free, and every request finds its page.
+    // Otherwise nothing is reserved and the answer is empty: complete the planned step first, as always.  A
+    // request that ends on the planned step's token after all (its end token) simply drops out of the step
+    // ahead: its row there is run for nothing and what it wrote goes back with everything else it holds.
+    const std::vector<PlannedEntry>& plan_ahead();
     // The planned step ran and its cache writes are committed.  `sampled` holds a token for every entry
-    // planned with `sample`.  Returns how many requests finished; they are the last of finished().
+    // planned with `sample`.  Returns how many requests finished; they are the last of finished().  A step
+    // planned ahead becomes the planned step (without the requests that have just finished).
     int complete(const std::unordered_map<RequestKey, std::int32_t>& sampled);
-    // The planned step failed: every request in it ends as aborted and gives back what it holds.
+    // The planned step failed (or the one ahead of it): every request in them ends as aborted and gives back
+    // what it holds.
     int abort();
 
     // The entries of the step that is planned and not yet completed or aborted (empty otherwise).
     const std::vector<PlannedEntry>& planned() const { return planned_; }
+    // The entries of the step planned beyond it (empty if there is none).
+    const std::vector<PlannedEntry>& ahead() const { return ahead_; }
     const std::vector<Finished>& finished() const { return finished_; }
     const std::vector<Event>& events() const { return events_; }
     const SchedulerStats& stats() const { return stats_; }
@@ -156,6 +172,8 @@ private:
     std::int64_t order_ = 0;
     bool planned_valid_ = false;
     std::vector<PlannedEntry> planned_;
+    bool ahead_valid_ = false;
+    std::vector<PlannedEntry> ahead_;
 };
 
 }  // namespace leone::host

@@ -13,6 +13,7 @@ reserved first, written by the kernels, and committed only if the step succeeds
 from __future__ import annotations
 
 import ctypes
+import math
 import time
 from ctypes import c_int, c_int64, c_long
 from dataclasses import dataclass, field
@@ -153,7 +154,8 @@ class _DecodeGraph:
         self.rows = rows
         self._pieces, self._tables = pieces, {g: pieces[5 + len(tilings) + g].view(rows, widths[g]) for g in range(groups)}
         self._engine_type = (engine.dtype, engine.device)
-        self.recordings: Dict[int, tuple] = {}        # context range -> (graph, its logits)
+        self.recordings: Dict[object, tuple] = {}     # context range -> (graph, its logits)
+        self.turn = 0
         self.copied = torch.cuda.Event()
 
     def context(self, bucket: int) -> StepContext:
@@ -209,6 +211,7 @@ class Engine:
         self.graphs = bool(graphs) and model.graph_safe
         self._decode_graphs: Dict[int, _DecodeGraph] = {}
         self._graph_pool = torch.cuda.graph_pool_handle() if self.graphs else None
+        self.twin_recordings = False
         self._staging: List[Optional[tuple]] = [None, None]
         self._staging_turn = 0
 
@@ -243,11 +246,12 @@ class Engine:
         if tokens is not None and tokens < length:
             raise StepError(f"a model with per-request state shares a prefix only at the parent's latest position "
                             f"({length} tokens), where its state is; asked for {tokens}")
-        held = self.cache.fork(parent, child, tokens)
-        if held != length:
-            self.cache.release(child)
+        unit = math.lcm(*[group.page_tokens for group in self.cache.groups]) if self.cache.groups else 1
+        if length % unit:
             raise StepError(f"a model with per-request state shares a prefix only at the parent's latest position "
-                            f"({length} tokens), and pages are shared whole: {held} tokens could be shared")
+                            f"({length} tokens), and pages are shared whole: every {unit} tokens")
+        held = self.cache.fork(parent, child, tokens)
+        assert held == length
         self.pools.copy_state(self.cache.slot(parent), self.cache.slot(child))
         return held
 
@@ -345,8 +349,9 @@ class Engine:
                 if not 0 <= int(w) < len(e.tokens):
                     raise StepError(f"request {e.request!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
 
-    def step(self, entries: Sequence[StepEntry]) -> StepOutput:
-        """Admits unknown requests, reserves pages, runs the tokens and commits.  All or nothing."""
+    def step(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> StepOutput:
+        """Admits unknown requests, reserves pages, runs the tokens and commits.  All or nothing.
+        ``device_tokens``: see ``run_reserved``."""
         self._validate(entries)
         admitted, reserved = [], []
         try:
@@ -362,10 +367,22 @@ class Engine:
             for request in admitted:
                 self.cache.release(request)
             raise
-        return self.run_reserved(entries)
+        return self.run_reserved(entries, device_tokens)
 
-    def run_reserved(self, entries: Sequence[StepEntry]) -> StepOutput:
-        """Runs a step whose pages the caller has reserved; commits on success, rolls back on failure."""
+    def run_reserved(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None) -> StepOutput:
+        """Runs a step whose pages the caller has reserved; commits on success, rolls back on failure.
+
+        ``device_tokens`` (int32 ``[entries]`` on the device, for a step of one token an entry): the rows' tokens
+        are these, not the entries' (which only stand in): the tokens an earlier step has chosen and that have
+        not left the device yet, so that this step can be issued before the host has seen them.  Everything is
+        ordered on the stream; a value outside the vocabulary (a row that found no finite logit gives -1) is
+        run as the nearest token, for the caller to throw away."""
+        if device_tokens is not None:
+            if any(len(e.tokens) != 1 for e in entries):
+                raise StepError("tokens can be taken from the device only for a step of one token an entry")
+            if (device_tokens.dtype != torch.int32 or device_tokens.device != self.device
+                    or tuple(device_tokens.shape) != (len(entries),)):
+                raise StepError(f"device tokens must be int32 [{len(entries)}] on {self.device}")
         self.poison_freed_pages()              # what a scheduler on the same manager has freed since the last step
         # A failed step gives its pages back (rollback) and leaves per-request state as it found it.
         saved_state = self.pools.snapshot_state([self.cache.slot(e.request) for e in entries])
@@ -375,9 +392,12 @@ class Engine:
                     self.pools.zero_state(self.cache.slot(e.request))   # a request's state starts from zero
             # A step that is being profiled runs call by call: a replayed recording has no calls to time.
             if self.graphs and not profile.recording() and all(len(e.tokens) == 1 for e in entries):
-                logits, rows = self._run_decode_graph(entries)
+                logits, rows = self._run_decode_graph(entries, device_tokens)
             else:
                 tokens, context, rows = self._build_context(entries)
+                if device_tokens is not None:
+                    # entries run in the order the layout gives them: rows of one token each keep the caller's
+                    torch.clamp(device_tokens, 0, self.vocab_size - 1, out=tokens)
                 caches = self.pools.views(context.block_tables)
                 with ops.one_stream():
                     logits = self.model.forward(tokens, context, caches)
@@ -392,14 +412,20 @@ class Engine:
         self.poison_freed_pages()              # pages a window has passed
         return StepOutput(logits, rows)
 
-    def _run_decode_graph(self, entries: Sequence[StepEntry]):
+    def _run_decode_graph(self, entries: Sequence[StepEntry], device_tokens: Optional[torch.Tensor] = None):
         """One decoded token for each entry, replayed from the recording for this batch size."""
         state = self._decode_graphs.get(len(entries))
         if state is None:
             state = self._decode_graphs[len(entries)] = _DecodeGraph(self, len(entries))
         packed = state.fill(self, entries)
+        if device_tokens is not None:                 # after the upload, on the same stream
+            torch.clamp(device_tokens, 0, self.vocab_size - 1, out=state.tokens)
         bucket = context_bucket(packed.max_position + 1, self.max_context)
-        recording = state.recordings.get(bucket)
+        key = bucket
+        if self.twin_recordings:
+            state.turn ^= 1
+            key = (bucket, state.turn)
+        recording = state.recordings.get(key)
         if recording is None:
             # First step of this size and context range: run it for real on the static buffers, then record
             # the same calls for later steps.  Recording executes nothing, so the cache is written once.
@@ -413,7 +439,7 @@ class Engine:
             # (errors of the capture are this thread's: an engine in another thread goes on with its own work)
             with torch.cuda.graph(graph, pool=self._graph_pool, capture_error_mode="thread_local"), ops.one_stream():
                 recorded_logits = self.model.forward(state.tokens, context, caches)
-            state.recordings[bucket] = (graph, recorded_logits)
+            state.recordings[key] = (graph, recorded_logits)
         else:
             recording[0].replay()
             logits = recording[1]

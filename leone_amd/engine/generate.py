@@ -32,6 +32,7 @@ class GenerationStats:
     prefill_tokens: int = 0
     decode_tokens: int = 0
     preemptions: int = 0
+    steps_ahead: int = 0             # steps issued before the tokens of the step before them had reached the host
 
     @property
     def prefill_rate(self) -> float:
@@ -132,8 +133,52 @@ def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params:
     return out
 
 
+def choose_on_device(logits: torch.Tensor, entries: Sequence[PlannedEntry],
+                     params: Dict[Hashable, SamplingParams]) -> Optional[torch.Tensor]:
+    """The tokens of the sampled entries as int32 on the device, in their order, without a copy to the host; None
+    unless every one of them is chosen by a device kernel (greedy, or plain temperature).  -1 stands for a row
+    without a finite logit."""
+    rows = [e for e in entries if e.sample]
+    policies = [params[e.request] or SamplingParams() for e in rows]
+    if not rows or not all(p.device_eligible for p in policies):
+        return None
+    for p in policies:
+        p.validate()
+    scaled = [not p.greedy for p in policies]
+    if not any(scaled):
+        return ops.argmax(logits)
+    temps = torch.tensor([p.temperature if s else 1.0 for p, s in zip(policies, scaled)], dtype=torch.float64,
+                         device=logits.device)
+    draws = torch.tensor([rng.uniform(p.seed, e.sample_position) for p, e in zip(policies, rows)], dtype=torch.float64,
+                         device=logits.device)
+    drawn = ops.sample_temperature(logits, temps, draws)
+    if all(scaled):
+        return drawn
+    return torch.where(torch.tensor(scaled, device=logits.device), drawn, ops.argmax(logits))
+
+
+@dataclass
+class _InFlight:
+    """A step that has been issued and whose tokens have not been reported to the scheduler yet."""
+    plan: List[PlannedEntry]
+    logits: Optional[torch.Tensor]
+    picked: Optional[torch.Tensor]       # the chosen tokens on the device, if device kernels chose them all
+    decoding: bool
+    started: float
+    recorder: Optional[Recorder] = None
+    exact: bool = True                   # its rows are still the scheduler's planned rows, one for one
+    host: Optional[torch.Tensor] = None  # the chosen tokens on their way into pinned host memory; `arrived` says when they are there
+    arrived: Optional[torch.cuda.Event] = None
+
+
 class Generator:
-    """Runs requests to completion: scheduler above, engine below."""
+    """Runs requests to completion: scheduler above, engine below.
+
+    ``look_ahead``: where the scheduler can plan the next step before the tokens of the one in flight are known
+    (a step of decoded tokens for the same requests; ``Scheduler.plan_ahead``) and device kernels choose those
+    tokens, the next step is issued with the tokens taken from the device, and only then are the earlier step's
+    tokens copied to the host and reported: planning, the step's metadata and the launch overlap the step in
+    flight instead of standing between two steps.  The tokens are the same either way."""
 
     def __init__(self, engine: Engine, policy: Optional[SchedulerPolicy] = None):
         self.engine = engine
@@ -147,6 +192,11 @@ class Generator:
         self.logit_observer: Optional[Callable[[Hashable, int, torch.Tensor], None]] = None
         # When set, the decode-only steps are timed operation by operation until it has its fill.
         self.decode_profile: Optional[Recorder] = None
+        self.look_ahead = True
+        self._flight: Optional[_InFlight] = None
+        self._last_finish = 0.0
+        self._token_buffers: List[Optional[torch.Tensor]] = [None, None, None]
+        self._token_turn = 0
 
     def submit(self, request_id: Hashable, prompt: Sequence[int], max_new_tokens: int,
                sampling: Optional[SamplingParams] = None, eos_token_id: Optional[int] = None) -> None:
@@ -164,46 +214,76 @@ class Generator:
             self.controllers[request_id] = MirostatState(*sampling.mirostat)
         self.stats.prompt_tokens += len(prompt)
 
-    def step(self, on_token: Optional[Callable[[Hashable, int], None]] = None) -> List[Finished]:
-        """Plans and runs one step.  Returns the requests that finished in it."""
-        scheduler = self.scheduler
-        plan = scheduler.plan()
-        if not plan:
-            return []
+    def _issue(self, plan: List[PlannedEntry], device_tokens: Optional[torch.Tensor] = None) -> _InFlight:
+        """Hands a planned step to the engine and, where device kernels choose all its tokens, has them chosen;
+        nothing is waited for."""
         decoding = all(len(e.tokens) == 1 and e.start > 0 for e in plan)
         recorder = self.decode_profile if decoding and self.decode_profile is not None \
             and not self.decode_profile.done else None
-        started = time.perf_counter()
-        try:
-            entries = [StepEntry(e.request, e.tokens, [len(e.tokens) - 1] if e.sample else []) for e in plan]
-            if recorder is not None:
-                recorder.begin_step()
-            output = self.engine.run_reserved(entries)
-            sampled = choose_tokens(output.logits, plan, self.params, scheduler.history, self.controllers) \
-                if output.logits is not None else {}
-            if recorder is not None:
-                recorder.end_step(len(plan))
-            if self.logit_observer is not None and output.logits is not None:
-                for row, e in enumerate([e for e in plan if e.sample]):
-                    self.logit_observer(e.request, e.sample_position, output.logits[row])
-        except Exception:
-            if recorder is not None:
-                recorder.abandon_step()
-            scheduler.abort()
-            raise
-        elapsed = time.perf_counter() - started
+        flight = _InFlight(plan, None, None, decoding, time.perf_counter(), recorder)
+        entries = [StepEntry(e.request, e.tokens, [len(e.tokens) - 1] if e.sample else []) for e in plan]
+        if recorder is not None:
+            recorder.begin_step()
+        output = self.engine.run_reserved(entries, device_tokens)
+        flight.logits = output.logits
+        if output.logits is not None and recorder is None and self.logit_observer is None \
+                and not any(e.request in self.controllers for e in plan):
+            flight.picked = choose_on_device(output.logits, plan, self.params)
+            if flight.picked is not None:
+                # The copy to the host is asked for now, behind the kernels that choose, and waited for by its
+                # event: a copy asked for later would queue behind whatever has been issued since (the step ahead).
+                flight.host = self._token_buffer(flight.picked.numel())
+                flight.host.copy_(flight.picked, non_blocking=True)
+                flight.arrived = torch.cuda.Event()
+                flight.arrived.record()
+        return flight
+
+    def _token_buffer(self, count: int) -> torch.Tensor:
+        """Pinned host memory for one step's chosen tokens; three take turns (a step, the one ahead of it, and one
+        whose tokens are being read)."""
+        self._token_turn = (self._token_turn + 1) % 3
+        held = self._token_buffers[self._token_turn]
+        if held is None or held.numel() < count:
+            held = self._token_buffers[self._token_turn] = torch.empty(max(count, 64), dtype=torch.int32).pin_memory()
+        return held[:count]
+
+    def _conclude(self, flight: _InFlight, on_token: Optional[Callable[[Hashable, int], None]]) -> List[Finished]:
+        """Brings the step's tokens to the host (or chooses them there), reports them and the time."""
+        plan, scheduler = flight.plan, self.scheduler
+        if flight.picked is not None:
+            rows = [e for e in plan if e.sample]
+            flight.arrived.synchronize()
+            sampled = dict(zip((e.request for e in rows), flight.host.tolist()))
+            for e in rows:
+                if sampled[e.request] < 0:
+                    raise SamplerError(f"request {e.request!r}: no finite logit at position {e.sample_position}")
+        else:
+            sampled = choose_tokens(flight.logits, plan, self.params, scheduler.history, self.controllers) \
+                if flight.logits is not None else {}
+        if flight.recorder is not None:
+            flight.recorder.end_step(len(plan))
+            flight.recorder = None
+        if self.logit_observer is not None and flight.logits is not None:
+            for row, e in enumerate([e for e in plan if e.sample]):
+                self.logit_observer(e.request, e.sample_position, flight.logits[row])
+        now = time.perf_counter()
+        elapsed = now - max(flight.started, self._last_finish)     # a step issued ahead counts from the end of the one before
+        self._last_finish = now
         rows = sum(len(e.tokens) for e in plan)
-        if decoding:
+        if flight.decoding:
             self.stats.decode_seconds += elapsed
             self.stats.decode_tokens += rows
         else:
             self.stats.prefill_seconds += elapsed
             self.stats.prefill_tokens += rows
         self.stats.steps += 1
+        live = scheduler.live if not flight.exact else None         # a request that has ended meanwhile is given nothing
+        if live is not None:
+            sampled = {name: token for name, token in sampled.items() if name in live}
         self.stats.emitted_tokens += len(sampled)
         if on_token is not None:
             for e in plan:
-                if e.sample:
+                if e.sample and e.request in sampled:
                     on_token(e.request, sampled[e.request])
         done = scheduler.complete(sampled)
         for f in done:
@@ -211,10 +291,51 @@ class Generator:
         self.stats.preemptions = scheduler.stats.preemptions
         return done
 
+    def _give_up(self, *flights: Optional[_InFlight]) -> None:
+        for flight in flights:
+            if flight is not None and flight.recorder is not None:
+                flight.recorder.abandon_step()
+        self._flight = None
+        self.scheduler.abort()
+
+    def step(self, on_token: Optional[Callable[[Hashable, int], None]] = None) -> List[Finished]:
+        """Brings one step to its end and returns the requests that finished in it: the step in flight if one was
+        issued ahead, else the next one the scheduler plans; before its tokens are waited for, the step after it
+        is issued if ``look_ahead`` is on and the scheduler can plan it (see the class)."""
+        scheduler = self.scheduler
+        flight = self._flight
+        if flight is None:
+            plan = scheduler.plan()
+            if not plan:
+                return []
+            try:
+                flight = self._issue(plan)
+            except Exception:
+                self._give_up(flight)
+                raise
+        self._flight = following = None
+        try:
+            if self.look_ahead and flight.exact and flight.picked is not None and flight.picked.numel() == len(flight.plan):
+                ahead = scheduler.plan_ahead()
+                if ahead:
+                    following = self._issue(ahead, device_tokens=flight.picked)
+                    self.stats.steps_ahead += 1
+            done = self._conclude(flight, on_token)
+        except Exception:
+            self._give_up(flight, following)
+            raise
+        if following is not None:
+            if done:                                   # somebody ended on this token: its row in the step ahead is void,
+                following.exact = False                # and the rows no longer stand one for one
+                if not any(e.request in scheduler.live for e in following.plan):
+                    following = None                   # everybody did: the scheduler has dropped the step
+            self._flight = following
+        return done
+
     def run(self, on_token: Optional[Callable[[Hashable, int], None]] = None,
             cancelled: Optional[Callable[[], bool]] = None) -> List[Finished]:
         finished: List[Finished] = []
-        while self.scheduler.has_work():
+        while self.scheduler.has_work() or self._flight is not None:
             if cancelled is not None and cancelled():
                 for rid in list(self.scheduler.live) + [q.request.id for q in self.scheduler.queue]:
                     self.scheduler.cancel(rid)
@@ -231,11 +352,12 @@ def generate_tokens(engine: Engine, prompts: Sequence[Sequence[int]], max_new_to
                     on_token: Optional[Callable[[Hashable, int], None]] = None,
                     logit_observer: Optional[Callable[[Hashable, int, torch.Tensor], None]] = None,
                     decode_profile: Optional[Recorder] = None,
-                    cancelled: Optional[Callable[[], bool]] = None):
+                    cancelled: Optional[Callable[[], bool]] = None, look_ahead: bool = True):
     """Generates for every prompt (token ids); returns results in prompt order and the run's statistics.
     ``cancelled`` is asked before every step; once it says yes, every request ends as "cancelled" with the
-    tokens it has."""
+    tokens it has.  ``look_ahead``: see ``Generator``."""
     generator = Generator(engine, policy)
+    generator.look_ahead = look_ahead
     generator.logit_observer = logit_observer
     generator.decode_profile = decode_profile
     for i, prompt in enumerate(prompts):

@@ -88,6 +88,7 @@ class PlannedEntry:
     tokens: List[int]
     start: int                           # absolute position of tokens[0]
     sample: bool                         # the portion ends the known tokens: its last row's logits are wanted
+    deferred: bool = False               # planned ahead: the token is the one the step before is still choosing
 
     @property
     def sample_position(self) -> int:
@@ -256,7 +257,8 @@ class Scheduler:
     @property
     def events(self) -> List[tuple]:
         """The decision log: ("reject", id, reason), ("submit", id, prompt tokens, most new tokens),
-        ("step", [(id, start, tokens, sample)]),
+        ("step", [(id, start, tokens, sample)]), ("ahead", [...]) for a step planned before the tokens of the one
+        before it were known,
         ("admit", id), ("preempt", id, tokens known), ("token", id, position, token), ("finish", id, reason)."""
         n = self._checked(self._lib.leone_scheduler_event_count(self.handle))
         kinds, a, b, c = (c_int * max(1, n))(), (c_int * max(1, n))(), (c_int * max(1, n))(), (c_int * max(1, n))()
@@ -283,6 +285,10 @@ class Scheduler:
                 out.append(("token", name, a[i], b[i]))
             elif kind == 7:
                 out.append(("finish", name, _REASONS[a[i]]))
+            elif kind == 8:
+                rows = [(self._names[keys[j]], a[j], b[j], bool(c[j])) for j in range(i + 1, i + 1 + a[i])]
+                out.append(("ahead", rows))
+                i += a[i]
             i += 1
         return out
 
@@ -305,6 +311,23 @@ class Scheduler:
             self._checked(self._lib.leone_scheduler_tokens(self.handle, key, start, count, tokens))
             entries.append(PlannedEntry(self._names[key], list(tokens), start, bool(self._samples[i])))
         return entries
+
+    def plan_ahead(self) -> List[PlannedEntry]:
+        """One step beyond the planned one, before that one's tokens are known: every request of the planned step
+        once more, one row at its next position, in the same order, pages reserved; the rows' tokens (``tokens``
+        holds a stand-in, ``deferred`` says so) are the ones the planned step is choosing, which the caller feeds
+        from the device.  Empty, with nothing reserved, wherever the next step cannot be known without those
+        tokens (a request uses up its budget, somebody waits for a free place, a page is missing, a portion of a
+        prompt is not the last): then the planned step is completed first, as always.  The planned step must
+        have run.  Once the planned step is completed the step ahead is the planned one; a request that ended
+        on its end token meanwhile is no longer in it, and a token reported for it is ignored."""
+        n = self._checked(self._lib.leone_scheduler_plan_ahead(self.handle))
+        if n == 0:
+            return []
+        self._grow(n)
+        self._checked(self._lib.leone_scheduler_ahead(self.handle, self._keys, self._starts, self._counts,
+                                                      self._samples, self._capacity))
+        return [PlannedEntry(self._names[self._keys[i]], [0], self._starts[i], True, deferred=True) for i in range(n)]
 
     # ---- after the step ----------------------------------------------------------------------
     def complete(self, sampled: Dict[Hashable, int]) -> List[Finished]:

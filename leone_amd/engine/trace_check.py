@@ -3,7 +3,10 @@
 It takes ``Scheduler.events`` (plain tuples) and the figures of the run (pages, page size, budgets) and
 re-derives from the events alone what must hold: every request goes submit, admit, (preempt, admit)*,
 finish; one step is in flight at a time and each of its sampling rows is answered by exactly one
-token before the next step; a request's portions follow each other without a gap or an overlap from
+token before the next step, except that one step may be planned ahead of a step whose rows all owe their
+tokens: the same requests once more, one row each at the next position, none of them at the end of its
+output, and nothing else may be decided until the owed tokens have come (a request that ends on its end
+token then drops out of the step ahead); a request's portions follow each other without a gap or an overlap from
 position 0 after every (re)admission; steps keep the token budget, the portion limit and the limit of
 live requests; the pages that the live requests' positions need never exceed the pool; nothing
 happens to a request that has finished; output limits hold.  It returns what each request was fed and
@@ -84,6 +87,7 @@ def verify_events(events: Iterable[tuple], figures: RunFigures) -> TraceReport:
     rejected: List[Tuple[Hashable, str]] = []
     awaiting: Dict[Hashable, int] = {}       # rows of the step in flight that still owe a token: id -> position
     in_flight: List[Hashable] = []           # requests of the step in flight
+    ahead: Optional[Dict[Hashable, int]] = None   # rows of a step planned ahead of it: id -> position
     steps = 0
     peak_pages = [0 for _ in figures.pools]
     peak_live = peak_tokens = 0
@@ -103,7 +107,8 @@ def verify_events(events: Iterable[tuple], figures: RunFigures) -> TraceReport:
         live = [t for t in requests.values() if t.state == "live"]
         return [sum(pool.pages_for(t.held_before, t.held) for t in live) for pool in figures.pools]
 
-    for index, event in enumerate(events):
+    events_list = list(events)
+    for index, event in enumerate(events_list):
         kind = event[0]
         if kind == "reject":
             rejected.append((event[1], event[2]))
@@ -122,6 +127,8 @@ def verify_events(events: Iterable[tuple], figures: RunFigures) -> TraceReport:
             if live > figures.max_live_requests:
                 fail(index, f"{live} live requests, the limit is {figures.max_live_requests}")
         elif kind == "preempt":
+            if ahead is not None:
+                fail(index, f"request {event[1]!r} preempted while a step is planned ahead")
             trace = known(index, event[1], "live")
             if event[1] in in_flight and event[1] in awaiting:
                 fail(index, f"request {event[1]!r} preempted while its row is in flight")
@@ -130,7 +137,42 @@ def verify_events(events: Iterable[tuple], figures: RunFigures) -> TraceReport:
                             f"{trace.prompt_tokens + len(trace.emitted)}")
             trace.state, trace.held = "queued", 0
             trace.preemptions += 1
+        elif kind == "ahead":
+            rows = event[1]
+            if ahead is not None:
+                fail(index, "a second step planned ahead")
+            if not in_flight or sorted(map(str, awaiting)) != sorted(map(str, in_flight)):
+                fail(index, "a step is planned ahead, but not every row of the step in flight owes a token")
+            if [name for name, _, _, _ in rows] != in_flight:
+                fail(index, "the step planned ahead does not hold the requests of the step in flight in their order")
+            live = [name for name, t in requests.items() if t.state == "live"]
+            if sorted(map(str, live)) != sorted(map(str, in_flight)):
+                fail(index, "a step is planned ahead although a live request is not in the step in flight")
+            steps += 1
+            ahead = {}
+            for name, start, count, sample in rows:
+                trace = known(index, name, "live")
+                if count != 1 or not sample:
+                    fail(index, f"request {name!r}: a step planned ahead holds one sampling row a request")
+                if start != trace.held or start != awaiting[name] + 1:
+                    fail(index, f"request {name!r} runs ahead from position {start}, it holds {trace.held} and is "
+                                f"owed the token of position {awaiting[name]}")
+                if len(trace.emitted) + 1 >= trace.max_new_tokens:
+                    fail(index, f"request {name!r} is planned beyond the last token it may be given")
+                trace.held_before = trace.held       # the step in flight is committed: what its window passed is back
+                trace.held += 1
+                trace.fed += 1
+                ahead[name] = start
+            peak_tokens = max(peak_tokens, len(rows))
+            if len(rows) > figures.max_step_tokens:
+                fail(index, f"a step of {len(rows)} tokens, the budget is {figures.max_step_tokens}")
+            for g, (pool, used) in enumerate(zip(figures.pools, pages_now())):
+                peak_pages[g] = max(peak_pages[g], used)
+                if used > pool.num_pages:
+                    fail(index, f"group {g} needs {used} pages, the pool has {pool.num_pages}")
         elif kind == "step":
+            if ahead is not None:
+                fail(index, "a step starts while another is planned ahead and not yet in flight")
             if awaiting:
                 fail(index, f"a step starts while rows of the last one still owe tokens: {sorted(map(str, awaiting))}")
             rows = event[1]
@@ -194,8 +236,18 @@ def verify_events(events: Iterable[tuple], figures: RunFigures) -> TraceReport:
             if reason == "eos" and not trace.emitted:
                 fail(index, f"request {name!r} finished on an end token it was never given")
             trace.state, trace.reason, trace.held = "finished", reason, 0
+            if ahead is not None:
+                ahead.pop(name, None)            # it drops out of the step ahead
         else:
             fail(index, f"unknown event {kind!r}")
+        # Once every row of the step in flight is answered (and the request of the last answer has had its chance
+        # to finish: its finish follows its token at once), the step planned ahead is the step in flight.
+        if ahead is not None and not awaiting and kind in ("token", "finish"):
+            following = events_list[index + 1] if index + 1 < len(events_list) else None
+            if not (following is not None and following[0] == "finish" and kind == "token" and following[1] == event[1]):
+                in_flight = [name for name in in_flight if name in ahead]
+                awaiting = dict(ahead)
+                ahead = None
     return TraceReport(requests, rejected, steps, peak_pages, peak_live, peak_tokens)
 
 

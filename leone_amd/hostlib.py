@@ -58,6 +58,8 @@ _PROTOTYPES = {
     "leone_scheduler_has_work": (c_int, [H]),
     "leone_scheduler_plan": (c_int, [H]),
     "leone_scheduler_planned": (c_int, [H, PI64, PI, PI, PI, c_int]),
+    "leone_scheduler_plan_ahead": (c_int, [H]),
+    "leone_scheduler_ahead": (c_int, [H, PI64, PI, PI, PI, c_int]),
     "leone_scheduler_complete": (c_int, [H, PI64, PI32, c_int]),
     "leone_scheduler_abort": (c_int, [H]),
     "leone_scheduler_history": (c_int, [H, c_int64, PI32, c_int]),

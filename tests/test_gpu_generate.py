@@ -116,6 +116,50 @@ def test_greedy_generation_at_the_widths_of_the_large_models(tmp_path):
             assert row[token] >= row.max() - 1.5e-2 * scale, (i, token, float(row[token]), float(row.max()))
 
 
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("temperature", [None, 0.9])
+def test_steps_issued_ahead_of_the_tokens_give_the_same_tokens(folders, tmp_path, dtype_name, temperature):
+    """Where device kernels choose the tokens, the next decode step is issued before the last step's tokens have
+    reached the host (they are fed from the device): the same tokens as step by step, with requests that end
+    on an end token at different times (their row in the step ahead is thrown away), with so few pages that
+    requests are preempted, greedy and with a temperature; the decision log still shows a sound run."""
+    from leone_amd.api import Runtime, sampling_params
+    from leone_amd.engine import trace_check
+    from leone_amd.engine.generate import Generator
+    from leone_amd.engine.scheduler import SchedulerPolicy
+    folder = folders["B"] if dtype_name == "float32" else make_model_dir(str(tmp_path / "m"), TINY["B"], 33, torch.bfloat16)
+    config = read_config(folder)
+    prompts = [random_tokens(70 + i, n, config["vocab_size"]) for i, n in enumerate([12, 31, 5, 44, 20])]
+    params = sampling_params(temperature=temperature, seed=99)
+    policy = SchedulerPolicy(max_live_requests=4, prefill_chunk_tokens=16, max_step_tokens=32)
+    runtime = Runtime.load(folder, dtype_name, num_pages=10, page_tokens=16, max_requests=4, poison_freed=True, policy=policy)
+    plain_run = runtime.generate_tokens(prompts, 40, params, eos_token_id=None, look_ahead=False)
+    assert runtime.last_stats.steps_ahead == 0 and runtime.last_stats.preemptions >= 1
+    ahead_run = runtime.generate_tokens(prompts, 40, params, eos_token_id=None)          # ahead by default
+    assert runtime.last_stats.steps_ahead > 10 and runtime.last_stats.preemptions >= 1
+    assert [r.tokens for r in ahead_run] == [r.tokens for r in plain_run]
+    # an end token that some requests meet early, some late and some never
+    seen = [t for r in plain_run for t in r.tokens[5:30]]
+    eos = max(set(seen), key=seen.count)
+    results = {}
+    for look_ahead in (False, True):
+        generator = Generator(runtime.engine, policy)
+        generator.look_ahead = look_ahead
+        for i, prompt in enumerate(prompts):
+            generator.submit(i, prompt, 40, params, eos)
+        finished = {f.id: f for f in generator.run()}
+        results[look_ahead] = [(finished[i].tokens, finished[i].reason) for i in range(len(prompts))]
+        report = trace_check.verify_events(generator.scheduler.events, trace_check.figures_of(generator.scheduler))
+        assert report.steps == generator.scheduler.stats.steps
+        assert (generator.stats.steps_ahead > 10) == look_ahead
+        assert any(kind == "ahead" for kind, *_ in generator.scheduler.events) == look_ahead
+        runtime.engine.cache.check()
+        assert not runtime.engine.cache.live_requests()
+    assert results[True] == results[False]
+    assert {reason for _, reason in results[True]} == {"eos", "length"}
+    assert any(tokens[-1] == eos and len(tokens) < 40 for tokens, _ in results[True])
+
+
 def test_temperature_sampling_matches_oracle_and_ignores_batching(folders):
     """Config B's workload: prompts 5/40/130, portions of 32, 24 tokens at temperature 0.8, seeded."""
     from leone_amd.api import Runtime, sampling_params

@@ -40,6 +40,44 @@ def run(scheduler, fail_at_step=None):
     return steps
 
 
+def run_ahead(scheduler, fail_at_step=None):
+    """The same with a step planned ahead wherever the scheduler allows one: the step that has run is completed
+    only after the next one has been planned and "launched" (its cache writes committed), as a caller does that
+    keeps the chosen tokens on the device.  Returns (steps, steps that were planned ahead)."""
+    steps = looked = 0
+    pending = None                                   # the step that has run and is not completed yet
+    while scheduler.has_work():
+        if pending is None:
+            pending = scheduler.plan()
+            steps += 1
+            for entry in pending:
+                assert scheduler.cache.length(entry.request) == entry.start
+                scheduler.cache.commit(entry.request, len(entry.tokens))
+        if fail_at_step == steps:
+            scheduler.abort()
+            pending = None
+            continue
+        ahead = scheduler.plan_ahead()
+        if ahead:
+            assert [(e.request, e.start, e.deferred) for e in ahead] == \
+                [(e.request, e.start + len(e.tokens), True) for e in pending]
+            steps += 1
+            looked += 1
+            for entry in ahead:
+                scheduler.cache.commit(entry.request, 1)
+            if fail_at_step == steps:                # the step ahead fails: both go
+                scheduler.abort()
+                pending = None
+                continue
+        sampled = {e.request: next_token(scheduler.live[e.request].tokens) for e in pending if e.sample}
+        scheduler.complete(sampled)
+        scheduler.cache.check()
+        live = scheduler.live
+        pending = [e for e in ahead if e.request in live] or None
+        assert steps < 100000
+    return steps, looked
+
+
 def isolated(prompt, n, eos=None):
     tokens = list(prompt)
     for _ in range(n):
@@ -221,7 +259,7 @@ def test_random_load_under_page_pressure(seed):
 
 # ---- the checker that works from the decision log alone ------------------------------------------
 
-def _loaded(seed, window=None):
+def _loaded(seed, window=None, ahead=False):
     from leone_amd.engine import trace_check
     rng = random.Random(500 + seed)
     page_tokens = rng.choice([4, 8])
@@ -239,17 +277,24 @@ def _loaded(seed, window=None):
             wanted[i] = (prompt, n)
     if seed % 2:
         s.cancel(3)
-    run(s, fail_at_step=7 if seed == 2 else None)
+    if ahead:
+        s.looked_ahead = run_ahead(s, fail_at_step=40 if seed == 2 else None)[1]
+    else:
+        run(s, fail_at_step=7 if seed == 2 else None)
     return s, wanted, trace_check
 
 
+@pytest.mark.parametrize("ahead", [False, True])
 @pytest.mark.parametrize("window", [None, 9])
 @pytest.mark.parametrize("seed", range(4))
-def test_the_log_alone_shows_a_sound_run(seed, window):
+def test_the_log_alone_shows_a_sound_run(seed, window, ahead):
     """Page conservation, budgets, one step in flight and contiguous positions are re-derived from the
     events by a checker that shares nothing with the scheduler, and the transcript it reads off the events
-    equals every request run alone (crates/leone/src/scheduler.rs:1349-1655)."""
-    s, wanted, trace_check = _loaded(seed, window)
+    equals every request run alone (crates/leone/src/scheduler.rs:1349-1655).  The same with a step planned
+    ahead of the tokens wherever the scheduler allows it: the tokens are the same, a request that ends on its
+    end token drops out of the step ahead, and a failed step takes the step ahead with it."""
+    s, wanted, trace_check = _loaded(seed, window, ahead)
+    assert not ahead or s.looked_ahead > 5
     figures = trace_check.figures_of(s)
     report = trace_check.verify_events(s.events, figures)
     assert report.steps == s.stats.steps and report.peak_live <= 4
@@ -298,3 +343,92 @@ def test_the_checker_refuses_a_log_that_breaks_a_rule():
         trace_check.verify_events(events, dataclasses.replace(figures, max_step_tokens=1))
     with pytest.raises(trace_check.TraceError, match="live requests"):
         trace_check.verify_events(events, dataclasses.replace(figures, max_live_requests=1))
+
+
+def test_a_step_is_planned_ahead_only_where_the_next_step_is_known():
+    s = make(pages=8, page_tokens=4, prefill_chunk_tokens=8, max_step_tokens=16, max_live_requests=2)
+    with pytest.raises(SchedulerError, match="no step is planned"):
+        s.plan_ahead()
+    assert s.submit(Request("a", list(range(12)), 6)) is None
+    s.plan()                                                           # a portion that does not end the prompt
+    s.cache.commit("a")
+    assert s.plan_ahead() == [] and s.cache.length("a") == 8
+    s.complete({})
+    s.plan()                                                           # the rest of the prompt: a token comes of it
+    with pytest.raises(SchedulerError, match="has not run"):
+        s.plan_ahead()
+    s.cache.commit("a")
+    free = s.cache.free_pages(0)
+    ahead = s.plan_ahead()
+    assert [(e.request, e.start, e.tokens, e.sample, e.deferred) for e in ahead] == [("a", 12, [0], True, True)]
+    assert s.cache.free_pages(0) == free - 1                           # position 12 opens a page: it is reserved
+    with pytest.raises(SchedulerError, match="already"):
+        s.plan_ahead()
+    with pytest.raises(SchedulerError, match="neither completed"):
+        s.plan()
+    s.cache.commit("a", 1)
+    assert s.complete({"a": 7}) == [] and s.history("a")[-1] == 7
+    # the step ahead is the planned one now; somebody in the queue with a place free: no looking ahead
+    assert s.submit(Request("b", [1, 2, 3], 9)) is None
+    assert s.plan_ahead() == []
+    s.complete({"a": 8})
+    both = s.plan()
+    assert [e.request for e in both] == ["a", "b"]
+    for e in both:
+        s.cache.commit(e.request)
+    # the queue is empty and both get a token: ahead, step after step, until "a" is one token from its sixth
+    token, given = 9, 2
+    while True:
+        ahead = s.plan_ahead()
+        if given + 1 >= 6:                         # the token the planned step is choosing is its last
+            assert ahead == []
+            break
+        assert [(e.request, e.start) for e in ahead] == [(e.request, e.start + len(e.tokens)) for e in both]
+        for e in ahead:
+            s.cache.commit(e.request, 1)
+        assert s.complete({"a": token, "b": token + 20}) == []
+        both, token, given = ahead, token + 1, given + 1
+    done = s.complete({"a": 50, "b": 51})
+    assert [f.id for f in done] == ["a"] and done[0].reason == "length" and done[0].tokens == [7, 8, 9, 10, 11, 50]
+    # an end token drops a request out of the step ahead, and what it held goes back
+    s2 = make(pages=8, page_tokens=4, max_live_requests=2)
+    s2.submit(Request("x", [1, 2, 3], 9, eos_token_id=5)), s2.submit(Request("y", [4, 5], 9, eos_token_id=5))
+    for e in s2.plan():
+        s2.cache.commit(e.request)
+    ahead = s2.plan_ahead()
+    assert len(ahead) == 2
+    for e in ahead:
+        s2.cache.commit(e.request, 1)
+    done = s2.complete({"x": 5, "y": 6})
+    assert [f.id for f in done] == ["x"] and done[0].reason == "eos" and not s2.cache.has("x")
+    assert [e.request for e in s2.plan_ahead()] == ["y"]               # the step that was ahead is the planned one: "y" alone
+    s2.cache.check()
+
+
+def test_the_checker_refuses_a_step_ahead_that_breaks_a_rule():
+    s, wanted, trace_check = _loaded(1, ahead=True)
+    figures = trace_check.figures_of(s)
+    events = s.events
+    trace_check.verify_events(events, figures)
+    first_ahead = next(i for i, e in enumerate(events) if e[0] == "ahead")
+    with_two = next(i for i, e in enumerate(events) if e[0] == "ahead" and len(e[1]) >= 2)
+
+    def broken(change):
+        changed = [list(e) if e[0] not in ("step", "ahead") else [e[0], [list(r) for r in e[1]]] for e in events]
+        change(changed)
+        with pytest.raises(trace_check.TraceError):
+            trace_check.verify_events([tuple(e) for e in changed], figures)
+
+    broken(lambda ev: ev.insert(first_ahead, ev[first_ahead]))                          # two steps ahead
+    broken(lambda ev: ev[with_two][1].pop())                                            # a request of the step in flight left out
+    broken(lambda ev: ev[with_two][1].reverse())                                        # another order than the step in flight
+    broken(lambda ev: ev[first_ahead][1][0].__setitem__(1, ev[first_ahead][1][0][1] + 1))   # a position skipped
+    broken(lambda ev: ev[first_ahead][1][0].__setitem__(2, 2))                          # two rows for a request
+    broken(lambda ev: ev.__setitem__(first_ahead, ["step", ev[first_ahead][1]]))        # an ordinary step before the tokens
+    broken(lambda ev: ev.insert(first_ahead + 1, ["preempt", ev[first_ahead][1][0][0], 1]))   # a decision while a step is ahead
+    # a step ahead after the first token of the step in flight has come: not every row owes its token
+    first_token_after = next(i for i in range(with_two, len(events)) if events[i][0] == "token")
+
+    def late(ev):
+        ev.insert(first_token_after + 1, ev.pop(with_two))
+    broken(late)
