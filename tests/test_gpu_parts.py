@@ -504,6 +504,30 @@ def test_toy_architecture_with_state_window_repeat_and_shared_cache(tmp_path, dt
         engine.release("p"), engine.release("c")
         engine.cache.check()
         assert all(engine.cache.free_pages(g) == 36 for g in range(3))
+        # The generation loop on this model (state, a window, pages of two sizes; no recording, one of its parts is
+        # not safe to record): steps issued ahead of the tokens give the tokens that steps one by one give, and
+        # the plain implementation's greedy choice in float32.
+        from leone_amd.engine.generate import Generator
+        from leone_amd.engine.scheduler import SchedulerPolicy
+        assert not engine.graphs
+        prompts = [requests["t0"][:19], requests["t1"][:7], requests["t3"][:30]]
+        outcomes = []
+        for look_ahead in (False, True):
+            generator = Generator(engine, SchedulerPolicy(max_live_requests=3, prefill_chunk_tokens=8, max_step_tokens=16))
+            generator.look_ahead = look_ahead
+            for i, prompt in enumerate(prompts):
+                generator.submit(i, prompt, 12, None, None)
+            finished = {f.id: f.tokens for f in generator.run()}
+            outcomes.append([finished[i] for i in range(len(prompts))])
+            assert (generator.stats.steps_ahead > 5) == look_ahead
+            engine.cache.check()
+        assert outcomes[0] == outcomes[1]
+        if dtype_name == "float32":
+            for prompt, tokens in zip(prompts, outcomes[1]):
+                history = list(prompt)
+                for token in tokens:
+                    assert int(toy_plain(weights, history)[-1].argmax()) == token
+                    history.append(token)
     finally:
         unregister_architecture("ToyForCausalLM")
         MIXERS.unregister("toy_decay")
