@@ -154,8 +154,7 @@ class _DecodeGraph:
         self.rows = rows
         self._pieces, self._tables = pieces, {g: pieces[5 + len(tilings) + g].view(rows, widths[g]) for g in range(groups)}
         self._engine_type = (engine.dtype, engine.device)
-        self.recordings: Dict[object, tuple] = {}     # context range -> (graph, its logits)
-        self.turn = 0
+        self.recordings: Dict[int, tuple] = {}        # context range -> (graph, its logits)
         self.copied = torch.cuda.Event()
 
     def context(self, bucket: int) -> StepContext:
@@ -211,7 +210,6 @@ class Engine:
         self.graphs = bool(graphs) and model.graph_safe
         self._decode_graphs: Dict[int, _DecodeGraph] = {}
         self._graph_pool = torch.cuda.graph_pool_handle() if self.graphs else None
-        self.twin_recordings = False
         self._staging: List[Optional[tuple]] = [None, None]
         self._staging_turn = 0
 
@@ -421,11 +419,7 @@ class Engine:
         if device_tokens is not None:                 # after the upload, on the same stream
             torch.clamp(device_tokens, 0, self.vocab_size - 1, out=state.tokens)
         bucket = context_bucket(packed.max_position + 1, self.max_context)
-        key = bucket
-        if self.twin_recordings:
-            state.turn ^= 1
-            key = (bucket, state.turn)
-        recording = state.recordings.get(key)
+        recording = state.recordings.get(bucket)
         if recording is None:
             # First step of this size and context range: run it for real on the static buffers, then record
             # the same calls for later steps.  Recording executes nothing, so the cache is written once.
@@ -439,7 +433,7 @@ class Engine:
             # (errors of the capture are this thread's: an engine in another thread goes on with its own work)
             with torch.cuda.graph(graph, pool=self._graph_pool, capture_error_mode="thread_local"), ops.one_stream():
                 recorded_logits = self.model.forward(state.tokens, context, caches)
-            state.recordings[key] = (graph, recorded_logits)
+            state.recordings[bucket] = (graph, recorded_logits)
         else:
             recording[0].replay()
             logits = recording[1]
