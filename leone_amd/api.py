@@ -110,12 +110,14 @@ class Runtime:
         return getattr(self.config, "eos_token_id", None)
 
     def generate_tokens(self, prompts: Sequence[Sequence[int]], max_new_tokens: int,
-                        sampling: Optional[SamplingParams] = None, eos_token_id: Union[int, None, str] = "config",
+                        sampling: Union[SamplingParams, Sequence[Optional[SamplingParams]], None] = None,
+                        eos_token_id: Union[int, None, str] = "config",
                         on_token: Optional[Callable[[Hashable, int], None]] = None,
                         logit_observer: Optional[Callable] = None,
                         profile_decode_steps: int = 0,
                         cancelled: Optional[Callable[[], bool]] = None, look_ahead: bool = True) -> List[GenerationResult]:
-        """Token ids in, token ids out, one result per prompt in order.  ``profile_decode_steps``: time
+        """Token ids in, token ids out, one result per prompt in order.  ``sampling``: one policy for all prompts,
+        or a list with one for each (None: greedy).  ``profile_decode_steps``: time
         that many decode steps operation by operation (they run without graph replay); the result is
         left in ``last_decode_profile``.  ``cancelled``: asked before every step; a yes ends every request
         with the tokens it has (the reference's cancellation flag, crates/leone-cli/src/main.rs:1600-1602).

@@ -180,9 +180,19 @@ int leone_sample_temperature(const float* logits, const double* temperature, con
 
 // The `wanted` best finite logits of each row (higher first, lower id on a tie), best first, for a sampler
 // that truncates to the k best before anything else.  out_values and out_ids have
-// leone_top_candidates_max() places a row; out_count[row] is the number filled, or -1 for a row that has
-// to be selected another way.
+// leone_top_candidates_max() places a row; out_count[row] is the number filled (fewer than wanted only if the
+// row has fewer finite logits).
 int leone_top_candidates_max();
 int leone_top_candidates(const float* logits, float* out_values, int* out_ids, int* out_count, int rows, int vocab,
                          int wanted, hipStream_t stream);
+
+// One token a row by temperature sampling with truncation stages, the first of which keeps the k best logits
+// (k at most leone_top_candidates_max()): selection, stages and draw in one launch, in double, by the host
+// sampler's rules.  `params` holds leone_sample_truncated_params() doubles a row: temperature, uniform value,
+// number of stages (1..leone_sample_truncated_stages(); 0: the row is skipped and gets -1), then (kind, value)
+// for each stage, kind 0 top-k, 1 top-p, 2 min-p.  out[row] is -1 for a row without a finite logit.
+int leone_sample_truncated_stages();
+int leone_sample_truncated_params();
+int leone_sample_truncated(const float* logits, const double* params, int* out, int rows, int vocab,
+                           hipStream_t stream);
 }

@@ -239,49 +239,234 @@ __device__ inline void sort_keys_descending(unsigned long long* keys, int n) {
     __syncthreads();
 }
 
-__global__ void __launch_bounds__(kSampleThreads)
-top_candidates_kernel(const float* __restrict__ logits, int k, float* __restrict__ out_values,
-                      int* __restrict__ out_ids, int* __restrict__ out_count, int vocab) {
-    __shared__ unsigned long long keys[kCandidateRoom];
-    __shared__ int collected;
-    const float* row = logits + static_cast<long>(blockIdx.x) * vocab;
+// The greatest key of the workgroup, for every thread; `scratch` holds one place a wave.
+__device__ inline unsigned long long block_max_key(unsigned long long mine, unsigned long long* scratch) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const unsigned long long other = __shfl_xor(mine, off, kWave);
+        mine = other > mine ? other : mine;
+    }
+    __syncthreads();                                        // what the call before this one left has been read
+    if (threadIdx.x % kWave == 0) scratch[threadIdx.x / kWave] = mine;
+    __syncthreads();
+    unsigned long long total = scratch[0];
+    for (int w = 1; w < kSampleThreads / kWave; ++w) total = scratch[w] > total ? scratch[w] : total;
+    return total;
+}
 
+struct Selection {
+    int kept;   // keys[0, kept) are the row's best keys, the best first: min(k, size) of them
+    int size;   // finite logits in the row
+};
+
+// The selection described above; every thread of the workgroup calls it.  `keys` has kCandidateRoom places,
+// `counters` two.  A row whose collection does not fit the room is selected the slow way instead, one key
+// after the other, each the greatest that lies behind the one before: k walks over the row, for rows that
+// are laid out against the deal of ids to threads and for no others.
+__device__ inline Selection select_best(const float* __restrict__ row, int vocab, int k, unsigned long long* keys,
+                                        int* counters) {
     unsigned long long best = 0ull;
+    int finite = 0;
     for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
         const unsigned long long key = candidate_key(row[i], i);
+        finite += key != 0ull;
         best = key > best ? key : best;
     }
     keys[threadIdx.x] = best;
-    if (threadIdx.x == 0) collected = 0;
+    if (threadIdx.x == 0) counters[0] = counters[1] = 0;
     sort_keys_descending(keys, kSampleThreads);
     // 0 if fewer than k threads own a finite value: then every finite value is collected.
     const unsigned long long bound = keys[k - 1];
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) finite += __shfl_xor(finite, off, kWave);
+    if (threadIdx.x % kWave == 0) atomicAdd(&counters[1], finite);
     __syncthreads();
 
     for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
         const unsigned long long key = candidate_key(row[i], i);
         if (key != 0ull && key >= bound) {
-            const int at = atomicAdd(&collected, 1);
+            const int at = atomicAdd(&counters[0], 1);
             if (at < kCandidateRoom) keys[at] = key;
         }
     }
     __syncthreads();
-    const int found = collected;
-    if (found > kCandidateRoom) {
-        if (threadIdx.x == 0) out_count[blockIdx.x] = -1;
-        return;
+    const int found = counters[0], size = counters[1];
+    if (found <= kCandidateRoom) {
+        int room = 1;
+        while (room < found) room <<= 1;
+        for (int i = found + threadIdx.x; i < room; i += kSampleThreads) keys[i] = 0ull;
+        sort_keys_descending(keys, room);
+        return Selection{found < k ? found : k, size};
     }
-    int room = 1;
-    while (room < found) room <<= 1;
-    for (int i = found + threadIdx.x; i < room; i += kSampleThreads) keys[i] = 0ull;
-    sort_keys_descending(keys, room);
-    const int kept = found < k ? found : k;
-    for (int i = threadIdx.x; i < kept; i += kSampleThreads) {
-        const int id = static_cast<int>(0xffffffffu - static_cast<unsigned>(keys[i] & 0xffffffffull));
+    unsigned long long* scratch = keys + kCandidateMaxK;
+    unsigned long long behind = ~0ull;
+    int kept = 0;
+    for (; kept < k; ++kept) {
+        unsigned long long mine = 0ull;
+        for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
+            const unsigned long long key = candidate_key(row[i], i);
+            if (key < behind && key > mine) mine = key;
+        }
+        mine = block_max_key(mine, scratch);
+        if (mine == 0ull) break;
+        if (threadIdx.x == 0) keys[kept] = mine;
+        behind = mine;
+    }
+    __syncthreads();
+    return Selection{kept, size};
+}
+
+__device__ inline int candidate_id(unsigned long long key) {
+    return static_cast<int>(0xffffffffu - static_cast<unsigned>(key & 0xffffffffull));
+}
+
+__global__ void __launch_bounds__(kSampleThreads)
+top_candidates_kernel(const float* __restrict__ logits, int k, float* __restrict__ out_values,
+                      int* __restrict__ out_ids, int* __restrict__ out_count, int vocab) {
+    __shared__ unsigned long long keys[kCandidateRoom];
+    __shared__ int counters[2];
+    const float* row = logits + static_cast<long>(blockIdx.x) * vocab;
+    const Selection chosen = select_best(row, vocab, k, keys, counters);
+    for (int i = threadIdx.x; i < chosen.kept; i += kSampleThreads) {
+        const int id = candidate_id(keys[i]);
         out_ids[static_cast<long>(blockIdx.x) * kCandidateMaxK + i] = id;
         out_values[static_cast<long>(blockIdx.x) * kCandidateMaxK + i] = row[id];
     }
-    if (threadIdx.x == 0) out_count[blockIdx.x] = kept;
+    if (threadIdx.x == 0) out_count[blockIdx.x] = chosen.kept;
+}
+
+// ---- temperature sampling with truncation stages, top-k first -------------------------------------------
+//
+// The host sampler's rules (csrc/host/sampler.cpp, after crates/leone/src/sampler.rs:502-606, 843-858) for the
+// policies whose first stage keeps the k best logits, k at most kCandidateMaxK: those k are all the sampler
+// ever looks at.  One workgroup a row selects them as above; the weights exp(l/t - l_max/t) are taken in
+// double, one thread a candidate; one thread then walks the stages in the order given, each on the
+// renormalised result of the one before, each keeping at least one token, with the sums taken from the left
+// as the host takes them; the token is the first of the kept ones, in id order, whose running share exceeds
+// the uniform value, the last with a share above zero if rounding leaves none.  A row without a finite logit
+// gives -1.
+//
+// A row's parameters are kDrawParams doubles: temperature, uniform value, the number of stages (0: the row
+// is not for this kernel and gets -1), then for each stage its kind (0 top-k, 1 top-p, 2 min-p) and value.
+constexpr int kDrawStages = 8;
+constexpr int kDrawParams = 3 + 2 * kDrawStages;
+
+__global__ void __launch_bounds__(kSampleThreads)
+sample_truncated_kernel(const float* __restrict__ logits, const double* __restrict__ params, int* __restrict__ out,
+                        int vocab) {
+    __shared__ unsigned long long keys[kCandidateRoom];
+    __shared__ int counters[2];
+    __shared__ double share[kCandidateMaxK];
+    __shared__ double mass;
+    __shared__ int keep;
+    const float* row = logits + static_cast<long>(blockIdx.x) * vocab;
+    const double* mine = params + static_cast<long>(blockIdx.x) * kDrawParams;
+    // The caller checks the table before it uploads it; whatever the memory holds, the kernel stays in its arrays.
+    const int stages = mine[2] >= 1.0 ? (mine[2] < kDrawStages ? static_cast<int>(mine[2]) : kDrawStages) : 0;
+    const bool cut = stages > 0 && static_cast<int>(mine[3]) == 0 && mine[4] >= 1.0 && mine[4] <= kCandidateMaxK;
+    if (!cut) {
+        if (threadIdx.x == 0) out[blockIdx.x] = -1;
+        return;
+    }
+    const int k = static_cast<int>(mine[4]);
+    const Selection chosen = select_best(row, vocab, k, keys, counters);
+    const int have = chosen.kept;
+    if (have == 0) {
+        if (threadIdx.x == 0) out[blockIdx.x] = -1;
+        return;
+    }
+    const double t = mine[0];
+    if (static_cast<int>(threadIdx.x) < have) {
+        const double shift = static_cast<double>(row[candidate_id(keys[0])]) / t;
+        share[threadIdx.x] = exp(static_cast<double>(row[candidate_id(keys[threadIdx.x])]) / t - shift);
+    }
+    // The candidates once more in id order, each with its rank: the order of the draw, and of the whole row's sum.
+    unsigned long long* by_id = keys + kCandidateMaxK;
+    int room = 1;
+    while (room < have) room <<= 1;
+    __syncthreads();
+    if (static_cast<int>(threadIdx.x) < room)
+        by_id[threadIdx.x] = static_cast<int>(threadIdx.x) < have
+                                 ? (keys[threadIdx.x] << 32) | static_cast<unsigned long long>(threadIdx.x) : 0ull;
+    sort_keys_descending(by_id, room);
+
+    // A first stage that cuts makes the sum over the whole row cancel in the renormalisation that follows: the
+    // weights stand for themselves.  Otherwise every finite logit is a candidate and the sum is theirs, in id
+    // order, compensated.
+    if (threadIdx.x == 0) {
+        double total = 1.0;
+        if (!(k < chosen.size)) {
+            double carry = 0.0;
+            total = 0.0;
+            for (int j = 0; j < have; ++j) {
+                const double y = share[by_id[j] & 0xffffffffull] - carry, sum = total + y;
+                carry = (sum - total) - y;
+                total = sum;
+            }
+        }
+        mass = total;
+    }
+    __syncthreads();
+    if (static_cast<int>(threadIdx.x) < have) share[threadIdx.x] /= mass;
+    __syncthreads();
+
+    int kept = chosen.size;                                 // tokens of the present distribution
+    for (int s = 0; s < stages; ++s) {
+        if (threadIdx.x == 0) {
+            const int kind = static_cast<int>(mine[3 + 2 * s]);
+            const double value = mine[4 + 2 * s];
+            const int seen = kept < have ? kept : have;
+            int n = seen;
+            if (kind == 0) {
+                n = value >= static_cast<double>(kept) ? kept : static_cast<int>(value);
+            } else if (kind == 1) {
+                double sum = 0.0;
+                for (int i = 0; i < seen; ++i) {
+                    sum += share[i];
+                    if (sum >= value) {
+                        n = i + 1;
+                        break;
+                    }
+                }
+            } else {
+                const double floor = value * share[0];
+                for (int i = 0; i < seen; ++i)
+                    if (!(share[i] >= floor)) {
+                        n = i;
+                        break;
+                    }
+            }
+            n = n < 1 ? 1 : n;
+            n = n > have ? have : n;                        // the first stage has cut to what is held, or the row is held whole
+            double sum = 0.0;
+            for (int i = 0; i < n; ++i) sum += share[i];
+            mass = sum;
+            keep = n;
+        }
+        __syncthreads();
+        const int n = keep;
+        if (n < kept) {
+            if (static_cast<int>(threadIdx.x) < n) share[threadIdx.x] /= mass;
+            kept = n;
+        }
+        __syncthreads();
+    }
+
+    if (threadIdx.x == 0) {
+        const double u = mine[1];
+        double running = 0.0;
+        int token = -1;
+        for (int j = 0; j < have; ++j) {
+            const int rank = static_cast<int>(by_id[j] & 0xffffffffull);
+            if (rank >= kept) continue;
+            const double p = share[rank];
+            if (!(p > 0.0)) continue;
+            token = candidate_id(keys[rank]);
+            running += p;
+            if (u < running) break;
+        }
+        out[blockIdx.x] = token;
+    }
 }
 
 }  // namespace leone
@@ -293,8 +478,7 @@ extern "C" int leone_top_candidates_max() { return kCandidateMaxK; }
 // For each row the `wanted` (1..leone_top_candidates_max()) best finite logits in the sampler's order,
 // best first (so that the first j of them are the row's j best): out_values and out_ids hold
 // leone_top_candidates_max() places a row, out_count[row] says how many are filled (fewer than wanted if
-// the row has fewer finite logits), or is -1 if the row's values are laid out so that the selection did
-// not fit: such a row must be selected another way.
+// the row has fewer finite logits).
 extern "C" int leone_top_candidates(const float* logits, float* out_values, int* out_ids, int* out_count, int rows,
                                     int vocab, int wanted, hipStream_t stream) {
     LEONE_REQUIRE(logits && out_values && out_ids && out_count, "top_candidates: null pointer");
@@ -303,6 +487,23 @@ extern "C" int leone_top_candidates(const float* logits, float* out_values, int*
                   "top_candidates: %d wanted, at most %d can be selected", wanted, kCandidateMaxK);
     top_candidates_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, wanted, out_values, out_ids, out_count, vocab);
     LEONE_LAUNCH_CHECK("top_candidates");
+    return 0;
+}
+
+extern "C" int leone_sample_truncated_stages() { return kDrawStages; }
+extern "C" int leone_sample_truncated_params() { return kDrawParams; }
+
+// One token a row by temperature sampling with truncation stages of which the first keeps the k best logits,
+// k at most leone_top_candidates_max().  `params` holds leone_sample_truncated_params() doubles a row:
+// temperature (above zero), the uniform value in [0, 1), the number of stages (1..leone_sample_truncated_stages();
+// 0 marks a row that is not to be sampled and gets -1), then a (kind, value) pair for each stage: 0 top-k,
+// 1 top-p, 2 min-p; the first stage's kind is 0.  out[row] is -1 for a row without a finite logit.
+extern "C" int leone_sample_truncated(const float* logits, const double* params, int* out, int rows, int vocab,
+                                      hipStream_t stream) {
+    LEONE_REQUIRE(logits && params && out, "sample_truncated: null pointer");
+    LEONE_REQUIRE(rows > 0 && vocab > 0, "sample_truncated: rows %d vocab %d must be positive", rows, vocab);
+    sample_truncated_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, params, out, vocab);
+    LEONE_LAUNCH_CHECK("sample_truncated");
     return 0;
 }
 

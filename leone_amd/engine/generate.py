@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import time
 from dataclasses import dataclass
-from typing import Callable, Dict, Hashable, List, Optional, Sequence
+from typing import Callable, Dict, Hashable, List, Optional, Sequence, Union
 
 import torch
 
@@ -16,7 +16,6 @@ from .. import ops
 from ..ops.profile import Recorder
 from ..sampling import rng
 from ..sampling.sampler import (MirostatState, SamplerError, SamplingParams, apply_penalties, native_eligible,
-                                preselect_count, sample_candidates_native,
                                 sample as host_sample, sample_rows_native)
 from .engine import Engine, StepEntry
 from .scheduler import Finished, PlannedEntry, Reject, Request, Scheduler, SchedulerPolicy
@@ -57,14 +56,51 @@ class RequestRejected(ValueError):
         self.reason = reason
 
 
+def device_kind(policy: SamplingParams) -> Optional[str]:
+    """Which device kernel chooses a row's token under this policy: "greedy", "temperature" (nothing cut), or
+    "truncated" (stages that begin with a top-k the selection kernel can serve); None if the row has to come
+    to the host: penalties, a Mirostat controller, other stages."""
+    if policy.penalties_active or policy.mirostat is not None:
+        return None
+    if policy.greedy:
+        return "greedy"
+    if not policy.truncations:
+        return "temperature"
+    return "truncated" if ops.truncated_draw_supported(policy.truncations) else None
+
+
+def _tokens_on_device(logits: torch.Tensor, rows: Sequence[PlannedEntry], policies: Sequence[SamplingParams],
+                      kinds: Sequence[Optional[str]]) -> torch.Tensor:
+    """int32 [rows] on the device: for every row whose kind is not None the token its kernel chose (-1 for a row
+    without a finite logit); the other rows hold nothing of meaning.  Each kernel runs once, over all rows."""
+    chosen = {}
+    if "greedy" in kinds:
+        chosen["greedy"] = ops.argmax(logits)
+    draws = [rng.uniform(p.seed, e.sample_position) if kind in ("temperature", "truncated") else 0.0
+             for p, e, kind in zip(policies, rows, kinds)]
+    if "temperature" in kinds:
+        table = torch.tensor([[p.temperature if kind == "temperature" else 1.0 for p, kind in zip(policies, kinds)], draws],
+                             dtype=torch.float64).to(logits.device)
+        chosen["temperature"] = ops.sample_temperature(logits, table[0], table[1])
+    if "truncated" in kinds:
+        chosen["truncated"] = ops.sample_truncated(
+            logits, [(p.temperature, u, p.truncations) if kind == "truncated" else None
+                     for p, u, kind in zip(policies, draws, kinds)])
+    names = list(chosen)
+    out = chosen[names[0]]
+    for name in names[1:]:
+        out = torch.where(torch.tensor([kind == name for kind in kinds], device=logits.device), chosen[name], out)
+    return out
+
+
 def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params: Dict[Hashable, SamplingParams],
                   history: Callable[[Hashable], Sequence[int]],
                   controllers: Optional[Dict[Hashable, MirostatState]] = None) -> Dict[Hashable, int]:
     """One token per sampled entry; ``logits`` has one row per such entry, in order.
 
-    Greedy and plain-temperature rows are chosen by the device kernels; rows with truncation stages
-    or penalties are copied to the host and go through the double-precision sampler, which reads a
-    request's tokens so far through ``history``."""
+    Greedy rows, plain-temperature rows and rows whose stages begin with a top-k of modest size are chosen by
+    the device kernels; rows with other stages, penalties or a controller are copied to the host and go through
+    the double-precision sampler, which reads a request's tokens so far through ``history``."""
     rows = [e for e in entries if e.sample]
     if not rows:
         return {}
@@ -72,39 +108,13 @@ def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params:
     for p in policies:
         p.validate()
     out: Dict[Hashable, int] = {}
-    on_device = [i for i, p in enumerate(policies) if p.device_eligible]
-    greedy = [i for i in on_device if policies[i].greedy]
-    scaled = [i for i in on_device if not policies[i].greedy]
-    if greedy:
-        picked = ops.argmax(logits).cpu().tolist()
-        for i in greedy:
-            out[rows[i].request] = picked[i]
-    if scaled:
-        temps = torch.tensor([policies[i].temperature if i in scaled else 1.0 for i in range(len(rows))],
-                             dtype=torch.float64, device=logits.device)
-        draws = torch.tensor([rng.uniform(policies[i].seed, rows[i].sample_position) for i in range(len(rows))],
-                             dtype=torch.float64, device=logits.device)
-        picked = ops.sample_temperature(logits, temps, draws).cpu().tolist()
-        for i in scaled:
-            out[rows[i].request] = picked[i]
-    host_rows = [i for i in range(len(rows)) if i not in on_device]
-    # Rows that keep their k best logits before anything else: the device selects those, and only they
-    # come to the host.  A row the selection could not serve goes the long way with the others.
-    narrow = [i for i in host_rows if preselect_count(policies[i], ops.TOP_CANDIDATES_MAX)
-              and rows[i].request not in (controllers or {})]
-    if narrow:
-        index = torch.tensor(narrow, dtype=torch.long, device=logits.device)
-        values, ids, counts = ops.top_candidates(logits.index_select(0, index),
-                                                 [preselect_count(policies[i], ops.TOP_CANDIDATES_MAX) for i in narrow])
-        served = [k for k in range(len(narrow)) if counts[k] >= 0]
-        if served:
-            drawn = sample_candidates_native(values[served], ids[served], counts[served],
-                                             [policies[narrow[k]] for k in served],
-                                             [rows[narrow[k]].sample_position for k in served])
-            for k, token in zip(served, drawn):
-                out[rows[narrow[k]].request] = token
-        done = {narrow[k] for k in served}
-        host_rows = [i for i in host_rows if i not in done]
+    kinds = [None if e.request in (controllers or {}) else device_kind(p) for e, p in zip(rows, policies)]
+    if any(kinds):
+        picked = _tokens_on_device(logits, rows, policies, kinds).cpu().tolist()
+        for e, kind, token in zip(rows, kinds, picked):
+            if kind is not None:
+                out[e.request] = token
+    host_rows = [i for i, kind in enumerate(kinds) if kind is None]
     if host_rows:
         index = torch.tensor(host_rows, dtype=torch.long, device=logits.device)
         copied = logits.index_select(0, index).cpu().numpy()
@@ -136,25 +146,16 @@ def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params:
 def choose_on_device(logits: torch.Tensor, entries: Sequence[PlannedEntry],
                      params: Dict[Hashable, SamplingParams]) -> Optional[torch.Tensor]:
     """The tokens of the sampled entries as int32 on the device, in their order, without a copy to the host; None
-    unless every one of them is chosen by a device kernel (greedy, or plain temperature).  -1 stands for a row
-    without a finite logit."""
+    unless every one of them is chosen by a device kernel (``device_kind``).  -1 stands for a row without a
+    finite logit."""
     rows = [e for e in entries if e.sample]
     policies = [params[e.request] or SamplingParams() for e in rows]
-    if not rows or not all(p.device_eligible for p in policies):
-        return None
     for p in policies:
         p.validate()
-    scaled = [not p.greedy for p in policies]
-    if not any(scaled):
-        return ops.argmax(logits)
-    temps = torch.tensor([p.temperature if s else 1.0 for p, s in zip(policies, scaled)], dtype=torch.float64,
-                         device=logits.device)
-    draws = torch.tensor([rng.uniform(p.seed, e.sample_position) for p, e in zip(policies, rows)], dtype=torch.float64,
-                         device=logits.device)
-    drawn = ops.sample_temperature(logits, temps, draws)
-    if all(scaled):
-        return drawn
-    return torch.where(torch.tensor(scaled, device=logits.device), drawn, ops.argmax(logits))
+    kinds = [device_kind(p) for p in policies]
+    if not rows or not all(kinds):
+        return None
+    return _tokens_on_device(logits, rows, policies, kinds)
 
 
 @dataclass
@@ -347,7 +348,7 @@ class Generator:
 
 
 def generate_tokens(engine: Engine, prompts: Sequence[Sequence[int]], max_new_tokens: int,
-                    sampling: Optional[SamplingParams] = None, eos_token_id: Optional[int] = None,
+                    sampling: Union[SamplingParams, Sequence[Optional[SamplingParams]], None] = None, eos_token_id: Optional[int] = None,
                     policy: Optional[SchedulerPolicy] = None,
                     on_token: Optional[Callable[[Hashable, int], None]] = None,
                     logit_observer: Optional[Callable[[Hashable, int, torch.Tensor], None]] = None,
@@ -355,13 +356,17 @@ def generate_tokens(engine: Engine, prompts: Sequence[Sequence[int]], max_new_to
                     cancelled: Optional[Callable[[], bool]] = None, look_ahead: bool = True):
     """Generates for every prompt (token ids); returns results in prompt order and the run's statistics.
     ``cancelled`` is asked before every step; once it says yes, every request ends as "cancelled" with the
-    tokens it has.  ``look_ahead``: see ``Generator``."""
+    tokens it has.  ``look_ahead``: see ``Generator``.  ``sampling`` is one policy for all prompts or a list
+    with one for each (None in it: greedy)."""
+    each = list(sampling) if isinstance(sampling, (list, tuple)) else [sampling] * len(prompts)
+    if len(each) != len(prompts):
+        raise ValueError(f"{len(prompts)} prompts, {len(each)} sampling policies")
     generator = Generator(engine, policy)
     generator.look_ahead = look_ahead
     generator.logit_observer = logit_observer
     generator.decode_profile = decode_profile
     for i, prompt in enumerate(prompts):
-        generator.submit(i, prompt, max_new_tokens, sampling, eos_token_id)
+        generator.submit(i, prompt, max_new_tokens, each[i], eos_token_id)
     finished = {f.id: f for f in generator.run(on_token, cancelled)}
     results = [GenerationResult(i, list(finished[i].prompt), list(finished[i].tokens), finished[i].reason)
                for i in range(len(prompts))]

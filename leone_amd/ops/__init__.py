@@ -9,6 +9,7 @@ from __future__ import annotations
 from typing import Optional
 
 import functools
+import math
 import threading
 import weakref
 
@@ -962,8 +963,7 @@ def top_candidates(logits: torch.Tensor, wanted) -> tuple:
     id on a tie), selected on the device and brought to the host in one copy.
 
     Returns numpy arrays: values float32 [rows, TOP_CANDIDATES_MAX], ids int32 likewise, counts int32
-    [rows]; row r is filled up to counts[r], and counts[r] is -1 for a row whose values are laid out so
-    that the selection did not fit, which the caller has to select from the whole row."""
+    [rows]; row r is filled up to counts[r] (fewer than it wanted only if it has fewer finite logits)."""
     if library().leone_top_candidates_max() != TOP_CANDIDATES_MAX:
         raise KernelError("the kernel library was built for another number of candidates")
     rows, vocab = logits.shape
@@ -980,6 +980,55 @@ def top_candidates(logits: torch.Tensor, wanted) -> tuple:
     counts = np.where(host[:rows] < 0, -1, np.minimum(host[:rows], np.asarray(wanted, dtype=np.int32)))
     return (host[rows:rows + room].view("float32").reshape(rows, TOP_CANDIDATES_MAX),
             host[rows + room:].reshape(rows, TOP_CANDIDATES_MAX), counts)
+
+
+TRUNCATED_STAGES = 8         # most truncation stages of a row that is drawn on the device (checked against the library)
+TRUNCATION_KINDS = {"top_k": 0, "top_p": 1, "min_p": 2}
+
+
+def truncated_draw_supported(stages) -> bool:
+    """Whether ``sample_truncated`` serves a row with these (stage, value) pairs: top-k first with k at most
+    TOP_CANDIDATES_MAX, then top-k, top-p and min-p in any order, TRUNCATED_STAGES at most in all."""
+    stages = list(stages)
+    return (0 < len(stages) <= TRUNCATED_STAGES and all(name in TRUNCATION_KINDS for name, _ in stages)
+            and stages[0][0] == "top_k" and 1 <= int(stages[0][1]) <= TOP_CANDIDATES_MAX)
+
+
+def sample_truncated(logits: torch.Tensor, draws) -> torch.Tensor:
+    """One token a row (int32 on the device) by temperature sampling with truncation stages, top-k first:
+    selection, stages and draw in one launch, nothing comes to the host.  ``draws`` holds for each row either
+    None (the row is skipped and gets -1) or (temperature, uniform value, [(stage, value), ...]) with stages
+    that ``truncated_draw_supported`` accepts.  -1 also for a row without a finite logit."""
+    lib = library()
+    if (lib.leone_sample_truncated_stages() != TRUNCATED_STAGES or lib.leone_top_candidates_max() != TOP_CANDIDATES_MAX
+            or lib.leone_sample_truncated_params() != 3 + 2 * TRUNCATED_STAGES):
+        raise KernelError("the kernel library was built for another table of truncation stages")
+    rows, vocab = logits.shape
+    draws = list(draws)
+    if len(draws) != rows:
+        raise KernelError(f"sample_truncated: {rows} rows of logits, {len(draws)} draws")
+    table = np.zeros((rows, 3 + 2 * TRUNCATED_STAGES), dtype=np.float64)
+    for r, draw in enumerate(draws):
+        if draw is None:
+            continue
+        temperature, uniform, stages = draw
+        stages = list(stages)
+        if not truncated_draw_supported(stages):
+            raise KernelError(f"sample_truncated: row {r}: stages {stages} are not drawn on the device")
+        if not (math.isfinite(temperature) and temperature > 0.0 and 0.0 <= uniform < 1.0):
+            raise KernelError(f"sample_truncated: row {r}: temperature {temperature} or uniform value {uniform} out of range")
+        for name, value in stages:
+            if name == "top_k" and not (value >= 1 and int(value) == value) or name != "top_k" and not 0.0 < value <= 1.0:
+                raise KernelError(f"sample_truncated: row {r}: {name} {value} out of range")
+        table[r, 0], table[r, 1], table[r, 2] = temperature, uniform, len(stages)
+        for s, (name, value) in enumerate(stages):
+            # top-k beyond every vocabulary keeps everything: the value only has to stay a number the kernel can compare
+            table[r, 3 + 2 * s], table[r, 4 + 2 * s] = TRUNCATION_KINDS[name], min(float(value), 2.0 ** 31)
+    params = torch.from_numpy(table).to(logits.device)
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    call("leone_sample_truncated", _dev(logits, "sample logits", torch.float32),
+         _dev(params, "sample stages", torch.float64), _dev(out, "sample out"), rows, vocab, _stream())
+    return out
 
 
 __all__ = [name for name in dir() if not name.startswith("_")]

@@ -51,6 +51,7 @@ _PROTOTYPES = {
     "leone_library_product_forget": [c_int, c_int, c_int, c_int, c_int],
     "leone_sample_temperature": [P, P, P, P, P, P, P, P, c_int, c_int, P],
     "leone_top_candidates": [P, P, P, P, c_int, c_int, c_int, P],
+    "leone_sample_truncated": [P, P, P, c_int, c_int, P],
 }
 
 
@@ -76,6 +77,10 @@ def library() -> ctypes.CDLL:
             lib.leone_top_candidates_max.argtypes = []
             lib.leone_argmax_chunk.restype = c_int
             lib.leone_argmax_chunk.argtypes = []
+            lib.leone_sample_truncated_stages.restype = c_int
+            lib.leone_sample_truncated_stages.argtypes = []
+            lib.leone_sample_truncated_params.restype = c_int
+            lib.leone_sample_truncated_params.argtypes = []
             lib.leone_peak_mfma_flops.restype = ctypes.c_double
             lib.leone_peak_mfma_flops.argtypes = [c_int, c_int]
             lib.leone_gemm_rows_max_rows.restype = c_int

@@ -103,11 +103,6 @@ class SamplingParams:
     def penalties_active(self) -> bool:
         return self.counting_active or self.dry_active
 
-    @property
-    def device_eligible(self) -> bool:
-        """Greedy or plain temperature without penalties can be sampled by the device kernels."""
-        return not self.truncations and not self.penalties_active and self.mirostat is None
-
 
 def apply_penalties(logits: np.ndarray, history: Sequence[int], params: SamplingParams) -> np.ndarray:
     """Positive logits of seen tokens are divided by the repeat penalty, negative ones multiplied;
@@ -332,33 +327,6 @@ def native_eligible(params: SamplingParams) -> bool:
     """Temperature with no stages other than top-k, top-p and min-p: the host library draws such rows
     without sorting the whole vocabulary (``csrc/host/sampler.cpp``, the same rules)."""
     return not params.greedy and all(stage in _NATIVE_STAGES for stage, _ in params.truncations)
-
-
-def preselect_count(params: SamplingParams, limit: int) -> int:
-    """If the policy truncates to its k best tokens before anything else and nothing changes the logits
-    first, k (when it is at most ``limit``): then those k logits are all the sampler ever looks at, and
-    they can be selected on the device.  0 otherwise."""
-    if not native_eligible(params) or params.penalties_active or not params.truncations:
-        return 0
-    stage, value = params.truncations[0]
-    return int(value) if stage == "top_k" and 1 <= int(value) <= limit else 0
-
-
-def sample_candidates_native(values: np.ndarray, ids: np.ndarray, counts: Sequence[int],
-                             params: Sequence[SamplingParams], positions: Sequence[int]) -> List[int]:
-    """One token for each row from its preselected candidates (``values``/``ids`` [rows, room], row r
-    filled up to counts[r], in any order): the candidates are put in id order, which is the order the
-    sampler walks a row in, and drawn from as a row of their own."""
-    rows, room = values.shape
-    table = np.full((rows, room), -np.inf, dtype=np.float32)
-    order = []
-    for r in range(rows):
-        n = int(counts[r])
-        by_id = np.argsort(ids[r, :n], kind="stable")
-        table[r, :n] = values[r, :n][by_id]
-        order.append(ids[r, :n][by_id])
-    picked = sample_rows_native(table, params, positions)
-    return [int(order[r][at]) if at >= 0 else -1 for r, at in enumerate(picked)]
 
 
 def sample_rows_native(logits: np.ndarray, params: Sequence[SamplingParams], positions: Sequence[int]) -> List[int]:

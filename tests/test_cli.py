@@ -39,7 +39,16 @@ def test_truncation_flags_keep_their_order():
         ["generate", "-m", "x", "--prompt-tokens", "1", "-n", "2", "--dry-multiplier", "0.8", "--dry-base", "2",
          "--dry-allowed-length", "3", "--dry-window", "16"]))
     assert (dry.dry_multiplier, dry.dry_base, dry.dry_allowed_length, dry.dry_window) == (0.8, 2.0, 3, 16)
-    assert dry.dry_active and not dry.device_eligible and not params.dry_active
+    assert dry.dry_active and dry.penalties_active and not params.dry_active
+    from leone_amd.engine.generate import device_kind
+    from leone_amd.sampling.sampler import SamplingParams
+    assert device_kind(dry) is None and device_kind(SamplingParams()) == "greedy"
+    assert device_kind(params) is None                                        # top-p comes first: the whole row is needed
+    assert device_kind(SamplingParams(temperature=0.7)) == "temperature"
+    assert device_kind(SamplingParams(temperature=0.7, truncations=[("top_k", 40.0), ("top_p", 0.9)])) == "truncated"
+    assert device_kind(SamplingParams(temperature=0.7, truncations=[("top_k", 300.0)])) is None
+    assert device_kind(SamplingParams(temperature=0.7, truncations=[("top_k", 40.0), ("tfs", 0.9)])) is None
+    assert device_kind(SamplingParams(temperature=0.7, truncations=[("top_k", 40.0)], mirostat=(3.0, 0.1))) is None
 
 
 def test_bench_refuses_several_gpus(capsys):

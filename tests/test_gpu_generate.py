@@ -338,38 +338,96 @@ def test_top_candidates_kernel():
     for t in range(39):
         against[1, t::1024] = 50.0 + t
     values, ids, counts = ops.top_candidates(torch.from_numpy(against).cuda(), [40, 40])
-    assert counts[0] == 40 and counts[1] == -1
+    assert counts.tolist() == [40, 40]
+    for r in range(2):
+        assert ids[r, :40].tolist() == best_in_sampler_order(against[r], 40)
+        assert np.array_equal(values[r, :40], against[r, ids[r, :40]])
     with pytest.raises(ops.KernelError):
         ops.top_candidates(torch.from_numpy(against).cuda(), [40, 257])
 
 
-def test_truncated_sampling_takes_the_candidates_and_matches_the_whole_row(folders, monkeypatch):
-    """top-k first: the device selects, the host draws from the selection; the tokens are those of the
-    sampler over whole rows, alone or in a batch, and a row the selection hands back goes the long way."""
+def test_truncated_sampling_kernel_against_the_double_precision_sampler():
+    """Selection, stages and draw in one launch against the plain sampler over the whole row: stages in every
+    order behind the first top-k, ties across the cut, values that are not finite, rows with fewer finite values
+    than k (the whole row's sum counts then), k of 1 and of 256, a uniform value of 0, rows that are skipped, a
+    row laid out against the selection's deal of ids to threads."""
+    from leone_amd import ops
+    from leone_amd.sampling.sampler import SamplingParams, distribution, select
+    gen = np.random.default_rng(23)
+    checked = 0
+    for vocab in (1, 3, 50, 777, 4097, 151936):
+        for case in range(6 if vocab > 10000 else 12):
+            rows = 8
+            logits = (gen.standard_normal((rows, vocab)) * gen.choice([0.3, 2.0, 8.0])).astype(np.float32)
+            logits[1] = np.round(logits[1])                                      # ties, also across the cut
+            logits[2, ::2] = np.nan
+            logits[3, 1::5] = -np.inf
+            logits[4] = 1.5
+            if vocab > 1024:
+                logits[5, :] = -5.0
+                for t in range(39):
+                    logits[5, t::1024] = 50.0 + t * 0.01
+            draws = []
+            for r in range(rows):
+                later = [(str(name), float(gen.integers(1, 300)) if name == "top_k" else float(gen.uniform(0.02, 1.0)))
+                         for name in gen.permutation(["top_p", "min_p", "top_k", "top_p"])[:int(gen.integers(0, 5))]]
+                k = float(gen.choice([1, 2, 12, 40, 255, 256]))
+                u = 0.0 if r == 6 and case == 0 else float(gen.random())
+                draws.append((float(gen.choice([0.3, 0.8, 1.0, 2.5])), u, [("top_k", k)] + later))
+            draws[7] = None
+            got = ops.sample_truncated(torch.from_numpy(logits).cuda(), draws).cpu().tolist()
+            assert got[7] == -1
+            for r in range(7):
+                t, u, stages = draws[r]
+                if not np.isfinite(logits[r]).any():
+                    assert got[r] == -1
+                    continue
+                probs = distribution(logits[r], SamplingParams(temperature=t, truncations=stages))
+                want = select(probs, u)
+                if got[r] != want:      # only a draw within rounding of a boundary may differ, and then by one neighbour
+                    eligible = np.nonzero(probs > 0.0)[0]
+                    cumulative = np.cumsum(probs[eligible])
+                    edge = cumulative[np.searchsorted(eligible, min(got[r], want))]
+                    assert probs[got[r]] > 0.0 and abs(edge - u) < 1e-9, (vocab, case, r, got[r], want)
+                checked += 1
+    assert checked > 300
+    nothing = torch.full((2, 50), float("nan"), device="cuda")
+    assert ops.sample_truncated(nothing, [(1.0, 0.5, [("top_k", 5.0)])] * 2).tolist() == [-1, -1]
+    for bad in ([("top_p", 0.9)], [("top_k", 257.0)], [("top_k", 5.0), ("tfs", 0.5)], [("top_k", 5.0)] * 9, []):
+        assert not ops.truncated_draw_supported(bad)
+        with pytest.raises(ops.KernelError):
+            ops.sample_truncated(nothing, [(1.0, 0.5, bad), None])
+    with pytest.raises(ops.KernelError):
+        ops.sample_truncated(nothing, [(0.0, 0.5, [("top_k", 5.0)]), None])
+    with pytest.raises(ops.KernelError):
+        ops.sample_truncated(nothing, [(1.0, 1.0, [("top_k", 5.0)]), None])
+
+
+def test_truncated_sampling_on_the_device_matches_the_whole_row_on_the_host(folders, monkeypatch):
+    """top-k first: the device selects, cuts and draws; the tokens are those of the host sampler over whole rows,
+    alone, in a batch, beside greedy and plain-temperature requests, and with steps issued ahead."""
     from leone_amd import ops
     from leone_amd.api import Runtime, sampling_params
-    from leone_amd.engine import generate
     folder = folders["B"]
     config = read_config(folder)
     prompts = [random_tokens(90 + i, n, config["vocab_size"]) for i, n in enumerate([9, 33, 70])]
     params = sampling_params(temperature=0.9, seed=4321, top_k=12, top_p=0.85, min_p=0.02)
+    mixed = [params, None, sampling_params(temperature=1.1, seed=5)]
     runtime = Runtime.load(folder, "float32", max_tokens=3 * 128, page_tokens=16, max_requests=3)
     calls = []
-    real = ops.top_candidates
-    monkeypatch.setattr(ops, "top_candidates", lambda *a: calls.append(1) or real(*a))
+    real = ops.sample_truncated
+    monkeypatch.setattr(ops, "sample_truncated", lambda *a: calls.append(1) or real(*a))
     narrow = [r.tokens for r in runtime.generate_tokens(prompts, 20, params, eos_token_id=None)]
-    assert len(calls) >= 20
-    monkeypatch.setattr(generate, "preselect_count", lambda policy, limit: 0)      # everything the long way
+    assert len(calls) >= 20 and runtime.last_stats.steps_ahead >= 15
+    one_by_one = [r.tokens for r in runtime.generate_tokens(prompts, 20, params, eos_token_id=None, look_ahead=False)]
+    assert one_by_one == narrow and runtime.last_stats.steps_ahead == 0
+    beside = [r.tokens for r in runtime.generate_tokens(prompts, 20, mixed, eos_token_id=None)]
+    assert beside[0] == narrow[0] and runtime.last_stats.steps_ahead >= 15
     calls.clear()
+    monkeypatch.setattr(ops, "truncated_draw_supported", lambda stages: False)      # everything the long way
     whole = [r.tokens for r in runtime.generate_tokens(prompts, 20, params, eos_token_id=None)]
-    assert not calls and whole == narrow
-    monkeypatch.undo()
-    # every row handed back: the same tokens again
-    def refused(logits, wanted):
-        values, ids, counts = real(logits, wanted)
-        return values, ids, np.full_like(counts, -1)
-    monkeypatch.setattr(ops, "top_candidates", refused)
-    assert [r.tokens for r in runtime.generate_tokens(prompts, 20, params, eos_token_id=None)] == narrow
+    assert not calls and whole == narrow and runtime.last_stats.steps_ahead == 0
+    assert [r.tokens for r in runtime.generate_tokens(prompts, 20, mixed, eos_token_id=None)] == beside
 
 
 def test_command_line_generate(folders, tmp_path):

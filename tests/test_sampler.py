@@ -203,43 +203,3 @@ def test_native_rows_against_the_general_sampler_and_the_oracle():
             assert got[r] == select(distribution(logits[r], policies[r]), u), (vocab, r)
     assert not native_eligible(SamplingParams(temperature=1.0, truncations=[("tfs", 0.9)]))
     assert sample_rows_native(np.full((1, 7), np.nan, dtype=np.float32), [SamplingParams(temperature=1.0)], [0]) == [-1]
-
-
-def test_candidates_draw_what_the_whole_row_draws():
-    """A policy whose first stage keeps the k best: drawing from those k alone, given in any order, is
-    drawing from the row (the selection here is a plain sort; the device's own is tested on the GPU)."""
-    from leone_amd.sampling.sampler import preselect_count, sample_candidates_native, sample_rows_native
-    gen = np.random.default_rng(99)
-    assert preselect_count(SamplingParams(temperature=1.0, truncations=[("top_k", 40), ("top_p", 0.9)]), 256) == 40
-    assert preselect_count(SamplingParams(temperature=1.0, truncations=[("top_p", 0.9), ("top_k", 40)]), 256) == 0
-    assert preselect_count(SamplingParams(temperature=1.0, truncations=[("top_k", 300)]), 256) == 0
-    assert preselect_count(SamplingParams(temperature=1.0, truncations=[("top_k", 40)], repeat_penalty=1.2), 256) == 0
-    assert preselect_count(SamplingParams(temperature=1.0, truncations=[("top_k", 40)], dry_multiplier=0.5), 256) == 0
-    assert preselect_count(SamplingParams(truncations=[("top_k", 40)]), 256) == 0          # greedy
-    for case in range(40):
-        vocab = int(gen.choice([3, 50, 5000]))
-        rows = 4
-        logits = (gen.standard_normal((rows, vocab)) * gen.choice([0.2, 2.0, 8.0])).astype(np.float32)
-        logits[1] = np.round(logits[1])                                      # ties, also across the cut
-        logits[2, ::2] = np.nan
-        policies = []
-        for r in range(rows):
-            later = [(str(name), float(gen.uniform(0.05, 1.0))) for name in gen.permutation(["top_p", "min_p"])
-                     [:int(gen.integers(0, 3))]]
-            policies.append(SamplingParams(temperature=float(gen.choice([0.3, 0.8, 1.5])), seed=int(gen.integers(0, 2**60)),
-                                           truncations=[("top_k", float(gen.integers(1, 60)))] + later))
-        positions = [int(p) for p in gen.integers(0, 5000, rows)]
-        room = 64
-        values = np.zeros((rows, room), dtype=np.float32)
-        ids = np.zeros((rows, room), dtype=np.int32)
-        counts = np.zeros(rows, dtype=np.int32)
-        for r in range(rows):
-            k = preselect_count(policies[r], room)
-            finite = [i for i in range(vocab) if np.isfinite(logits[r, i])]
-            finite.sort(key=lambda i: (-float(logits[r, i]), i))
-            best = [finite[i] for i in gen.permutation(min(k, len(finite)))]     # in no particular order
-            counts[r] = len(best)
-            ids[r, :len(best)] = best
-            values[r, :len(best)] = logits[r, best]
-        assert sample_candidates_native(values, ids, counts, policies, positions) == \
-            sample_rows_native(logits, policies, positions), case
