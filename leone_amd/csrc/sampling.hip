@@ -202,13 +202,15 @@ temperature_pick_kernel(const float* __restrict__ logits, const double* __restri
 // lower id on a tie.  A logit and its id become one 64-bit key whose unsigned order is that order
 // (0 for a value that is not finite, behind every finite one), so that selection is a sort of integers.
 //
-// One workgroup a row.  Every thread finds the best key among the ids it owns (t, t + 1024, ...); the
-// k-th best of these 1024 keys is a bound that the row's k-th best key cannot lie behind.  A second walk
+// One workgroup a row.  Every thread finds the best key among the ids it owns (four neighbours out of every 4,096),
+// four neighbouring threads make a cell; the k-th best of the 256 cells' keys is a bound that the row's k-th best
+// key cannot lie behind.  A second walk
 // collects every key not behind the bound (for k <= 256 and a vocabulary of 150,000 a few hundred), the
 // collection is sorted and its first k keys are the result.  A row whose collection would not fit
-// (values arranged against the deal) reports -1 and is left to the host.
+// (values arranged against the deal) is selected key by key instead.
 constexpr int kCandidateMaxK = 256;
 constexpr int kCandidateRoom = 4096;
+constexpr int kCellThreads = 4;                              // threads whose ids make one cell
 
 __device__ inline unsigned long long candidate_key(float v, int id) {
     v += 0.0f;                                              // -0 and +0 are one value
@@ -218,25 +220,22 @@ __device__ inline unsigned long long candidate_key(float v, int id) {
     return (static_cast<unsigned long long>(ordered) << 32) | (0xffffffffu - static_cast<unsigned>(id));
 }
 
-// Sorts keys[0, n) (n a power of two) so that the greatest comes first; every thread of the workgroup calls it.
-__device__ inline void sort_keys_descending(unsigned long long* keys, int n) {
-    for (int width = 2; width <= n; width <<= 1) {
-        for (int stride = width >> 1; stride > 0; stride >>= 1) {
-            __syncthreads();
-            for (int i = threadIdx.x; i < n; i += kSampleThreads) {
-                const int partner = i ^ stride;
-                if (partner > i) {
-                    const unsigned long long a = keys[i], b = keys[partner];
-                    const bool descending = (i & width) == 0;
-                    if (descending ? a < b : a > b) {
-                        keys[i] = b;
-                        keys[partner] = a;
-                    }
-                }
-            }
-        }
+__device__ inline int candidate_id(unsigned long long key) {
+    return static_cast<int>(0xffffffffu - static_cast<unsigned>(key & 0xffffffffull));
+}
+
+// How many of keys[0, n) are greater than `key`: its place when the keys are put in falling order (the keys of
+// finite logits are all different).  Every lane reads the same place at a time, which shared memory serves as one
+// read; for the few hundred keys this is asked of it is much cheaper than a sort with a barrier a step.
+__device__ inline int rank_among(const unsigned long long* keys, int n, unsigned long long key) {
+    int greater = 0;
+    int i = 0;
+    for (; i + 2 <= n; i += 2) {
+        const ulonglong2 two = *reinterpret_cast<const ulonglong2*>(keys + i);
+        greater += (two.x > key) + (two.y > key);
     }
-    __syncthreads();
+    if (i < n) greater += keys[i] > key;
+    return greater;
 }
 
 // The greatest key of the workgroup, for every thread; `scratch` holds one place a wave.
@@ -259,43 +258,121 @@ struct Selection {
     int size;   // finite logits in the row
 };
 
-// The selection described above; every thread of the workgroup calls it.  `keys` has kCandidateRoom places,
-// `counters` two.  A row whose collection does not fit the room is selected the slow way instead, one key
-// after the other, each the greatest that lies behind the one before: k walks over the row, for rows that
-// are laid out against the deal of ids to threads and for no others.
-__device__ inline Selection select_best(const float* __restrict__ row, int vocab, int k, unsigned long long* keys,
-                                        int* counters) {
-    unsigned long long best = 0ull;
-    int finite = 0;
-    for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
-        const unsigned long long key = candidate_key(row[i], i);
-        finite += key != 0ull;
-        best = key > best ? key : best;
+// Thread t owns the ids 4 q .. 4 q + 3 of every q with q % 1024 == t.  The four logits at ids 4 q .. 4 q + 3, NaN
+// (which never counts) beyond the row's end; one 16-byte load where the row allows it.
+__device__ inline float4 row_quad(const float* __restrict__ row, int q, int vocab, bool aligned) {
+    const int id = 4 * q;
+    if (aligned && id + 4 <= vocab) return *reinterpret_cast<const float4*>(row + id);
+    float4 v;
+    v.x = id < vocab ? row[id] : NAN;
+    v.y = id + 1 < vocab ? row[id + 1] : NAN;
+    v.z = id + 2 < vocab ? row[id + 2] : NAN;
+    v.w = id + 3 < vocab ? row[id + 3] : NAN;
+    return v;
+}
+
+// Calls use(value, id) for every id this thread owns, in rising order, eight quads' loads on their way at a time;
+// beyond the row's end the value is NaN.
+template <typename Use>
+__device__ inline void for_own_ids(const float* __restrict__ row, int vocab, Use use) {
+    const bool aligned = (reinterpret_cast<unsigned long long>(row) & 15ull) == 0ull;
+    const int quads = (vocab + 3) / 4;
+    constexpr int kAhead = 8;
+    for (int q0 = threadIdx.x; q0 < quads; q0 += kAhead * kSampleThreads) {
+        float4 v[kAhead];
+#pragma unroll
+        for (int a = 0; a < kAhead; ++a) {
+            const int q = q0 + a * kSampleThreads;
+            v[a] = q < quads ? row_quad(row, q, vocab, aligned) : float4{NAN, NAN, NAN, NAN};
+        }
+#pragma unroll
+        for (int a = 0; a < kAhead; ++a) {
+            const int id = 4 * (q0 + a * kSampleThreads);
+            use(v[a].x, id);
+            use(v[a].y, id + 1);
+            use(v[a].z, id + 2);
+            use(v[a].w, id + 3);
+        }
     }
-    keys[threadIdx.x] = best;
-    if (threadIdx.x == 0) counters[0] = counters[1] = 0;
-    sort_keys_descending(keys, kSampleThreads);
-    // 0 if fewer than k threads own a finite value: then every finite value is collected.
-    const unsigned long long bound = keys[k - 1];
+}
+
+__device__ inline bool is_finite(float v) { return (__float_as_uint(v) & 0x7f800000u) != 0x7f800000u; }
+
+// The selection described above; every thread of the workgroup calls it.  `keys` has kCandidateRoom places,
+// `counters` two, `bound_at` one.  A row whose collection does not fit the room is selected the slow way instead,
+// one key after the other, each the greatest that lies behind the one before: k walks over the row, for rows that
+// are laid out against the deal of ids to cells and for no others.
+//
+// The walks compare logits as numbers (a greater value, or an equal one at a lower id, is the greater key) and
+// make keys only of what they keep: the walks are bound by their arithmetic, not by memory.
+__device__ inline Selection select_best(const float* __restrict__ row, int vocab, int k, unsigned long long* keys,
+                                        int* counters, unsigned long long* bound_at) {
+    static_assert(kSampleThreads / kCellThreads == kCandidateMaxK, "one cell for each candidate that may be asked for");
+    float best_value = 0.f;
+    int best_id = -1, finite = 0;
+    for_own_ids(row, vocab, [&](float v, int id) {
+        const bool counts = is_finite(v);
+        finite += counts;
+        if (counts && (best_id < 0 || v > best_value)) {      // ids come in rising order: of equal values the first stays
+            best_value = v;
+            best_id = id;
+        }
+    });
+    // A cell is kCellThreads neighbouring threads; its best key goes to keys[cell].
+    unsigned long long best = best_id < 0 ? 0ull : candidate_key(best_value, best_id);
+#pragma unroll
+    for (int off = 1; off < kCellThreads; off <<= 1) {
+        const unsigned long long other = __shfl_xor(best, off, kWave);
+        best = other > best ? other : best;
+    }
+    if (threadIdx.x % kCellThreads == 0) keys[threadIdx.x / kCellThreads] = best;
+    if (threadIdx.x == 0) {
+        counters[0] = counters[1] = 0;
+        *bound_at = 0ull;
+    }
+    __syncthreads();
+    // The k-th best of the cells' bests: 0 if fewer than k cells hold a finite value, then every finite value is
+    // collected.
+    if (threadIdx.x < kCandidateMaxK) {
+        const unsigned long long mine = keys[threadIdx.x];
+        if (mine != 0ull && rank_among(keys, kCandidateMaxK, mine) == k - 1) *bound_at = mine;
+    }
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) finite += __shfl_xor(finite, off, kWave);
     if (threadIdx.x % kWave == 0) atomicAdd(&counters[1], finite);
     __syncthreads();
+    const unsigned long long bound = *bound_at;
+    __syncthreads();                                        // the cells' bests have been read: their places are free
 
-    for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
-        const unsigned long long key = candidate_key(row[i], i);
-        if (key != 0ull && key >= bound) {
+    const bool all = bound == 0ull;
+    const int bound_id = candidate_id(bound);
+    const float bound_value = all ? 0.f : row[bound_id];
+    for_own_ids(row, vocab, [&](float v, int id) {
+        if (is_finite(v) && (all || v > bound_value || (v == bound_value && id <= bound_id))) {
             const int at = atomicAdd(&counters[0], 1);
-            if (at < kCandidateRoom) keys[at] = key;
+            if (at < kCandidateRoom) keys[at] = candidate_key(v, id);
         }
-    }
+    });
     __syncthreads();
     const int found = counters[0], size = counters[1];
     if (found <= kCandidateRoom) {
-        int room = 1;
-        while (room < found) room <<= 1;
-        for (int i = found + threadIdx.x; i < room; i += kSampleThreads) keys[i] = 0ull;
-        sort_keys_descending(keys, room);
+        // every collected key finds its place by itself; the first k places are the result
+        unsigned long long mine[kCandidateRoom / kSampleThreads];
+        int place[kCandidateRoom / kSampleThreads];
+#pragma unroll
+        for (int n = 0; n < kCandidateRoom / kSampleThreads; ++n) {
+            const int i = threadIdx.x + n * kSampleThreads;
+            place[n] = k;
+            if (i < found) {
+                mine[n] = keys[i];
+                place[n] = rank_among(keys, found, mine[n]);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int n = 0; n < kCandidateRoom / kSampleThreads; ++n)
+            if (place[n] < k) keys[place[n]] = mine[n];
+        __syncthreads();
         return Selection{found < k ? found : k, size};
     }
     unsigned long long* scratch = keys + kCandidateMaxK;
@@ -303,10 +380,10 @@ __device__ inline Selection select_best(const float* __restrict__ row, int vocab
     int kept = 0;
     for (; kept < k; ++kept) {
         unsigned long long mine = 0ull;
-        for (int i = threadIdx.x; i < vocab; i += kSampleThreads) {
-            const unsigned long long key = candidate_key(row[i], i);
+        for_own_ids(row, vocab, [&](float v, int id) {
+            const unsigned long long key = candidate_key(v, id);
             if (key < behind && key > mine) mine = key;
-        }
+        });
         mine = block_max_key(mine, scratch);
         if (mine == 0ull) break;
         if (threadIdx.x == 0) keys[kept] = mine;
@@ -316,17 +393,14 @@ __device__ inline Selection select_best(const float* __restrict__ row, int vocab
     return Selection{kept, size};
 }
 
-__device__ inline int candidate_id(unsigned long long key) {
-    return static_cast<int>(0xffffffffu - static_cast<unsigned>(key & 0xffffffffull));
-}
-
 __global__ void __launch_bounds__(kSampleThreads)
 top_candidates_kernel(const float* __restrict__ logits, int k, float* __restrict__ out_values,
                       int* __restrict__ out_ids, int* __restrict__ out_count, int vocab) {
-    __shared__ unsigned long long keys[kCandidateRoom];
+    __shared__ __align__(16) unsigned long long keys[kCandidateRoom];
     __shared__ int counters[2];
+    __shared__ unsigned long long bound;
     const float* row = logits + static_cast<long>(blockIdx.x) * vocab;
-    const Selection chosen = select_best(row, vocab, k, keys, counters);
+    const Selection chosen = select_best(row, vocab, k, keys, counters, &bound);
     for (int i = threadIdx.x; i < chosen.kept; i += kSampleThreads) {
         const int id = candidate_id(keys[i]);
         out_ids[static_cast<long>(blockIdx.x) * kCandidateMaxK + i] = id;
@@ -354,8 +428,10 @@ constexpr int kDrawParams = 3 + 2 * kDrawStages;
 __global__ void __launch_bounds__(kSampleThreads)
 sample_truncated_kernel(const float* __restrict__ logits, const double* __restrict__ params, int* __restrict__ out,
                         int vocab) {
-    __shared__ unsigned long long keys[kCandidateRoom];
+    __shared__ __align__(16) unsigned long long keys[kCandidateRoom];
     __shared__ int counters[2];
+    __shared__ unsigned long long bound;
+    __shared__ int by_id[kCandidateMaxK];
     __shared__ double share[kCandidateMaxK];
     __shared__ double mass;
     __shared__ int keep;
@@ -369,7 +445,7 @@ sample_truncated_kernel(const float* __restrict__ logits, const double* __restri
         return;
     }
     const int k = static_cast<int>(mine[4]);
-    const Selection chosen = select_best(row, vocab, k, keys, counters);
+    const Selection chosen = select_best(row, vocab, k, keys, counters, &bound);
     const int have = chosen.kept;
     if (have == 0) {
         if (threadIdx.x == 0) out[blockIdx.x] = -1;
@@ -380,15 +456,15 @@ sample_truncated_kernel(const float* __restrict__ logits, const double* __restri
         const double shift = static_cast<double>(row[candidate_id(keys[0])]) / t;
         share[threadIdx.x] = exp(static_cast<double>(row[candidate_id(keys[threadIdx.x])]) / t - shift);
     }
-    // The candidates once more in id order, each with its rank: the order of the draw, and of the whole row's sum.
-    unsigned long long* by_id = keys + kCandidateMaxK;
-    int room = 1;
-    while (room < have) room <<= 1;
+    // The candidates once more in id order: by_id[n] is the rank of the candidate with the n-th lowest id.  The
+    // order of the draw, and of the whole row's sum.
+    if (static_cast<int>(threadIdx.x) < have) {
+        const unsigned my_id = static_cast<unsigned>(keys[threadIdx.x] & 0xffffffffull);   // the greater, the lower the id
+        int lower = 0;
+        for (int i = 0; i < have; ++i) lower += static_cast<unsigned>(keys[i] & 0xffffffffull) > my_id;
+        by_id[lower] = threadIdx.x;
+    }
     __syncthreads();
-    if (static_cast<int>(threadIdx.x) < room)
-        by_id[threadIdx.x] = static_cast<int>(threadIdx.x) < have
-                                 ? (keys[threadIdx.x] << 32) | static_cast<unsigned long long>(threadIdx.x) : 0ull;
-    sort_keys_descending(by_id, room);
 
     // A first stage that cuts makes the sum over the whole row cancel in the renormalisation that follows: the
     // weights stand for themselves.  Otherwise every finite logit is a candidate and the sum is theirs, in id
@@ -399,7 +475,7 @@ sample_truncated_kernel(const float* __restrict__ logits, const double* __restri
             double carry = 0.0;
             total = 0.0;
             for (int j = 0; j < have; ++j) {
-                const double y = share[by_id[j] & 0xffffffffull] - carry, sum = total + y;
+                const double y = share[by_id[j]] - carry, sum = total + y;
                 carry = (sum - total) - y;
                 total = sum;
             }
@@ -457,7 +533,7 @@ sample_truncated_kernel(const float* __restrict__ logits, const double* __restri
         double running = 0.0;
         int token = -1;
         for (int j = 0; j < have; ++j) {
-            const int rank = static_cast<int>(by_id[j] & 0xffffffffull);
+            const int rank = by_id[j];
             if (rank >= kept) continue;
             const double p = share[rank];
             if (!(p > 0.0)) continue;

@@ -69,28 +69,53 @@ def device_kind(policy: SamplingParams) -> Optional[str]:
     return "truncated" if ops.truncated_draw_supported(policy.truncations) else None
 
 
-def _tokens_on_device(logits: torch.Tensor, rows: Sequence[PlannedEntry], policies: Sequence[SamplingParams],
-                      kinds: Sequence[Optional[str]]) -> torch.Tensor:
-    """int32 [rows] on the device: for every row whose kind is not None the token its kernel chose (-1 for a row
-    without a finite logit); the other rows hold nothing of meaning.  Each kernel runs once, over all rows."""
-    chosen = {}
-    if "greedy" in kinds:
-        chosen["greedy"] = ops.argmax(logits)
-    draws = [rng.uniform(p.seed, e.sample_position) if kind in ("temperature", "truncated") else 0.0
-             for p, e, kind in zip(policies, rows, kinds)]
-    if "temperature" in kinds:
-        table = torch.tensor([[p.temperature if kind == "temperature" else 1.0 for p, kind in zip(policies, kinds)], draws],
-                             dtype=torch.float64).to(logits.device)
-        chosen["temperature"] = ops.sample_temperature(logits, table[0], table[1])
-    if "truncated" in kinds:
-        chosen["truncated"] = ops.sample_truncated(
-            logits, [(p.temperature, u, p.truncations) if kind == "truncated" else None
-                     for p, u, kind in zip(policies, draws, kinds)])
-    names = list(chosen)
-    out = chosen[names[0]]
-    for name in names[1:]:
-        out = torch.where(torch.tensor([kind == name for kind in kinds], device=logits.device), chosen[name], out)
-    return out
+class DeviceChoice:
+    """What the device kernels need to choose a step's tokens, uploaded before the step's logits exist (so that
+    the upload does not stand between the step and the kernels that choose): temperatures and uniform values, the
+    table of truncation stages, and which kernel's answer each row takes.  ``kinds`` holds for every sampled row
+    its ``device_kind`` or None; rows with None get nothing of meaning."""
+
+    def __init__(self, rows: Sequence[PlannedEntry], policies: Sequence[SamplingParams],
+                 kinds: Sequence[Optional[str]], device):
+        self.kinds = list(kinds)
+        draws = [rng.uniform(p.seed, e.sample_position) if kind in ("temperature", "truncated") else 0.0
+                 for p, e, kind in zip(policies, rows, kinds)]
+        self.scaled = self.truncated = None
+        if "temperature" in kinds:
+            self.scaled = torch.tensor([[p.temperature if kind == "temperature" else 1.0 for p, kind in zip(policies, kinds)],
+                                        draws], dtype=torch.float64).to(device)
+        if "truncated" in kinds:
+            self.truncated = ops.truncated_table([(p.temperature, u, p.truncations) if kind == "truncated" else None
+                                                  for p, u, kind in zip(policies, draws, kinds)], device)
+        self.names = [name for name in ("greedy", "temperature", "truncated") if name in kinds]
+        self.masks = {name: torch.tensor([kind == name for kind in kinds], device=device) for name in self.names[1:]}
+
+    def choose(self, logits: torch.Tensor) -> torch.Tensor:
+        """int32 [rows] on the device: the token each row's kernel chose, -1 for a row without a finite logit.
+        Each kernel runs once, over all rows."""
+        out = None
+        for name in self.names:
+            if name == "greedy":
+                chosen = ops.argmax(logits)
+            elif name == "temperature":
+                chosen = ops.sample_temperature(logits, self.scaled[0], self.scaled[1])
+            else:
+                chosen = ops.sample_truncated(logits, self.truncated)
+            out = chosen if out is None else torch.where(self.masks[name], chosen, out)
+        return out
+
+
+def plan_device_choice(entries: Sequence[PlannedEntry], params: Dict[Hashable, SamplingParams],
+                       device) -> Optional[DeviceChoice]:
+    """The ``DeviceChoice`` of a step if device kernels choose every one of its tokens; None otherwise."""
+    rows = [e for e in entries if e.sample]
+    policies = [params[e.request] or SamplingParams() for e in rows]
+    for p in policies:
+        p.validate()
+    kinds = [device_kind(p) for p in policies]
+    if not rows or not all(kinds):
+        return None
+    return DeviceChoice(rows, policies, kinds, device)
 
 
 def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params: Dict[Hashable, SamplingParams],
@@ -110,7 +135,7 @@ def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params:
     out: Dict[Hashable, int] = {}
     kinds = [None if e.request in (controllers or {}) else device_kind(p) for e, p in zip(rows, policies)]
     if any(kinds):
-        picked = _tokens_on_device(logits, rows, policies, kinds).cpu().tolist()
+        picked = DeviceChoice(rows, policies, kinds, logits.device).choose(logits).cpu().tolist()
         for e, kind, token in zip(rows, kinds, picked):
             if kind is not None:
                 out[e.request] = token
@@ -148,14 +173,8 @@ def choose_on_device(logits: torch.Tensor, entries: Sequence[PlannedEntry],
     """The tokens of the sampled entries as int32 on the device, in their order, without a copy to the host; None
     unless every one of them is chosen by a device kernel (``device_kind``).  -1 stands for a row without a
     finite logit."""
-    rows = [e for e in entries if e.sample]
-    policies = [params[e.request] or SamplingParams() for e in rows]
-    for p in policies:
-        p.validate()
-    kinds = [device_kind(p) for p in policies]
-    if not rows or not all(kinds):
-        return None
-    return _tokens_on_device(logits, rows, policies, kinds)
+    choice = plan_device_choice(entries, params, logits.device)
+    return None if choice is None else choice.choose(logits)
 
 
 @dataclass
@@ -223,13 +242,16 @@ class Generator:
             and not self.decode_profile.done else None
         flight = _InFlight(plan, None, None, decoding, time.perf_counter(), recorder)
         entries = [StepEntry(e.request, e.tokens, [len(e.tokens) - 1] if e.sample else []) for e in plan]
+        # What the kernels that choose the tokens need goes to the device before the step, not between the two.
+        choice = None
+        if recorder is None and self.logit_observer is None and not any(e.request in self.controllers for e in plan):
+            choice = plan_device_choice(plan, self.params, self.engine.device)
         if recorder is not None:
             recorder.begin_step()
         output = self.engine.run_reserved(entries, device_tokens)
         flight.logits = output.logits
-        if output.logits is not None and recorder is None and self.logit_observer is None \
-                and not any(e.request in self.controllers for e in plan):
-            flight.picked = choose_on_device(output.logits, plan, self.params)
+        if output.logits is not None and choice is not None:
+            flight.picked = choice.choose(output.logits)
             if flight.picked is not None:
                 # The copy to the host is asked for now, behind the kernels that choose, and waited for by its
                 # event: a copy asked for later would queue behind whatever has been issued since (the step ahead).

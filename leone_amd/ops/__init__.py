@@ -994,20 +994,16 @@ def truncated_draw_supported(stages) -> bool:
             and stages[0][0] == "top_k" and 1 <= int(stages[0][1]) <= TOP_CANDIDATES_MAX)
 
 
-def sample_truncated(logits: torch.Tensor, draws) -> torch.Tensor:
-    """One token a row (int32 on the device) by temperature sampling with truncation stages, top-k first:
-    selection, stages and draw in one launch, nothing comes to the host.  ``draws`` holds for each row either
-    None (the row is skipped and gets -1) or (temperature, uniform value, [(stage, value), ...]) with stages
-    that ``truncated_draw_supported`` accepts.  -1 also for a row without a finite logit."""
+def truncated_table(draws, device) -> torch.Tensor:
+    """The parameters of ``sample_truncated`` on the device (one upload): ``draws`` holds for each row either None
+    (the row is skipped and gets -1) or (temperature, uniform value, [(stage, value), ...]) with stages that
+    ``truncated_draw_supported`` accepts."""
     lib = library()
     if (lib.leone_sample_truncated_stages() != TRUNCATED_STAGES or lib.leone_top_candidates_max() != TOP_CANDIDATES_MAX
             or lib.leone_sample_truncated_params() != 3 + 2 * TRUNCATED_STAGES):
         raise KernelError("the kernel library was built for another table of truncation stages")
-    rows, vocab = logits.shape
     draws = list(draws)
-    if len(draws) != rows:
-        raise KernelError(f"sample_truncated: {rows} rows of logits, {len(draws)} draws")
-    table = np.zeros((rows, 3 + 2 * TRUNCATED_STAGES), dtype=np.float64)
+    table = np.zeros((len(draws), 3 + 2 * TRUNCATED_STAGES), dtype=np.float64)
     for r, draw in enumerate(draws):
         if draw is None:
             continue
@@ -1024,7 +1020,18 @@ def sample_truncated(logits: torch.Tensor, draws) -> torch.Tensor:
         for s, (name, value) in enumerate(stages):
             # top-k beyond every vocabulary keeps everything: the value only has to stay a number the kernel can compare
             table[r, 3 + 2 * s], table[r, 4 + 2 * s] = TRUNCATION_KINDS[name], min(float(value), 2.0 ** 31)
-    params = torch.from_numpy(table).to(logits.device)
+    return torch.from_numpy(table).to(device)
+
+
+def sample_truncated(logits: torch.Tensor, draws) -> torch.Tensor:
+    """One token a row (int32 on the device) by temperature sampling with truncation stages, top-k first:
+    selection, stages and draw in one launch, nothing comes to the host.  ``draws``: what ``truncated_table``
+    takes, or the table it made (float64 on the device).  -1 for a skipped row and for a row without a finite
+    logit."""
+    rows, vocab = logits.shape
+    params = draws if isinstance(draws, torch.Tensor) else truncated_table(draws, logits.device)
+    if params.shape != (rows, 3 + 2 * TRUNCATED_STAGES):
+        raise KernelError(f"sample_truncated: {rows} rows of logits, a table of {tuple(params.shape)}")
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
     call("leone_sample_truncated", _dev(logits, "sample logits", torch.float32),
          _dev(params, "sample stages", torch.float64), _dev(out, "sample out"), rows, vocab, _stream())
