@@ -196,18 +196,18 @@ temperature_pick_kernel(const float* __restrict__ logits, const double* __restri
     }
 }
 
-// ---- the best k logits of a row, for the host sampler ---------------------------------------------------
+// ---- the best k logits of a row ---------------------------------------------------------------------------
 //
 // The sampler's order (crates/leone/src/sampler.rs:502-534): finite logits only, the higher first, the
 // lower id on a tie.  A logit and its id become one 64-bit key whose unsigned order is that order
-// (0 for a value that is not finite, behind every finite one), so that selection is a sort of integers.
+// (0 for a value that is not finite, behind every finite one), so that selection is a matter of integers.
 //
-// One workgroup a row.  Every thread finds the best key among the ids it owns (four neighbours out of every 4,096),
-// four neighbouring threads make a cell; the k-th best of the 256 cells' keys is a bound that the row's k-th best
-// key cannot lie behind.  A second walk
-// collects every key not behind the bound (for k <= 256 and a vocabulary of 150,000 a few hundred), the
-// collection is sorted and its first k keys are the result.  A row whose collection would not fit
-// (values arranged against the deal) is selected key by key instead.
+// One workgroup a row.  Every thread finds the best among the ids it owns (four neighbours out of every
+// 4,096), four neighbouring threads make a cell; the k-th best of the 256 cells' keys is a bound that the
+// row's k-th best key cannot lie behind.  A second walk collects every key not behind the bound (for
+// k <= 256 and a vocabulary of 150,000 a few hundred), every collected key finds its place by counting the
+// keys before it, and the first k places are the result.  A row whose collection would not fit (values
+// arranged against the deal of ids to cells) is selected key by key instead.
 constexpr int kCandidateMaxK = 256;
 constexpr int kCandidateRoom = 4096;
 constexpr int kCellThreads = 4;                              // threads whose ids make one cell
@@ -558,7 +558,7 @@ extern "C" int leone_top_candidates_max() { return kCandidateMaxK; }
 extern "C" int leone_top_candidates(const float* logits, float* out_values, int* out_ids, int* out_count, int rows,
                                     int vocab, int wanted, hipStream_t stream) {
     LEONE_REQUIRE(logits && out_values && out_ids && out_count, "top_candidates: null pointer");
-    LEONE_REQUIRE(rows > 0 && vocab > 0, "top_candidates: rows %d vocab %d must be positive", rows, vocab);
+    LEONE_REQUIRE(rows > 0 && vocab > 0 && vocab <= (1 << 30), "top_candidates: rows %d vocab %d out of range", rows, vocab);
     LEONE_REQUIRE(wanted >= 1 && wanted <= kCandidateMaxK,
                   "top_candidates: %d wanted, at most %d can be selected", wanted, kCandidateMaxK);
     top_candidates_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, wanted, out_values, out_ids, out_count, vocab);
@@ -577,7 +577,7 @@ extern "C" int leone_sample_truncated_params() { return kDrawParams; }
 extern "C" int leone_sample_truncated(const float* logits, const double* params, int* out, int rows, int vocab,
                                       hipStream_t stream) {
     LEONE_REQUIRE(logits && params && out, "sample_truncated: null pointer");
-    LEONE_REQUIRE(rows > 0 && vocab > 0, "sample_truncated: rows %d vocab %d must be positive", rows, vocab);
+    LEONE_REQUIRE(rows > 0 && vocab > 0 && vocab <= (1 << 30), "sample_truncated: rows %d vocab %d out of range", rows, vocab);
     sample_truncated_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, params, out, vocab);
     LEONE_LAUNCH_CHECK("sample_truncated");
     return 0;
