@@ -177,12 +177,12 @@ def time_decode(engine, batch: int, start_context: int, steps: int, warmup: int,
     return (elapsed, mean_context, profiled) if profile_steps else (elapsed, mean_context)
 
 
-def time_generate(engine, batch: int, prompt_tokens: int, new_tokens: int, seed: int = 3) -> dict:
+def time_generate(engine, batch: int, prompt_tokens: int, new_tokens: int, seed: int = 3, sampling=None) -> dict:
     """The stated workload through the generation loop itself, as the reference's bench runs it (prefill the
     prompt, sample, then time decoding: crates/leone/src/runtime.rs:2006-2050): ``batch`` prompts of
     ``prompt_tokens`` random tokens are submitted to a ``Generator`` (scheduler, real prefill a whole prompt a
     step, pages taken as tokens arrive, greedy choice on the device, tokens reported back), ``new_tokens``
-    tokens each.  Timed, on the wall clock around ``Generator.step`` (planning, the step, sampling, the copy of
+    tokens each (``sampling``: another policy than greedy for all of them).  Timed, on the wall clock around ``Generator.step`` (planning, the step, sampling, the copy of
     the tokens, completion), are the steps that hold one decoded token of every request and nothing else: the
     same work as the bare step loop of ``time_decode`` plus everything the loop leaves out."""
     import torch
@@ -196,7 +196,7 @@ def time_generate(engine, batch: int, prompt_tokens: int, new_tokens: int, seed:
                              max_step_tokens=prompt_tokens + 256 * -(-batch // 256))
     generator = Generator(engine, policy)
     for i, prompt in enumerate(prompts):
-        generator.submit(("generate", i), prompt, new_tokens, SamplingParams(), None)
+        generator.submit(("generate", i), prompt, new_tokens, sampling or SamplingParams(), None)
     seconds, tokens, steps, total_started = 0.0, 0, 0, time.perf_counter()
     while generator.scheduler.has_work():
         before = (generator.stats.decode_tokens, generator.stats.prefill_tokens)
@@ -472,6 +472,11 @@ def main(argv: Optional[List[str]] = None) -> int:
         for batch in sorted({1, args.batch, 64}):
             run = time_generate(engine, batch, STATED_PROMPT, STATED_NEW)
             points[f"generate_b{batch}"] = round(run["tok_s"], 2)
+        # and with a sampler that cuts: temperature 0.8, the 40 best, then 0.9 of their mass (chosen on the device)
+        from .sampling.sampler import SamplingParams
+        cut = SamplingParams(temperature=0.8, truncations=[("top_k", 40.0), ("top_p", 0.9)], seed=11)
+        run = time_generate(engine, args.batch, STATED_PROMPT, STATED_NEW, sampling=cut)
+        points[f"generate_b{args.batch}_top_k40_top_p0.9"] = round(run["tok_s"], 2)
     # A second engine, built for the model's whole context: decoding at context 32,768, decoding a short
     # context on an engine that could hold 40,960 positions (recordings are per context range), a long prompt.
     if not (args.no_points or args.no_long) and config.max_position_embeddings >= 32768 + 64:

@@ -10,6 +10,7 @@ import time
 from dataclasses import dataclass
 from typing import Callable, Dict, Hashable, List, Optional, Sequence, Union
 
+import numpy as np
 import torch
 
 from .. import ops
@@ -76,19 +77,46 @@ class DeviceChoice:
     its ``device_kind`` or None; rows with None get nothing of meaning."""
 
     def __init__(self, rows: Sequence[PlannedEntry], policies: Sequence[SamplingParams],
-                 kinds: Sequence[Optional[str]], device):
+                 kinds: Sequence[Optional[str]], device, staging: Optional[Callable[[int], torch.Tensor]] = None):
+        """``staging(n)``: pinned host memory for n float64 values that stays untouched until the upload has
+        happened; the upload then waits for nothing and holds nobody up (a copy out of ordinary memory makes the
+        host wait for everything the stream still has to do: the step in flight)."""
         self.kinds = list(kinds)
+        count = len(rows)
         draws = [rng.uniform(p.seed, e.sample_position) if kind in ("temperature", "truncated") else 0.0
                  for p, e, kind in zip(policies, rows, kinds)]
-        self.scaled = self.truncated = None
+        pieces = []
         if "temperature" in kinds:
-            self.scaled = torch.tensor([[p.temperature if kind == "temperature" else 1.0 for p, kind in zip(policies, kinds)],
-                                        draws], dtype=torch.float64).to(device)
+            pieces.append(np.array([[p.temperature if kind == "temperature" else 1.0 for p, kind in zip(policies, kinds)],
+                                    draws], dtype=np.float64).reshape(-1))
         if "truncated" in kinds:
-            self.truncated = ops.truncated_table([(p.temperature, u, p.truncations) if kind == "truncated" else None
-                                                  for p, u, kind in zip(policies, draws, kinds)], device)
+            pieces.append(ops.truncated_rows([(p.temperature, u, p.truncations) if kind == "truncated" else None
+                                              for p, u, kind in zip(policies, draws, kinds)]).reshape(-1))
+        # which rows take the answer of the second and third kernel (a batch of one kind needs none)
         self.names = [name for name in ("greedy", "temperature", "truncated") if name in kinds]
-        self.masks = {name: torch.tensor([kind == name for kind in kinds], device=device) for name in self.names[1:]}
+        for name in self.names[1:]:
+            pieces.append(np.array([1.0 if kind == name else 0.0 for kind in kinds], dtype=np.float64))
+        self.scaled = self.truncated = None
+        self.masks = {}
+        if pieces:
+            flat = np.concatenate(pieces)
+            if staging is not None:
+                host = staging(flat.size)
+                host.numpy()[:] = flat
+                on_device = host.to(device, non_blocking=True)
+            else:
+                on_device = torch.from_numpy(flat).to(device)
+            at = 0
+            if "temperature" in kinds:
+                self.scaled = on_device[:2 * count].view(2, count)
+                at = 2 * count
+            if "truncated" in kinds:
+                width = 3 + 2 * ops.TRUNCATED_STAGES
+                self.truncated = on_device[at:at + count * width].view(count, width)
+                at += count * width
+            for name in self.names[1:]:
+                self.masks[name] = on_device[at:at + count] != 0.0
+                at += count
 
     def choose(self, logits: torch.Tensor) -> torch.Tensor:
         """int32 [rows] on the device: the token each row's kernel chose, -1 for a row without a finite logit.
@@ -105,8 +133,8 @@ class DeviceChoice:
         return out
 
 
-def plan_device_choice(entries: Sequence[PlannedEntry], params: Dict[Hashable, SamplingParams],
-                       device) -> Optional[DeviceChoice]:
+def plan_device_choice(entries: Sequence[PlannedEntry], params: Dict[Hashable, SamplingParams], device,
+                       staging: Optional[Callable[[int], torch.Tensor]] = None) -> Optional[DeviceChoice]:
     """The ``DeviceChoice`` of a step if device kernels choose every one of its tokens; None otherwise."""
     rows = [e for e in entries if e.sample]
     policies = [params[e.request] or SamplingParams() for e in rows]
@@ -115,7 +143,7 @@ def plan_device_choice(entries: Sequence[PlannedEntry], params: Dict[Hashable, S
     kinds = [device_kind(p) for p in policies]
     if not rows or not all(kinds):
         return None
-    return DeviceChoice(rows, policies, kinds, device)
+    return DeviceChoice(rows, policies, kinds, device, staging)
 
 
 def choose_tokens(logits: torch.Tensor, entries: Sequence[PlannedEntry], params: Dict[Hashable, SamplingParams],
@@ -217,6 +245,8 @@ class Generator:
         self._last_finish = 0.0
         self._token_buffers: List[Optional[torch.Tensor]] = [None, None, None]
         self._token_turn = 0
+        self._choice_buffers: List[Optional[torch.Tensor]] = [None, None, None]
+        self._choice_turn = 0
 
     def submit(self, request_id: Hashable, prompt: Sequence[int], max_new_tokens: int,
                sampling: Optional[SamplingParams] = None, eos_token_id: Optional[int] = None) -> None:
@@ -245,7 +275,7 @@ class Generator:
         # What the kernels that choose the tokens need goes to the device before the step, not between the two.
         choice = None
         if recorder is None and self.logit_observer is None and not any(e.request in self.controllers for e in plan):
-            choice = plan_device_choice(plan, self.params, self.engine.device)
+            choice = plan_device_choice(plan, self.params, self.engine.device, self._choice_buffer)
         if recorder is not None:
             recorder.begin_step()
         output = self.engine.run_reserved(entries, device_tokens)
@@ -260,6 +290,15 @@ class Generator:
                 flight.arrived = torch.cuda.Event()
                 flight.arrived.record()
         return flight
+
+    def _choice_buffer(self, count: int) -> torch.Tensor:
+        """Pinned host memory for what one step's choosing kernels are given; three take turns, as for the tokens:
+        by the time a buffer's turn comes again, the step it served has been concluded."""
+        self._choice_turn = (self._choice_turn + 1) % 3
+        held = self._choice_buffers[self._choice_turn]
+        if held is None or held.numel() < count:
+            held = self._choice_buffers[self._choice_turn] = torch.empty(max(count, 256), dtype=torch.float64).pin_memory()
+        return held[:count]
 
     def _token_buffer(self, count: int) -> torch.Tensor:
         """Pinned host memory for one step's chosen tokens; three take turns (a step, the one ahead of it, and one

@@ -994,10 +994,10 @@ def truncated_draw_supported(stages) -> bool:
             and stages[0][0] == "top_k" and 1 <= int(stages[0][1]) <= TOP_CANDIDATES_MAX)
 
 
-def truncated_table(draws, device) -> torch.Tensor:
-    """The parameters of ``sample_truncated`` on the device (one upload): ``draws`` holds for each row either None
-    (the row is skipped and gets -1) or (temperature, uniform value, [(stage, value), ...]) with stages that
-    ``truncated_draw_supported`` accepts."""
+def truncated_rows(draws) -> np.ndarray:
+    """The parameters of ``sample_truncated`` as a host array, float64 [rows, 3 + 2 * TRUNCATED_STAGES]: ``draws``
+    holds for each row either None (the row is skipped and gets -1) or (temperature, uniform value,
+    [(stage, value), ...]) with stages that ``truncated_draw_supported`` accepts."""
     lib = library()
     if (lib.leone_sample_truncated_stages() != TRUNCATED_STAGES or lib.leone_top_candidates_max() != TOP_CANDIDATES_MAX
             or lib.leone_sample_truncated_params() != 3 + 2 * TRUNCATED_STAGES):
@@ -1020,7 +1020,12 @@ def truncated_table(draws, device) -> torch.Tensor:
         for s, (name, value) in enumerate(stages):
             # top-k beyond every vocabulary keeps everything: the value only has to stay a number the kernel can compare
             table[r, 3 + 2 * s], table[r, 4 + 2 * s] = TRUNCATION_KINDS[name], min(float(value), 2.0 ** 31)
-    return torch.from_numpy(table).to(device)
+    return table
+
+
+def truncated_table(draws, device) -> torch.Tensor:
+    """``truncated_rows`` on the device."""
+    return torch.from_numpy(truncated_rows(draws)).to(device)
 
 
 def sample_truncated(logits: torch.Tensor, draws) -> torch.Tensor:

@@ -44,6 +44,7 @@ def test_the_record_of_a_short_run(capsys):
     # the stated workload as a bare step loop and through the generation loop, and the second engine's points
     for batch in (1, 8, 64):
         assert {f"decode_b{batch}_prompt2048_new256", f"generate_b{batch}"} <= set(record["points"])
+    assert "generate_b8_top_k40_top_p0.9" in record["points"]
     assert {"decode_b1_context32768", "decode_b8_context32768", "decode_b1_context512_of_40960",
             "decode_b8_context512_of_40960", "prefill_8192"} <= set(record["points"])
 
